@@ -1,0 +1,219 @@
+"""ctypes view of the CPU oracle (oracle/libkvoracle.so) — TEST INFRASTRUCTURE, NOT PRODUCT.
+
+Only the tests, the smoke check and the benchmark's CPU-baseline leg import this module. The
+shipped package (rivoli_amd) never does. Arrays cross as numpy; every function mirrors one in
+kvcache_oracle.h, which carries the reference citations.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libkvoracle.so")
+REF_LIB_PATH = os.path.join(HERE, "_ref", "librivoli_ref_kernels.so")
+
+
+def build(with_ref: bool = True) -> None:
+    """Compile the oracle; also the reference's own launchers when its tree is mounted."""
+    subprocess.run(["make", "-C", HERE, "-B", "all"], check=True)
+    if with_ref and os.path.isdir("/root/reference/crates/backend/kernels"):
+        subprocess.run(["make", "-C", HERE, "-B", "ref"], check=True)
+
+
+def _ptr(a: np.ndarray, ctype):
+    return a.ctypes.data_as(C.POINTER(ctype))
+
+
+def _c(a, dtype) -> np.ndarray:
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+class Oracle:
+    def __init__(self, path: str = LIB_PATH):
+        if not os.path.exists(path):
+            build(with_ref=False)
+        self.lib = lib = C.CDLL(path)
+        u8p, u16p, u32p = C.POINTER(C.c_uint8), C.POINTER(C.c_uint16), C.POINTER(C.c_uint32)
+        i32p, f32p = C.POINTER(C.c_int32), C.POINTER(C.c_float)
+        sig = {
+            "ro_f32_to_e4m3": (C.c_uint8, [C.c_float]),
+            "ro_e4m3_to_f32": (C.c_float, [C.c_uint8]),
+            "ro_f32_to_bf16": (C.c_uint16, [C.c_float]),
+            "ro_bf16_to_f32": (C.c_float, [C.c_uint16]),
+            "ro_f32_to_e4m3_n": (None, [f32p, u8p, C.c_size_t]),
+            "ro_e4m3_to_f32_n": (None, [u8p, f32p, C.c_size_t]),
+            "ro_f32_to_bf16_n": (None, [f32p, u16p, C.c_size_t]),
+            "ro_selftest_bf16_exhaustive": (C.c_uint64, []),
+            "ro_lcg_f": (C.c_float, [C.POINTER(C.c_uint64)]),
+            "ro_lcg_fill": (None, [C.POINTER(C.c_uint64), f32p, C.c_size_t]),
+            "ro_quant_block": (None, [f32p, C.c_int, u8p, f32p]),
+            "ro_append_kv": (C.c_int, [f32p, f32p, u8p, f32p, u16p] + [C.c_int] * 4),
+            "ro_index_append": (C.c_int, [f32p, u16p, C.c_int, C.c_int]),
+            "ro_kv_page_bytes": (C.c_size_t, [C.c_int, C.c_int]),
+            "ro_kv_append_paged": (C.c_int, [u16p, i32p, u8p] + [C.c_int] * 4),
+            "ro_kv_append_paged_mt": (None, [u16p, i32p, u8p] + [C.c_int] * 5),
+            "ro_kv_gather_paged": (None, [u8p, i32p, i32p, i32p, u16p] + [C.c_int] * 4),
+            "ro_kv_gather_paged_mt": (None, [u8p, i32p, i32p, i32p, u16p] + [C.c_int] * 5),
+            "ro_kv_gather_rows_paged": (None, [u8p, i32p, u32p, i32p, u16p] + [C.c_int] * 5),
+            "ro_topk": (C.c_int, [f32p, C.c_int, C.c_int, u32p]),
+            "ro_topk_batched": (None, [f32p, C.c_int, C.c_int, i32p, C.c_int, C.c_int, u32p, C.c_int]),
+            "ro_fnv1a": (C.c_uint64, [u8p, C.c_size_t]),
+            "ro_splitmix_finalize": (C.c_uint64, [C.c_uint64]),
+            "ro_xor_fold": (C.c_uint64, [u32p, C.c_size_t, C.c_uint64, C.c_size_t]),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+
+    # ---- codecs -------------------------------------------------------------------------
+    def f32_to_e4m3(self, x) -> np.ndarray:
+        x = _c(x, np.float32)
+        out = np.empty(x.shape, np.uint8)
+        self.lib.ro_f32_to_e4m3_n(_ptr(x, C.c_float), _ptr(out, C.c_uint8), x.size)
+        return out
+
+    def e4m3_to_f32(self, c) -> np.ndarray:
+        c = _c(c, np.uint8)
+        out = np.empty(c.shape, np.float32)
+        self.lib.ro_e4m3_to_f32_n(_ptr(c, C.c_uint8), _ptr(out, C.c_float), c.size)
+        return out
+
+    def f32_to_bf16(self, x) -> np.ndarray:
+        x = _c(x, np.float32)
+        out = np.empty(x.shape, np.uint16)
+        self.lib.ro_f32_to_bf16_n(_ptr(x, C.c_float), _ptr(out, C.c_uint16), x.size)
+        return out
+
+    def selftest_bf16_exhaustive(self) -> int:
+        return int(self.lib.ro_selftest_bf16_exhaustive())
+
+    # ---- the reference tests' input stream ----------------------------------------------
+    def lcg(self, seed: int) -> "Lcg":
+        return Lcg(self, seed)
+
+    # ---- quantization -------------------------------------------------------------------
+    def quant_block(self, v):
+        v = _c(v, np.float32).ravel()
+        codes = np.empty(v.size, np.uint8)
+        scale = C.c_float()
+        self.lib.ro_quant_block(_ptr(v, C.c_float), v.size, _ptr(codes, C.c_uint8), C.byref(scale))
+        return codes, np.float32(scale.value)
+
+    def append_kv(self, latent, rope, lc8, lscale, rc, pos, kvl, ropn, n_blocks) -> int:
+        latent, rope = _c(latent, np.float32), _c(rope, np.float32)
+        return int(self.lib.ro_append_kv(
+            _ptr(latent, C.c_float), _ptr(rope, C.c_float), _ptr(lc8, C.c_uint8),
+            _ptr(lscale, C.c_float), _ptr(rc, C.c_uint16), pos, kvl, ropn, n_blocks))
+
+    def index_append(self, k, kcache, pos, hd) -> int:
+        k = _c(k, np.float32)
+        return int(self.lib.ro_index_append(_ptr(k, C.c_float), _ptr(kcache, C.c_uint16), pos, hd))
+
+    # ---- paged cache --------------------------------------------------------------------
+    def kv_page_bytes(self, page_tokens: int, width: int) -> int:
+        return int(self.lib.ro_kv_page_bytes(page_tokens, width))
+
+    def kv_append_paged(self, rows_bf16, slot_mapping, pool, width, page_tokens, n_pages,
+                        n_threads: int = 0) -> int:
+        rows_bf16, slot_mapping = _c(rows_bf16, np.uint16), _c(slot_mapping, np.int32)
+        assert pool.dtype == np.uint8 and pool.flags.c_contiguous
+        n = slot_mapping.size
+        if n_threads > 0:
+            self.lib.ro_kv_append_paged_mt(_ptr(rows_bf16, C.c_uint16), _ptr(slot_mapping, C.c_int32),
+                                           _ptr(pool, C.c_uint8), n, width, page_tokens, n_pages,
+                                           n_threads)
+            return 0
+        return int(self.lib.ro_kv_append_paged(_ptr(rows_bf16, C.c_uint16),
+                                               _ptr(slot_mapping, C.c_int32),
+                                               _ptr(pool, C.c_uint8), n, width, page_tokens,
+                                               n_pages))
+
+    def kv_gather_paged(self, pool, block_table, seq_lens, width, page_tokens,
+                        n_threads: int = 0, out=None) -> np.ndarray:
+        block_table, seq_lens = _c(block_table, np.int32), _c(seq_lens, np.int32)
+        n_seqs, max_blocks = block_table.shape
+        cu = np.zeros(n_seqs + 1, np.int32)
+        np.cumsum(seq_lens, out=cu[1:])
+        if out is None:
+            out = np.zeros((int(cu[-1]), width), np.uint16)
+        args = (_ptr(pool, C.c_uint8), _ptr(block_table, C.c_int32), _ptr(seq_lens, C.c_int32),
+                _ptr(cu, C.c_int32), _ptr(out, C.c_uint16), n_seqs, max_blocks, width, page_tokens)
+        if n_threads > 0:
+            self.lib.ro_kv_gather_paged_mt(*args, n_threads)
+        else:
+            self.lib.ro_kv_gather_paged(*args)
+        return out
+
+    def kv_gather_rows_paged(self, pool, block_table, rows, width, page_tokens,
+                             n_rows=None) -> np.ndarray:
+        block_table, rows = _c(block_table, np.int32), _c(rows, np.uint32)
+        n_q, max_blocks = block_table.shape
+        k = rows.shape[1]
+        out = np.zeros((n_q, k, width), np.uint16)
+        nr = None if n_rows is None else _c(n_rows, np.int32)
+        self.lib.ro_kv_gather_rows_paged(
+            _ptr(pool, C.c_uint8), _ptr(block_table, C.c_int32), _ptr(rows, C.c_uint32),
+            None if nr is None else _ptr(nr, C.c_int32), _ptr(out, C.c_uint16), n_q, k,
+            max_blocks, width, page_tokens)
+        return out
+
+    # ---- selection ----------------------------------------------------------------------
+    def topk(self, scores, k: int) -> np.ndarray:
+        scores = _c(scores, np.float32).ravel()
+        rows = np.empty(max(min(k, scores.size), 0), np.uint32)
+        n = self.lib.ro_topk(_ptr(scores, C.c_float), scores.size, k, _ptr(rows, C.c_uint32))
+        return rows[:n]
+
+    def topk_batched(self, scores, k: int, nts=None, n_threads: int = 1) -> np.ndarray:
+        scores = _c(scores, np.float32)
+        n_q, stride = scores.shape
+        rows = np.full((n_q, k), 0xFFFFFFFF, np.uint32)
+        nt_arr = None if nts is None else _c(nts, np.int32)
+        self.lib.ro_topk_batched(_ptr(scores, C.c_float), n_q, stride,
+                                 None if nt_arr is None else _ptr(nt_arr, C.c_int32), stride, k,
+                                 _ptr(rows, C.c_uint32), n_threads)
+        return rows
+
+    # ---- content pinning ----------------------------------------------------------------
+    def fnv1a(self, data: bytes) -> int:
+        buf = np.frombuffer(data, np.uint8) if len(data) else np.zeros(0, np.uint8)
+        return int(self.lib.ro_fnv1a(_ptr(buf, C.c_uint8) if buf.size else None, buf.size))
+
+    def splitmix_finalize(self, z: int) -> int:
+        return int(self.lib.ro_splitmix_finalize(C.c_uint64(z)))
+
+    def xor_fold(self, buf, i_base: int = 0, stride: int = 1) -> int:
+        """Fold over the buffer's 32-bit words (its byte length must be a multiple of 4)."""
+        words = np.ascontiguousarray(buf).view(np.uint8).ravel().view(np.uint32)
+        return int(self.lib.ro_xor_fold(_ptr(words, C.c_uint32), words.size, i_base, stride))
+
+
+class Lcg:
+    """crates/engine/tests/common/reference.rs:141-162 — uniform in [-1, 1)."""
+
+    def __init__(self, oracle: Oracle, seed: int):
+        self._o = oracle
+        self._state = C.c_uint64(seed)
+
+    def f(self) -> np.float32:
+        return np.float32(self._o.lib.ro_lcg_f(C.byref(self._state)))
+
+    def fill(self, n: int) -> np.ndarray:
+        out = np.empty(n, np.float32)
+        self._o.lib.ro_lcg_fill(C.byref(self._state), _ptr(out, C.c_float), n)
+        return out
+
+
+_ORACLE = None
+
+
+def oracle() -> Oracle:
+    global _ORACLE
+    if _ORACLE is None:
+        _ORACLE = Oracle()
+    return _ORACLE
