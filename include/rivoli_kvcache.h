@@ -1,0 +1,129 @@
+/* rivoli fp8 MLA KV-cache hot path for gfx950 (MI355X) — C ABI.
+ *
+ * The entry points below are what rivoli's backend FFI binds for this path. They follow the
+ * house launcher convention (crates/backend/kernels/fwd.hip:1-4, crates/backend/src/hip.rs:
+ * 328-336): return 0 on success, a POSITIVE argument-guard code when the call is refused
+ * before anything is launched (1001 non-positive / null argument, 1002 size bound,
+ * 1004 divisibility), or -(int)hipError_t from the launch. Launch-only: no allocation, no
+ * copy, no synchronisation. Every pointer is a device pointer owned by the caller and must
+ * stay live until `stream` (nullptr = the null stream) has drained. Dims cross as int
+ * (the Rust side narrows usize as i32); all byte offsets are formed in 64 bits inside.
+ *
+ * Paged cache layout ("page"): page_tokens rows of `width` e4m3 codes, then page_tokens f32
+ * scales — rivoli_kv_page_bytes(page_tokens, width) bytes, one scale per token (the whole
+ * row is one quantization block). A pool is n_pages such pages, contiguous.
+ * slot = page * page_tokens + offset_in_page.
+ */
+#ifndef RIVOLI_KVCACHE_H
+#define RIVOLI_KVCACHE_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------
+ * Entry points that keep a reference signature byte for byte (drop-in for gfx950)
+ * ---------------------------------------------------------------------------------------- */
+
+/* Replaces crates/backend/kernels/fwd.hip:224-235 (Rust: launch_append_kv,
+ * crates/backend/src/hip_attn.rs:137-147). One token into the LINEAR slabs at row `pos`:
+ * latent as e4m3 with one f32 scale per 128 values, roped key as bf16. Null stream.
+ * Guards: 1001 pos<0 or a non-positive dim; 1002 kvl not a multiple of 128 in [128,1024]
+ * or ropn > kvl. */
+int rivoli_append_kv(const float* latent, const float* rope, unsigned char* lc8, float* lscale,
+                     unsigned short* rc, int pos, int kvl, int ropn, int n_blocks);
+
+/* Replaces crates/backend/kernels/indexer.hip:268-276 (launch_index_append,
+ * crates/backend/src/hip_attn.rs:450-455): kcache[pos*hd + i] = bf16(k[i]). */
+int rivoli_index_append(const float* k, unsigned short* kcache, int pos, int hd);
+
+/* Replaces crates/backend/kernels/indexer.hip:327-335 (launch_index_topk,
+ * crates/backend/src/hip_attn.rs:490-495): rows[0..min(k,nt)) = the k best-scoring token
+ * indices (score descending, ties to the lowest index, -0.0 == +0.0), emitted ASCENDING.
+ * Entries past min(k,nt) are not written. Guard 1001: nt<=0 or k<=0. Null stream. */
+int rivoli_index_topk(const float* scores, int nt, int k, unsigned int* rows);
+
+/* Replaces crates/backend/kernels/fwd.hip:411-427 (launch_hash_rows,
+ * crates/backend/src/hip.rs:581-603): XOR-folds splitmix64(((i_base+i)<<32) ^ bits(x[i]))
+ * over i = 0, stride, 2*stride, ... < n INTO *out (the caller zeroes it). */
+int rivoli_hash_rows(const float* x, int n, int stride, unsigned long long i_base,
+                     unsigned long long* out, void* stream);
+
+/* Replaces crates/backend/src/hip.rs:339-342's rivoli_device_sync: hipDeviceSynchronize. */
+int rivoli_device_sync(void);
+
+/* ------------------------------------------------------------------------------------------
+ * New entry points (same convention, trailing stream): the paged, batched path
+ * ---------------------------------------------------------------------------------------- */
+
+/* Pure function, like rivoli_mla_attend_scratch_floats (crates/backend/kernels/attn.hip:
+ * 100-103): bytes of one page. 64 x 576 -> 37120. */
+size_t rivoli_kv_page_bytes(int page_tokens, int width);
+
+/* Quantize-and-append (the paged, many-token form of append_kv, crates/backend/kernels/
+ * fwd.hip:51-71 with the block widened to the whole row): for each token t < n_tokens,
+ * rows[t*width .. +width) (bf16) -> amax, scale = amax>0 ? amax/448 : 1, codes =
+ * e4m3(v/scale), stored at slot_mapping[t]. A negative slot skips the token (padding). A
+ * slot >= n_pages*page_tokens is never written; it is counted in *bad_slots when that
+ * pointer is non-null.
+ * Guards: 1001 null pointer / non-positive dim; 1002 width > 1024; 1004 width % 16 or
+ * page_tokens % 4. */
+int rivoli_kv_append_paged(const unsigned short* rows, const int* slot_mapping,
+                           unsigned char* pool, int n_tokens, int width, int page_tokens,
+                           int n_pages, unsigned int* bad_slots, void* stream);
+
+/* Linear-slab append of n_tokens consecutive rows starting at pos0 — rivoli_append_kv for a
+ * prefill chunk in ONE launch and on a stream (the reference loops rows on the host,
+ * crates/engine/src/glm/attn.rs:135-160). latent is [n_tokens][kvl] f32, rope
+ * [n_tokens][ropn] f32. Same guards as rivoli_append_kv plus 1001 for n_tokens <= 0. */
+int rivoli_append_kv_rows(const float* latent, const float* rope, unsigned char* lc8,
+                          float* lscale, unsigned short* rc, int pos0, int n_tokens, int kvl,
+                          int ropn, int n_blocks, void* stream);
+
+/* Block-table gather + dequantize (the tile load of mla_latent_attend with rows == null,
+ * crates/backend/kernels/attn.hip:168-177, materialised): for each sequence s < n_seqs and
+ * t < seq_lens[s]:
+ *   out[(cu_seqlens[s] + t)*width + i] = bf16(e4m3_to_f32(code) * scale)
+ * where the token lives in page block_table[s*max_blocks_per_seq + t/page_tokens].
+ * cu_seqlens has n_seqs+1 entries (exclusive prefix sum of seq_lens, in tokens). A page id
+ * outside [0, n_pages) is skipped and counted in *bad_pages when non-null.
+ * Guards: 1001, 1004 as above. */
+int rivoli_kv_gather_paged(const unsigned char* pool, const int* block_table,
+                           const int* seq_lens, const int* cu_seqlens, unsigned short* out,
+                           int n_seqs, int max_blocks_per_seq, int width, int page_tokens,
+                           int n_pages, unsigned int* bad_pages, void* stream);
+
+/* Sparse row gather + dequantize (the `rows` argument of rivoli_mla_attend,
+ * crates/backend/kernels/attn.hip:125,175): for query q < n_queries and j < n_rows[q]
+ * (k when n_rows is null): out[(q*k + j)*width ..] = dequantized token rows[q*k + j] of
+ * sequence q. Row indices >= max_blocks_per_seq*page_tokens or pages outside the pool are
+ * skipped and counted in *bad_rows when non-null. */
+int rivoli_kv_gather_rows_paged(const unsigned char* pool, const int* block_table,
+                                const unsigned int* rows, const int* n_rows,
+                                unsigned short* out, int n_queries, int k,
+                                int max_blocks_per_seq, int width, int page_tokens, int n_pages,
+                                unsigned int* bad_rows, void* stream);
+
+/* Batched rivoli_index_topk: query q reads scores[q*stride .. +nts[q]) (nt for every query
+ * when nts is null) and writes rows[q*k .. +min(k, nt_q)), ascending. One launch for all
+ * queries; the selection rule is the single-query one.
+ * Guards: 1001 null / non-positive; 1002 stride < nt. */
+int rivoli_index_topk_batched(const float* scores, int n_queries, int stride, const int* nts,
+                              int nt, int k, unsigned int* rows, void* stream);
+
+/* Element codecs as launchers (what formats.hpp:42-57,99-106 and fwd.hip:20-45 are to the
+ * reference's kernels), for census tests of the device codecs on arbitrary inputs:
+ *   e4m3_encode: out[i] = f32_to_e4m3(x[i])            (rule of crates/core/src/num.rs:128-152)
+ *   e4m3_dequant_bf16: out[i] = bf16(e4m3_to_f32(c[i]) * scale)
+ *   bf16_encode: out[i] = f32_to_bf16(x[i]) */
+int rivoli_codec_e4m3_encode(const float* x, unsigned char* out, long long n, void* stream);
+int rivoli_codec_e4m3_dequant_bf16(const unsigned char* codes, float scale, unsigned short* out,
+                                   long long n, void* stream);
+int rivoli_codec_bf16_encode(const float* x, unsigned short* out, long long n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,62 @@
+"""Builds the HIP library in-tree: rivoli_amd/csrc/*.hip -> rivoli_amd/csrc/librivoli_kvcache.so.
+
+Mirrors how the reference builds its kernels (crates/backend/build.rs:103-183: hipcc,
+--offload-arch from the environment, -O3 -fPIC, link amdhip64), except that the default
+architecture here is gfx950 and the product is one shared library behind a C ABI.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIB_PATH = os.path.join(CSRC, "librivoli_kvcache.so")
+HOST_LIB_PATH = os.path.join(CSRC, "librivoli_pagepool.so")
+KERNELS = ["kv_append.hip", "kv_gather.hip", "index_topk.hip", "hash_rows.hip"]
+HOST_SOURCES = ["pagepool.cpp"]
+
+
+def hipcc() -> str:
+    return os.environ.get("HIPCC", "hipcc")
+
+
+def offload_arch() -> str:
+    return os.environ.get("RIVOLI_OFFLOAD_ARCH", "gfx950")
+
+
+def build_kernels(verbose: bool = False) -> str:
+    cmd = [hipcc(), f"--offload-arch={offload_arch()}", "-O3", "-std=c++17", "-fPIC", "-shared",
+           # packed-f32 instructions stay off: plain f32 math only
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I", os.path.join(os.path.dirname(CSRC), "..", "include"),
+           "-o", LIB_PATH] + [os.path.join(CSRC, k) for k in KERNELS]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed building " + LIB_PATH)
+    return LIB_PATH
+
+
+def build_host(verbose: bool = False) -> str:
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
+           "-I", os.path.join(os.path.dirname(CSRC), "..", "include"),
+           "-o", HOST_LIB_PATH] + [os.path.join(CSRC, s) for s in HOST_SOURCES]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+    if res.returncode != 0:
+        raise RuntimeError("g++ failed building " + HOST_LIB_PATH)
+    return HOST_LIB_PATH
+
+
+def build_all(verbose: bool = False) -> None:
+    build_kernels(verbose)
+    build_host(verbose)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)
+    print(LIB_PATH)
+    print(HOST_LIB_PATH)

@@ -1,0 +1,99 @@
+// Device element codecs and wave64 helpers for the fp8 KV-cache kernels (gfx950 only).
+//
+// Arithmetic contract (must stay bit-identical to rivoli_core::num, crates/core/src/num.rs):
+//   * e4m3 encode: round to nearest even on normals, round HALF AWAY from zero in the
+//     subnormal band, saturate |x| >= 448 to 0x7e, |x| < 2^-10 to signed zero, NaN -> 0x7f.
+//   * e4m3 decode is exact; gfx950's v_cvt_pk_f32_fp8 decodes OCP e4m3 and is used as is.
+//   * bf16 encode is round to nearest even; gfx950's v_cvt_pk_bf16_f32 does exactly that.
+//   * scale = amax > 0 ? amax / 448 : 1 and v / scale are IEEE-correct f32 divides (hipcc's
+//     default); nothing here may be built with fast-math.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rk {
+
+constexpr int kWave = 64;
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf16_lo_to_f32(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16_hi_to_f32(uint32_t pair) {
+    return __uint_as_float(pair & 0xffff0000u);
+}
+
+// Two f32 -> two bf16 packed (lo in the low half), round to nearest even.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    bf16x2 p = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, p);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16(float x) {
+    __bf16 h = (__bf16)x;
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+// f32 -> OCP e4m3 byte, the KV-cache rule (crates/core/src/num.rs:128-182; device twin in the
+// reference at crates/backend/kernels/fwd.hip:20-45). Written as straight-line selects.
+__device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
+    uint32_t xb = __float_as_uint(x);
+    uint32_t sign = (xb >> 24) & 0x80u;
+    uint32_t ab = xb & 0x7fffffffu;
+    float a = __uint_as_float(ab);
+    // normal path: keep 3 mantissa bits, nearest even over the 20 dropped ones. Adding
+    // 0x7ffff + lsb carries into the exponent field by itself when the mantissa wraps.
+    uint32_t r = ab + 0x0007ffffu + ((ab >> 20) & 1u);
+    uint32_t normal = (r >> 20) - (120u << 3);  // exponent rebias 127 -> 7
+    // subnormal band [2^-10, 2^-6): m = floor(a*512 + 0.5); m == 8 is code 0x08 by itself.
+    uint32_t sub = (uint32_t)(a * 512.0f + 0.5f);
+    uint32_t mag = a < 0.015625f ? sub : normal;
+    mag = a < 0.0009765625f ? 0u : mag;
+    mag = a >= 448.0f ? 0x7eu : mag;  // also catches +-inf
+    uint32_t code = sign | mag;
+    return ab > 0x7f800000u ? 0x7fu : code;
+}
+
+// Four packed e4m3 codes -> four f32, exact.
+__device__ __forceinline__ void e4m3x4_to_f32(uint32_t w, float (&v)[4]) {
+    f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+    f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+    v[0] = lo.x;
+    v[1] = lo.y;
+    v[2] = hi.x;
+    v[3] = hi.y;
+}
+
+// Four packed e4m3 codes times one scale -> four bf16 in two dwords.
+__device__ __forceinline__ u32x2 dequant4_bf16(uint32_t w, float scale) {
+    float v[4];
+    e4m3x4_to_f32(w, v);
+    u32x2 r = {pack_bf16x2(v[0] * scale, v[1] * scale), pack_bf16x2(v[2] * scale, v[3] * scale)};
+    return r;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ __forceinline__ unsigned long long wave_xor(unsigned long long v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v ^= __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// Launcher epilogue shared by every entry point: 0 or -(hipError_t).
+inline int launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : -(int)e;
+}
+
+}  // namespace rk

@@ -1,0 +1,231 @@
+// Gather + dequantize: fp8 pages -> bf16 rows, dense (block table) and sparse (row list).
+//
+// The arithmetic is the tile load of the reference's attention kernel
+// (crates/backend/kernels/attn.hip:168-177): val = e4m3_to_f32(code) * scale in f32, here
+// rounded to nearest even into bf16. Both decodes are exact, the multiply is one IEEE
+// operation and the narrowing is one rounding, so the result is bit-identical to the CPU
+// rule whatever the schedule.
+//
+// Dense: one workgroup per (sequence, page). A page's codes are one contiguous run and so is
+// its destination (tokens of a page are consecutive in the output), so the kernel is a
+// streaming transform: every lane loads 8 bytes of codes (a wave covers 512 contiguous
+// bytes) and stores 16 bytes of bf16 (a wave covers 1 KiB contiguous). All of a thread's
+// loads are issued before the first use to keep enough bytes in flight for HBM.
+// Sparse: one workgroup per 32 selected rows of one query; the 32 row bases and scales are
+// resolved once into LDS (block-table lookup), then the same 8-in/16-out streaming body runs
+// over the 32 x width bytes.
+// Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
+#include "codec.hpp"
+
+namespace rk {
+
+constexpr int kGatherThreads = 256;
+constexpr int kRowsPerGroup = 32;  // sparse gather: rows resolved per workgroup
+
+__device__ __forceinline__ u32x4 dequant8_bf16(u32x2 codes, float scale) {
+    u32x2 a = dequant4_bf16(codes.x, scale);
+    u32x2 b = dequant4_bf16(codes.y, scale);
+    u32x4 r = {a.x, a.y, b.x, b.y};
+    return r;
+}
+
+// W / PT are the compile-time row width and page size (0 = take the runtime value), so the
+// flagship 576 x 64 shape gets constant divisors and a fully unrolled body.
+template <int W, int PT, int UNROLL>
+__global__ __launch_bounds__(kGatherThreads) void kv_gather_paged_kernel(
+    const uint8_t* __restrict__ pool, const int* __restrict__ block_table,
+    const int* __restrict__ seq_lens, const int* __restrict__ cu_seqlens,
+    uint16_t* __restrict__ out, int max_blocks_per_seq, int width_rt, int page_tokens_rt,
+    int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_pages) {
+    const int width = W ? W : width_rt;
+    const int pt = PT ? PT : page_tokens_rt;
+    const int s = blockIdx.y;
+    const int t0 = (int)blockIdx.x * pt;
+    const int len = seq_lens[s];
+    if (t0 >= len) return;
+    const int valid = min(pt, len - t0);
+    const int page = block_table[(size_t)s * max_blocks_per_seq + blockIdx.x];
+    if ((unsigned)page >= (unsigned)n_pages) {
+        if (threadIdx.x == 0 && bad_pages) atomicAdd(bad_pages, 1u);
+        return;
+    }
+    const uint8_t* pg = pool + (size_t)page * page_bytes;
+    const u32x2* src = reinterpret_cast<const u32x2*>(pg);
+    const float* scales = reinterpret_cast<const float*>(pg + (size_t)pt * width);
+    u32x4* dst = reinterpret_cast<u32x4*>(out + ((size_t)cu_seqlens[s] + t0) * width);
+    const int cpr = width >> 3;  // 8-byte chunks per row
+    const int n_chunks = valid * cpr;
+
+    for (int base = threadIdx.x; base < n_chunks; base += kGatherThreads * UNROLL) {
+        u32x2 raw[UNROLL];
+        float scl[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int c = base + u * kGatherThreads;
+            if (c < n_chunks) {
+                raw[u] = __builtin_nontemporal_load(src + c);
+                scl[u] = scales[c / cpr];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int c = base + u * kGatherThreads;
+            if (c < n_chunks) __builtin_nontemporal_store(dequant8_bf16(raw[u], scl[u]), dst + c);
+        }
+    }
+}
+
+template <int W, int PT, int UNROLL>
+__global__ __launch_bounds__(kGatherThreads) void kv_gather_rows_kernel(
+    const uint8_t* __restrict__ pool, const int* __restrict__ block_table,
+    const unsigned int* __restrict__ rows, const int* __restrict__ n_rows,
+    uint16_t* __restrict__ out, int k, int max_blocks_per_seq, int width_rt, int page_tokens_rt,
+    int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_rows) {
+    const int width = W ? W : width_rt;
+    const int pt = PT ? PT : page_tokens_rt;
+    __shared__ unsigned long long s_base[kRowsPerGroup];
+    __shared__ float s_scale[kRowsPerGroup];
+    constexpr unsigned long long kSkip = ~0ull;
+
+    const int q = blockIdx.y;
+    const int r0 = (int)blockIdx.x * kRowsPerGroup;
+    const int nr = n_rows ? min(n_rows[q], k) : k;
+    if (r0 >= nr) return;
+    const int cnt = min(kRowsPerGroup, nr - r0);
+
+    if (threadIdx.x < kRowsPerGroup) {
+        unsigned long long base = kSkip;
+        float scale = 0.0f;
+        if ((int)threadIdx.x < cnt) {
+            const unsigned int tok = rows[(size_t)q * k + r0 + threadIdx.x];
+            const unsigned int blk = tok / (unsigned)pt;
+            const unsigned int off = tok - blk * (unsigned)pt;
+            int page = -1;
+            if (blk < (unsigned)max_blocks_per_seq)
+                page = block_table[(size_t)q * max_blocks_per_seq + blk];
+            if ((unsigned)page < (unsigned)n_pages) {
+                const size_t pbase = (size_t)page * page_bytes;
+                base = pbase + (size_t)off * width;
+                scale = *reinterpret_cast<const float*>(pool + pbase + (size_t)pt * width +
+                                                        (size_t)off * 4);
+            } else if (bad_rows) {
+                atomicAdd(bad_rows, 1u);
+            }
+        }
+        s_base[threadIdx.x] = base;
+        s_scale[threadIdx.x] = scale;
+    }
+    __syncthreads();
+
+    const int cpr = width >> 3;
+    const int n_chunks = cnt * cpr;
+    u32x4* dst = reinterpret_cast<u32x4*>(out + ((size_t)q * k + r0) * width);
+    for (int cb = threadIdx.x; cb < n_chunks; cb += kGatherThreads * UNROLL) {
+        u32x2 raw[UNROLL];
+        float scl[UNROLL];
+        bool live[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int c = cb + u * kGatherThreads;
+            live[u] = false;
+            if (c < n_chunks) {
+                int r = c / cpr;
+                int col = c - r * cpr;
+                unsigned long long base = s_base[r];
+                if (base != kSkip) {
+                    live[u] = true;
+                    raw[u] = __builtin_nontemporal_load(
+                        reinterpret_cast<const u32x2*>(pool + base) + col);
+                    scl[u] = s_scale[r];
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int c = cb + u * kGatherThreads;
+            if (live[u]) __builtin_nontemporal_store(dequant8_bf16(raw[u], scl[u]), dst + c);
+        }
+    }
+}
+
+// out[i] = bf16(e4m3_to_f32(codes[i]) * scale): the dequant body alone, for codec census tests.
+__global__ void e4m3_dequant_bf16_kernel(const uint8_t* __restrict__ codes, float scale,
+                                         uint16_t* __restrict__ out, long long n) {
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long step = (long long)gridDim.x * blockDim.x;
+    for (; i < n; i += step) {
+        // the packed decoder is the product path; feed it the byte in lane 0 of a dword
+        u32x2 r = dequant4_bf16((uint32_t)codes[i], scale);
+        out[i] = (uint16_t)(r.x & 0xffffu);
+    }
+}
+
+static inline bool shape_ok(int width, int page_tokens) {
+    return (width % 16) == 0 && (page_tokens % 4) == 0;
+}
+
+}  // namespace rk
+
+extern "C" int rivoli_kv_gather_paged(const unsigned char* pool, const int* block_table,
+                                      const int* seq_lens, const int* cu_seqlens,
+                                      unsigned short* out, int n_seqs, int max_blocks_per_seq,
+                                      int width, int page_tokens, int n_pages,
+                                      unsigned int* bad_pages, void* stream) {
+    using namespace rk;
+    if (!pool || !block_table || !seq_lens || !cu_seqlens || !out) return 1001;
+    if (n_seqs <= 0 || max_blocks_per_seq <= 0 || width <= 0 || page_tokens <= 0 || n_pages <= 0)
+        return 1001;
+    if (n_seqs > 65535) return 1002;
+    if (!shape_ok(width, page_tokens)) return 1004;
+    const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
+    dim3 grid((unsigned)max_blocks_per_seq, (unsigned)n_seqs);
+    (void)hipGetLastError();
+    if (width == 576 && page_tokens == 64) {
+        hipLaunchKernelGGL((kv_gather_paged_kernel<576, 64, 18>), grid, dim3(kGatherThreads), 0,
+                           (hipStream_t)stream, pool, block_table, seq_lens, cu_seqlens, out,
+                           max_blocks_per_seq, width, page_tokens, n_pages, page_bytes, bad_pages);
+    } else {
+        hipLaunchKernelGGL((kv_gather_paged_kernel<0, 0, 4>), grid, dim3(kGatherThreads), 0,
+                           (hipStream_t)stream, pool, block_table, seq_lens, cu_seqlens, out,
+                           max_blocks_per_seq, width, page_tokens, n_pages, page_bytes, bad_pages);
+    }
+    return launch_status();
+}
+
+extern "C" int rivoli_kv_gather_rows_paged(const unsigned char* pool, const int* block_table,
+                                           const unsigned int* rows, const int* n_rows,
+                                           unsigned short* out, int n_queries, int k,
+                                           int max_blocks_per_seq, int width, int page_tokens,
+                                           int n_pages, unsigned int* bad_rows, void* stream) {
+    using namespace rk;
+    if (!pool || !block_table || !rows || !out) return 1001;
+    if (n_queries <= 0 || k <= 0 || max_blocks_per_seq <= 0 || width <= 0 || page_tokens <= 0 ||
+        n_pages <= 0)
+        return 1001;
+    if (n_queries > 65535) return 1002;
+    if (!shape_ok(width, page_tokens)) return 1004;
+    const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
+    dim3 grid((unsigned)((k + kRowsPerGroup - 1) / kRowsPerGroup), (unsigned)n_queries);
+    (void)hipGetLastError();
+    if (width == 576 && page_tokens == 64) {
+        hipLaunchKernelGGL((kv_gather_rows_kernel<576, 64, 9>), grid, dim3(kGatherThreads), 0,
+                           (hipStream_t)stream, pool, block_table, rows, n_rows, out, k,
+                           max_blocks_per_seq, width, page_tokens, n_pages, page_bytes, bad_rows);
+    } else {
+        hipLaunchKernelGGL((kv_gather_rows_kernel<0, 0, 4>), grid, dim3(kGatherThreads), 0,
+                           (hipStream_t)stream, pool, block_table, rows, n_rows, out, k,
+                           max_blocks_per_seq, width, page_tokens, n_pages, page_bytes, bad_rows);
+    }
+    return launch_status();
+}
+
+extern "C" int rivoli_codec_e4m3_dequant_bf16(const unsigned char* codes, float scale,
+                                              unsigned short* out, long long n, void* stream) {
+    if (!codes || !out || n <= 0) return 1001;
+    long long blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    (void)hipGetLastError();
+    hipLaunchKernelGGL(rk::e4m3_dequant_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                       (hipStream_t)stream, codes, scale, out, n);
+    return rk::launch_status();
+}

@@ -1,0 +1,180 @@
+"""The launcher wall: one `launch_*` per `extern "C" int rivoli_*` entry point.
+
+Host-side mirror of the reference's `launchers!` rows (crates/backend/src/hip.rs:196-221,
+crates/backend/src/hip_attn.rs:113-147,450-495): every wrapper narrows its dims to C int,
+calls the symbol, and maps the return code the way `ensure_hip_status` does
+(crates/backend/src/hip.rs:328-336) — 0 ok, positive = argument guard, negative = HIP error.
+Pointers are device addresses: pass a torch tensor (its data_ptr is taken), an int, or None.
+There is no fallback: if the HIP library has not been built, importing a launcher fails.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+from .build import LIB_PATH
+
+NULL_STREAM = None
+
+
+class LaunchError(RuntimeError):
+    """What `ensure_hip_status` bails with; `.code` keeps the raw launcher return."""
+
+    def __init__(self, name: str, code: int):
+        self.name, self.code = name, code
+        if code > 0:
+            super().__init__(f"{name}: argument guard rejected ({code})")
+        else:
+            super().__init__(f"{name}: HIP error {-code}")
+
+
+def ensure_hip_status(code: int, name: str) -> None:
+    if code != 0:
+        raise LaunchError(name, code)
+
+
+_LIB = None
+
+_VP, _I, _LL, _ULL, _F = C.c_void_p, C.c_int, C.c_longlong, C.c_ulonglong, C.c_float
+_SIGNATURES = {
+    "rivoli_append_kv": [_VP] * 5 + [_I] * 4,
+    "rivoli_append_kv_rows": [_VP] * 5 + [_I] * 5 + [_VP],
+    "rivoli_index_append": [_VP, _VP, _I, _I],
+    "rivoli_index_topk": [_VP, _I, _I, _VP],
+    "rivoli_index_topk_batched": [_VP, _I, _I, _VP, _I, _I, _VP, _VP],
+    "rivoli_hash_rows": [_VP, _I, _I, _ULL, _VP, _VP],
+    "rivoli_device_sync": [],
+    "rivoli_kv_append_paged": [_VP, _VP, _VP, _I, _I, _I, _I, _VP, _VP],
+    "rivoli_kv_gather_paged": [_VP] * 5 + [_I] * 5 + [_VP, _VP],
+    "rivoli_kv_gather_rows_paged": [_VP] * 5 + [_I] * 6 + [_VP, _VP],
+    "rivoli_codec_e4m3_encode": [_VP, _VP, _LL, _VP],
+    "rivoli_codec_e4m3_dequant_bf16": [_VP, _F, _VP, _LL, _VP],
+    "rivoli_codec_bf16_encode": [_VP, _VP, _LL, _VP],
+}
+
+
+def lib() -> C.CDLL:
+    """The loaded HIP library. Raises if it was never built — there is no other path."""
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(
+                f"{LIB_PATH} is missing: build it with `python -m rivoli_amd.build` "
+                "(hipcc, gfx950); this package has no CPU fallback")
+        handle = C.CDLL(LIB_PATH)
+        for name, args in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = C.c_int, args
+        handle.rivoli_kv_page_bytes.restype = C.c_size_t
+        handle.rivoli_kv_page_bytes.argtypes = [_I, _I]
+        _LIB = handle
+    return _LIB
+
+
+def exported_symbols() -> list[str]:
+    return sorted(list(_SIGNATURES) + ["rivoli_kv_page_bytes"])
+
+
+def _p(x):
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    return x.data_ptr()  # torch tensor
+
+
+def _s(stream):
+    if stream is None:
+        return None
+    if isinstance(stream, int):
+        return stream
+    return stream.cuda_stream  # torch.cuda.Stream
+
+
+def device_sync() -> None:
+    ensure_hip_status(lib().rivoli_device_sync(), "device_sync")
+
+
+def kv_page_bytes(page_tokens: int, width: int) -> int:
+    return int(lib().rivoli_kv_page_bytes(page_tokens, width))
+
+
+# ---- reference-signature launchers --------------------------------------------------------
+
+def launch_append_kv(latent, rope, lc8, lscale, rc, pos, kvl, ropn, n_blocks) -> None:
+    ensure_hip_status(lib().rivoli_append_kv(_p(latent), _p(rope), _p(lc8), _p(lscale), _p(rc),
+                                             pos, kvl, ropn, n_blocks), "append_kv")
+
+
+def launch_append_kv_rows(latent, rope, lc8, lscale, rc, pos0, n_tokens, kvl, ropn, n_blocks,
+                          stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_append_kv_rows(_p(latent), _p(rope), _p(lc8), _p(lscale),
+                                                  _p(rc), pos0, n_tokens, kvl, ropn, n_blocks,
+                                                  _s(stream)), "append_kv_rows")
+
+
+def launch_index_append(k, kcache, pos, hd) -> None:
+    ensure_hip_status(lib().rivoli_index_append(_p(k), _p(kcache), pos, hd), "index_append")
+
+
+def launch_index_topk(scores, nt, k, rows) -> None:
+    ensure_hip_status(lib().rivoli_index_topk(_p(scores), nt, k, _p(rows)), "index_topk")
+
+
+def launch_hash_rows(x, n, stride, i_base, out, stream=NULL_STREAM) -> None:
+    if n > 2 ** 31 - 1:
+        raise LaunchError("hash_rows", 1002)  # exceeds the i32 ABI, crates/backend/src/hip.rs:595-598
+    ensure_hip_status(lib().rivoli_hash_rows(_p(x), n, stride, i_base, _p(out), _s(stream)),
+                      "hash_rows")
+
+
+# ---- paged, batched launchers -------------------------------------------------------------
+
+def launch_kv_append_paged(rows, slot_mapping, pool, n_tokens, width, page_tokens, n_pages,
+                           bad_slots=None, stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_kv_append_paged(_p(rows), _p(slot_mapping), _p(pool), n_tokens,
+                                                   width, page_tokens, n_pages, _p(bad_slots),
+                                                   _s(stream)), "kv_append_paged")
+
+
+def launch_kv_gather_paged(pool, block_table, seq_lens, cu_seqlens, out, n_seqs,
+                           max_blocks_per_seq, width, page_tokens, n_pages, bad_pages=None,
+                           stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_kv_gather_paged(_p(pool), _p(block_table), _p(seq_lens),
+                                                   _p(cu_seqlens), _p(out), n_seqs,
+                                                   max_blocks_per_seq, width, page_tokens, n_pages,
+                                                   _p(bad_pages), _s(stream)), "kv_gather_paged")
+
+
+def launch_kv_gather_rows_paged(pool, block_table, rows, n_rows, out, n_queries, k,
+                                max_blocks_per_seq, width, page_tokens, n_pages, bad_rows=None,
+                                stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_kv_gather_rows_paged(_p(pool), _p(block_table), _p(rows),
+                                                        _p(n_rows), _p(out), n_queries, k,
+                                                        max_blocks_per_seq, width, page_tokens,
+                                                        n_pages, _p(bad_rows), _s(stream)),
+                      "kv_gather_rows_paged")
+
+
+def launch_index_topk_batched(scores, n_queries, stride, nts, nt, k, rows,
+                              stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_index_topk_batched(_p(scores), n_queries, stride, _p(nts), nt,
+                                                      k, _p(rows), _s(stream)),
+                      "index_topk_batched")
+
+
+# ---- element codecs -----------------------------------------------------------------------
+
+def launch_codec_e4m3_encode(x, out, n, stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_codec_e4m3_encode(_p(x), _p(out), n, _s(stream)),
+                      "codec_e4m3_encode")
+
+
+def launch_codec_e4m3_dequant_bf16(codes, scale, out, n, stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_codec_e4m3_dequant_bf16(_p(codes), scale, _p(out), n,
+                                                           _s(stream)), "codec_e4m3_dequant_bf16")
+
+
+def launch_codec_bf16_encode(x, out, n, stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_codec_bf16_encode(_p(x), _p(out), n, _s(stream)),
+                      "codec_bf16_encode")

@@ -1,0 +1,53 @@
+"""Device-buffer plumbing for the GPU parity tests: torch only allocates and copies."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+REF_LIB = os.path.join(ROOT, "oracle", "_ref", "librivoli_ref_kernels.so")
+
+
+def torch_cuda():
+    import torch
+
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch
+
+
+def dev(a: np.ndarray):
+    """Upload any numpy array as raw bytes (a uint8 device tensor)."""
+    torch = torch_cuda()
+    b = np.ascontiguousarray(a).view(np.uint8).reshape(-1)
+    return torch.from_numpy(b.copy()).cuda()
+
+
+def dzeros(nbytes: int, fill: int = 0):
+    torch = torch_cuda()
+    return torch.full((int(nbytes),), fill, dtype=torch.uint8, device="cuda")
+
+
+def back(t, dtype=np.uint8) -> np.ndarray:
+    """Synchronise and download as `dtype`."""
+    return t.cpu().numpy().view(dtype)
+
+
+_REF = None
+
+
+def ref_kernels():
+    """The reference's own launchers compiled for gfx950 (oracle/Makefile `ref`), or None.
+    They run on the null stream like every launch in these tests."""
+    global _REF
+    if _REF is None and os.path.exists(REF_LIB):
+        h = C.CDLL(REF_LIB)
+        vp, i = C.c_void_p, C.c_int
+        h.rivoli_append_kv.restype, h.rivoli_append_kv.argtypes = i, [vp] * 5 + [i] * 4
+        h.rivoli_index_append.restype, h.rivoli_index_append.argtypes = i, [vp, vp, i, i]
+        h.rivoli_index_topk.restype, h.rivoli_index_topk.argtypes = i, [vp, i, i, vp]
+        h.rivoli_hash_rows.restype = i
+        h.rivoli_hash_rows.argtypes = [vp, i, i, C.c_ulonglong, vp, vp]
+        _REF = h
+    return _REF

@@ -1,0 +1,182 @@
+"""Quantize-and-append on the device against the CPU oracle (bit-exact codes, scales, bf16
+keys), on the reference's own fixture, on BASELINE configs 1 and 2, and on rows built to sit
+on the quantizer's rounding ties."""
+import numpy as np
+import pytest
+
+from rivoli_amd import hip
+from tests.gpu_util import back, dev, dzeros, ref_kernels
+from tests.test_oracle_quant import fixture_a99e
+from tests.util import f32_to_bf16_rne, make_rows_bf16, shuffled_block_tables, slots_for
+
+pytestmark = pytest.mark.gpu
+W, PT = 576, 64
+
+
+def test_append_kv_reference_fixture(oracle):
+    """crates/engine/tests/fwd_kernel.rs:139-214 — five-row slabs, row 3 written."""
+    rows, kvl, ropn, pos, nb = 5, 256, 64, 3, 2
+    latent, rope = fixture_a99e(oracle)
+    want = [np.zeros(rows * kvl, np.uint8), np.zeros(rows * nb, np.float32),
+            np.zeros(rows * ropn, np.uint16)]
+    assert oracle.append_kv(latent, rope, *want, pos, kvl, ropn, nb) == 0
+    c8, ls, rc = dzeros(rows * kvl), dzeros(rows * nb * 4), dzeros(rows * ropn * 2)
+    hip.launch_append_kv(dev(latent), dev(rope), c8, ls, rc, pos, kvl, ropn, nb)
+    assert np.count_nonzero(want[0]) > kvl // 2
+    assert np.array_equal(back(c8), want[0])
+    assert np.array_equal(back(ls, np.uint32), want[1].view(np.uint32))
+    assert np.array_equal(back(rc, np.uint16), want[2])
+    ref = ref_kernels()
+    if ref is not None:  # the reference's own kernel, compiled for this GPU, agrees too
+        r8, rs, rr = dzeros(rows * kvl), dzeros(rows * nb * 4), dzeros(rows * ropn * 2)
+        lat_d, rope_d = dev(latent), dev(rope)
+        assert ref.rivoli_append_kv(lat_d.data_ptr(), rope_d.data_ptr(), r8.data_ptr(),
+                                    rs.data_ptr(), rr.data_ptr(), pos, kvl, ropn, nb) == 0
+        assert np.array_equal(back(r8), want[0])
+        assert np.array_equal(back(rs, np.uint32), want[1].view(np.uint32))
+        assert np.array_equal(back(rr, np.uint16), want[2])
+
+
+def test_append_kv_guards():
+    b = dzeros(4096)
+    for args, code in (((-1, 256, 64, 2), 1001), ((0, 0, 64, 2), 1001), ((0, 192, 64, 2), 1002),
+                       ((0, 2048, 64, 16), 1002), ((0, 128, 256, 1), 1002)):
+        with pytest.raises(hip.LaunchError) as e:
+            hip.launch_append_kv(b, b, b, b, b, *args)
+        assert e.value.code == code
+    assert str(e.value) == "append_kv: argument guard rejected (1002)"
+
+
+def test_append_kv_rows_matches_per_token_oracle(oracle):
+    """GLM dims (kvl 512, rope 64, 4 block scales), 37 tokens from pos 5, in one launch."""
+    n, kvl, ropn, nb, pos0, rows = 37, 512, 64, 4, 5, 50
+    rng = np.random.default_rng(12)
+    latent = (rng.standard_normal((n, kvl)) * rng.choice([0.01, 1, 30], (n, 1))).astype(np.float32)
+    latent[3, 128:256] = 0.0                      # an all-zero block: scale 1.0, codes 0
+    rope = rng.standard_normal((n, ropn)).astype(np.float32)
+    want = [np.full(rows * kvl, 0xEE, np.uint8), np.full(rows * nb, 7.0, np.float32),
+            np.full(rows * ropn, 0xABCD, np.uint16)]
+    for t in range(n):
+        oracle.append_kv(latent[t], rope[t], *want, pos0 + t, kvl, ropn, nb)
+    c8, ls, rc = dev(np.full(rows * kvl, 0xEE, np.uint8)), dev(np.full(rows * nb, 7.0, np.float32)), \
+        dev(np.full(rows * ropn, 0xABCD, np.uint16))
+    hip.launch_append_kv_rows(dev(latent), dev(rope), c8, ls, rc, pos0, n, kvl, ropn, nb)
+    assert np.array_equal(back(c8), want[0])
+    assert np.array_equal(back(ls, np.uint32), want[1].view(np.uint32))
+    assert np.array_equal(back(rc, np.uint16), want[2])
+
+
+def test_index_append_reference_fixture(oracle):
+    """crates/engine/tests/indexer_kernel.rs:119-140 — seven-row slab, row 5."""
+    rows, hd, pos = 7, 128, 5
+    k = oracle.lcg(0xC0DE).fill(hd) * np.float32(8.0)
+    want = np.zeros(rows * hd, np.uint16)
+    oracle.index_append(k, want, pos, hd)
+    cache = dzeros(rows * hd * 2)
+    hip.launch_index_append(dev(k), cache, pos, hd)
+    assert np.array_equal(back(cache, np.uint16), want)
+    ref = ref_kernels()
+    if ref is not None:
+        rcache, kd = dzeros(rows * hd * 2), dev(k)
+        assert ref.rivoli_index_append(kd.data_ptr(), rcache.data_ptr(), pos, hd) == 0
+        assert np.array_equal(back(rcache, np.uint16), want)
+    with pytest.raises(hip.LaunchError):
+        hip.launch_index_append(dev(k), cache, -1, hd)
+
+
+def paged_append_both(oracle, rows, slots, n_pages, fill=0xA5):
+    page_bytes = oracle.kv_page_bytes(PT, W)
+    assert hip.kv_page_bytes(PT, W) == page_bytes
+    want = np.full(n_pages * page_bytes, fill, np.uint8)
+    bad_want = oracle.kv_append_paged(rows, slots, want, W, PT, n_pages)
+    pool, bad = dzeros(n_pages * page_bytes, fill), dzeros(4)
+    hip.launch_kv_append_paged(dev(rows), dev(slots), pool, slots.size, W, PT, n_pages, bad)
+    return back(pool), want, int(back(bad, np.uint32)[0]), bad_want
+
+
+def test_config1_append_one_token_after_4095(oracle):
+    """BASELINE config 1: 4095 cached tokens, block table = seeded permutation of 64 pages,
+    append the 4096th."""
+    table = shuffled_block_tables(1, 64, 64, seed=0x5EED0001)[0]
+    rows = make_rows_bf16(4096, W, seed=0x5EED0001)
+    slots = slots_for(table, np.arange(4096))
+    got, want, bad, bad_want = paged_append_both(oracle, rows[:4095], slots[:4095], 64)
+    assert np.array_equal(got, want) and bad == bad_want == 0
+    # now the decode step: one token into the live pool
+    pool = dev(got)
+    hip.launch_kv_append_paged(dev(rows[4095:]), dev(slots[4095:]), pool, 1, W, PT, 64)
+    oracle.kv_append_paged(rows[4095:], slots[4095:], want, W, PT, 64)
+    assert np.array_equal(back(pool), want)
+
+
+def test_config2_prefill_bulk_append_with_outlier_rows(oracle):
+    """BASELINE config 2: 8192 rows, 0.5% of rows x50, 128 shuffled pages."""
+    table = shuffled_block_tables(1, 128, 128, seed=0x5EED0002)[0]
+    rows = make_rows_bf16(8192, W, seed=0x5EED0002, outlier_frac=0.005, outlier_mul=50.0)
+    slots = slots_for(table, np.arange(8192))
+    got, want, bad, _ = paged_append_both(oracle, rows, slots, 128)
+    assert bad == 0
+    mism = np.flatnonzero(got != want)
+    assert mism.size == 0, mism[:10]
+    scales = got.reshape(128, -1)[:, PT * W:].copy().view(np.float32)
+    assert scales.max() / np.median(scales) > 20      # the outlier rows really moved the scale
+
+
+def test_append_rounding_ties_saturation_and_special_rows(oracle):
+    f32 = np.zeros((16, W), np.float32)
+    q = np.float32(2.0 ** -10)
+    # row 0: a 448 pins scale == 1; the rest are multiples and half-multiples of the subnormal
+    # quantum in both signs, so exact subnormal ties reach the encoder
+    f32[0, 0] = 448.0
+    m = (np.arange(1, W) % 32).astype(np.float32) * q
+    f32[0, 1:] = np.where(np.arange(1, W) % 2 == 0, m, -m)
+    # row 1: normal-range ties (k + 1/2 mantissa steps) under scale 1
+    f32[1, 0] = -448.0
+    f32[1, 1:] = (1.0 + (np.arange(1, W) % 16) / 16.0) * np.where(np.arange(1, W) % 3 == 0, -4.0, 0.25)
+    f32[2] = 0.0                                           # all zero -> scale 1.0
+    f32[3, ::2] = -0.0                                     # signed zeros only
+    f32[4] = np.random.default_rng(1).standard_normal(W) * 1e-38   # denormal-range amax
+    f32[5] = np.random.default_rng(2).standard_normal(W) * 1e37    # huge
+    f32[6] = np.random.default_rng(3).standard_normal(W)
+    f32[6, 17] *= 200.0                                    # one outlier crushes the rest
+    f32[7, 5] = 3.0                                        # single non-zero
+    f32[8] = np.random.default_rng(4).standard_normal(W) * 200.0   # the x200 outlier-token case
+    f32[9:] = np.random.default_rng(5).standard_normal((7, W)) * np.float32(2.0) ** np.arange(-60, 61, 20)[:, None]
+    rows = f32_to_bf16_rne(f32)
+    slots = np.arange(16, dtype=np.int32) * 3
+    got, want, bad, _ = paged_append_both(oracle, rows, slots, 1)
+    assert bad == 0 and np.array_equal(got, want)
+    codes0 = want[: W]
+    assert {1, 3, 5, 7}.issubset(set(codes0.tolist()))      # half-away results are present
+    # anti-vacuity: nearest-even on those ties would have produced a different row
+    assert np.count_nonzero(codes0 & 0x7F) > W // 2
+
+
+def test_append_padding_bad_slots_and_guards(oracle):
+    rows = make_rows_bf16(6, W, seed=8)
+    slots = np.array([5, -1, 128, 2 ** 31 - 1, 64, -7], np.int32)
+    got, want, bad, bad_want = paged_append_both(oracle, rows, slots, 2, fill=0)
+    assert bad == bad_want == 2 and np.array_equal(got, want)
+    b = dzeros(4096)
+    for args, code in (((0, W, PT, 1), 1001), ((1, 0, PT, 1), 1001), ((1, W, PT, 0), 1001),
+                       ((1, 2048, PT, 1), 1002), ((1, 570, PT, 1), 1004), ((1, W, 6, 1), 1004)):
+        with pytest.raises(hip.LaunchError) as e:
+            hip.launch_kv_append_paged(b, b, b, *args)
+        assert e.value.code == code, args
+    with pytest.raises(hip.LaunchError) as e:
+        hip.launch_kv_append_paged(None, b, b, 1, W, PT, 1)
+    assert e.value.code == 1001
+
+
+def test_append_other_widths(oracle):
+    """Non-flagship shapes: width 512 (one step per lane), 128, 1024; page of 16 tokens."""
+    for width, pt in ((512, 64), (128, 16), (1024, 32), (64, 4)):
+        n, n_pages = 100, 8 * 64 // pt
+        rows = make_rows_bf16(n, width, seed=width)
+        slots = np.random.default_rng(width).permutation(n_pages * pt)[:n].astype(np.int32)
+        pb = oracle.kv_page_bytes(pt, width)
+        want = np.zeros(n_pages * pb, np.uint8)
+        oracle.kv_append_paged(rows, slots, want, width, pt, n_pages)
+        pool = dzeros(n_pages * pb)
+        hip.launch_kv_append_paged(dev(rows), dev(slots), pool, n, width, pt, n_pages)
+        assert np.array_equal(back(pool), want), (width, pt)
