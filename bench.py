@@ -40,6 +40,14 @@ def parse():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=32768)
+    ap.add_argument("--workload", choices=["decode", "prefill", "dsa"], default="decode",
+                    help="decode = BASELINE config 3 (the headline line); prefill = config 2 "
+                         "bulk append; dsa = config 4 top-k + sparse gather")
+    ap.add_argument("--tokens", type=int, default=8192, help="prefill: new tokens per step")
+    ap.add_argument("--topk", type=int, default=2048)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy (a known-size kernel to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     return ap.parse_args()
@@ -58,6 +66,16 @@ def main():
         sys.exit("bench.py needs a GPU (cuda:0); there is no CPU fallback for the product path")
     torch.cuda.set_device(0)
     hip.lib()
+    if a.calibrate_copy:
+        src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    if a.workload == "prefill":
+        return bench_prefill(a, torch, hip)
+    if a.workload == "dsa":
+        return bench_dsa(a, torch, hip)
     L, B, ctx = a.layers, a.batch, a.ctx
     blocks = -(-ctx // PT)
     n_pages = B * blocks
@@ -143,13 +161,191 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "kv_gather_paged_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": round(achieved * 1e9 / HBM_PEAK, 4),
                      "avg_launch_ms": round(gather_ms, 5), "bytes_per_launch": gather_bytes_layer,
-                     "traffic": None},
+                     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+                     # this workload, scaled by a known 1 GiB copy (profiles/); it cannot be
+                     # read live, so it is only reported for the shape it was measured on
+                     "traffic": 1821500000 if (B, ctx) == (32, 32768) else None},
     }
 
     if not a.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(pools[0], tables_np, seq_lens_np, out, a.cpu_seconds,
                                               hip, tables, seq_lens, cu, B, blocks, n_pages)
     print(json.dumps(result), flush=True)
+
+
+def timed(torch, stream, steps, warmup, step):
+    """Warm up, then time `steps` calls of step(events) with HIP events on `stream`."""
+    for _ in range(warmup):
+        step(None)
+    stream.synchronize()
+    torch.cuda.synchronize()
+    t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    events = {}
+    t0.record(stream)
+    for _ in range(steps):
+        step(events)
+    t1.record(stream)
+    stream.synchronize()
+    torch.cuda.synchronize()
+    per_kernel = {k: float(np.mean([a.elapsed_time(b) for a, b in v])) for k, v in events.items()}
+    return t0.elapsed_time(t1) / steps, per_kernel
+
+
+def bracket(torch, stream, events, name, launch):
+    if events is None:
+        return launch()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    launch()
+    e1.record(stream)
+    events.setdefault(name, []).append((e0, e1))
+
+
+def bench_prefill(a, torch, hip):
+    """BASELINE config 2: `tokens` new 576-wide bf16 rows (0.5% of rows x50) quantize-appended
+    into shuffled pages, one layer, one launch per step."""
+    n = a.tokens
+    n_pages = -(-n // PT)
+    page_bytes = hip.kv_page_bytes(PT, W)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0x5EED0002)
+    rng = np.random.default_rng(0x5EED0002)
+    rows = torch.randn(n, W, generator=g, device="cuda", dtype=torch.float32)
+    hit = torch.rand(n, generator=g, device="cuda") < 0.005
+    rows[hit] *= 50.0
+    rows = rows.to(torch.bfloat16)
+    table = rng.permutation(n_pages).astype(np.int32)
+    pos = np.arange(n)
+    slots = torch.from_numpy((table[pos // PT] * PT + pos % PT).astype(np.int32)).cuda()
+    pool = torch.zeros(n_pages * page_bytes, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.Stream()
+    sh = stream.cuda_stream
+
+    def step(events):
+        bracket(torch, stream, events, "append",
+                lambda: hip.launch_kv_append_paged(rows, slots, pool, n, W, PT, n_pages, None, sh))
+
+    ms, per = timed(torch, stream, a.steps, a.warmup, step)
+    nbytes = n * (ROW_IN + 4 + REC)
+    res = {"metric": "kv_append_GBps", "value": round(nbytes / (ms * 1e-3) / 1e9, 2), "unit": "GB/s",
+           "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+           "data": "synthetic",
+           "config": {"workload": "prefill bulk append (BASELINE config 2)", "tokens": n,
+                      "pages": n_pages, "width": W, "page_tokens": PT},
+           "tokens_per_s": round(n / (ms * 1e-3), 1),
+           "roofline": {"bound": "hbm", "kernel": "kv_append_paged_kernel",
+                        "achieved": round(nbytes / (per["append"] * 1e-3) / 1e9, 2),
+                        "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                        "frac": round(nbytes / (per["append"] * 1e-3) / HBM_PEAK, 5),
+                        "avg_launch_ms": round(per["append"], 5), "bytes_per_launch": nbytes,
+                        "traffic": None}}
+    if not a.no_cpu_baseline:
+        from oracle.kvoracle import oracle as get_oracle
+
+        ora, cores = get_oracle(), max(1, min(16, os.cpu_count() or 1))
+        rows_h = rows.view(torch.int16).cpu().numpy().view(np.uint16)
+        slots_h, pool_h = slots.cpu().numpy(), np.zeros(n_pages * page_bytes, np.uint8)
+        reps, spent = 0, 0.0
+        while spent < a.cpu_seconds and reps < 200:
+            t0 = time.perf_counter()
+            ora.kv_append_paged(rows_h, slots_h, pool_h, W, PT, n_pages, n_threads=cores)
+            spent += time.perf_counter() - t0
+            reps += 1
+        if not np.array_equal(pool.cpu().numpy(), pool_h):
+            raise SystemExit("bench: GPU append differs from the CPU oracle")
+        res["cpu_baseline"] = {"value": round(nbytes / (spent / reps) / 1e9, 3), "unit": "GB/s",
+                               "cores": cores, "kind": "port",
+                               "sample": f"the same {n}-token append x{reps} reps, {cores} host "
+                                         "threads; GPU pool bytes checked equal"}
+    print(json.dumps(res), flush=True)
+
+
+def bench_dsa(a, torch, hip):
+    """BASELINE config 4: per layer, select the top-k of 65536 indexer scores for each of 16
+    queries (ties to the lowest index), then gather + dequantize those rows from fragmented
+    pages. One step = all layers."""
+    L, B, nt, k = a.layers, (16 if a.batch == 32 else a.batch), (65536 if a.ctx == 32768 else a.ctx), a.topk
+    blocks = -(-nt // PT)
+    n_pages = B * blocks
+    page_bytes = hip.kv_page_bytes(PT, W)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0x5EED0004)
+    rng = np.random.default_rng(0x5EED0004)
+    tables_np = rng.permutation(n_pages).astype(np.int32).reshape(B, blocks)
+    pos = np.arange(nt)
+    slots_np = np.concatenate([tables_np[s][pos // PT] * PT + pos % PT for s in range(B)]).astype(np.int32)
+    tables, slots_all = torch.from_numpy(tables_np.copy()).cuda(), torch.from_numpy(slots_np).cuda()
+    kv_rows = torch.randn(B * nt, W, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    pools = []
+    for _ in range(L):
+        pool = torch.empty(n_pages * page_bytes, dtype=torch.uint8, device="cuda")
+        hip.launch_kv_append_paged(kv_rows, slots_all, pool, B * nt, W, PT, n_pages)
+        pools.append(pool)
+    del kv_rows
+    scores = []
+    for _ in range(L):
+        sc = torch.randn(B, nt, generator=g, device="cuda", dtype=torch.float32)
+        sc[:, -64:] += 4.0                                       # recency boost
+        scores.append(sc)
+    sel = torch.empty(B * k, dtype=torch.int32, device="cuda")
+    out = torch.empty(B * k * W, dtype=torch.bfloat16, device="cuda")
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    sh = stream.cuda_stream
+
+    def step(events):
+        for layer in range(L):
+            bracket(torch, stream, events, "topk",
+                    lambda: hip.launch_index_topk_batched(scores[layer], B, nt, None, nt, k, sel, sh))
+            bracket(torch, stream, events, "gather_rows",
+                    lambda: hip.launch_kv_gather_rows_paged(pools[layer], tables, sel, None, out, B, k,
+                                                            blocks, W, PT, n_pages, None, sh))
+
+    ms, per = timed(torch, stream, a.steps, a.warmup, step)
+    topk_bytes = B * nt * 4 + B * k * 4
+    rows_bytes = B * k * (4 + REC + ROW_IN) + B * blocks * 4
+    layer_bytes = topk_bytes + rows_bytes
+    res = {"metric": "kv_dsa_topk_gather_GBps", "value": round(L * layer_bytes / (ms * 1e-3) / 1e9, 2),
+           "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+           "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "DSA sparse path (BASELINE config 4): top-k then sparse row gather",
+                      "layers": L, "batch": B, "ctx": nt, "k": k, "width": W, "page_tokens": PT},
+           "rows_per_s": round(L * B * k / (ms * 1e-3), 1),
+           "kernels_ms": {n: round(v, 5) for n, v in per.items()},
+           "roofline": {"bound": "hbm", "kernel": "kv_gather_rows_kernel",
+                        "achieved": round(rows_bytes / (per["gather_rows"] * 1e-3) / 1e9, 2),
+                        "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                        "frac": round(rows_bytes / (per["gather_rows"] * 1e-3) / HBM_PEAK, 5),
+                        "avg_launch_ms": round(per["gather_rows"], 5),
+                        "bytes_per_launch": rows_bytes, "traffic": None},
+           "topk": {"achieved": round(topk_bytes / (per["topk"] * 1e-3) / 1e9, 2), "unit": "GB/s",
+                    "avg_launch_ms": round(per["topk"], 5), "bytes_per_launch": topk_bytes}}
+    if not a.no_cpu_baseline:
+        from oracle.kvoracle import oracle as get_oracle
+
+        ora, cores = get_oracle(), max(1, min(16, os.cpu_count() or 1))
+        sc_h, pool_h = scores[0].cpu().numpy(), pools[0].cpu().numpy()
+        reps, spent = 0, 0.0
+        while spent < a.cpu_seconds and reps < 50:
+            t0 = time.perf_counter()
+            want_sel = ora.topk_batched(sc_h, k, n_threads=cores)
+            want_rows = ora.kv_gather_rows_paged(pool_h, tables_np, want_sel, W, PT)
+            spent += time.perf_counter() - t0
+            reps += 1
+        hip.launch_index_topk_batched(scores[0], B, nt, None, nt, k, sel)
+        hip.launch_kv_gather_rows_paged(pools[0], tables, sel, None, out, B, k, blocks, W, PT, n_pages)
+        torch.cuda.synchronize()
+        if not np.array_equal(sel.cpu().numpy().view(np.uint32).reshape(B, k), want_sel):
+            raise SystemExit("bench: GPU top-k differs from the CPU oracle")
+        if not np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16).reshape(B, k, W), want_rows):
+            raise SystemExit("bench: GPU sparse gather differs from the CPU oracle")
+        res["cpu_baseline"] = {"value": round(layer_bytes / (spent / reps) / 1e9, 3), "unit": "GB/s",
+                               "cores": cores, "kind": "port",
+                               "sample": f"one layer (top-k on {cores} host threads, sparse gather "
+                                         f"single-threaded) x{reps} reps; GPU indices and rows checked equal"}
+    print(json.dumps(res), flush=True)
 
 
 def cpu_baseline(pool0, tables_np, seq_lens_np, out, budget_s, hip, tables, seq_lens, cu, B, blocks,

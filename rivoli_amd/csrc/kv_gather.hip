@@ -6,11 +6,12 @@
 // operation and the narrowing is one rounding, so the result is bit-identical to the CPU
 // rule whatever the schedule.
 //
-// Dense: one workgroup per (sequence, page). A page's codes are one contiguous run and so is
-// its destination (tokens of a page are consecutive in the output), so the kernel is a
-// streaming transform: every lane loads 8 bytes of codes (a wave covers 512 contiguous
-// bytes) and stores 16 bytes of bf16 (a wave covers 1 KiB contiguous). All of a thread's
-// loads are issued before the first use to keep enough bytes in flight for HBM.
+// Dense: one workgroup per 16 rows of a (sequence, page). A page's codes are one contiguous
+// run and so is its destination (tokens of a page are consecutive in the output), so the
+// kernel is a streaming transform: every lane loads 8 bytes of codes (a wave covers 512
+// contiguous bytes) and stores 16 bytes of bf16 (a wave covers 1 KiB contiguous). All of a
+// thread's loads are issued before the first use. Loads and stores carry the nontemporal
+// hint: nothing here is read twice, and without it the kernel runs ~10% slower.
 // Sparse: one workgroup per 32 selected rows of one query; the 32 row bases and scales are
 // resolved once into LDS (block-table lookup), then the same 8-in/16-out streaming body runs
 // over the 32 x width bytes.
@@ -30,46 +31,55 @@ __device__ __forceinline__ u32x4 dequant8_bf16(u32x2 codes, float scale) {
 }
 
 // W / PT are the compile-time row width and page size (0 = take the runtime value), so the
-// flagship 576 x 64 shape gets constant divisors and a fully unrolled body.
-template <int W, int PT, int UNROLL>
-__global__ __launch_bounds__(kGatherThreads) void kv_gather_paged_kernel(
+// flagship 576 x 64 shape gets constant divisors and a fully unrolled body. A workgroup owns
+// ROWS consecutive rows of one page (PT / ROWS workgroups per page): measured on MI355X,
+// work units of 8-16 rows with one or two chunks per thread keep the chip's in-flight writes
+// on a compact, nearly sequential frontier of the output and run ~7% faster than one
+// workgroup per page.
+template <int W, int PT, int THREADS, int ROWS>
+__global__ __launch_bounds__(THREADS) void kv_gather_paged_kernel(
     const uint8_t* __restrict__ pool, const int* __restrict__ block_table,
     const int* __restrict__ seq_lens, const int* __restrict__ cu_seqlens,
     uint16_t* __restrict__ out, int max_blocks_per_seq, int width_rt, int page_tokens_rt,
     int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_pages) {
     const int width = W ? W : width_rt;
     const int pt = PT ? PT : page_tokens_rt;
+    const int parts = pt / ROWS;
     const int s = blockIdx.y;
-    const int t0 = (int)blockIdx.x * pt;
+    const int blk = (int)blockIdx.x / parts;
+    const int part = (int)blockIdx.x - blk * parts;
+    const int t0 = blk * pt + part * ROWS;
     const int len = seq_lens[s];
     if (t0 >= len) return;
-    const int valid = min(pt, len - t0);
-    const int page = block_table[(size_t)s * max_blocks_per_seq + blockIdx.x];
+    const int valid = min(ROWS, len - t0);
+    const int page = block_table[(size_t)s * max_blocks_per_seq + blk];
     if ((unsigned)page >= (unsigned)n_pages) {
-        if (threadIdx.x == 0 && bad_pages) atomicAdd(bad_pages, 1u);
+        if (threadIdx.x == 0 && part == 0 && bad_pages) atomicAdd(bad_pages, 1u);
         return;
     }
     const uint8_t* pg = pool + (size_t)page * page_bytes;
-    const u32x2* src = reinterpret_cast<const u32x2*>(pg);
-    const float* scales = reinterpret_cast<const float*>(pg + (size_t)pt * width);
+    const u32x2* src = reinterpret_cast<const u32x2*>(pg + (size_t)part * ROWS * width);
+    const float* scales = reinterpret_cast<const float*>(pg + (size_t)pt * width) + part * ROWS;
     u32x4* dst = reinterpret_cast<u32x4*>(out + ((size_t)cu_seqlens[s] + t0) * width);
     const int cpr = width >> 3;  // 8-byte chunks per row
     const int n_chunks = valid * cpr;
+    // trips is a constant for a compile-time width, so the two loops below unroll fully
+    constexpr int kMaxTrips = W ? (ROWS * (W / 8) + THREADS - 1) / THREADS : 4;
 
-    for (int base = threadIdx.x; base < n_chunks; base += kGatherThreads * UNROLL) {
-        u32x2 raw[UNROLL];
-        float scl[UNROLL];
+    for (int base = threadIdx.x; base < n_chunks; base += THREADS * kMaxTrips) {
+        u32x2 raw[kMaxTrips];
+        float scl[kMaxTrips];
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            int c = base + u * kGatherThreads;
+        for (int u = 0; u < kMaxTrips; ++u) {
+            int c = base + u * THREADS;
             if (c < n_chunks) {
                 raw[u] = __builtin_nontemporal_load(src + c);
                 scl[u] = scales[c / cpr];
             }
         }
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            int c = base + u * kGatherThreads;
+        for (int u = 0; u < kMaxTrips; ++u) {
+            int c = base + u * THREADS;
             if (c < n_chunks) __builtin_nontemporal_store(dequant8_bf16(raw[u], scl[u]), dst + c);
         }
     }
@@ -178,16 +188,25 @@ extern "C" int rivoli_kv_gather_paged(const unsigned char* pool, const int* bloc
     if (n_seqs > 65535) return 1002;
     if (!shape_ok(width, page_tokens)) return 1004;
     const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
-    dim3 grid((unsigned)max_blocks_per_seq, (unsigned)n_seqs);
     (void)hipGetLastError();
     if (width == 576 && page_tokens == 64) {
-        hipLaunchKernelGGL((kv_gather_paged_kernel<576, 64, 18>), grid, dim3(kGatherThreads), 0,
-                           (hipStream_t)stream, pool, block_table, seq_lens, cu_seqlens, out,
+        constexpr int kRows = 16, kThreads = 768;
+        dim3 grid((unsigned)max_blocks_per_seq * (64 / kRows), (unsigned)n_seqs);
+        hipLaunchKernelGGL((kv_gather_paged_kernel<576, 64, kThreads, kRows>), grid, dim3(kThreads),
+                           0, (hipStream_t)stream, pool, block_table, seq_lens, cu_seqlens, out,
                            max_blocks_per_seq, width, page_tokens, n_pages, page_bytes, bad_pages);
+    } else if (page_tokens % 16 == 0) {
+        dim3 grid((unsigned)max_blocks_per_seq * (unsigned)(page_tokens / 16), (unsigned)n_seqs);
+        hipLaunchKernelGGL((kv_gather_paged_kernel<0, 0, kGatherThreads, 16>), grid,
+                           dim3(kGatherThreads), 0, (hipStream_t)stream, pool, block_table,
+                           seq_lens, cu_seqlens, out, max_blocks_per_seq, width, page_tokens,
+                           n_pages, page_bytes, bad_pages);
     } else {
-        hipLaunchKernelGGL((kv_gather_paged_kernel<0, 0, 4>), grid, dim3(kGatherThreads), 0,
-                           (hipStream_t)stream, pool, block_table, seq_lens, cu_seqlens, out,
-                           max_blocks_per_seq, width, page_tokens, n_pages, page_bytes, bad_pages);
+        dim3 grid((unsigned)max_blocks_per_seq * (unsigned)(page_tokens / 4), (unsigned)n_seqs);
+        hipLaunchKernelGGL((kv_gather_paged_kernel<0, 0, kGatherThreads, 4>), grid,
+                           dim3(kGatherThreads), 0, (hipStream_t)stream, pool, block_table,
+                           seq_lens, cu_seqlens, out, max_blocks_per_seq, width, page_tokens,
+                           n_pages, page_bytes, bad_pages);
     }
     return launch_status();
 }
