@@ -1,0 +1,122 @@
+"""BASELINE configs 3 and 4 at their real per-layer shapes: byte comparison against the
+oracle where the host can hold it, and size-independent properties (page-permutation
+invariance, sparse == dense[rows], the XOR fold computed on the device equal to the oracle's
+fold) for the rest."""
+import numpy as np
+import pytest
+
+from rivoli_amd import hip
+from tests.churn import token_rows
+from tests.gpu_util import back, dev, dzeros, torch_cuda
+from tests.util import shuffled_block_tables
+
+pytestmark = pytest.mark.gpu
+W, PT = 576, 64
+
+
+def device_fold(t, n_words):
+    out = dzeros(8)
+    hip.launch_hash_rows(t, n_words, 1, 0, out)
+    return int(back(out, np.uint64)[0])
+
+
+def test_config3_one_layer_ragged_batch32(oracle):
+    """48 layers repeat this; one layer at the config's shape: batch 32, ctx ~ U[1024, 32768]
+    from seed, pages from a shuffled global pool; append everything, then append one more
+    token per sequence (the decode step), then gather every sequence's full context."""
+    rng = np.random.default_rng(0x5EED0003)
+    B = 32
+    ctx = rng.integers(1024, 32769, B).astype(np.int32)
+    blocks = -(-(ctx + 1) // PT)
+    max_blocks = int(blocks.max())
+    n_pages = int(blocks.sum()) + 7
+    perm = rng.permutation(n_pages).astype(np.int32)
+    tables = np.zeros((B, max_blocks), np.int32)
+    at = 0
+    for s in range(B):
+        tables[s, : blocks[s]] = perm[at: at + blocks[s]]
+        at += blocks[s]
+    slots = np.concatenate([tables[s][np.arange(ctx[s]) // PT] * PT + np.arange(ctx[s]) % PT
+                            for s in range(B)]).astype(np.int32)
+    rows = token_rows(rng, int(ctx.sum()))
+    page_bytes = oracle.kv_page_bytes(PT, W)
+    want_pool = np.zeros(n_pages * page_bytes, np.uint8)
+    oracle.kv_append_paged(rows, slots, want_pool, W, PT, n_pages, n_threads=8)
+    pool = dzeros(n_pages * page_bytes)
+    hip.launch_kv_append_paged(dev(rows), dev(slots), pool, slots.size, W, PT, n_pages)
+    # the decode step: one new token per sequence at position ctx[s]
+    new_rows = token_rows(rng, B)
+    new_slots = (tables[np.arange(B), ctx // PT] * PT + ctx % PT).astype(np.int32)
+    oracle.kv_append_paged(new_rows, new_slots, want_pool, W, PT, n_pages)
+    hip.launch_kv_append_paged(dev(new_rows), dev(new_slots), pool, B, W, PT, n_pages)
+    assert np.array_equal(back(pool), want_pool)
+
+    lens = (ctx + 1).astype(np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    out = dzeros(int(cu[-1]) * W * 2)
+    hip.launch_kv_gather_paged(pool, dev(tables), dev(lens), dev(cu), out, B, max_blocks, W, PT,
+                               n_pages)
+    want = oracle.kv_gather_paged(want_pool, tables, lens, W, PT, n_threads=8)
+    n_words = int(cu[-1]) * W // 2
+    assert device_fold(out, n_words) == oracle.xor_fold(want)      # one u64 for 600+ MB
+    assert np.array_equal(back(out, np.uint16).reshape(-1, W), want)
+
+
+def test_config4_one_layer_topk_then_sparse_gather(oracle):
+    """16 queries x 65536 tokens, k = 2048, fragmented pages: the selected rows gathered
+    sparsely equal the dense gather indexed by the same rows, and both equal the oracle."""
+    torch = torch_cuda()
+    rng = np.random.default_rng(0x5EED0004)
+    B, nt, k = 16, 65536, 2048
+    blocks = nt // PT
+    n_pages = B * blocks
+    tables = shuffled_block_tables(B, blocks, n_pages, seed=0x5EED0004 % 9973)
+    pos = np.arange(nt)
+    page_bytes = oracle.kv_page_bytes(PT, W)
+    pool = dzeros(n_pages * page_bytes)
+    for s in range(B):      # sequence by sequence keeps the host arrays small
+        rows = token_rows(rng, nt)
+        slots = (tables[s][pos // PT] * PT + pos % PT).astype(np.int32)
+        hip.launch_kv_append_paged(dev(rows), dev(slots), pool, nt, W, PT, n_pages)
+    scores = rng.standard_normal((B, nt), dtype=np.float32)
+    scores[:, -64:] += np.float32(4.0)
+    sel = dzeros(B * k * 4, 0xFF)
+    hip.launch_index_topk_batched(dev(scores), B, nt, None, nt, k, sel)
+    sel_np = back(sel, np.uint32).reshape(B, k)
+    assert np.array_equal(sel_np, oracle.topk_batched(scores, k, n_threads=8))
+    sparse = dzeros(B * k * W * 2)
+    tables_d = dev(tables)
+    hip.launch_kv_gather_rows_paged(pool, tables_d, sel, None, sparse, B, k, blocks, W, PT, n_pages)
+    lens = np.full(B, nt, np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    dense = dzeros(B * nt * W * 2)
+    hip.launch_kv_gather_paged(pool, tables_d, dev(lens), dev(cu), dense, B, blocks, W, PT, n_pages)
+    idx = torch.from_numpy(sel_np.astype(np.int64) + (np.arange(B, dtype=np.int64) * nt)[:, None]).cuda()
+    picked = dense.view(torch.int16).view(B * nt, W)[idx.reshape(-1)]
+    assert torch.equal(picked, sparse.view(torch.int16).view(B * k, W))
+    # and against the oracle on the host for the first two queries' pages
+    host_pool = back(pool)
+    want = oracle.kv_gather_rows_paged(host_pool, tables[:2], sel_np[:2], W, PT)
+    assert np.array_equal(back(sparse, np.uint16).reshape(B, k, W)[:2], want)
+
+
+def test_gather_output_is_independent_of_page_placement_at_scale(oracle):
+    """The same 8 x 8192 tokens through two different shuffles of a 1024-page pool fold to the
+    same u64 on the device."""
+    rng = np.random.default_rng(77)
+    B, ctx, n_pages = 8, 8192, 1100
+    rows = token_rows(rng, B * ctx)
+    folds = []
+    for seed in (1, 2):
+        tables = shuffled_block_tables(B, ctx // PT, n_pages, seed)
+        pos = np.arange(ctx)
+        slots = np.concatenate([tables[s][pos // PT] * PT + pos % PT for s in range(B)]).astype(np.int32)
+        pool = dzeros(n_pages * oracle.kv_page_bytes(PT, W), 0xEE)
+        hip.launch_kv_append_paged(dev(rows), dev(slots), pool, B * ctx, W, PT, n_pages)
+        lens = np.full(B, ctx, np.int32)
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        out = dzeros(B * ctx * W * 2)
+        hip.launch_kv_gather_paged(pool, dev(tables), dev(lens), dev(cu), out, B, ctx // PT, W, PT,
+                                   n_pages)
+        folds.append(device_fold(out, B * ctx * W // 2))
+    assert folds[0] == folds[1] and folds[0] != 0

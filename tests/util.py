@@ -4,8 +4,13 @@ import numpy as np
 
 def f32_to_bf16_rne(x: np.ndarray) -> np.ndarray:
     """Textbook integer round-to-nearest-even; finite inputs only."""
-    b = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
-    return ((b + 0x7FFF + ((b >> 16) & 1)) >> 16).astype(np.uint16)
+    b = np.ascontiguousarray(x, np.float32).view(np.uint32)
+    # uint32 arithmetic cannot wrap for finite inputs (|bits| <= 0x7f7fffff before the add)
+    r = (b >> np.uint32(16)) & np.uint32(1)
+    r += np.uint32(0x7FFF)
+    r += b
+    r >>= np.uint32(16)
+    return r.astype(np.uint16)
 
 
 def bf16_to_f32(b: np.ndarray) -> np.ndarray:
