@@ -290,6 +290,7 @@ def bench_dsa(a, torch, hip):
         scores.append(sc)
     sel = torch.empty(B * k, dtype=torch.int32, device="cuda")
     out = torch.empty(B * k * W, dtype=torch.bfloat16, device="cuda")
+    ws = torch.zeros(hip.index_topk_workspace_bytes(B, nt), dtype=torch.uint8, device="cuda")
     torch.cuda.synchronize()
     stream = torch.cuda.Stream()
     sh = stream.cuda_stream
@@ -297,7 +298,7 @@ def bench_dsa(a, torch, hip):
     def step(events):
         for layer in range(L):
             bracket(torch, stream, events, "topk",
-                    lambda: hip.launch_index_topk_batched(scores[layer], B, nt, None, nt, k, sel, sh))
+                    lambda: hip.launch_index_topk_batched(scores[layer], B, nt, None, nt, k, sel, ws, sh))
             bracket(torch, stream, events, "gather_rows",
                     lambda: hip.launch_kv_gather_rows_paged(pools[layer], tables, sel, None, out, B, k,
                                                             blocks, W, PT, n_pages, None, sh))
@@ -334,7 +335,7 @@ def bench_dsa(a, torch, hip):
             want_rows = ora.kv_gather_rows_paged(pool_h, tables_np, want_sel, W, PT)
             spent += time.perf_counter() - t0
             reps += 1
-        hip.launch_index_topk_batched(scores[0], B, nt, None, nt, k, sel)
+        hip.launch_index_topk_batched(scores[0], B, nt, None, nt, k, sel, ws)
         hip.launch_kv_gather_rows_paged(pools[0], tables, sel, None, out, B, k, blocks, W, PT, n_pages)
         torch.cuda.synchronize()
         if not np.array_equal(sel.cpu().numpy().view(np.uint32).reshape(B, k), want_sel):

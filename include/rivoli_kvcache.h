@@ -107,11 +107,17 @@ int rivoli_kv_gather_rows_paged(const unsigned char* pool, const int* block_tabl
                                 unsigned int* bad_rows, void* stream);
 
 /* Batched rivoli_index_topk: query q reads scores[q*stride .. +nts[q]) (nt for every query
- * when nts is null) and writes rows[q*k .. +min(k, nt_q)), ascending. One launch for all
+ * when nts is null) and writes rows[q*k .. +min(k, nt_q)), ascending. One call for all
  * queries; the selection rule is the single-query one.
+ * `workspace` (nullable) lets the call spread every query over many workgroups instead of
+ * one: rivoli_index_topk_workspace_bytes(n_queries, nt) bytes of device memory that the
+ * caller zero-fills ONCE (hipMemset) before its first use; every call puts back to zero
+ * whatever has to start at zero, so it can be reused call after call on one stream (calls
+ * that share a workspace must not overlap). With a null workspace each query is selected by a single workgroup.
  * Guards: 1001 null / non-positive; 1002 stride < nt. */
+size_t rivoli_index_topk_workspace_bytes(int n_queries, int nt);
 int rivoli_index_topk_batched(const float* scores, int n_queries, int stride, const int* nts,
-                              int nt, int k, unsigned int* rows, void* stream);
+                              int nt, int k, unsigned int* rows, void* workspace, void* stream);
 
 /* Element codecs as launchers (what formats.hpp:42-57,99-106 and fwd.hip:20-45 are to the
  * reference's kernels), for census tests of the device codecs on arbitrary inputs:

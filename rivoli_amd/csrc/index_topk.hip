@@ -5,25 +5,38 @@
 // ties by index ascending; take the first min(k, nt); write that SET in index order. Entries
 // past min(k, nt) are not written. NaN scores are out of contract on both sides.
 //
-// Shape: one 1024-thread workgroup (16 wave64) per query, all queries in one launch. Each
-// wave owns a contiguous segment of the score array and keeps its order-preserving u32 keys
-// in registers (up to 64 per lane = 65536 scores per query), so the scores are read from
-// memory once. Selection is a 4-pass, 8-bit, MSB-first radix select of the k-th largest key.
-// Score arrays concentrate in a handful of exponent bytes, so each histogram bin is
-// replicated 32 times in LDS, one copy per bank (copy = lane mod 32): a wave's 64 atomic
-// increments then never collide inside one instruction whatever the digit distribution.
-// Compaction needs no atomics: a selected element's slot is
-//   (# keys > pivot before it) + min(# keys == pivot before it, need),
-// monotone in the index; within a wave those prefixes are ballots and popcounts, across
-// waves one 16-entry prefix. Longer arrays (nt > 65536) stream the keys from memory on every
-// sweep with the same code.
+// Two shapes share one selection rule.
+//
+// (1) One workgroup per query (`topk_block`): each wave owns a contiguous segment of the
+//     score array and keeps its order-preserving u32 keys in registers (up to 64 per lane),
+//     so the scores are read once. Selection is a 4-pass, 8-bit, MSB-first radix select of the
+//     k-th largest key. Score arrays concentrate in a handful of exponent bytes, so each
+//     histogram bin is replicated 32 times in LDS, one copy per bank (copy = lane mod 32): a
+//     wave's 64 atomic increments never collide inside one instruction whatever the digit
+//     distribution. Compaction needs no atomics: a selected element's slot is
+//       (# keys > pivot before it) + min(# keys == pivot before it, need),
+//     monotone in the index; within a wave those prefixes are ballots and popcounts, across
+//     waves one short prefix. It needs no scratch memory, so it serves the reference-signature
+//     entry point; but 65536 keys x several sweeps on ONE compute unit is issue-bound.
+//
+// (2) Split across the chip (`topk_hist_kernel` + `topk_select_kernel`), used when the caller
+//     supplies a workspace: every 4096-score segment of every query gets its own workgroup.
+//     Kernel A histograms the top 12 key bits per query in global memory (LDS histogram first,
+//     then one atomic per non-empty bin); the LAST workgroup of a query to finish — decided by
+//     a ticket, never by waiting — walks the histogram for the bin that holds the k-th key.
+//     Kernel B writes, per segment and in index order, the indices whose key is in that bin or
+//     above (at least k of them, typically ~1.5 k); the last workgroup of the query pulls those
+//     candidates into LDS, finishes the radix select on the low 20 bits among the bin's
+//     members, and emits the selection in index order. If the candidates do not fit in LDS
+//     (degenerate score arrays: huge ties) that workgroup runs shape (1) over the query
+//     instead — slower, same answer. The workspace is left zeroed for the next call.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
+#include <type_traits>
+
 #include "codec.hpp"
 
 namespace rk {
 
-constexpr int kTopkThreads = 1024;
-constexpr int kTopkWaves = kTopkThreads / kWave;
 constexpr int kBins = 256;
 constexpr int kCopies = 32;
 
@@ -39,41 +52,82 @@ __device__ __forceinline__ uint32_t lanes_below(unsigned long long mask) {
                                      __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
 
+// A load that other workgroups' writes (made visible by a fence + ticket) are seen by.
+__device__ __forceinline__ uint32_t load_agent(const uint32_t* p) {
+    return __hip_atomic_load(const_cast<uint32_t*>(p), __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // One sweep over a lane's elements: a compile-time trip count when the keys live in
 // registers (so every key[j] is a register, never scratch), a runtime one when streaming.
 template <int ITEMS, class F>
 __device__ __forceinline__ void sweep(int steps, F&& body) {
     if constexpr (ITEMS > 0) {
 #pragma unroll
-        for (int j = 0; j < ITEMS; ++j)
+        for (int j = 0; j < ITEMS; ++j) {
             if (j < steps) body(j);
+            // keep each step's temporaries from being hoisted across steps: with 64 keys per
+            // lane live, the register budget (128 at 1024 threads) has no room for that
+            __builtin_amdgcn_sched_barrier(0);
+        }
     } else {
         for (int j = 0; j < steps; ++j) body(j);
     }
 }
 
-// ITEMS: keys per lane kept in registers; 0 = re-read the scores on every sweep.
-template <int ITEMS>
-__global__ __launch_bounds__(kTopkThreads) void index_topk_kernel(
-    const float* __restrict__ scores, int stride, const int* __restrict__ nts, int nt_all, int k,
-    uint32_t* __restrict__ rows) {
-    __shared__ uint32_t s_hist[kBins * kCopies];
-    __shared__ uint32_t s_bins[kBins];
-    __shared__ uint32_t s_wave[kTopkWaves];
-    __shared__ uint32_t s_pivot, s_need;
+// Wave 0 only. bins[256] hold counts; finds the highest bin b with
+// (count of bins >= b) >= need and publishes {b, need - count of bins > b} to pn[0..1].
+// Exactly one lane publishes when the total is >= need.
+__device__ __forceinline__ void find_pivot_bin(const uint32_t* bins, uint32_t need, uint32_t* pn,
+                                               int lane) {
+    uint32_t c[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) c[b] = bins[lane * 4 + b];
+    const uint32_t tot = c[0] + c[1] + c[2] + c[3];
+    uint32_t suffix = tot;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        uint32_t v = __shfl_down(suffix, off, kWave);
+        if (lane + off < kWave) suffix += v;
+    }
+    const uint32_t above = suffix - tot;
+    if (above < need && need <= suffix) {
+        uint32_t acc = above;
+        int b = 3;
+        for (; b > 0; --b) {
+            if (acc + c[b] >= need) break;
+            acc += c[b];
+        }
+        pn[0] = (uint32_t)(lane * 4 + b);
+        pn[1] = need - acc;
+    }
+}
 
-    const int q = blockIdx.x;
-    int nt = nts ? min(nts[q], nt_all) : nt_all;
-    if (nt <= 0) return;
-    const uint32_t kq = (uint32_t)min(k, nt);
-    const float* s = scores + (size_t)q * stride;
-    uint32_t* out = rows + (size_t)q * k;
+// LDS a workgroup of THREADS needs for topk_block, in u32 words.
+template <int THREADS>
+constexpr int topk_block_lds_words() {
+    return kBins * kCopies + kBins + 2 * (THREADS / kWave) + 2;
+}
+
+// Shape (1): the whole selection for one query by one workgroup of THREADS threads.
+// ITEMS: keys per lane kept in registers; 0 = re-read the scores on every sweep.
+template <int THREADS, int ITEMS>
+__device__ __forceinline__ void topk_block(const float* __restrict__ s, int nt, uint32_t kq,
+                                           uint32_t* __restrict__ out, uint32_t* lds) {
+    constexpr int WAVES = THREADS / kWave;
+    constexpr int TPB = THREADS / kBins;  // threads that share one bin's copies
+    static_assert(TPB == 1 || TPB == 4, "256 or 1024 threads");
+    uint32_t* s_hist = lds;
+    uint32_t* s_bins = s_hist + kBins * kCopies;
+    uint32_t* s_gt = s_bins + kBins;
+    uint32_t* s_eq = s_gt + WAVES;
+    uint32_t* s_pn = s_eq + WAVES;
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid >> 6;
     // Each wave owns per_wave consecutive scores, a multiple of 64, walked 64 at a time.
-    const int per_wave = ((nt + kTopkThreads - 1) / kTopkThreads) * kWave;
+    const int per_wave = ((nt + THREADS - 1) / THREADS) * kWave;
     const int steps = per_wave / kWave;
     const long long seg0 = (long long)wave * per_wave;
     // element (j, lane) is index seg0 + j*64 + lane; it exists iff j*64 < limit
@@ -81,19 +135,32 @@ __global__ __launch_bounds__(kTopkThreads) void index_topk_kernel(
     const int limit = (int)(rem < per_wave ? rem : per_wave) - lane;
 
     uint32_t key[ITEMS ? ITEMS : 1];
-    if (ITEMS) {
+    if constexpr (ITEMS > 0) {
+        // A wave whose whole segment exists (wave-uniform test) issues every load off one
+        // base register before the first use; only the array's last, partial segment takes
+        // the predicated path.
+        const float* sp = s + seg0 + lane;
+        if (rem >= per_wave) {
 #pragma unroll
-        for (int j = 0; j < ITEMS; ++j)
-            key[j] = (j * kWave < limit) ? topk_key(s[seg0 + j * kWave + lane]) : 0u;
+            for (int j = 0; j < ITEMS; ++j)
+                key[j] = j < steps ? __float_as_uint(sp[j * kWave]) : 0u;
+#pragma unroll
+            for (int j = 0; j < ITEMS; ++j)
+                key[j] = j < steps ? topk_key(__uint_as_float(key[j])) : 0u;
+        } else {
+#pragma unroll
+            for (int j = 0; j < ITEMS; ++j)
+                key[j] = (j * kWave < limit) ? topk_key(sp[j * kWave]) : 0u;
+        }
     }
     auto key_at = [&](int j) -> uint32_t {
-        if (ITEMS) return key[j];
+        if constexpr (ITEMS > 0) return key[j];
         return (j * kWave < limit) ? topk_key(s[seg0 + (long long)j * kWave + lane]) : 0u;
     };
 
     uint32_t pivot = 0u, mask = 0u, need = kq;
     for (int shift = 24; shift >= 0; shift -= 8) {
-        for (int i = tid; i < kBins * kCopies; i += kTopkThreads) s_hist[i] = 0u;
+        for (int i = tid; i < kBins * kCopies; i += THREADS) s_hist[i] = 0u;
         __syncthreads();
         sweep<ITEMS>(steps, [&](int j) {
             const uint32_t u = key_at(j);
@@ -102,44 +169,24 @@ __global__ __launch_bounds__(kTopkThreads) void index_topk_kernel(
         });
         __syncthreads();
         {
-            // four threads per bin, eight copies each, rotated so a wave spreads over banks
-            const int bin = tid >> 2, part = tid & 3;
+            // TPB threads per bin, 32/TPB copies each, rotated so a wave spreads over banks
+            constexpr int PER = kCopies / TPB;
+            const int bin = tid / TPB, part = tid % TPB;
             uint32_t sum = 0;
 #pragma unroll
-            for (int c = 0; c < 8; ++c) sum += s_hist[bin * kCopies + part * 8 + ((c + lane) & 7)];
-            sum += __shfl_xor(sum, 1, kWave);
-            sum += __shfl_xor(sum, 2, kWave);
+            for (int c = 0; c < PER; ++c)
+                sum += s_hist[bin * kCopies + part * PER + ((c + lane) & (PER - 1))];
+            if (TPB == 4) {
+                sum += __shfl_xor(sum, 1, kWave);
+                sum += __shfl_xor(sum, 2, kWave);
+            }
             if (part == 0) s_bins[bin] = sum;
         }
         __syncthreads();
-        if (wave == 0) {
-            // lane L owns bins 4L..4L+3. Walk from the top bin down for the one holding the
-            // need-th candidate: the lane whose inclusive suffix count first reaches need.
-            uint32_t c[4];
-#pragma unroll
-            for (int b = 0; b < 4; ++b) c[b] = s_bins[lane * 4 + b];
-            const uint32_t tot = c[0] + c[1] + c[2] + c[3];
-            uint32_t suffix = tot;
-#pragma unroll
-            for (int off = 1; off < kWave; off <<= 1) {
-                uint32_t v = __shfl_down(suffix, off, kWave);
-                if (lane + off < kWave) suffix += v;
-            }
-            const uint32_t above = suffix - tot;
-            if (above < need && need <= suffix) {
-                uint32_t acc = above;
-                int b = 3;
-                for (; b > 0; --b) {
-                    if (acc + c[b] >= need) break;
-                    acc += c[b];
-                }
-                s_pivot = pivot | ((uint32_t)(lane * 4 + b) << shift);
-                s_need = need - acc;
-            }
-        }
+        if (wave == 0) find_pivot_bin(s_bins, need, s_pn, lane);
         __syncthreads();
-        pivot = s_pivot;
-        need = s_need;
+        pivot |= s_pn[0] << shift;
+        need = s_pn[1];
         mask |= 0xffu << shift;
     }
 
@@ -154,14 +201,14 @@ __global__ __launch_bounds__(kTopkThreads) void index_topk_kernel(
     });
     const uint32_t gt_total = wave_sum(cnt_gt), eq_total = wave_sum(cnt_eq);
     if (lane == 0) {
-        s_wave[wave] = gt_total;
-        s_bins[wave] = eq_total;
+        s_gt[wave] = gt_total;
+        s_eq[wave] = eq_total;
     }
     __syncthreads();
     uint32_t run_gt = 0, run_eq = 0;
     for (int w = 0; w < wave; ++w) {
-        run_gt += s_wave[w];
-        run_eq += s_bins[w];
+        run_gt += s_gt[w];
+        run_eq += s_eq[w];
     }
     sweep<ITEMS>(steps, [&](int j) {
         const uint32_t u = key_at(j);
@@ -169,6 +216,7 @@ __global__ __launch_bounds__(kTopkThreads) void index_topk_kernel(
         const bool g = live && u > pivot;
         const bool e = live && u == pivot;
         const unsigned long long mg = __ballot(g), me = __ballot(e);
+        if ((mg | me) == 0ull) return;  // wave-uniform: most steps select nothing
         const uint32_t G = run_gt + lanes_below(mg);
         const uint32_t E = run_eq + lanes_below(me);
         const uint32_t slot = G + (E < need ? E : need);
@@ -181,36 +229,590 @@ __global__ __launch_bounds__(kTopkThreads) void index_topk_kernel(
     });
 }
 
+constexpr int kTopkThreads = 1024;
+constexpr int kTopkWaves = kTopkThreads / kWave;
+
+// Shape (1), lean form for register-resident queries (nt <= 65536). A compute unit issues
+// about one wave-instruction per cycle, so what a single workgroup pays for is instructions
+// per key; sweeping all keys four times plus two compaction sweeps (topk_block) costs ~110 of
+// them. Here all keys are swept three times with a few instructions each — one 10-bit
+// histogram pass (1024 bins x 8 bank copies), one count, one ordered compaction of the keys
+// in the pivot bin or above into LDS — and everything after that (the remaining 22 bits of
+// the radix select, the ordered emission) runs over those few thousand candidates only.
+// Falls back to topk_block when the candidates do not fit (degenerate score arrays).
+constexpr int kLeanBits = 10;
+constexpr int kLeanBins = 1 << kLeanBits;  // == kTopkThreads: one thread per bin
+constexpr int kLeanCopies = 8;
+constexpr int kLeanLow = 32 - kLeanBits;
+constexpr int kLeanCap = 12288;  // candidates held in LDS (index + key)
+static_assert(kLeanBins == kTopkThreads, "one thread per bin");
+constexpr int kLeanLdsWords = 2 * kLeanCap + kLeanBins * kLeanCopies + 4 * kTopkWaves + 8;
+static_assert(topk_block_lds_words<kTopkThreads>() <= kLeanLdsWords, "fallback fits");
+static_assert(kLeanCap < 65536, "emission packs two counts into 16 bits each");
+
+// Sum over the 16 wave slots of v[w] for w < wave (*before) and over all of them (*all).
+// Lanes 0..15 read one slot each and a 4-step butterfly adds them: a couple of registers and
+// no dependent chain of LDS reads. Every lane of the wave must call it.
+__device__ __forceinline__ void wave_slots_prefix(const uint32_t* v, int wave, uint32_t* before,
+                                                  uint32_t* all) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t x = lane < kTopkWaves ? v[lane] : 0u;
+    uint32_t a = x, b = lane < wave ? x : 0u;
+#pragma unroll
+    for (int off = kTopkWaves / 2; off > 0; off >>= 1) {
+        a += __shfl_xor(a, off, kWave);
+        b += __shfl_xor(b, off, kWave);
+    }
+    *all = __builtin_amdgcn_readfirstlane(a);
+    *before = __builtin_amdgcn_readfirstlane(b);
+}
+
+template <int ITEMS>
+__device__ __forceinline__ void topk_block_lean(const float* __restrict__ s, int nt, uint32_t kq,
+                                                uint32_t* __restrict__ out, uint32_t* lds) {
+    uint32_t* c_idx = lds;  // the candidates, in index order
+    uint32_t* c_key = lds + kLeanCap;
+    uint32_t* s_hist = lds + 2 * kLeanCap;        // later reused as the 256-bin histogram
+    uint32_t* s_wa = s_hist + kLeanBins * kLeanCopies;
+    uint32_t* s_wb = s_wa + kTopkWaves;
+    uint32_t* s_pn = s_wb + kTopkWaves;  // [0] bin, [1] need, [2] candidate total
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    // the wave index as a scalar: everything derived from it (segment base, bounds, the load
+    // addresses' base) then lives in scalar registers instead of one vector register per use
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int per_wave = ((nt + kTopkThreads - 1) / kTopkThreads) * kWave;
+    const int steps = per_wave / kWave;
+    const int seg0 = wave * per_wave;
+    const int rem = nt - seg0;
+    const int limit = (rem < per_wave ? rem : per_wave) - lane;
+    // Wave-uniform: a wave whose whole segment exists needs no per-key bounds test. Each pass
+    // below is instantiated for both cases and the wave picks one.
+    const bool full = rem >= per_wave;
+    auto both = [&](auto&& pass) {
+        if (full) pass(std::true_type{});
+        else pass(std::false_type{});
+    };
+
+    uint32_t key[ITEMS];
+    {
+        // a scalar base per step plus one per-lane offset register for all 64 loads
+        const float* sw = s + seg0;
+        if (full) {  // all issued before the first use
+#pragma unroll
+            for (int j = 0; j < ITEMS; ++j)
+                key[j] = j < steps ? __float_as_uint((sw + j * kWave)[lane]) : 0u;
+#pragma unroll
+            for (int j = 0; j < ITEMS; ++j)
+                key[j] = j < steps ? topk_key(__uint_as_float(key[j])) : 0u;
+        } else {
+#pragma unroll
+            for (int j = 0; j < ITEMS; ++j)
+                key[j] = (j * kWave < limit) ? topk_key((sw + j * kWave)[lane]) : 0u;
+        }
+    }
+
+    // ---- pass 1: histogram of the top 10 bits ----
+    for (int i = tid; i < kLeanBins * kLeanCopies; i += kTopkThreads) s_hist[i] = 0u;
+    __syncthreads();
+    uint32_t* my_copy = s_hist + (lane & (kLeanCopies - 1));
+    both([&](auto F) {
+        sweep<ITEMS>(steps, [&](int j) {
+            if (decltype(F)::value || j * kWave < limit)
+                atomicAdd(&my_copy[(key[j] >> kLeanLow) * kLeanCopies], 1u);
+        });
+    });
+    __syncthreads();
+    uint32_t cnt = 0;
+#pragma unroll
+    for (int c = 0; c < kLeanCopies; ++c)
+        cnt += s_hist[tid * kLeanCopies + ((c + lane) & (kLeanCopies - 1))];
+    // suffix counts over threads (= bins): how many keys sit in higher bins than mine
+    uint32_t suffix = cnt;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        uint32_t v = __shfl_down(suffix, off, kWave);
+        if (lane + off < kWave) suffix += v;
+    }
+    if (lane == 0) s_wa[wave] = suffix;  // the wave's total
+    __syncthreads();
+    uint32_t lower, all;
+    wave_slots_prefix(s_wa, wave + 1, &lower, &all);
+    const uint32_t above = all - lower + (suffix - cnt);  // higher waves + higher lanes
+    if (above < kq && kq <= above + cnt) {
+        s_pn[0] = (uint32_t)tid;
+        s_pn[1] = kq - above;
+        s_pn[2] = above + cnt;
+    }
+    __syncthreads();
+    const uint32_t pbin = s_pn[0];
+    uint32_t need = s_pn[1];
+    const uint32_t total = s_pn[2];
+    if (total > (uint32_t)kLeanCap) {
+        // rare (huge ties): the streaming form re-reads the scores and needs no key registers
+        topk_block<kTopkThreads, 0>(s, nt, kq, out, lds);
+        return;
+    }
+
+    // ---- pass 2: candidates per wave (a candidate is key >= the pivot bin's first key) ----
+    const uint32_t thr = pbin << kLeanLow;
+    uint32_t mine = 0;
+    both([&](auto F) {
+        sweep<ITEMS>(steps, [&](int j) {
+            const bool is = (decltype(F)::value || j * kWave < limit) && key[j] >= thr;
+            mine += (uint32_t)__popcll(__ballot(is));  // scalar popcount: one VALU op per key
+        });
+    });
+    if (lane == 0) s_wb[wave] = mine;
+    __syncthreads();
+    uint32_t run, unused;
+    wave_slots_prefix(s_wb, wave, &run, &unused);
+
+    // ---- pass 3: ordered compaction of (index, key) into LDS ----
+    // the element index is carried as a running register (a per-step constant would be
+    // materialised 64 times over and spill)
+    uint32_t idx = (uint32_t)(seg0 + lane);
+    both([&](auto F) {
+        sweep<ITEMS>(steps, [&](int j) {
+            const bool is = (decltype(F)::value || j * kWave < limit) && key[j] >= thr;
+            const unsigned long long m = __ballot(is);
+            if (is) {
+                const uint32_t pos = run + lanes_below(m);
+                c_idx[pos] = idx;
+                c_key[pos] = key[j];
+            }
+            run += (uint32_t)__popcll(m);
+            idx += kWave;
+            asm volatile("" : "+v"(idx));  // keep the add where it is
+        });
+    });
+    __syncthreads();
+
+    // ---- the remaining 22 bits among the pivot bin's members: 8 + 8 + 6 ----
+    uint32_t* s_bins = s_hist;
+    uint32_t pivot = thr, mask = ~0u << kLeanLow;
+    for (int shift = kLeanLow - 8;; shift = shift >= 8 ? shift - 8 : 0) {
+        const uint32_t dmask = (shift == 0 && (kLeanLow % 8)) ? (1u << (kLeanLow % 8)) - 1u : 0xffu;
+        if (tid < kBins) s_bins[tid] = 0u;
+        __syncthreads();
+        for (uint32_t c = tid; c < total; c += kTopkThreads) {
+            const uint32_t u = c_key[c];
+            if ((u & mask) == pivot) atomicAdd(&s_bins[(u >> shift) & dmask], 1u);
+        }
+        __syncthreads();
+        if (wave == 0) find_pivot_bin(s_bins, need, s_pn, lane);
+        __syncthreads();
+        pivot |= s_pn[0] << shift;
+        need = s_pn[1];
+        mask |= dmask << shift;
+        if (shift == 0) break;
+    }
+
+    // ---- ordered emission: each thread owns a run of consecutive candidates ----
+    const uint32_t chunk = (total + kTopkThreads - 1) / kTopkThreads;
+    const uint32_t c_lo = min((uint32_t)tid * chunk, total), c_hi = min(c_lo + chunk, total);
+    uint32_t my_gt = 0, my_eq = 0;
+    for (uint32_t c = c_lo; c < c_hi; ++c) {
+        const uint32_t u = c_key[c];
+        my_gt += u > pivot ? 1u : 0u;
+        my_eq += u == pivot ? 1u : 0u;
+    }
+    // block-wide exclusive prefix of both counts, packed 16:16 (each total <= kLeanCap)
+    const uint32_t packed = my_gt | (my_eq << 16);
+    uint32_t incl = packed;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        uint32_t v = __shfl_up(incl, off, kWave);
+        if (lane >= off) incl += v;
+    }
+    if (lane == kWave - 1) s_wa[wave] = incl;
+    __syncthreads();
+    uint32_t before;
+    wave_slots_prefix(s_wa, wave, &before, &unused);
+    const uint32_t excl = before + incl - packed;
+    uint32_t G = excl & 0xffffu, E = excl >> 16;
+    for (uint32_t c = c_lo; c < c_hi; ++c) {
+        const uint32_t u = c_key[c];
+        const bool g = u > pivot, e = u == pivot;
+        const uint32_t slot = G + (E < need ? E : need);
+        // slot < kq holds by construction; the compare keeps a wrong pivot from ever
+        // turning into a write outside the caller's buffer
+        if ((g || (e && E < need)) && slot < kq) out[slot] = c_idx[c];
+        G += g ? 1u : 0u;
+        E += e ? 1u : 0u;
+    }
+}
+
+template <int ITEMS>
+__global__ __launch_bounds__(kTopkThreads) void index_topk_kernel(
+    const float* __restrict__ scores, int stride, const int* __restrict__ nts, int nt_all, int k,
+    uint32_t* __restrict__ rows) {
+    // static LDS: 128 KiB for the lean form (gfx950 has 160 KiB per workgroup), 33 KiB streaming
+    __shared__ uint32_t lds[ITEMS > 0 ? kLeanLdsWords : topk_block_lds_words<kTopkThreads>()];
+    const int q = blockIdx.x;
+    const int nt = nts ? min(nts[q], nt_all) : nt_all;
+    if (nt <= 0) return;
+    const float* s = scores + (size_t)q * stride;
+    uint32_t* out = rows + (size_t)q * k;
+    if constexpr (ITEMS > 0)
+        topk_block_lean<ITEMS>(s, nt, (uint32_t)min(k, nt), out, lds);
+    else
+        topk_block<kTopkThreads, 0>(s, nt, (uint32_t)min(k, nt), out, lds);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Shape (2): a query split over many workgroups.
+// ---------------------------------------------------------------------------------------------
+constexpr int kSegThreads = 256;
+constexpr int kSegWaves = kSegThreads / kWave;
+constexpr int kSegKeys = 4096;                     // scores per workgroup
+constexpr int kSegItems = kSegKeys / kSegThreads;  // 16 per thread
+constexpr int kTopBits = 12;
+constexpr int kTopBins = 1 << kTopBits;  // global histogram bins per query
+constexpr int kLowBits = 32 - kTopBits;
+constexpr int kCandCap = 8192;  // candidates the finishing workgroup can cache in LDS
+constexpr int kMaxSegs = 1024;  // segment prefix table held in LDS
+
+// Workspace, u32 words per query: [0,4096) histogram | 4096 ticket A | 4097 ticket B |
+// 4098 pivot bin | 4099 need | [4100, 4100+S) per-segment candidate counts | (pad to 4) |
+// S x 4096 candidate indices.
+constexpr int kWsTicketA = kTopBins, kWsTicketB = kTopBins + 1, kWsPivot = kTopBins + 2,
+              kWsNeed = kTopBins + 3, kWsCounts = kTopBins + 4;
+__host__ __device__ inline size_t topk_ws_cand_offset(int n_segs) {
+    return ((size_t)kWsCounts + (size_t)n_segs + 3) & ~(size_t)3;
+}
+static inline size_t topk_ws_words(int n_segs) {
+    return topk_ws_cand_offset(n_segs) + (size_t)n_segs * kSegKeys;
+}
+
+// A workgroup's 4096 keys: element (j, tid) is index seg*4096 + j*256 + tid.
+__device__ __forceinline__ void load_segment_keys(const float* __restrict__ s, int nt, int seg,
+                                                  uint32_t (&key)[kSegItems], int& limit) {
+    const int base = seg * kSegKeys + (int)threadIdx.x;
+    limit = nt - base;  // element j exists iff j*256 < limit
+    float raw[kSegItems];
+#pragma unroll
+    for (int j = 0; j < kSegItems; ++j) {
+        int i = base + j * kSegThreads;
+        raw[j] = s[i < nt ? i : nt - 1];
+    }
+#pragma unroll
+    for (int j = 0; j < kSegItems; ++j) key[j] = topk_key(raw[j]);
+}
+
+// Exclusive prefix sum of one value per thread over a 256-thread workgroup, in thread order;
+// *total receives the workgroup sum. tmp holds kSegWaves words. Every thread must call it.
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* tmp,
+                                                         uint32_t* total) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    uint32_t incl = v;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        uint32_t t = __shfl_up(incl, off, kWave);
+        if (lane >= off) incl += t;
+    }
+    __syncthreads();  // tmp may still be read from a previous use
+    if (lane == kWave - 1) tmp[wave] = incl;
+    __syncthreads();
+    uint32_t before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < kSegWaves; ++w) {
+        if (w < wave) before += tmp[w];
+        all += tmp[w];
+    }
+    *total = all;
+    return before + incl - v;
+}
+
+// True in exactly one workgroup of the n that share `ticket`: the last to arrive. Nobody
+// waits: the others simply leave. Every wave first drains its own stores into L2, then ONE
+// wave publishes the workgroup's writes device-wide (an L2 write-back is expensive, and 256
+// workgroups x 4 waves of them were measured to cost more than the kernel's real work).
+__device__ __forceinline__ bool last_to_arrive(uint32_t* ticket, uint32_t n, uint32_t* s_flag) {
+    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wave's global stores have completed
+    __syncthreads();
+    if (threadIdx.x < kWave) {
+        __threadfence();
+        if (threadIdx.x == 0) *s_flag = atomicAdd(ticket, 1u);
+    }
+    __syncthreads();
+    const bool last = *s_flag == n - 1;
+    if (last) __threadfence();  // the others' writes are visible after the last ticket
+    return last;
+}
+
+__global__ __launch_bounds__(kSegThreads) void topk_hist_kernel(
+    const float* __restrict__ scores, int stride, const int* __restrict__ nts, int nt_all, int k,
+    uint32_t* __restrict__ ws, size_t ws_stride) {
+    __shared__ uint32_t s_hist[kTopBins];
+    __shared__ uint32_t s_scan[kSegWaves];
+    __shared__ uint32_t s_flag;
+    const int q = blockIdx.y, seg = blockIdx.x, tid = threadIdx.x;
+    const int nt = nts ? min(nts[q], nt_all) : nt_all;
+    if (nt <= 0) return;
+    const uint32_t kq = (uint32_t)min(k, nt);
+    uint32_t* w = ws + (size_t)q * ws_stride;
+
+    for (int i = tid; i < kTopBins; i += kSegThreads) s_hist[i] = 0u;
+    __syncthreads();
+    if (seg * kSegKeys < nt) {
+        uint32_t key[kSegItems];
+        int limit;
+        load_segment_keys(scores + (size_t)q * stride, nt, seg, key, limit);
+#pragma unroll
+        for (int j = 0; j < kSegItems; ++j)
+            if (j * kSegThreads < limit) atomicAdd(&s_hist[key[j] >> kLowBits], 1u);
+    }
+    __syncthreads();
+    for (int b = tid; b < kTopBins; b += kSegThreads) {
+        const uint32_t c = s_hist[b];
+        if (c) atomicAdd(&w[b], c);
+    }
+    if (!last_to_arrive(&w[kWsTicketA], gridDim.x, &s_flag)) return;
+
+    // The query's histogram is complete. Thread t owns bins [16t, 16t+16); find the highest
+    // bin b with (count of bins >= b) >= kq.
+    constexpr int OWN = kTopBins / kSegThreads;
+    uint32_t c[OWN], sum = 0;
+#pragma unroll
+    for (int m = 0; m < OWN; ++m) {
+        c[m] = load_agent(&w[tid * OWN + m]);
+        sum += c[m];
+    }
+    uint32_t all = 0;
+    const uint32_t below = block_exclusive_scan(sum, s_scan, &all);
+    const uint32_t above = all - below - sum;  // candidates in bins owned by higher threads
+    if (above < kq && kq <= above + sum) {
+        uint32_t acc = above;
+        int m = OWN - 1;
+        for (; m > 0; --m) {
+            if (acc + c[m] >= kq) break;
+            acc += c[m];
+        }
+        w[kWsPivot] = (uint32_t)(tid * OWN + m);
+        w[kWsNeed] = kq - acc;
+    }
+    // leave the histogram and the ticket zeroed for the next call
+#pragma unroll
+    for (int m = 0; m < OWN; ++m) w[tid * OWN + m] = 0u;
+    if (tid == 0) w[kWsTicketA] = 0u;
+}
+
+__global__ __launch_bounds__(kSegThreads) void topk_select_kernel(
+    const float* __restrict__ scores, int stride, const int* __restrict__ nts, int nt_all, int k,
+    uint32_t* __restrict__ rows, uint32_t* __restrict__ ws, size_t ws_stride) {
+    // the finishing workgroup's candidate cache (indices, keys); the fallback's LDS aliases it
+    __shared__ uint32_t s_mem[2 * kCandCap];
+    __shared__ uint32_t s_pref[kMaxSegs + 1];
+    __shared__ uint32_t s_cnt[kSegItems * kSegWaves];
+    __shared__ uint32_t s_bins[kBins];
+    __shared__ uint32_t s_pn[2];
+    __shared__ uint32_t s_flag;
+    static_assert(topk_block_lds_words<kSegThreads>() <= 2 * kCandCap, "fallback fits the cache");
+    static_assert(kSegItems * kSegWaves == kWave, "one wave scans the (step, wave) counts");
+
+    const int q = blockIdx.y, seg = blockIdx.x, tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    const int n_segs = gridDim.x;
+    const int nt = nts ? min(nts[q], nt_all) : nt_all;
+    if (nt <= 0) return;
+    const uint32_t kq = (uint32_t)min(k, nt);
+    const float* s = scores + (size_t)q * stride;
+    uint32_t* w = ws + (size_t)q * ws_stride;
+    uint32_t* cand = w + topk_ws_cand_offset(n_segs);
+    const uint32_t p12 = w[kWsPivot];
+
+    // ---- this segment's candidates (key's top bits >= pivot bin), in index order ----
+    uint32_t key[kSegItems];
+    int limit = 0;
+    if (seg * kSegKeys < nt) {
+        load_segment_keys(s, nt, seg, key, limit);
+    } else {
+#pragma unroll
+        for (int j = 0; j < kSegItems; ++j) key[j] = 0u;
+    }
+    uint32_t rank[kSegItems];
+    bool sel[kSegItems];
+#pragma unroll
+    for (int j = 0; j < kSegItems; ++j) {
+        sel[j] = j * kSegThreads < limit && (key[j] >> kLowBits) >= p12;
+        const unsigned long long m = __ballot(sel[j]);
+        rank[j] = lanes_below(m);
+        if (lane == 0) s_cnt[j * kSegWaves + wave] = (uint32_t)__popcll(m);
+    }
+    __syncthreads();
+    if (wave == 0) {  // exclusive scan of the 64 (step, wave) counts, which is element order
+        const uint32_t v = s_cnt[lane];
+        uint32_t incl = v;
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            uint32_t t = __shfl_up(incl, off, kWave);
+            if (lane >= off) incl += t;
+        }
+        s_cnt[lane] = incl - v;
+        if (lane == kWave - 1) w[kWsCounts + seg] = incl;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kSegItems; ++j)
+        if (sel[j])
+            cand[(size_t)seg * kSegKeys + s_cnt[j * kSegWaves + wave] + rank[j]] =
+                (uint32_t)(seg * kSegKeys + j * kSegThreads + tid);
+    if (!last_to_arrive(&w[kWsTicketB], (uint32_t)n_segs, &s_flag)) return;
+
+    // ---- the query's last workgroup finishes the selection ----
+    if (tid == 0) w[kWsTicketB] = 0u;  // left zeroed for the next call
+    uint32_t* out = rows + (size_t)q * k;
+    uint32_t total = 0;
+    bool cached = n_segs <= kMaxSegs;
+    if (cached) {
+        // thread t owns `per` consecutive segments: load their counts at once, scan, publish
+        constexpr int PER_MAX = kMaxSegs / kSegThreads;
+        const int per = (n_segs + kSegThreads - 1) / kSegThreads;
+        uint32_t cnt[PER_MAX], mine = 0;
+#pragma unroll
+        for (int i = 0; i < PER_MAX; ++i) {
+            const int sg = tid * per + i;
+            cnt[i] = (i < per && sg < n_segs) ? load_agent(&w[kWsCounts + sg]) : 0u;
+            mine += cnt[i];
+        }
+        uint32_t acc = block_exclusive_scan(mine, s_cnt, &total);
+#pragma unroll
+        for (int i = 0; i < PER_MAX; ++i) {
+            const int sg = tid * per + i;
+            if (i < per && sg < n_segs) s_pref[sg] = acc;
+            acc += cnt[i];
+        }
+        if (tid == 0) s_pref[n_segs] = total;
+        __syncthreads();
+        cached = total <= (uint32_t)kCandCap;
+    }
+    if (!cached) {
+        // too many candidates to hold (heavy ties): select over the whole query directly
+        topk_block<kSegThreads, 0>(s, nt, kq, out, s_mem);
+        return;
+    }
+    // Pull the candidates into LDS in index order: a group of threads per segment, so no
+    // thread has to search for the segment an output position belongs to.
+    uint32_t* c_idx = s_mem;
+    uint32_t* c_key = s_mem + kCandCap;
+    {
+        const int tps = n_segs < kSegThreads ? kSegThreads / n_segs : 1;  // threads per segment
+        const int groups = kSegThreads / tps;
+        const int sub = tid % tps;
+        for (int sg = tid / tps; sg < n_segs; sg += groups) {
+            const uint32_t base = s_pref[sg], n = s_pref[sg + 1] - base;
+            const uint32_t* src = cand + (size_t)sg * kSegKeys;
+#pragma unroll 4
+            for (uint32_t i = sub; i < n; i += tps) {
+                const uint32_t idx = load_agent(&src[i]);
+                c_idx[base + i] = idx;
+                c_key[base + i] = topk_key(s[idx]);
+            }
+        }
+    }
+    __syncthreads();
+
+    // Radix select on the low 20 bits among the pivot bin's members: 8 + 8 + 4 bits.
+    uint32_t need = w[kWsNeed];
+    uint32_t pivot = p12 << kLowBits, mask = ~0u << kLowBits;
+    for (int shift = kLowBits - 8;; shift = shift >= 8 ? shift - 8 : 0) {
+        const uint32_t dmask = (shift == 0 && (kLowBits % 8)) ? (1u << (kLowBits % 8)) - 1u : 0xffu;
+        s_bins[tid] = 0u;
+        __syncthreads();
+        for (uint32_t c = tid; c < total; c += kSegThreads) {
+            const uint32_t u = c_key[c];
+            if ((u & mask) == pivot) atomicAdd(&s_bins[(u >> shift) & dmask], 1u);
+        }
+        __syncthreads();
+        if (wave == 0) find_pivot_bin(s_bins, need, s_pn, lane);
+        __syncthreads();
+        pivot |= s_pn[0] << shift;
+        need = s_pn[1];
+        mask |= dmask << shift;
+        __syncthreads();
+        if (shift == 0) break;
+    }
+
+    // Ordered emission: 256 candidates per round, running (gt, eq) counts carried across.
+    uint32_t run_gt = 0, run_eq = 0;
+    for (uint32_t c0 = 0; c0 < total; c0 += kSegThreads) {
+        const uint32_t c = c0 + tid;
+        const bool live = c < total;
+        const uint32_t u = live ? c_key[c] : 0u;
+        const bool g = live && u > pivot, e = live && u == pivot;
+        const unsigned long long mg = __ballot(g), me = __ballot(e);
+        if (lane == 0) {
+            s_cnt[wave] = (uint32_t)__popcll(mg);
+            s_cnt[kSegWaves + wave] = (uint32_t)__popcll(me);
+        }
+        __syncthreads();
+        uint32_t G = run_gt + lanes_below(mg), E = run_eq + lanes_below(me);
+        for (int wv = 0; wv < kSegWaves; ++wv) {
+            if (wv < wave) {
+                G += s_cnt[wv];
+                E += s_cnt[kSegWaves + wv];
+            }
+            run_gt += s_cnt[wv];
+            run_eq += s_cnt[kSegWaves + wv];
+        }
+        const uint32_t slot = G + (E < need ? E : need);
+        if ((g || (e && E < need)) && slot < kq) out[slot] = c_idx[c];
+        __syncthreads();
+    }
+}
+
 static int index_topk_launch(const float* scores, int n_queries, int stride, const int* nts,
-                             int nt, int k, unsigned int* rows, hipStream_t stream) {
+                             int nt, int k, unsigned int* rows, void* workspace,
+                             hipStream_t stream) {
     if (!scores || !rows) return 1001;
     if (n_queries <= 0 || nt <= 0 || k <= 0) return 1001;
     if (stride < nt) return 1002;
-    dim3 grid((unsigned)n_queries), block(kTopkThreads);
     (void)hipGetLastError();
+    const int n_segs = (nt + kSegKeys - 1) / kSegKeys;
+    // A query that fits one workgroup's registers (<= 65536 scores) is fastest there; longer
+    // ones are split over the chip when the caller brought a workspace. 65535 bounds grid.y.
+    if (workspace && nt > kTopkThreads * 64 && n_queries <= 65535) {
+        const size_t ws_stride = topk_ws_words(n_segs);
+        dim3 grid((unsigned)n_segs, (unsigned)n_queries), block(kSegThreads);
+        hipLaunchKernelGGL(topk_hist_kernel, grid, block, 0, stream, scores, stride, nts, nt, k,
+                           (uint32_t*)workspace, ws_stride);
+        hipLaunchKernelGGL(topk_select_kernel, grid, block, 0, stream, scores, stride, nts, nt, k,
+                           rows, (uint32_t*)workspace, ws_stride);
+        return launch_status();
+    }
+    dim3 grid((unsigned)n_queries), block(kTopkThreads);
     if (nt <= kTopkThreads * 4)
-        hipLaunchKernelGGL(index_topk_kernel<4>, grid, block, 0, stream, scores, stride, nts, nt, k,
-                           rows);
+        hipLaunchKernelGGL(index_topk_kernel<4>, grid, block, 0, stream, scores, stride, nts,
+                           nt, k, rows);
     else if (nt <= kTopkThreads * 16)
-        hipLaunchKernelGGL(index_topk_kernel<16>, grid, block, 0, stream, scores, stride, nts, nt,
-                           k, rows);
+        hipLaunchKernelGGL(index_topk_kernel<16>, grid, block, 0, stream, scores, stride,
+                           nts, nt, k, rows);
     else if (nt <= kTopkThreads * 64)
-        hipLaunchKernelGGL(index_topk_kernel<64>, grid, block, 0, stream, scores, stride, nts, nt,
-                           k, rows);
+        hipLaunchKernelGGL(index_topk_kernel<64>, grid, block, 0, stream, scores, stride,
+                           nts, nt, k, rows);
     else
-        hipLaunchKernelGGL(index_topk_kernel<0>, grid, block, 0, stream, scores, stride, nts, nt, k,
-                           rows);
+        hipLaunchKernelGGL(index_topk_kernel<0>, grid, block, 0, stream, scores, stride,
+                           nts, nt, k, rows);
     return launch_status();
 }
 
 }  // namespace rk
 
+extern "C" size_t rivoli_index_topk_workspace_bytes(int n_queries, int nt) {
+    if (n_queries <= 0 || nt <= 0) return 0;
+    const int n_segs = (nt + rk::kSegKeys - 1) / rk::kSegKeys;
+    return (size_t)n_queries * rk::topk_ws_words(n_segs) * sizeof(uint32_t);
+}
+
 extern "C" int rivoli_index_topk_batched(const float* scores, int n_queries, int stride,
                                          const int* nts, int nt, int k, unsigned int* rows,
-                                         void* stream) {
-    return rk::index_topk_launch(scores, n_queries, stride, nts, nt, k, rows, (hipStream_t)stream);
+                                         void* workspace, void* stream) {
+    return rk::index_topk_launch(scores, n_queries, stride, nts, nt, k, rows, workspace,
+                                 (hipStream_t)stream);
 }
 
 extern "C" int rivoli_index_topk(const float* scores, int nt, int k, unsigned int* rows) {
-    return rk::index_topk_launch(scores, 1, nt, nullptr, nt, k, rows, nullptr);
+    return rk::index_topk_launch(scores, 1, nt, nullptr, nt, k, rows, nullptr, nullptr);
 }

@@ -41,7 +41,7 @@ _SIGNATURES = {
     "rivoli_append_kv_rows": [_VP] * 5 + [_I] * 5 + [_VP],
     "rivoli_index_append": [_VP, _VP, _I, _I],
     "rivoli_index_topk": [_VP, _I, _I, _VP],
-    "rivoli_index_topk_batched": [_VP, _I, _I, _VP, _I, _I, _VP, _VP],
+    "rivoli_index_topk_batched": [_VP, _I, _I, _VP, _I, _I, _VP, _VP, _VP],
     "rivoli_hash_rows": [_VP, _I, _I, _ULL, _VP, _VP],
     "rivoli_device_sync": [],
     "rivoli_kv_append_paged": [_VP, _VP, _VP, _I, _I, _I, _I, _VP, _VP],
@@ -65,14 +65,15 @@ def lib() -> C.CDLL:
         for name, args in _SIGNATURES.items():
             fn = getattr(handle, name)
             fn.restype, fn.argtypes = C.c_int, args
-        handle.rivoli_kv_page_bytes.restype = C.c_size_t
-        handle.rivoli_kv_page_bytes.argtypes = [_I, _I]
+        for name in ("rivoli_kv_page_bytes", "rivoli_index_topk_workspace_bytes"):
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = C.c_size_t, [_I, _I]
         _LIB = handle
     return _LIB
 
 
 def exported_symbols() -> list[str]:
-    return sorted(list(_SIGNATURES) + ["rivoli_kv_page_bytes"])
+    return sorted(list(_SIGNATURES) + ["rivoli_kv_page_bytes", "rivoli_index_topk_workspace_bytes"])
 
 
 def _p(x):
@@ -156,10 +157,16 @@ def launch_kv_gather_rows_paged(pool, block_table, rows, n_rows, out, n_queries,
                       "kv_gather_rows_paged")
 
 
-def launch_index_topk_batched(scores, n_queries, stride, nts, nt, k, rows,
+def index_topk_workspace_bytes(n_queries: int, nt: int) -> int:
+    return int(lib().rivoli_index_topk_workspace_bytes(n_queries, nt))
+
+
+def launch_index_topk_batched(scores, n_queries, stride, nts, nt, k, rows, workspace=None,
                               stream=NULL_STREAM) -> None:
+    """`workspace`: a zero-filled device buffer of index_topk_workspace_bytes(n_queries, nt)
+    bytes (left zero-filled by every call), or None for one workgroup per query."""
     ensure_hip_status(lib().rivoli_index_topk_batched(_p(scores), n_queries, stride, _p(nts), nt,
-                                                      k, _p(rows), _s(stream)),
+                                                      k, _p(rows), _p(workspace), _s(stream)),
                       "index_topk_batched")
 
 

@@ -81,7 +81,8 @@ def test_config4_one_layer_topk_then_sparse_gather(oracle):
     scores = rng.standard_normal((B, nt), dtype=np.float32)
     scores[:, -64:] += np.float32(4.0)
     sel = dzeros(B * k * 4, 0xFF)
-    hip.launch_index_topk_batched(dev(scores), B, nt, None, nt, k, sel)
+    ws = dzeros(hip.index_topk_workspace_bytes(B, nt))
+    hip.launch_index_topk_batched(dev(scores), B, nt, None, nt, k, sel, ws)
     sel_np = back(sel, np.uint32).reshape(B, k)
     assert np.array_equal(sel_np, oracle.topk_batched(scores, k, n_threads=8))
     sparse = dzeros(B * k * W * 2)

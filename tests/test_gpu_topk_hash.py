@@ -47,6 +47,24 @@ def test_index_topk_guards():
     assert e.value.code == 1002
 
 
+def batched_topk(scores, nts, k, split):
+    """Runs the batched entry point without (one workgroup per query) or with a workspace
+    (each query split over the chip), twice in the latter case on the SAME workspace so the
+    second call sees what the first one left behind."""
+    n_q, stride = scores.shape
+    sd = dev(scores)
+    ntd = None if nts is None else dev(np.asarray(nts, np.int32))
+    ws = dzeros(hip.index_topk_workspace_bytes(n_q, stride)) if split else None
+    got = None
+    for _ in range(2 if split else 1):
+        rows = dzeros(n_q * k * 4, 0xFF)
+        hip.launch_index_topk_batched(sd, n_q, stride, ntd, stride, k, rows, ws)
+        got = back(rows, np.uint32).reshape(n_q, k)
+    if split:   # the histogram and both tickets are back to zero
+        assert not back(ws, np.uint32).reshape(n_q, -1)[:, :4098].any()
+    return got
+
+
 def dsa_scores(n_q, nt, seed):
     """BASELINE config 4's score shape: N(0,1) plus a boost on the last 64 tokens."""
     rng = np.random.default_rng(seed)
@@ -55,16 +73,16 @@ def dsa_scores(n_q, nt, seed):
     return s
 
 
-@pytest.mark.parametrize("nt", [1, 63, 64, 65, 1023, 1024, 1025, 4096, 4097, 5185, 16384, 16385,
-                                65535, 65536, 65537, 200_000])
-def test_batched_topk_sizes(oracle, nt):
-    """Every register-resident variant's boundary, and the streaming path past 65536."""
+@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("nt", [1, 63, 64, 65, 1023, 1024, 1025, 4096, 4097, 5185, 8192, 16384,
+                                16385, 65535, 65536, 65537, 200_000])
+def test_batched_topk_sizes(oracle, nt, split):
+    """Every register-resident variant's boundary, the streaming path past 65536, and the
+    segment boundaries of the split form."""
     n_q, k = 3, 2048
     s = dsa_scores(n_q, nt, seed=nt)
-    s[1, :: 3] = np.float32(0.25)               # a tie-heavy query
-    rows = dzeros(n_q * k * 4, 0xFF)
-    hip.launch_index_topk_batched(dev(s), n_q, nt, None, nt, k, rows)
-    got = back(rows, np.uint32).reshape(n_q, k)
+    s[1, :: 3] = np.float32(0.25)               # a tie-heavy query (overflows the candidate cache)
+    got = batched_topk(s, None, k, split)
     for q in range(n_q):
         want = oracle.topk(s[q], k)
         assert np.array_equal(got[q, : want.size], want), (nt, q)
@@ -73,31 +91,30 @@ def test_batched_topk_sizes(oracle, nt):
         assert np.array_equal(got[0, : min(k, nt)], brute_force_topk(s[0], k))
 
 
-def test_config4_shape_16_queries_of_65536(oracle):
+@pytest.mark.parametrize("split", [False, True])
+def test_config4_shape_16_queries_of_65536(oracle, split):
     n_q, nt, k = 16, 65536, 2048
     s = dsa_scores(n_q, nt, seed=0x5EED0004)
-    rows = dzeros(n_q * k * 4, 0xFF)
-    hip.launch_index_topk_batched(dev(s), n_q, nt, None, nt, k, rows)
-    got = back(rows, np.uint32).reshape(n_q, k)
+    got = batched_topk(s, None, k, split)
     want = oracle.topk_batched(s, k, n_threads=8)
     assert np.array_equal(got, want)
     assert np.all(np.isin(np.arange(nt - 64, nt), got[0]))   # the recency window is selected
 
 
-def test_batched_topk_per_query_lengths_and_strides(oracle):
+@pytest.mark.parametrize("split", [False, True])
+def test_batched_topk_per_query_lengths_and_strides(oracle, split):
     n_q, stride, k = 6, 9000, 512
     s = dsa_scores(n_q, stride, seed=4)
     nts = np.array([9000, 1, 0, 511, 512, 8999], np.int32)
-    rows = dzeros(n_q * k * 4, 0xFF)
-    hip.launch_index_topk_batched(dev(s), n_q, stride, dev(nts), stride, k, rows)
-    got = back(rows, np.uint32).reshape(n_q, k)
+    got = batched_topk(s, nts, k, split)
     for q in range(n_q):
         want = oracle.topk(s[q, : nts[q]], k)
         assert np.array_equal(got[q, : want.size], want), q
         assert np.all(got[q, want.size:] == SENTINEL), q
 
 
-def test_topk_adversarial_values(oracle):
+@pytest.mark.parametrize("split", [False, True])
+def test_topk_adversarial_values(oracle, split):
     nt, k = 70000, 2048
     rng = np.random.default_rng(8)
     cases = {
@@ -111,9 +128,20 @@ def test_topk_adversarial_values(oracle):
     }
     for name, s in cases.items():
         for n in (nt, 65536, 3000):
-            rows = dzeros(k * 4, 0xFF)
-            hip.launch_index_topk_batched(dev(s[:n]), 1, n, None, n, k, rows)
-            assert np.array_equal(back(rows, np.uint32), oracle.topk(s[:n], k)), (name, n)
+            got = batched_topk(np.ascontiguousarray(s[None, :n]), None, k, split)[0]
+            assert np.array_equal(got, oracle.topk(s[:n], k)), (name, n)
+
+
+@pytest.mark.parametrize("split", [False, True])
+def test_topk_small_k_and_k_beyond_nt(oracle, split):
+    rng = np.random.default_rng(15)
+    s = rng.standard_normal((4, 20000)).astype(np.float32)
+    for k in (1, 2, 63, 64, 4095, 4096, 4097, 20000, 25000):
+        got = batched_topk(s, None, k, split)
+        for q in range(4):
+            want = oracle.topk(s[q], k)
+            assert np.array_equal(got[q, : want.size], want), (k, q)
+            assert np.all(got[q, want.size:] == SENTINEL), (k, q)
 
 
 def test_hash_rows_matches_the_host_fold(oracle):
