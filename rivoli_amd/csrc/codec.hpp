@@ -3,6 +3,8 @@
 // Arithmetic contract (must stay bit-identical to rivoli_core::num, crates/core/src/num.rs):
 //   * e4m3 encode: round to nearest even on normals, round HALF AWAY from zero in the
 //     subnormal band, saturate |x| >= 448 to 0x7e, |x| < 2^-10 to signed zero, NaN -> 0x7f.
+//     gfx950's v_cvt_pk_fp8_f32 is nearest-even everywhere, so it is used only where the two
+//     rules coincide; the rest goes through the integer form.
 //   * e4m3 decode is exact; gfx950's v_cvt_pk_f32_fp8 decodes OCP e4m3 and is used as is.
 //   * bf16 encode is round to nearest even; gfx950's v_cvt_pk_bf16_f32 does exactly that.
 //   * scale = amax > 0 ? amax / 448 : 1 and v / scale are IEEE-correct f32 divides (hipcc's
@@ -37,8 +39,9 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float x) {
 }
 
 // f32 -> OCP e4m3 byte, the KV-cache rule (crates/core/src/num.rs:128-182; device twin in the
-// reference at crates/backend/kernels/fwd.hip:20-45). Written as straight-line selects.
-__device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
+// reference at crates/backend/kernels/fwd.hip:20-45), in integer arithmetic: the software
+// form, valid for every input.
+__device__ __forceinline__ uint32_t f32_to_e4m3_sw(float x) {
     uint32_t xb = __float_as_uint(x);
     uint32_t sign = (xb >> 24) & 0x80u;
     uint32_t ab = xb & 0x7fffffffu;
@@ -54,6 +57,72 @@ __device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
     mag = a >= 448.0f ? 0x7eu : mag;  // also catches +-inf
     uint32_t code = sign | mag;
     return ab > 0x7f800000u ? 0x7fu : code;
+}
+
+// Two / four values through gfx950's v_cvt_pk_fp8_f32 (OCP e4m3, round to nearest even
+// everywhere). It agrees with the KV-cache rule exactly where that rule is nearest-even and
+// does not saturate: 2^-6 <= |x| < 464 (448..464 rounds down to 448), and at +-0. It differs
+// on subnormal-band ties (the rule rounds those half AWAY), so callers route |x| < 2^-6,
+// |x| >= 464 and NaN to the software form.
+__device__ __forceinline__ uint32_t e4m3x4_hw(float q0, float q1, float q2, float q3) {
+    int w = __builtin_amdgcn_cvt_pk_fp8_f32(q0, q1, 0, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(q2, q3, w, true);
+    return (uint32_t)w;
+}
+__device__ __forceinline__ bool e4m3_hw_exact_domain(float x) {
+    const float a = fabsf(x);
+    return (a >= 0.015625f && a < 464.0f) || a == 0.0f;  // false for NaN
+}
+
+// The rule for one value: hardware conversion inside its exact domain, software outside.
+__device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
+    if (e4m3_hw_exact_domain(x)) return e4m3x4_hw(x, 0.0f, 0.0f, 0.0f) & 0xffu;
+    return f32_to_e4m3_sw(x);
+}
+
+// The append quantizer divides by the row scale before encoding: code = rule(RN(x / scl)).
+// A correctly rounded divide costs ~11 instructions, so the fast path multiplies by the
+// correctly rounded reciprocal instead: q' = RN(x * RN(1/scl)) is within 3 ulps of RN(x/scl)
+// (two roundings of 2^-24 relative each against one). The e4m3 code of both is the same
+// unless a rounding tie lies between them; ties sit where the 20 dropped mantissa bits equal
+// 0x80000, so a q' farther than 8 ulps from that pattern, inside the hardware converter's
+// exact domain, is safe to convert directly. Everything else takes the exact divide and the
+// software encoder. Requires scl and 1/scl normal and finite (the caller checks the row).
+__device__ __forceinline__ bool quotient_needs_exact(float q) {
+    const uint32_t b = __float_as_uint(q);
+    const float a = fabsf(q);
+    const bool out_of_domain = !(a >= 0.015625f) && a != 0.0f;  // subnormal band, or NaN
+    const bool near_tie = ((b & 0x000fffffu) - 0x0007fff8u) < 16u;
+    return out_of_domain || near_tie;
+}
+
+// Eight consecutive bf16 (four dwords) -> eight e4m3 codes (two dwords) under one row scale.
+__device__ __forceinline__ u32x2 quantize8(const uint32_t (&w)[4], float scl, float rinv,
+                                           bool row_fast) {
+    float x[8], q[8];
+    bool exact = !row_fast;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        x[2 * i] = bf16_lo_to_f32(w[i]);
+        x[2 * i + 1] = bf16_hi_to_f32(w[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        q[i] = x[i] * rinv;
+        exact = exact || quotient_needs_exact(q[i]);
+    }
+    if (!exact) {
+        u32x2 r = {e4m3x4_hw(q[0], q[1], q[2], q[3]), e4m3x4_hw(q[4], q[5], q[6], q[7])};
+        return r;
+    }
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        lo |= f32_to_e4m3_sw(x[i] / scl) << (8 * i);
+        hi |= f32_to_e4m3_sw(x[4 + i] / scl) << (8 * i);
+    }
+    u32x2 r = {lo, hi};
+    return r;
 }
 
 // Four packed e4m3 codes -> four f32, exact.

@@ -6,20 +6,138 @@
 //   * the reference's linear slabs: f32 input, one scale per 128 latent values, the roped
 //     key kept as bf16 (crates/backend/kernels/fwd.hip:51-71).
 //
-// One wave64 owns one token. A lane holds 8 consecutive elements per step (one 16-byte load
-// of bf16), so a 576-wide row is one full step plus an 8-lane tail; the per-token amax is a
-// register max followed by a wave butterfly, which is exact and order-free, so it equals
-// the reference's LDS tree bit for bit. Codes leave as 8-byte stores, contiguous per wave.
+// Paged: one wave64 owns 8 tokens (see the kernel). Linear: one wave64 owns one token. Either
+// way the amax is a max over registers, LDS and wave butterflies — exact and order-free, so
+// it equals the reference's LDS tree bit for bit.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
 #include "codec.hpp"
 
 namespace rk {
 
-constexpr int kAppendWaves = 4;  // tokens per workgroup
+constexpr int kAppendWaves = 4;   // linear-slab kernel: tokens per workgroup
+constexpr int kRowsPerWave = 8;   // paged kernel: tokens per (one-wave) workgroup
+constexpr int kMaxChunksPerRow = 128;  // width <= 1024
+// Batches at least this large take the 8-rows-per-wave kernel (throughput); smaller ones the
+// one-wave-per-token kernel (latency). RIVOLI_BULK_APPEND_TOKENS overrides it at build time.
+#ifndef RIVOLI_BULK_APPEND_TOKENS
+#define RIVOLI_BULK_APPEND_TOKENS 32768
+#endif
+constexpr int kBulkAppendTokens = RIVOLI_BULK_APPEND_TOKENS;
 
-// STEPS = ceil(width / 512): how many 8-element chunks a lane may own.
+// Paged append. One wave64 workgroup owns 8 consecutive tokens = one contiguous run of the
+// input, cut into 16-byte chunks (8 bf16) dealt round-robin to the lanes: for a 576-wide row
+// that is 8 x 72 = 576 chunks, exactly 9 per lane, so no lane idles and every load is a full
+// 1 KiB wave access. Per-chunk maxima go through LDS to a segmented reduce (8 lanes per row),
+// which is exact and order-free like the reference's LDS tree; one lane per row derives the
+// scale, its reciprocal and the row's destination. Codes leave as 8-byte stores.
+// CPR = chunks per row at compile time (0 = runtime, up to 128).
+template <int CPR>
+__global__ __launch_bounds__(kWave) void kv_append_paged_kernel(
+    const uint16_t* __restrict__ rows, const int* __restrict__ slot_mapping,
+    uint8_t* __restrict__ pool, int n_tokens, int width, int page_tokens, long long n_slots,
+    size_t page_bytes, unsigned int* __restrict__ bad_slots) {
+    constexpr int MAXJ = CPR ? (kRowsPerWave * CPR + kWave - 1) / kWave
+                             : kRowsPerWave * kMaxChunksPerRow / kWave;
+    constexpr unsigned long long kSkip = ~0ull;
+    __shared__ float s_amax[kRowsPerWave * (CPR ? CPR : kMaxChunksPerRow)];
+    __shared__ float s_scl[kRowsPerWave], s_rinv[kRowsPerWave];
+    __shared__ int s_fast[kRowsPerWave];
+    __shared__ unsigned long long s_dst[kRowsPerWave], s_sdst[kRowsPerWave];
+
+    const int cpr = CPR ? CPR : width >> 3;
+    const int lane = threadIdx.x;
+    const int t0 = (int)blockIdx.x * kRowsPerWave;
+    const int nrows = min(kRowsPerWave, n_tokens - t0);
+    const int n_chunks = nrows * cpr;
+    const u32x4* src = reinterpret_cast<const u32x4*>(rows + (size_t)t0 * width);
+
+    u32x4 raw[MAXJ];
+#pragma unroll
+    for (int j = 0; j < MAXJ; ++j) {
+        const int c = lane + j * kWave;
+        raw[j] = c < n_chunks ? __builtin_nontemporal_load(src + c) : u32x4{0, 0, 0, 0};
+    }
+    if (lane < kRowsPerWave) {  // where each row goes (or nowhere)
+        unsigned long long dst = kSkip, sdst = 0;
+        if (lane < nrows) {
+            const int slot = slot_mapping[t0 + lane];
+            if (slot >= 0) {
+                if ((long long)slot < n_slots) {
+                    const int page = slot / page_tokens, off = slot - page * page_tokens;
+                    dst = (size_t)page * page_bytes + (size_t)off * width;
+                    sdst = (size_t)page * page_bytes + (size_t)page_tokens * width + (size_t)off * 4;
+                } else if (bad_slots) {
+                    atomicAdd(bad_slots, 1u);
+                }
+            }
+        }
+        s_dst[lane] = dst;
+        s_sdst[lane] = sdst;
+    }
+#pragma unroll
+    for (int j = 0; j < MAXJ; ++j) {
+        const int c = lane + j * kWave;
+        if (c < n_chunks) {
+            const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+            float m = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                m = fmaxf(m, fmaxf(fabsf(bf16_lo_to_f32(w[i])), fabsf(bf16_hi_to_f32(w[i]))));
+            s_amax[c] = m;
+        }
+    }
+    __syncthreads();
+    {
+        // lane = (row, part): each of a row's 8 lanes folds a slice of its chunk maxima
+        const int r = lane >> 3, part = lane & 7;
+        const int per = (cpr + 7) >> 3;
+        constexpr int PER_MAX = CPR ? (CPR + 7) / 8 : kMaxChunksPerRow / 8;
+        float m = 0.0f;
+        if (r < nrows) {
+#pragma unroll
+            for (int i = 0; i < PER_MAX; ++i) {  // independent LDS reads, not a dependent loop
+                const int at = part * per + i;
+                if (i < per && at < cpr) m = fmaxf(m, s_amax[r * cpr + at]);
+            }
+        }
+        m = fmaxf(m, __shfl_xor(m, 1, kWave));
+        m = fmaxf(m, __shfl_xor(m, 2, kWave));
+        m = fmaxf(m, __shfl_xor(m, 4, kWave));
+        if (part == 0 && r < nrows) {
+            const float scl = m > 0.0f ? m / 448.0f : 1.0f;
+            s_scl[r] = scl;
+            s_rinv[r] = 1.0f / scl;
+            // the reciprocal shortcut needs scl and 1/scl comfortably normal and finite
+            s_fast[r] = (scl >= 1e-30f && scl <= 1e30f) ? 1 : 0;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < MAXJ; ++j) {
+        const int c = lane + j * kWave;
+        if (c < n_chunks) {
+            const int r = c / cpr, col = c - r * cpr;
+            const unsigned long long dst = s_dst[r];
+            if (dst != kSkip) {
+                const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+                reinterpret_cast<u32x2*>(pool + dst)[col] =
+                    quantize8(w, s_scl[r], s_rinv[r], s_fast[r] != 0);
+            }
+        }
+    }
+    // the scales last: a global store ahead of a barrier would make the barrier wait for it
+    if (lane < nrows && s_dst[lane] != kSkip)
+        *reinterpret_cast<float*>(pool + s_sdst[lane]) = s_scl[lane];
+}
+
+// Paged append, low-latency form for small batches (decode steps, short prefill chunks): one
+// wave64 per token, 4 tokens per workgroup, no LDS and no barrier. A lane holds 8 consecutive
+// elements per step (one 16-byte load), so a 576-wide row is one full step plus an 8-lane
+// tail; the amax is a register max plus a wave butterfly. Half the lanes idle in the tail
+// step, which is why large batches use the 8-rows-per-wave kernel above instead.
+// STEPS = ceil(width / 512).
 template <int STEPS>
-__global__ __launch_bounds__(kAppendWaves* kWave) void kv_append_paged_kernel(
+__global__ __launch_bounds__(kAppendWaves* kWave) void kv_append_paged_token_kernel(
     const uint16_t* __restrict__ rows, const int* __restrict__ slot_mapping,
     uint8_t* __restrict__ pool, int n_tokens, int width, int page_tokens, long long n_slots,
     size_t page_bytes, unsigned int* __restrict__ bad_slots) {
@@ -42,20 +160,18 @@ __global__ __launch_bounds__(kAppendWaves* kWave) void kv_append_paged_kernel(
         int c = lane + s * kWave;
         raw[s] = c < n_chunks ? __builtin_nontemporal_load(src + c) : u32x4{0, 0, 0, 0};
     }
-    float v[STEPS][8];
     float amax = 0.0f;
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
         const uint32_t w[4] = {raw[s].x, raw[s].y, raw[s].z, raw[s].w};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            v[s][2 * i] = bf16_lo_to_f32(w[i]);
-            v[s][2 * i + 1] = bf16_hi_to_f32(w[i]);
-            amax = fmaxf(amax, fmaxf(fabsf(v[s][2 * i]), fabsf(v[s][2 * i + 1])));
-        }
+        for (int i = 0; i < 4; ++i)
+            amax = fmaxf(amax, fmaxf(fabsf(bf16_lo_to_f32(w[i])), fabsf(bf16_hi_to_f32(w[i]))));
     }
     amax = wave_max(amax);
     const float scl = amax > 0.0f ? amax / 448.0f : 1.0f;
+    const float rinv = 1.0f / scl;
+    const bool row_fast = scl >= 1e-30f && scl <= 1e30f;
 
     const int page = slot / page_tokens;
     const int off = slot - page * page_tokens;
@@ -65,13 +181,8 @@ __global__ __launch_bounds__(kAppendWaves* kWave) void kv_append_paged_kernel(
     for (int s = 0; s < STEPS; ++s) {
         int c = lane + s * kWave;
         if (c < n_chunks) {
-            uint32_t lo = 0, hi = 0;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                lo |= f32_to_e4m3(v[s][i] / scl) << (8 * i);
-                hi |= f32_to_e4m3(v[s][4 + i] / scl) << (8 * i);
-            }
-            dst[c] = u32x2{lo, hi};
+            const uint32_t w[4] = {raw[s].x, raw[s].y, raw[s].z, raw[s].w};
+            dst[c] = quantize8(w, scl, rinv, row_fast);
         }
     }
     if (lane == 0)
@@ -142,15 +253,28 @@ extern "C" int rivoli_kv_append_paged(const unsigned short* rows, const int* slo
     if ((width % 16) != 0 || (page_tokens % 4) != 0) return 1004;
     const size_t page_bytes = rivoli_kv_page_bytes(page_tokens, width);
     const long long n_slots = (long long)n_pages * page_tokens;
-    dim3 grid((unsigned)((n_tokens + kAppendWaves - 1) / kAppendWaves));
-    dim3 block(kAppendWaves * kWave);
     (void)hipGetLastError();
-    if (width <= 512) {
-        hipLaunchKernelGGL(kv_append_paged_kernel<1>, grid, block, 0, (hipStream_t)stream, rows,
+    if (n_tokens < kBulkAppendTokens) {
+        dim3 grid((unsigned)((n_tokens + kAppendWaves - 1) / kAppendWaves));
+        dim3 block(kAppendWaves * kWave);
+        if (width <= 512)
+            hipLaunchKernelGGL(kv_append_paged_token_kernel<1>, grid, block, 0,
+                               (hipStream_t)stream, rows, slot_mapping, pool, n_tokens, width,
+                               page_tokens, n_slots, page_bytes, bad_slots);
+        else
+            hipLaunchKernelGGL(kv_append_paged_token_kernel<2>, grid, block, 0,
+                               (hipStream_t)stream, rows, slot_mapping, pool, n_tokens, width,
+                               page_tokens, n_slots, page_bytes, bad_slots);
+        return launch_status();
+    }
+    dim3 grid((unsigned)((n_tokens + kRowsPerWave - 1) / kRowsPerWave));
+    dim3 block(kWave);
+    if (width == 576) {
+        hipLaunchKernelGGL(kv_append_paged_kernel<72>, grid, block, 0, (hipStream_t)stream, rows,
                            slot_mapping, pool, n_tokens, width, page_tokens, n_slots, page_bytes,
                            bad_slots);
     } else {
-        hipLaunchKernelGGL(kv_append_paged_kernel<2>, grid, block, 0, (hipStream_t)stream, rows,
+        hipLaunchKernelGGL(kv_append_paged_kernel<0>, grid, block, 0, (hipStream_t)stream, rows,
                            slot_mapping, pool, n_tokens, width, page_tokens, n_slots, page_bytes,
                            bad_slots);
     }
