@@ -1,6 +1,6 @@
 """Benchmark of the fp8 MLA KV-cache hot path on one MI355X.
 
-Workload (default): BASELINE config 3 at its metric point — 48 layers, batch 32, every
+Workload (default): benchmark configuration 3 at its metric point — 48 layers, batch 32, every
 sequence at 32768 tokens of context, pages of 64 tokens drawn from a shuffled global pool. One
 "step" is one decode step's KV work: per layer, quantize-append one new 576-wide row per
 sequence, then gather + dequantize every sequence's full context to bf16. All inputs are
@@ -41,7 +41,7 @@ def parse():
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=32768)
     ap.add_argument("--workload", choices=["decode", "prefill", "dsa"], default="decode",
-                    help="decode = BASELINE config 3 (the headline line); prefill = config 2 "
+                    help="decode = benchmark configuration 3 (the headline line); prefill = config 2 "
                          "bulk append; dsa = config 4 top-k + sparse gather")
     ap.add_argument("--tokens", type=int, default=8192, help="prefill: new tokens per step")
     ap.add_argument("--topk", type=int, default=2048)
@@ -151,7 +151,7 @@ def main():
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "batched decode (BASELINE config 3, metric point): append 1 token/"
+        "config": {"workload": "batched decode (benchmark configuration 3, metric point): append 1 token/"
                                "seq/layer then gather+dequantize every sequence's full context",
                    "layers": L, "batch": B, "ctx": ctx, "page_tokens": PT, "width": W,
                    "stored": "fp8 e4m3 + 1 f32 scale/token", "out": "bf16"},
@@ -202,7 +202,7 @@ def bracket(torch, stream, events, name, launch):
 
 
 def bench_prefill(a, torch, hip):
-    """BASELINE config 2: `tokens` new 576-wide bf16 rows (0.5% of rows x50) quantize-appended
+    """benchmark configuration 2: `tokens` new 576-wide bf16 rows (0.5% of rows x50) quantize-appended
     into shuffled pages, one layer, one launch per step."""
     n = a.tokens
     n_pages = -(-n // PT)
@@ -231,7 +231,7 @@ def bench_prefill(a, torch, hip):
            "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
            "data": "synthetic",
-           "config": {"workload": "prefill bulk append (BASELINE config 2)", "tokens": n,
+           "config": {"workload": "prefill bulk append (benchmark configuration 2)", "tokens": n,
                       "pages": n_pages, "width": W, "page_tokens": PT},
            "tokens_per_s": round(n / (ms * 1e-3), 1),
            "roofline": {"bound": "hbm", "kernel": "kv_append_paged_kernel",
@@ -262,7 +262,7 @@ def bench_prefill(a, torch, hip):
 
 
 def bench_dsa(a, torch, hip):
-    """BASELINE config 4: per layer, select the top-k of 65536 indexer scores for each of 16
+    """benchmark configuration 4: per layer, select the top-k of 65536 indexer scores for each of 16
     queries (ties to the lowest index), then gather + dequantize those rows from fragmented
     pages. One step = all layers."""
     L, B, nt, k = a.layers, (16 if a.batch == 32 else a.batch), (65536 if a.ctx == 32768 else a.ctx), a.topk
@@ -311,7 +311,7 @@ def bench_dsa(a, torch, hip):
            "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-           "config": {"workload": "DSA sparse path (BASELINE config 4): top-k then sparse row gather",
+           "config": {"workload": "DSA sparse path (benchmark configuration 4): top-k then sparse row gather",
                       "layers": L, "batch": B, "ctx": nt, "k": k, "width": W, "page_tokens": PT},
            "rows_per_s": round(L * B * k / (ms * 1e-3), 1),
            "kernels_ms": {n: round(v, 5) for n, v in per.items()},

@@ -1,4 +1,4 @@
-"""BASELINE config 5 as a seeded event stream: a 2048-page pool kept ~80% full by up to 64
+"""benchmark configuration 5 as a seeded event stream: a 2048-page pool kept ~80% full by up to 64
 sequences of 512 to 128K tokens, decode appends interleaved with whole-sequence frees whose
 pages are reused LIFO; 1% of tokens are x200 outliers. Shared by the CPU and GPU tests."""
 import numpy as np

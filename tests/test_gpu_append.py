@@ -1,5 +1,5 @@
 """Quantize-and-append on the device against the CPU oracle (bit-exact codes, scales, bf16
-keys), on the reference's own fixture, on BASELINE configs 1 and 2, and on rows built to sit
+keys), on the reference's own fixture, on benchmark configurations 1 and 2, and on rows built to sit
 on the quantizer's rounding ties."""
 import numpy as np
 import pytest
@@ -95,7 +95,7 @@ def paged_append_both(oracle, rows, slots, n_pages, fill=0xA5):
 
 
 def test_config1_append_one_token_after_4095(oracle):
-    """BASELINE config 1: 4095 cached tokens, block table = seeded permutation of 64 pages,
+    """benchmark configuration 1: 4095 cached tokens, block table = seeded permutation of 64 pages,
     append the 4096th."""
     table = shuffled_block_tables(1, 64, 64, seed=0x5EED0001)[0]
     rows = make_rows_bf16(4096, W, seed=0x5EED0001)
@@ -110,7 +110,7 @@ def test_config1_append_one_token_after_4095(oracle):
 
 
 def test_config2_prefill_bulk_append_with_outlier_rows(oracle):
-    """BASELINE config 2: 8192 rows, 0.5% of rows x50, 128 shuffled pages."""
+    """benchmark configuration 2: 8192 rows, 0.5% of rows x50, 128 shuffled pages."""
     table = shuffled_block_tables(1, 128, 128, seed=0x5EED0002)[0]
     rows = make_rows_bf16(8192, W, seed=0x5EED0002, outlier_frac=0.005, outlier_mul=50.0)
     slots = slots_for(table, np.arange(8192))

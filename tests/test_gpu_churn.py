@@ -1,4 +1,4 @@
-"""BASELINE config 5 on the device: 10k seeded steps of appends and whole-sequence frees with
+"""benchmark configuration 5 on the device: 10k seeded steps of appends and whole-sequence frees with
 LIFO page reuse and x200 outlier tokens; the device pool must equal the oracle's byte for byte
 throughout, and every surviving sequence must gather identically."""
 import numpy as np

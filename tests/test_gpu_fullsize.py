@@ -1,4 +1,4 @@
-"""BASELINE configs 3 and 4 at their real per-layer shapes: byte comparison against the
+"""benchmark configurations 3 and 4 at their real per-layer shapes: byte comparison against the
 oracle where the host can hold it, and size-independent properties (page-permutation
 invariance, sparse == dense[rows], the XOR fold computed on the device equal to the oracle's
 fold) for the rest."""

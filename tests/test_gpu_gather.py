@@ -38,7 +38,7 @@ def gpu_gather(pool, tables, seq_lens, width=W, pt=PT, n_pages=None, fill=0x5A):
 
 
 def test_config1_gather_full_context(oracle):
-    """BASELINE config 1: batch 1, ctx 4096, block table a seeded permutation of 64 pages."""
+    """benchmark configuration 1: batch 1, ctx 4096, block table a seeded permutation of 64 pages."""
     pool, tables = build_pool(oracle, [4096], 64, seed=0x5EED0001 % 10007)
     want = oracle.kv_gather_paged(pool, tables, [4096], W, PT)
     got, bad = gpu_gather(pool, tables, [4096])

@@ -66,7 +66,7 @@ def batched_topk(scores, nts, k, split):
 
 
 def dsa_scores(n_q, nt, seed):
-    """BASELINE config 4's score shape: N(0,1) plus a boost on the last 64 tokens."""
+    """benchmark configuration 4's score shape: N(0,1) plus a boost on the last 64 tokens."""
     rng = np.random.default_rng(seed)
     s = rng.standard_normal((n_q, nt), dtype=np.float32)
     s[:, -64:] += np.float32(4.0)
