@@ -119,6 +119,35 @@ size_t rivoli_index_topk_workspace_bytes(int n_queries, int nt);
 int rivoli_index_topk_batched(const float* scores, int n_queries, int stride, const int* nts,
                               int nt, int k, unsigned int* rows, void* workspace, void* stream);
 
+/* Replaces crates/backend/kernels/indexer.hip:278-295 (launch_index_score,
+ * crates/backend/src/hip_attn.rs:464-476): scores[t] = sum over the active heads h of
+ * w[h]*wscale*max((q_h . k_t)*dscale, 0) for t < nt, over the LINEAR bf16 key cache
+ * kcache[nt][hd]. q is [nh][hd] f32, w [nh] f32; heads (nullable) lists the nact active
+ * heads, null = heads 0..nact-1. Results agree with the reference's within 1e-5 of the
+ * largest score (its own test bar), not bit for bit: the dots run on the matrix cores.
+ * Guards: 1001 as the reference (non-positive dims, nact > nh); 1002 nact > 64 or hd > 128
+ * (the reference allows up to 1024 heads); 1004 hd % 16. Null stream. */
+int rivoli_index_score(const float* q, const float* w, const unsigned short* kcache,
+                       const unsigned int* heads, int nt, int nh, int nact, int hd, float wscale,
+                       float dscale, float* scores);
+
+/* The paged, batched form: query qi (q [n_queries][nh][hd], w [n_queries][nh]) scores its
+ * first nts[qi] tokens (nt when nts is null) through block_table[qi] over the paged key
+ * cache kpool[n_pages*page_tokens][hd] bf16, into scores[qi*stride + t]. Tokens whose page id
+ * is outside [0, n_pages) are not written. Same guards, plus 1002 for stride < nt. */
+int rivoli_index_score_paged(const float* q, const float* w, const unsigned short* kpool,
+                             const int* block_table, const int* nts, const unsigned int* heads,
+                             int n_queries, int max_blocks_per_seq, int stride, int nt, int nh,
+                             int nact, int hd, int page_tokens, int n_pages, float wscale,
+                             float dscale, float* scores, void* stream);
+
+/* Paged form of rivoli_index_append for many tokens: kpool[slot_mapping[t]*hd + i] =
+ * bf16(k[t*hd + i]). Negative slots are padding; slots >= n_pages*page_tokens are counted in
+ * *bad_slots (nullable) and never written. Guards: 1001; 1004 hd % 8. */
+int rivoli_index_append_paged(const float* k, const int* slot_mapping, unsigned short* kpool,
+                              int n_tokens, int hd, int page_tokens, int n_pages,
+                              unsigned int* bad_slots, void* stream);
+
 /* Element codecs as launchers (what formats.hpp:42-57,99-106 and fwd.hip:20-45 are to the
  * reference's kernels), for census tests of the device codecs on arbitrary inputs:
  *   e4m3_encode: out[i] = f32_to_e4m3(x[i])            (rule of crates/core/src/num.rs:128-152)

@@ -152,6 +152,96 @@ int ro_index_append(const float* k, uint16_t* kcache, int pos, int hd) {
 }
 
 /* ------------------------------------------------------------------------------------------
+ * Indexer scores
+ * ---------------------------------------------------------------------------------------- */
+
+/* One token's score in the host reference's order (crates/engine/tests/indexer_kernel.rs:
+ * 240-249): per head a left fold of q*k products, then acc + w*wscale*max(dot*dscale, 0). */
+static float score_one(const float* q, const float* w, const uint16_t* krow,
+                       const uint32_t* heads, int nact, int hd, float wscale, float dscale) {
+    float acc = 0.0f;
+    for (int a = 0; a < nact; ++a) {
+        int h = heads ? (int)heads[a] : a;
+        const float* qh = q + (size_t)h * hd;
+        float dot = 0.0f;
+        for (int i = 0; i < hd; ++i) dot += qh[i] * ro_bf16_to_f32(krow[i]);
+        acc = acc + w[h] * wscale * fmaxf(dot * dscale, 0.0f);
+    }
+    return acc;
+}
+
+int ro_index_score(const float* q, const float* w, const uint16_t* kcache, const uint32_t* heads,
+                   int nt, int nh, int nact, int hd, float wscale, float dscale, float* scores) {
+    if (nt <= 0 || nh <= 0 || nact <= 0 || nact > nh || hd <= 0) return 1001;
+    for (int t = 0; t < nt; ++t)
+        scores[t] = score_one(q, w, kcache + (size_t)t * hd, heads, nact, hd, wscale, dscale);
+    return 0;
+}
+
+int ro_index_append_paged(const float* k, const int32_t* slot_mapping, uint16_t* kpool,
+                          int n_tokens, int hd, int page_tokens, int n_pages) {
+    int bad = 0;
+    for (int t = 0; t < n_tokens; ++t) {
+        int32_t slot = slot_mapping[t];
+        if (slot < 0) continue;
+        if ((int64_t)slot >= (int64_t)n_pages * page_tokens) {
+            ++bad;
+            continue;
+        }
+        for (int i = 0; i < hd; ++i)
+            kpool[(size_t)slot * hd + i] = ro_f32_to_bf16(k[(size_t)t * hd + i]);
+    }
+    return bad;
+}
+
+typedef struct {
+    const float *q, *w;
+    const uint16_t* kpool;
+    const int32_t *block_table, *nts;
+    const uint32_t* heads;
+    float* scores;
+    int n_queries, max_blocks_per_seq, stride, nh, nact, hd, page_tokens, tid, n_threads;
+    float wscale, dscale;
+} score_job;
+
+static void* score_worker(void* p) {
+    score_job* j = (score_job*)p;
+    long item = 0;
+    for (int qi = 0; qi < j->n_queries; ++qi) {
+        const float* q = j->q + (size_t)qi * j->nh * j->hd;
+        const float* w = j->w + (size_t)qi * j->nh;
+        for (int t = 0; t < j->nts[qi]; ++t, ++item) {
+            if ((item >> 6) % j->n_threads != j->tid) continue; /* 64-token slices per thread */
+            int page = j->block_table[(size_t)qi * j->max_blocks_per_seq + t / j->page_tokens];
+            size_t slot = (size_t)page * j->page_tokens + (size_t)(t % j->page_tokens);
+            j->scores[(size_t)qi * j->stride + t] = score_one(
+                q, w, j->kpool + slot * j->hd, j->heads, j->nact, j->hd, j->wscale, j->dscale);
+        }
+    }
+    return NULL;
+}
+
+void ro_index_score_paged(const float* q, const float* w, const uint16_t* kpool,
+                          const int32_t* block_table, const int32_t* nts, const uint32_t* heads,
+                          int n_queries, int max_blocks_per_seq, int stride, int nh, int nact,
+                          int hd, int page_tokens, float wscale, float dscale, float* scores,
+                          int n_threads) {
+    if (n_threads < 1) n_threads = 1;
+    pthread_t* th = (pthread_t*)malloc(sizeof(pthread_t) * (size_t)n_threads);
+    score_job* jobs = (score_job*)malloc(sizeof(score_job) * (size_t)n_threads);
+    for (int i = 0; i < n_threads; ++i) {
+        score_job j = {q, w, kpool, block_table, nts, heads, scores, n_queries,
+                       max_blocks_per_seq, stride, nh, nact, hd, page_tokens, i, n_threads,
+                       wscale, dscale};
+        jobs[i] = j;
+        pthread_create(&th[i], NULL, score_worker, &jobs[i]);
+    }
+    for (int i = 0; i < n_threads; ++i) pthread_join(th[i], NULL);
+    free(jobs);
+    free(th);
+}
+
+/* ------------------------------------------------------------------------------------------
  * Paged cache, one scale per token
  * ---------------------------------------------------------------------------------------- */
 

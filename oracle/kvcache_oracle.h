@@ -21,6 +21,9 @@
  *   paged addressing    NEW in this build (the reference has a linear slab): pinned by
  *                       identity-table equivalence with the linear slab and by permutation
  *                       invariance, not by any reference test
+ *   ro_index_score      float64 restatement within 1e-6 of the scale; the reference test's
+ *                       own separation property (head subset [5,0,6,2] vs all heads > 1e-2);
+ *                       single-head / all-negative closed forms
  *   ro_kv_gather_rows   parity unpinned by reference tests (no reference test passes
  *                       rows != null, crates/engine/tests/kernel_attend.rs:114); pinned
  *                       here by gather_rows(rows) == gather_dense()[rows]
@@ -61,6 +64,23 @@ int ro_append_kv(const float* latent, const float* rope, uint8_t* lc8, float* ls
                  uint16_t* rc, int pos, int kvl, int ropn, int n_blocks);
 /* crates/backend/kernels/indexer.hip:54-58 */
 int ro_index_append(const float* k, uint16_t* kcache, int pos, int hd);
+
+/* ---- indexer scores: crates/backend/kernels/indexer.hip:60-93, host restatement
+ *      crates/engine/tests/indexer_kernel.rs:238-250 (same fold order):
+ *      scores[t] = sum over active heads h of w[h]*wscale*max((q_h . k_t)*dscale, 0).
+ *      kcache is [nt][hd] bf16; heads (nullable) lists the nact active heads. Returns the
+ *      launcher's guard code (crates/backend/kernels/indexer.hip:281). ---- */
+int ro_index_score(const float* q, const float* w, const uint16_t* kcache, const uint32_t* heads,
+                   int nt, int nh, int nact, int hd, float wscale, float dscale, float* scores);
+/* Paged forms (new here): the key cache is [n_pages*page_tokens][hd] bf16 addressed by slot;
+ * query qi scores its first nts[qi] tokens through block_table[qi]. */
+int ro_index_append_paged(const float* k, const int32_t* slot_mapping, uint16_t* kpool,
+                          int n_tokens, int hd, int page_tokens, int n_pages);
+void ro_index_score_paged(const float* q, const float* w, const uint16_t* kpool,
+                          const int32_t* block_table, const int32_t* nts, const uint32_t* heads,
+                          int n_queries, int max_blocks_per_seq, int stride, int nh, int nact,
+                          int hd, int page_tokens, float wscale, float dscale, float* scores,
+                          int n_threads);
 
 /* ---- paged fp8 cache, one f32 scale per token (block = whole row) ----
  * Page layout: [page_tokens][width] u8 codes, then [page_tokens] f32 scales. */

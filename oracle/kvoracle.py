@@ -54,6 +54,10 @@ class Oracle:
             "ro_quant_block": (None, [f32p, C.c_int, u8p, f32p]),
             "ro_append_kv": (C.c_int, [f32p, f32p, u8p, f32p, u16p] + [C.c_int] * 4),
             "ro_index_append": (C.c_int, [f32p, u16p, C.c_int, C.c_int]),
+            "ro_index_score": (C.c_int, [f32p, f32p, u16p, u32p] + [C.c_int] * 4 + [C.c_float] * 2 + [f32p]),
+            "ro_index_append_paged": (C.c_int, [f32p, i32p, u16p] + [C.c_int] * 4),
+            "ro_index_score_paged": (None, [f32p, f32p, u16p, i32p, i32p, u32p] + [C.c_int] * 7
+                                     + [C.c_float] * 2 + [f32p, C.c_int]),
             "ro_kv_page_bytes": (C.c_size_t, [C.c_int, C.c_int]),
             "ro_kv_append_paged": (C.c_int, [u16p, i32p, u8p] + [C.c_int] * 4),
             "ro_kv_append_paged_mt": (None, [u16p, i32p, u8p] + [C.c_int] * 5),
@@ -113,6 +117,40 @@ class Oracle:
     def index_append(self, k, kcache, pos, hd) -> int:
         k = _c(k, np.float32)
         return int(self.lib.ro_index_append(_ptr(k, C.c_float), _ptr(kcache, C.c_uint16), pos, hd))
+
+    # ---- indexer scores -----------------------------------------------------------------
+    def index_score(self, q, w, kcache_bf16, heads, nh, hd, wscale, dscale):
+        """Returns (guard code, scores[nt])."""
+        q, w, kc = _c(q, np.float32), _c(w, np.float32), _c(kcache_bf16, np.uint16)
+        nt = kc.size // hd
+        hs = None if heads is None else _c(heads, np.uint32)
+        nact = nh if hs is None else hs.size
+        scores = np.zeros(max(nt, 0), np.float32)
+        rc = self.lib.ro_index_score(_ptr(q, C.c_float), _ptr(w, C.c_float), _ptr(kc, C.c_uint16),
+                                     None if hs is None else _ptr(hs, C.c_uint32), nt, nh, nact,
+                                     hd, wscale, dscale, _ptr(scores, C.c_float))
+        return int(rc), scores
+
+    def index_append_paged(self, k, slot_mapping, kpool, hd, page_tokens, n_pages) -> int:
+        k, slot_mapping = _c(k, np.float32), _c(slot_mapping, np.int32)
+        return int(self.lib.ro_index_append_paged(_ptr(k, C.c_float), _ptr(slot_mapping, C.c_int32),
+                                                  _ptr(kpool, C.c_uint16), slot_mapping.size, hd,
+                                                  page_tokens, n_pages))
+
+    def index_score_paged(self, q, w, kpool, block_table, nts, heads, stride, hd, page_tokens,
+                          wscale, dscale, n_threads: int = 1) -> np.ndarray:
+        q, w = _c(q, np.float32), _c(w, np.float32)
+        block_table, nts = _c(block_table, np.int32), _c(nts, np.int32)
+        n_q, nh = w.shape
+        hs = None if heads is None else _c(heads, np.uint32)
+        nact = nh if hs is None else hs.size
+        scores = np.zeros((n_q, stride), np.float32)
+        self.lib.ro_index_score_paged(
+            _ptr(q, C.c_float), _ptr(w, C.c_float), _ptr(kpool, C.c_uint16),
+            _ptr(block_table, C.c_int32), _ptr(nts, C.c_int32),
+            None if hs is None else _ptr(hs, C.c_uint32), n_q, block_table.shape[1], stride, nh,
+            nact, hd, page_tokens, wscale, dscale, _ptr(scores, C.c_float), n_threads)
+        return scores
 
     # ---- paged cache --------------------------------------------------------------------
     def kv_page_bytes(self, page_tokens: int, width: int) -> int:

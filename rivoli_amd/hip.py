@@ -42,6 +42,9 @@ _SIGNATURES = {
     "rivoli_index_append": [_VP, _VP, _I, _I],
     "rivoli_index_topk": [_VP, _I, _I, _VP],
     "rivoli_index_topk_batched": [_VP, _I, _I, _VP, _I, _I, _VP, _VP, _VP],
+    "rivoli_index_score": [_VP] * 4 + [_I] * 4 + [_F, _F, _VP],
+    "rivoli_index_score_paged": [_VP] * 6 + [_I] * 9 + [_F, _F, _VP, _VP],
+    "rivoli_index_append_paged": [_VP, _VP, _VP, _I, _I, _I, _I, _VP, _VP],
     "rivoli_hash_rows": [_VP, _I, _I, _ULL, _VP, _VP],
     "rivoli_device_sync": [],
     "rivoli_kv_append_paged": [_VP, _VP, _VP, _I, _I, _I, _I, _VP, _VP],
@@ -120,6 +123,27 @@ def launch_index_append(k, kcache, pos, hd) -> None:
 
 def launch_index_topk(scores, nt, k, rows) -> None:
     ensure_hip_status(lib().rivoli_index_topk(_p(scores), nt, k, _p(rows)), "index_topk")
+
+
+def launch_index_score(q, w, kcache, heads, nt, nh, nact, hd, wscale, dscale, scores) -> None:
+    ensure_hip_status(lib().rivoli_index_score(_p(q), _p(w), _p(kcache), _p(heads), nt, nh, nact,
+                                               hd, wscale, dscale, _p(scores)), "index_score")
+
+
+def launch_index_score_paged(q, w, kpool, block_table, nts, heads, n_queries, max_blocks_per_seq,
+                             stride, nt, nh, nact, hd, page_tokens, n_pages, wscale, dscale,
+                             scores, stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_index_score_paged(
+        _p(q), _p(w), _p(kpool), _p(block_table), _p(nts), _p(heads), n_queries,
+        max_blocks_per_seq, stride, nt, nh, nact, hd, page_tokens, n_pages, wscale, dscale,
+        _p(scores), _s(stream)), "index_score_paged")
+
+
+def launch_index_append_paged(k, slot_mapping, kpool, n_tokens, hd, page_tokens, n_pages,
+                              bad_slots=None, stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_index_append_paged(_p(k), _p(slot_mapping), _p(kpool), n_tokens,
+                                                      hd, page_tokens, n_pages, _p(bad_slots),
+                                                      _s(stream)), "index_append_paged")
 
 
 def launch_hash_rows(x, n, stride, i_base, out, stream=NULL_STREAM) -> None:
