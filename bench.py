@@ -40,9 +40,10 @@ def parse():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=32768)
-    ap.add_argument("--workload", choices=["decode", "prefill", "dsa"], default="decode",
-                    help="decode = benchmark configuration 3 (the headline line); prefill = config 2 "
-                         "bulk append; dsa = config 4 top-k + sparse gather")
+    ap.add_argument("--workload", choices=["decode", "prefill", "dsa", "dsa_scored"], default="decode",
+                    help="decode = configuration 3 (the headline line); prefill = configuration 2 "
+                         "bulk append; dsa = configuration 4 top-k + sparse gather on synthetic "
+                         "scores; dsa_scored = the same with the scores computed on the device")
     ap.add_argument("--tokens", type=int, default=8192, help="prefill: new tokens per step")
     ap.add_argument("--topk", type=int, default=2048)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -74,8 +75,8 @@ def main():
         del src, dst
     if a.workload == "prefill":
         return bench_prefill(a, torch, hip)
-    if a.workload == "dsa":
-        return bench_dsa(a, torch, hip)
+    if a.workload in ("dsa", "dsa_scored"):
+        return bench_dsa(a, torch, hip, scored=a.workload == "dsa_scored")
     L, B, ctx = a.layers, a.batch, a.ctx
     blocks = -(-ctx // PT)
     n_pages = B * blocks
@@ -261,7 +262,7 @@ def bench_prefill(a, torch, hip):
     print(json.dumps(res), flush=True)
 
 
-def bench_dsa(a, torch, hip):
+def bench_dsa(a, torch, hip, scored=False):
     """benchmark configuration 4: per layer, select the top-k of 65536 indexer scores for each of 16
     queries (ties to the lowest index), then gather + dequantize those rows from fragmented
     pages. One step = all layers."""
@@ -284,21 +285,42 @@ def bench_dsa(a, torch, hip):
         pools.append(pool)
     del kv_rows
     scores = []
-    for _ in range(L):
-        sc = torch.randn(B, nt, generator=g, device="cuda", dtype=torch.float32)
-        sc[:, -64:] += 4.0                                       # recency boost
-        scores.append(sc)
+    NH, HD = 64, 128                                             # indexer heads x head dim
+    if scored:
+        # one paged bf16 key cache per layer (same block tables), filled by index_append_paged;
+        # every layer gets its own queries and head weights
+        keys = torch.randn(B * nt, HD, generator=g, device="cuda", dtype=torch.float32)
+        kpools, qs, ws = [], [], []
+        for _ in range(L):
+            kp = torch.empty(n_pages * PT * HD, dtype=torch.bfloat16, device="cuda")
+            hip.launch_index_append_paged(keys, slots_all, kp, B * nt, HD, PT, n_pages)
+            kpools.append(kp)
+            qs.append(torch.randn(B, NH, HD, generator=g, device="cuda", dtype=torch.float32))
+            ws.append(torch.rand(B, NH, generator=g, device="cuda", dtype=torch.float32))
+        del keys
+        score_buf = torch.empty(B, nt, dtype=torch.float32, device="cuda")
+    else:
+        for _ in range(L):
+            sc = torch.randn(B, nt, generator=g, device="cuda", dtype=torch.float32)
+            sc[:, -64:] += 4.0                                   # recency boost
+            scores.append(sc)
     sel = torch.empty(B * k, dtype=torch.int32, device="cuda")
     out = torch.empty(B * k * W, dtype=torch.bfloat16, device="cuda")
-    ws = torch.zeros(hip.index_topk_workspace_bytes(B, nt), dtype=torch.uint8, device="cuda")
+    ws_topk = torch.zeros(hip.index_topk_workspace_bytes(B, nt), dtype=torch.uint8, device="cuda")
     torch.cuda.synchronize()
     stream = torch.cuda.Stream()
     sh = stream.cuda_stream
 
     def step(events):
         for layer in range(L):
+            if scored:
+                bracket(torch, stream, events, "score",
+                        lambda: hip.launch_index_score_paged(
+                            qs[layer], ws[layer], kpools[layer], tables, None, None, B, blocks, nt,
+                            nt, NH, NH, HD, PT, n_pages, HD ** -0.5, 1.0, score_buf, sh))
+            sc_in = score_buf if scored else scores[layer]
             bracket(torch, stream, events, "topk",
-                    lambda: hip.launch_index_topk_batched(scores[layer], B, nt, None, nt, k, sel, ws, sh))
+                    lambda: hip.launch_index_topk_batched(sc_in, B, nt, None, nt, k, sel, ws_topk, sh))
             bracket(torch, stream, events, "gather_rows",
                     lambda: hip.launch_kv_gather_rows_paged(pools[layer], tables, sel, None, out, B, k,
                                                             blocks, W, PT, n_pages, None, sh))
@@ -306,7 +328,8 @@ def bench_dsa(a, torch, hip):
     ms, per = timed(torch, stream, a.steps, a.warmup, step)
     topk_bytes = B * nt * 4 + B * k * 4
     rows_bytes = B * k * (4 + REC + ROW_IN) + B * blocks * 4
-    layer_bytes = topk_bytes + rows_bytes
+    score_bytes = (B * nt * (HD * 2 + 4) + B * NH * (HD + 1) * 4 + B * blocks * 4) if scored else 0
+    layer_bytes = topk_bytes + rows_bytes + score_bytes
     res = {"metric": "kv_dsa_topk_gather_GBps", "value": round(L * layer_bytes / (ms * 1e-3) / 1e9, 2),
            "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
@@ -323,7 +346,14 @@ def bench_dsa(a, torch, hip):
                         "bytes_per_launch": rows_bytes, "traffic": None},
            "topk": {"achieved": round(topk_bytes / (per["topk"] * 1e-3) / 1e9, 2), "unit": "GB/s",
                     "avg_launch_ms": round(per["topk"], 5), "bytes_per_launch": topk_bytes}}
-    if not a.no_cpu_baseline:
+    if scored:
+        res["config"]["workload"] = ("DSA sparse path with device scores: index_score (64 heads x "
+                                     "128, paged bf16 keys) -> top-k -> sparse row gather")
+        res["index_score"] = {"achieved": round(score_bytes / (per["score"] * 1e-3) / 1e9, 2),
+                              "unit": "GB/s", "frac": round(score_bytes / (per["score"] * 1e-3) / HBM_PEAK, 4),
+                              "avg_launch_ms": round(per["score"], 5), "bytes_per_launch": score_bytes,
+                              "tflops": round(B * nt * NH * HD * 2 * 2 / (per["score"] * 1e-3) / 1e12, 1)}
+    if not a.no_cpu_baseline and not scored:
         from oracle.kvoracle import oracle as get_oracle
 
         ora, cores = get_oracle(), max(1, min(16, os.cpu_count() or 1))
@@ -335,7 +365,7 @@ def bench_dsa(a, torch, hip):
             want_rows = ora.kv_gather_rows_paged(pool_h, tables_np, want_sel, W, PT)
             spent += time.perf_counter() - t0
             reps += 1
-        hip.launch_index_topk_batched(scores[0], B, nt, None, nt, k, sel, ws)
+        hip.launch_index_topk_batched(scores[0], B, nt, None, nt, k, sel, ws_topk)
         hip.launch_kv_gather_rows_paged(pools[0], tables, sel, None, out, B, k, blocks, W, PT, n_pages)
         torch.cuda.synchronize()
         if not np.array_equal(sel.cpu().numpy().view(np.uint32).reshape(B, k), want_sel):

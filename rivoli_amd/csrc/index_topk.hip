@@ -239,7 +239,9 @@ constexpr int kTopkWaves = kTopkThreads / kWave;
 // histogram pass (1024 bins x 8 bank copies), one count, one ordered compaction of the keys
 // in the pivot bin or above into LDS — and everything after that (the remaining 22 bits of
 // the radix select, the ordered emission) runs over those few thousand candidates only.
-// Falls back to topk_block when the candidates do not fit (degenerate score arrays).
+// The histogram window adapts to the data (it starts at the highest bit in which the keys
+// differ and descends into the pivot bin while that bin is too full), and a pivot value tied
+// more often than LDS can list is emitted straight from the registers.
 constexpr int kLeanBits = 10;
 constexpr int kLeanBins = 1 << kLeanBits;  // == kTopkThreads: one thread per bin
 constexpr int kLeanCopies = 8;
@@ -247,7 +249,6 @@ constexpr int kLeanLow = 32 - kLeanBits;
 constexpr int kLeanCap = 12288;  // candidates held in LDS (index + key)
 static_assert(kLeanBins == kTopkThreads, "one thread per bin");
 constexpr int kLeanLdsWords = 2 * kLeanCap + kLeanBins * kLeanCopies + 4 * kTopkWaves + 8;
-static_assert(topk_block_lds_words<kTopkThreads>() <= kLeanLdsWords, "fallback fits");
 static_assert(kLeanCap < 65536, "emission packs two counts into 16 bits each");
 
 // Sum over the 16 wave slots of v[w] for w < wave (*before) and over all of them (*all).
@@ -267,15 +268,29 @@ __device__ __forceinline__ void wave_slots_prefix(const uint32_t* v, int wave, u
     *before = __builtin_amdgcn_readfirstlane(b);
 }
 
+// Min and max over the 16 wave slots of lo[w] / hi[w]; every lane of the wave must call it.
+__device__ __forceinline__ void wave_slots_minmax(const uint32_t* lo, const uint32_t* hi,
+                                                  uint32_t* mn, uint32_t* mx) {
+    const int lane = threadIdx.x & (kWave - 1);
+    uint32_t a = lane < kTopkWaves ? lo[lane] : ~0u, b = lane < kTopkWaves ? hi[lane] : 0u;
+#pragma unroll
+    for (int off = kTopkWaves / 2; off > 0; off >>= 1) {
+        a = min(a, (uint32_t)__shfl_xor(a, off, kWave));
+        b = max(b, (uint32_t)__shfl_xor(b, off, kWave));
+    }
+    *mn = __builtin_amdgcn_readfirstlane(a);
+    *mx = __builtin_amdgcn_readfirstlane(b);
+}
+
 template <int ITEMS>
 __device__ __forceinline__ void topk_block_lean(const float* __restrict__ s, int nt, uint32_t kq,
                                                 uint32_t* __restrict__ out, uint32_t* lds) {
     uint32_t* c_idx = lds;  // the candidates, in index order
     uint32_t* c_key = lds + kLeanCap;
-    uint32_t* s_hist = lds + 2 * kLeanCap;        // later reused as the 256-bin histogram
+    uint32_t* s_hist = lds + 2 * kLeanCap;  // later reused as the 256-bin histogram
     uint32_t* s_wa = s_hist + kLeanBins * kLeanCopies;
     uint32_t* s_wb = s_wa + kTopkWaves;
-    uint32_t* s_pn = s_wb + kTopkWaves;  // [0] bin, [1] need, [2] candidate total
+    uint32_t* s_pn = s_wb + kTopkWaves;  // [0] bin, [1] need inside it, [2] its count
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -313,50 +328,128 @@ __device__ __forceinline__ void topk_block_lean(const float* __restrict__ s, int
         }
     }
 
-    // ---- pass 1: histogram of the top 10 bits ----
-    for (int i = tid; i < kLeanBins * kLeanCopies; i += kTopkThreads) s_hist[i] = 0u;
-    __syncthreads();
-    uint32_t* my_copy = s_hist + (lane & (kLeanCopies - 1));
+    // ---- where the keys differ: real score arrays (sums of ReLU'd terms, all positive) sit
+    // in two or three binades, so a fixed window on the top bits would put nearly every key
+    // in one bin. The histogram window starts at the highest bit in which max and min differ.
+    uint32_t kmin = ~0u, kmax = 0u;
     both([&](auto F) {
         sweep<ITEMS>(steps, [&](int j) {
-            if (decltype(F)::value || j * kWave < limit)
-                atomicAdd(&my_copy[(key[j] >> kLeanLow) * kLeanCopies], 1u);
+            if (decltype(F)::value || j * kWave < limit) {
+                kmin = min(kmin, key[j]);
+                kmax = max(kmax, key[j]);
+            }
         });
     });
-    __syncthreads();
-    uint32_t cnt = 0;
 #pragma unroll
-    for (int c = 0; c < kLeanCopies; ++c)
-        cnt += s_hist[tid * kLeanCopies + ((c + lane) & (kLeanCopies - 1))];
-    // suffix counts over threads (= bins): how many keys sit in higher bins than mine
-    uint32_t suffix = cnt;
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        uint32_t v = __shfl_down(suffix, off, kWave);
-        if (lane + off < kWave) suffix += v;
+    for (int off = 32; off > 0; off >>= 1) {
+        kmin = min(kmin, (uint32_t)__shfl_xor(kmin, off, kWave));
+        kmax = max(kmax, (uint32_t)__shfl_xor(kmax, off, kWave));
     }
-    if (lane == 0) s_wa[wave] = suffix;  // the wave's total
-    __syncthreads();
-    uint32_t lower, all;
-    wave_slots_prefix(s_wa, wave + 1, &lower, &all);
-    const uint32_t above = all - lower + (suffix - cnt);  // higher waves + higher lanes
-    if (above < kq && kq <= above + cnt) {
-        s_pn[0] = (uint32_t)tid;
-        s_pn[1] = kq - above;
-        s_pn[2] = above + cnt;
+    if (lane == 0) {
+        s_wa[wave] = kmin;
+        s_wb[wave] = kmax;
     }
     __syncthreads();
-    const uint32_t pbin = s_pn[0];
-    uint32_t need = s_pn[1];
-    const uint32_t total = s_pn[2];
+    wave_slots_minmax(s_wa, s_wb, &kmin, &kmax);
+    const uint32_t diff = kmin ^ kmax;
+    const int top = diff ? 31 - __builtin_clz(diff) : 0;  // highest bit that is not common
+    int shift = top > kLeanBits - 1 ? top - (kLeanBits - 1) : 0;
+    int width = top + 1 - shift;
+    uint32_t mask = top == 31 ? 0u : (~0u << (top + 1));  // bits every key shares
+    uint32_t prefix = kmax & mask;
+    uint32_t need = kq;  // how many are still to be taken from the keys matching `prefix`
+    uint32_t total;      // how many keys are >= the pivot bin's first key
+
+    // ---- histogram levels: 10 bits at a time below the common prefix, descending into the
+    // pivot bin only while it and everything above it are too many to hold as candidates ----
+    uint32_t* my_copy = s_hist + (lane & (kLeanCopies - 1));
+    for (;;) {
+        __syncthreads();  // s_wa / s_pn / s_hist from the previous use are no longer read
+        for (int i = tid; i < kLeanBins * kLeanCopies; i += kTopkThreads) s_hist[i] = 0u;
+        __syncthreads();
+        const uint32_t dmask = (1u << width) - 1u;
+        // (conditional on purpose: with unconditional LDS atomics the compiler runs all 64
+        // address computations ahead of them and spills the key registers)
+        both([&](auto F) {
+            sweep<ITEMS>(steps, [&](int j) {
+                if ((decltype(F)::value || j * kWave < limit) && (key[j] & mask) == prefix)
+                    atomicAdd(&my_copy[__builtin_amdgcn_ubfe(key[j], shift, width) * kLeanCopies], 1u);
+            });
+        });
+        __syncthreads();
+        uint32_t cnt = 0;  // thread tid owns bin tid
+#pragma unroll
+        for (int c = 0; c < kLeanCopies; ++c)
+            cnt += s_hist[tid * kLeanCopies + ((c + lane) & (kLeanCopies - 1))];
+        uint32_t suffix = cnt;  // keys in this bin and the higher bins of this wave
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            uint32_t v = __shfl_down(suffix, off, kWave);
+            if (lane + off < kWave) suffix += v;
+        }
+        if (lane == 0) s_wa[wave] = suffix;
+        __syncthreads();
+        uint32_t lower, all;
+        wave_slots_prefix(s_wa, wave + 1, &lower, &all);
+        const uint32_t above = all - lower + (suffix - cnt);  // higher waves + higher lanes
+        if (above < need && need <= above + cnt) {
+            s_pn[0] = (uint32_t)tid;
+            s_pn[1] = need - above;
+            s_pn[2] = cnt;
+        }
+        __syncthreads();
+        prefix |= s_pn[0] << shift;
+        mask |= dmask << shift;
+        need = s_pn[1];
+        total = kq - need + s_pn[2];  // everything already sure (kq - need) plus the pivot bin
+        if (total <= (uint32_t)kLeanCap || shift == 0) break;
+        const int next = shift > kLeanBits ? shift - kLeanBits : 0;
+        width = shift - next;
+        shift = next;
+    }
+
     if (total > (uint32_t)kLeanCap) {
-        // rare (huge ties): the streaming form re-reads the scores and needs no key registers
-        topk_block<kTopkThreads, 0>(s, nt, kq, out, lds);
+        // Every bit is fixed and the pivot VALUE itself is tied too often to list (e.g. a
+        // ReLU-sparse array whose tail is all zeros): emit straight from the registers —
+        // every key above the pivot, and the first `need` keys equal to it, in index order.
+        const uint32_t pivot = prefix;
+        uint32_t cnt_gt = 0, cnt_eq = 0;
+        both([&](auto F) {
+            sweep<ITEMS>(steps, [&](int j) {
+                const bool live = decltype(F)::value || j * kWave < limit;
+                cnt_gt += (uint32_t)__popcll(__ballot(live && key[j] > pivot));
+                cnt_eq += (uint32_t)__popcll(__ballot(live && key[j] == pivot));
+            });
+        });
+        __syncthreads();
+        if (lane == 0) {
+            s_wa[wave] = cnt_gt;
+            s_wb[wave] = cnt_eq;
+        }
+        __syncthreads();
+        uint32_t run_gt, run_eq, unused;
+        wave_slots_prefix(s_wa, wave, &run_gt, &unused);
+        wave_slots_prefix(s_wb, wave, &run_eq, &unused);
+        uint32_t idx = (uint32_t)(seg0 + lane);
+        both([&](auto F) {
+            sweep<ITEMS>(steps, [&](int j) {
+                const bool live = decltype(F)::value || j * kWave < limit;
+                const bool g = live && key[j] > pivot, e = live && key[j] == pivot;
+                const unsigned long long mg = __ballot(g), me = __ballot(e);
+                const uint32_t G = run_gt + lanes_below(mg), E = run_eq + lanes_below(me);
+                const uint32_t slot = G + (E < need ? E : need);
+                if ((g || (e && E < need)) && slot < kq) out[slot] = idx;
+                run_gt += (uint32_t)__popcll(mg);
+                run_eq += (uint32_t)__popcll(me);
+                idx += kWave;
+                asm volatile("" : "+v"(idx));
+            });
+        });
         return;
     }
 
-    // ---- pass 2: candidates per wave (a candidate is key >= the pivot bin's first key) ----
-    const uint32_t thr = pbin << kLeanLow;
+    // ---- candidates per wave (a candidate is key >= the pivot bin's first key) ----
+    const uint32_t thr = prefix;
     uint32_t mine = 0;
     both([&](auto F) {
         sweep<ITEMS>(steps, [&](int j) {
@@ -364,12 +457,13 @@ __device__ __forceinline__ void topk_block_lean(const float* __restrict__ s, int
             mine += (uint32_t)__popcll(__ballot(is));  // scalar popcount: one VALU op per key
         });
     });
+    __syncthreads();
     if (lane == 0) s_wb[wave] = mine;
     __syncthreads();
     uint32_t run, unused;
     wave_slots_prefix(s_wb, wave, &run, &unused);
 
-    // ---- pass 3: ordered compaction of (index, key) into LDS ----
+    // ---- ordered compaction of (index, key) into LDS ----
     // the element index is carried as a running register (a per-step constant would be
     // materialised 64 times over and spill)
     uint32_t idx = (uint32_t)(seg0 + lane);
@@ -389,24 +483,27 @@ __device__ __forceinline__ void topk_block_lean(const float* __restrict__ s, int
     });
     __syncthreads();
 
-    // ---- the remaining 22 bits among the pivot bin's members: 8 + 8 + 6 ----
+    // ---- the bits below the last window, among the pivot bin's members, 8 at a time ----
     uint32_t* s_bins = s_hist;
-    uint32_t pivot = thr, mask = ~0u << kLeanLow;
-    for (int shift = kLeanLow - 8;; shift = shift >= 8 ? shift - 8 : 0) {
-        const uint32_t dmask = (shift == 0 && (kLeanLow % 8)) ? (1u << (kLeanLow % 8)) - 1u : 0xffu;
+    uint32_t pivot = prefix;
+    for (int left = shift; left > 0;) {
+        const int take = left < 8 ? left : 8;
+        const int sh = left - take;
+        const uint32_t dmask = (1u << take) - 1u;
         if (tid < kBins) s_bins[tid] = 0u;
         __syncthreads();
         for (uint32_t c = tid; c < total; c += kTopkThreads) {
             const uint32_t u = c_key[c];
-            if ((u & mask) == pivot) atomicAdd(&s_bins[(u >> shift) & dmask], 1u);
+            if ((u & mask) == pivot) atomicAdd(&s_bins[(u >> sh) & dmask], 1u);
         }
         __syncthreads();
         if (wave == 0) find_pivot_bin(s_bins, need, s_pn, lane);
         __syncthreads();
-        pivot |= s_pn[0] << shift;
+        pivot |= s_pn[0] << sh;
         need = s_pn[1];
-        mask |= dmask << shift;
-        if (shift == 0) break;
+        mask |= dmask << sh;
+        left = sh;
+        __syncthreads();
     }
 
     // ---- ordered emission: each thread owns a run of consecutive candidates ----
