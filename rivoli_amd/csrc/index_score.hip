@@ -16,7 +16,7 @@
 // bf16 rounding of q would miss. With heads as the tile's ROWS a lane holds 16 heads of one
 // token, so ReLU, the head weights and the sum over heads are register arithmetic plus one
 // cross-half shuffle; nothing goes through LDS after the query is staged.
-// A workgroup stages its query once and walks 512 tokens (4 waves x 4 blocks of 32). The
+// A workgroup stages its query once and walks 2048 tokens (4 waves x 16 blocks of 32). The
 // kernel reads hd*2 bytes per token and is bound by that stream, not by the matrix cores.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
 #include "codec.hpp"
@@ -30,7 +30,7 @@ constexpr int kScoreThreads = 256;
 constexpr int kScoreWaves = kScoreThreads / kWave;
 constexpr int kScoreMaxHeads = 64;   // active heads, padded to a multiple of 32
 constexpr int kScoreMaxHd = 128;     // head dimension, a multiple of 16
-constexpr int kScoreBlocks = 4;      // 32-token blocks per wave
+constexpr int kScoreBlocks = 16;     // 32-token blocks per wave
 constexpr int kScoreTokensPerGroup = kScoreWaves * kScoreBlocks * 32;
 constexpr int kScoreRowPad = 8;      // bf16 of padding per staged query row
 
@@ -45,6 +45,8 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
     __shared__ __attribute__((aligned(16))) uint16_t s_qh[RB * 32][kScoreMaxHd + kScoreRowPad];
     __shared__ __attribute__((aligned(16))) uint16_t s_ql[RB * 32][kScoreMaxHd + kScoreRowPad];
     __shared__ float s_w[RB * 32];
+    __shared__ __attribute__((aligned(16)))
+    uint16_t s_k[kScoreWaves][32][kScoreMaxHd + kScoreRowPad];  // one key tile per wave
 
     const int qi = blockIdx.y;
     const int nt = nts ? min(nts[qi], nt_all) : nt_all;
@@ -55,17 +57,30 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     // ---- stage the active heads: q = hi + lo in bf16, and the per-head weight ----
-    for (int idx = tid; idx < RB * 32 * hd; idx += kScoreThreads) {
-        const int a = idx / hd, d = idx - a * hd;
-        float val = 0.0f;
+    // eight consecutive query values per step: two 16-byte loads in, two 16-byte LDS stores out
+    const int cpr = hd >> 3;
+    for (int c = tid; c < RB * 32 * cpr; c += kScoreThreads) {
+        const int a = c / cpr, d = (c - a * cpr) * 8;
+        float val[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         if (a < nact) {
             const int h = heads ? (int)heads[a] : a;
-            if ((unsigned)h < (unsigned)nh) val = q[((size_t)qi * nh + h) * hd + d];
+            if ((unsigned)h < (unsigned)nh) {
+                const float4* src =
+                    reinterpret_cast<const float4*>(q + ((size_t)qi * nh + h) * hd + d);
+                const float4 v0 = src[0], v1 = src[1];
+                val[0] = v0.x, val[1] = v0.y, val[2] = v0.z, val[3] = v0.w;
+                val[4] = v1.x, val[5] = v1.y, val[6] = v1.z, val[7] = v1.w;
+            }
         }
-        const uint16_t hi = f32_to_bf16(val);
-        const uint16_t lo = f32_to_bf16(val - __uint_as_float((uint32_t)hi << 16));
-        s_qh[a][d] = hi;
-        s_ql[a][d] = lo;
+        uint32_t hi[4], lo[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            hi[i] = pack_bf16x2(val[2 * i], val[2 * i + 1]);
+            lo[i] = pack_bf16x2(val[2 * i] - bf16_lo_to_f32(hi[i]),
+                                val[2 * i + 1] - bf16_hi_to_f32(hi[i]));
+        }
+        *reinterpret_cast<u32x4*>(&s_qh[a][d]) = u32x4{hi[0], hi[1], hi[2], hi[3]};
+        *reinterpret_cast<u32x4*>(&s_ql[a][d]) = u32x4{lo[0], lo[1], lo[2], lo[3]};
     }
     if (tid < RB * 32) {
         float wv = 0.0f;  // padding heads weigh nothing
@@ -80,24 +95,66 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
     const int col = lane & 31;        // the lane's token within a block / head within a row block
     const int khalf = (lane >> 5) * 8;  // which 8 of each 16-wide K-step this lane carries
     const int ksteps = hd >> 4;
-    for (int it = 0; it < kScoreBlocks; ++it) {
-        const int tb = t0 + (it * kScoreWaves + wave) * 32;
-        if (tb >= nt) break;  // wave-uniform
-        const int token = tb + col;
-        bool valid = token < nt;
-        const int tc = valid ? token : nt - 1;  // a clamped, always readable token
-        size_t slot = (size_t)tc;
-        if (block_table) {
-            const int page = block_table[(size_t)qi * max_blocks_per_seq + tc / page_tokens];
-            const bool ok = (unsigned)page < (unsigned)n_pages;
-            valid = valid && ok;
-            slot = ok ? (size_t)page * page_tokens + (size_t)(tc % page_tokens) : 0;
-        }
-        const uint16_t* krow = kpool + slot * hd + khalf;
-        bf16x8 kb[kScoreMaxHd / 16];
+    // accumulator element v of a lane is head row 8*(v/4) + 4*(lane/32) + v%4, token `col`:
+    // the lane's 16 (32) head weights are fixed for the whole kernel, so they sit in registers
+    float wv[RB][16];
 #pragma unroll
-        for (int s = 0; s < kScoreMaxHd / 16; ++s)
-            if (s < ksteps) kb[s] = *reinterpret_cast<const bf16x8*>(krow + 16 * s);
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            wv[rb][v] = s_w[rb * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)];
+
+    // A block's 32 key rows are one contiguous run (consecutive tokens of one page, or of the
+    // linear cache), so the wave fetches it with fully coalesced 16-byte loads, parks it in its
+    // own LDS tile and reads it back in the matrix core's operand layout. Fetching each lane's
+    // operand straight from memory instead touches 32 different rows per instruction and was
+    // measured ~1.6x slower. The next block's fetch is issued before this block's MFMAs.
+    constexpr int kChunks = 32 * kScoreMaxHd / 8 / kWave;  // 16-byte chunks per lane per block
+    uint16_t(*tile)[kScoreMaxHd + kScoreRowPad] = s_k[wave];
+    const int cprk = hd >> 3;                               // 16-byte chunks per key row
+    auto block_base = [&](int tb, int& rows_ok) -> const uint16_t* {
+        rows_ok = min(32, nt - tb);
+        size_t slot = (size_t)tb;
+        if (block_table) {
+            const int page = block_table[(size_t)qi * max_blocks_per_seq + tb / page_tokens];
+            if ((unsigned)page >= (unsigned)n_pages) {
+                rows_ok = 0;  // nothing of this block is readable or written
+                return kpool;
+            }
+            slot = (size_t)page * page_tokens + (size_t)(tb % page_tokens);
+        }
+        return kpool + slot * hd;
+    };
+    auto fetch = [&](const uint16_t* base, int rows_ok, u32x4 (&raw)[kChunks]) {
+#pragma unroll
+        for (int j = 0; j < kChunks; ++j) {
+            const int c = lane + j * kWave;
+            raw[j] = (c < rows_ok * cprk) ? reinterpret_cast<const u32x4*>(base)[c]
+                                          : u32x4{0, 0, 0, 0};
+        }
+    };
+
+    int tb = t0 + wave * 32, rows_ok = 0;
+    u32x4 raw[kChunks];
+    if (tb < nt) fetch(block_base(tb, rows_ok), rows_ok, raw);
+    for (int it = 0; it < kScoreBlocks && tb < nt; ++it) {
+        // park this block; the wave's LDS operations execute in order, the fences only keep
+        // the compiler from moving the reads above the writes (and the next writes above them)
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+        for (int j = 0; j < kChunks; ++j) {
+            const int c = lane + j * kWave;
+            if (c < 32 * cprk) {
+                const int r = c / cprk, cc = c - r * cprk;
+                *reinterpret_cast<u32x4*>(&tile[r][cc * 8]) = raw[j];
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        const int token = tb + col;
+        const bool valid = col < rows_ok;
+        const int tb_next = tb + kScoreWaves * 32;
+        int rows_next = 0;
+        if (it + 1 < kScoreBlocks && tb_next < nt) fetch(block_base(tb_next, rows_next), rows_next, raw);
 
         f32x16 acc[RB];
 #pragma unroll
@@ -107,28 +164,27 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
 #pragma unroll
         for (int s = 0; s < kScoreMaxHd / 16; ++s) {
             if (s < ksteps) {
+                const bf16x8 kb = *reinterpret_cast<const bf16x8*>(&tile[col][khalf + 16 * s]);
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb) {
                     const bf16x8 ah =
                         *reinterpret_cast<const bf16x8*>(&s_qh[rb * 32 + col][khalf + 16 * s]);
                     const bf16x8 al =
                         *reinterpret_cast<const bf16x8*>(&s_ql[rb * 32 + col][khalf + 16 * s]);
-                    acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, kb[s], acc[rb], 0, 0, 0);
-                    acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, kb[s], acc[rb], 0, 0, 0);
+                    acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, kb, acc[rb], 0, 0, 0);
+                    acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, kb, acc[rb], 0, 0, 0);
                 }
             }
         }
-        // accumulator element v of a lane is head row 8*(v/4) + 4*(lane/32) + v%4, token `col`
         float sum = 0.0f;
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = rb * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                sum += s_w[row] * fmaxf(acc[rb][v] * dscale, 0.0f);
-            }
+            for (int v = 0; v < 16; ++v) sum += wv[rb][v] * fmaxf(acc[rb][v] * dscale, 0.0f);
         sum += __shfl_xor(sum, 32, kWave);
         if (lane < 32 && valid) scores[(size_t)qi * stride + token] = sum;
+        tb = tb_next;
+        rows_ok = rows_next;
     }
 }
 
@@ -165,7 +221,7 @@ static int index_score_launch(const float* q, const float* w, const unsigned sho
     if (n_queries <= 0 || nt <= 0 || nh <= 0 || nact <= 0 || nact > nh || hd <= 0) return 1001;
     if (block_table && (max_blocks_per_seq <= 0 || page_tokens <= 0 || n_pages <= 0)) return 1001;
     if (nact > kScoreMaxHeads || hd > kScoreMaxHd || stride < nt || n_queries > 65535) return 1002;
-    if ((hd % 16) != 0) return 1004;
+    if ((hd % 16) != 0 || (block_table && (page_tokens % 32) != 0)) return 1004;
     dim3 grid((unsigned)((nt + kScoreTokensPerGroup - 1) / kScoreTokensPerGroup),
               (unsigned)n_queries);
     (void)hipGetLastError();
