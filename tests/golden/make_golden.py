@@ -1,0 +1,121 @@
+"""Writes tests/golden/kvcache_golden.json from the CPU oracle.
+
+The reference stores no vectors for this path (its tests compute every expectation at run
+time), so the committed vectors are the oracle's own outputs, taken only AFTER the oracle has
+passed the reference's known answers and the invariant checks in tests/test_oracle_*.py —
+this script runs those first and refuses to write when any fails. Small outputs are stored
+in full (hex); large ones as the reference's own pinning idiom, an FNV-1a hash of the bytes
+(crates/core/src/hash.rs:1-25), together with a few leading values.
+
+    python -m tests.golden.make_golden
+"""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+OUT = os.path.join(HERE, "kvcache_golden.json")
+W, PT = 576, 64
+
+
+def fnv(oracle, a) -> str:
+    return f"{oracle.fnv1a(np.ascontiguousarray(a).tobytes()):016x}"
+
+
+def hexs(a) -> str:
+    return np.ascontiguousarray(a).tobytes().hex()
+
+
+def build_cases(oracle) -> dict:
+    """Every golden case, computed by the oracle. Shared with the tests, which recompute the
+    same dict (from the oracle, or from the device) and compare it with the stored one."""
+    from tests.golden import inputs
+    from tests.test_oracle_quant import fixture_a99e
+    from tests.topk_cases import reference_topk_cases
+
+    g = {}
+    # -- codecs: the whole decode table and an encode sweep over every f32 exponent ----------
+    codes = np.arange(256, dtype=np.uint8)
+    g["e4m3_decode_table_u32"] = hexs(oracle.e4m3_to_f32(codes).view(np.uint32))
+    sweep = (np.arange(1 << 16, dtype=np.uint32) << np.uint32(16)).view(np.float32)  # all bf16 values
+    finite = sweep[np.isfinite(sweep)]
+    g["e4m3_encode_all_bf16_values"] = {"n": int(finite.size), "fnv": fnv(oracle, oracle.f32_to_e4m3(finite))}
+    g["subnormal_tie_codes"] = [int(c) for c in oracle.f32_to_e4m3(
+        np.array([1, 5, 9, 13, 15], np.float32) * np.float32(2.0 ** -10))]
+
+    # -- the reference's append_kv fixture (crates/engine/tests/fwd_kernel.rs:139-214) -------
+    rows, kvl, ropn, pos, nb = 5, 256, 64, 3, 2
+    latent, rope = fixture_a99e(oracle)
+    lc8, ls, rc = np.zeros(rows * kvl, np.uint8), np.zeros(rows * nb, np.float32), np.zeros(rows * ropn, np.uint16)
+    assert oracle.append_kv(latent, rope, lc8, ls, rc, pos, kvl, ropn, nb) == 0
+    g["append_kv_a99e"] = {
+        "latent_fnv": fnv(oracle, latent), "rope_fnv": fnv(oracle, rope),
+        "codes_row3": hexs(lc8[pos * kvl:(pos + 1) * kvl]),
+        "scales_row3_u32": hexs(ls[pos * nb:(pos + 1) * nb].view(np.uint32)),
+        "rope_row3_bf16": hexs(rc[pos * ropn:(pos + 1) * ropn]),
+    }
+
+    # -- the ten index_topk cases (crates/engine/tests/kernel_vector.rs:132-170) -------------
+    tk = {}
+    for name, scores, k in reference_topk_cases(oracle):
+        sel = oracle.topk(scores, k)
+        tk[name] = {"scores_fnv": fnv(oracle, scores), "n": int(sel.size), "fnv": fnv(oracle, sel),
+                    "head": [int(v) for v in sel[:6]], "tail": [int(v) for v in sel[-3:]]}
+    g["index_topk_cases"] = tk
+
+    # -- benchmark configuration 1: append the last token, gather the whole context ----------
+    rows1, table1, slots1 = inputs.config1(oracle)
+    pb = oracle.kv_page_bytes(PT, W)
+    pool = np.zeros(table1.size * pb, np.uint8)
+    oracle.kv_append_paged(rows1[:-1], slots1[:-1], pool, W, PT, table1.size)
+    before = fnv(oracle, pool)
+    oracle.kv_append_paged(rows1[-1:], slots1[-1:], pool, W, PT, table1.size)
+    out1 = oracle.kv_gather_paged(pool, table1, np.array([rows1.shape[0]], np.int32), W, PT)
+    g["config1"] = {"rows_fnv": fnv(oracle, rows1), "table_fnv": fnv(oracle, table1),
+                    "pool_before_last_fnv": before, "pool_fnv": fnv(oracle, pool),
+                    "gather_fnv": fnv(oracle, out1), "gather_row0_head": hexs(out1[0, :8]),
+                    "last_scale_u32": hexs(pool[int(slots1[-1]) // PT * pb + PT * W + (int(slots1[-1]) % PT) * 4:][:4])}
+
+    # -- benchmark configuration 2: bulk append with x50 outlier rows ------------------------
+    rows2, table2, slots2 = inputs.config2(oracle)
+    pool2 = np.zeros(table2.size * pb, np.uint8)
+    oracle.kv_append_paged(rows2, slots2, pool2, W, PT, table2.size)
+    g["config2"] = {"rows_fnv": fnv(oracle, rows2), "slots_fnv": fnv(oracle, slots2),
+                    "pool_fnv": fnv(oracle, pool2)}
+
+    # -- benchmark configuration 4, small: top-k then sparse gather --------------------------
+    rows4, table4, slots4, scores4, k4 = inputs.config4_small(oracle)
+    pool4 = np.zeros(table4.size * pb, np.uint8)
+    oracle.kv_append_paged(rows4, slots4, pool4, W, PT, table4.size)
+    sel4 = oracle.topk_batched(scores4, k4)
+    out4 = oracle.kv_gather_rows_paged(pool4, table4, sel4, W, PT)
+    g["config4_small"] = {"rows_fnv": fnv(oracle, rows4), "scores_fnv": fnv(oracle, scores4),
+                          "table_fnv": fnv(oracle, table4), "pool_fnv": fnv(oracle, pool4),
+                          "selected_fnv": fnv(oracle, sel4), "selected_q0_head": [int(v) for v in sel4[0, :6]],
+                          "gather_rows_fnv": fnv(oracle, out4)}
+    return g
+
+
+def main() -> None:
+    sys.path.insert(0, ROOT)
+    rc = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "not gpu",
+                         os.path.join(ROOT, "tests", "test_oracle_codecs.py"),
+                         os.path.join(ROOT, "tests", "test_oracle_quant.py"),
+                         os.path.join(ROOT, "tests", "test_oracle_topk_hash.py")], cwd=ROOT).returncode
+    if rc != 0:
+        sys.exit("the oracle does not pass its known-answer tests: no vectors written")
+    from oracle.kvoracle import oracle as get_oracle
+
+    g = build_cases(get_oracle())
+    with open(OUT, "w") as f:
+        json.dump(g, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print("wrote", OUT, os.path.getsize(OUT), "bytes")
+
+
+if __name__ == "__main__":
+    main()

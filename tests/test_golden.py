@@ -1,0 +1,123 @@
+"""The committed golden vectors (tests/golden/kvcache_golden.json, written by
+tests/golden/make_golden.py): the oracle must still reproduce them, and the device path must
+reproduce them through the C ABI without the oracle in the loop."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from tests.golden import inputs
+from tests.golden.make_golden import OUT, PT, W, build_cases, fnv, hexs
+from tests.test_oracle_quant import fixture_a99e
+from tests.topk_cases import reference_topk_cases
+
+
+@pytest.fixture(scope="module")
+def golden():
+    assert os.path.exists(OUT), "run python -m tests.golden.make_golden"
+    with open(OUT) as f:
+        return json.load(f)
+
+
+def test_oracle_reproduces_golden(oracle, golden):
+    got = build_cases(oracle)
+    assert sorted(got) == sorted(golden)
+    for key in golden:
+        assert got[key] == golden[key], key
+
+
+def test_golden_known_values(golden):
+    """Values in the file that the reference documents itself: decode(0x38) = 1.0,
+    decode(0x7e) = 448, decode(0xc0) = -2.0 (crates/core/src/routing.rs:338-362); the
+    half-away subnormal ties; the top-k KAT's shape (k clamps to nt)."""
+    table = np.frombuffer(bytes.fromhex(golden["e4m3_decode_table_u32"]), np.uint32).view(np.float32)
+    assert table[0x38] == 1.0 and table[0x7E] == 448.0 and table[0xC0] == -2.0
+    assert table[0x3C] == 1.5 and table[0x18] == 0.0625 and np.isnan(table[0x7F])
+    assert golden["subnormal_tie_codes"] == [1, 3, 5, 7, 8]
+    assert golden["index_topk_cases"]["k > nt (wrapper clamp)"]["n"] == 500
+    assert golden["index_topk_cases"]["ReLU-sparse (prefix answer)"]["head"] == [0, 1, 2, 3, 4, 5]
+
+
+@pytest.mark.gpu
+def test_device_reproduces_golden(oracle, golden):
+    """Same inputs (their hashes are checked first), outputs from the HIP library only."""
+    from rivoli_amd import hip
+    from tests.gpu_util import back, dev, dzeros
+
+    # codecs
+    sweep = (np.arange(1 << 16, dtype=np.uint32) << np.uint32(16)).view(np.float32)
+    finite = sweep[np.isfinite(sweep)]
+    codes = dzeros(finite.size)
+    hip.launch_codec_e4m3_encode(dev(finite), codes, finite.size)
+    assert fnv(oracle, back(codes)) == golden["e4m3_encode_all_bf16_values"]["fnv"]
+    dec = dzeros(256 * 2)
+    hip.launch_codec_e4m3_dequant_bf16(dev(np.arange(256, dtype=np.uint8)), 1.0, dec, 256)
+    table = np.frombuffer(bytes.fromhex(golden["e4m3_decode_table_u32"]), np.uint32)
+    finite_codes = (np.arange(256) & 0x7F) != 0x7F
+    assert np.array_equal(back(dec, np.uint16)[finite_codes], (table >> 16).astype(np.uint16)[finite_codes])
+
+    # the reference's append_kv fixture
+    g = golden["append_kv_a99e"]
+    rows, kvl, ropn, pos, nb = 5, 256, 64, 3, 2
+    latent, rope = fixture_a99e(oracle)
+    assert fnv(oracle, latent) == g["latent_fnv"] and fnv(oracle, rope) == g["rope_fnv"]
+    c8, ls, rc = dzeros(rows * kvl), dzeros(rows * nb * 4), dzeros(rows * ropn * 2)
+    hip.launch_append_kv(dev(latent), dev(rope), c8, ls, rc, pos, kvl, ropn, nb)
+    assert hexs(back(c8)[pos * kvl:(pos + 1) * kvl]) == g["codes_row3"]
+    assert hexs(back(ls, np.uint32)[pos * nb:(pos + 1) * nb]) == g["scales_row3_u32"]
+    assert hexs(back(rc, np.uint16)[pos * ropn:(pos + 1) * ropn]) == g["rope_row3_bf16"]
+
+    # the ten index_topk cases
+    for name, scores, k in reference_topk_cases(oracle):
+        c = golden["index_topk_cases"][name]
+        assert fnv(oracle, scores) == c["scores_fnv"], name
+        out = dzeros(max(scores.size, k) * 4, 0xFF)
+        hip.launch_index_topk(dev(scores), scores.size, k, out)
+        sel = back(out, np.uint32)[:c["n"]]
+        assert fnv(oracle, sel) == c["fnv"], name
+        assert [int(v) for v in sel[:6]] == c["head"] and [int(v) for v in sel[-3:]] == c["tail"], name
+
+    # configuration 1: all but the last token, then the last token, then the full gather
+    g = golden["config1"]
+    rows1, table1, slots1 = inputs.config1(oracle)
+    assert fnv(oracle, rows1) == g["rows_fnv"] and fnv(oracle, table1) == g["table_fnv"]
+    n, pb = rows1.shape[0], hip.kv_page_bytes(PT, W)
+    pool, rows_d, slots_d = dzeros(table1.size * pb), dev(rows1), dev(slots1)
+    hip.launch_kv_append_paged(rows_d, slots_d, pool, n - 1, W, PT, table1.size)
+    assert fnv(oracle, back(pool)) == g["pool_before_last_fnv"]
+    hip.launch_kv_append_paged(rows_d[(n - 1) * W * 2:], slots_d[(n - 1) * 4:], pool, 1, W, PT, table1.size)
+    assert fnv(oracle, back(pool)) == g["pool_fnv"]
+    out = dzeros(n * W * 2)
+    lens = np.array([n], np.int32)
+    hip.launch_kv_gather_paged(pool, dev(table1), dev(lens), dev(np.array([0, n], np.int32)), out, 1,
+                               table1.shape[1], W, PT, table1.size)
+    got = back(out, np.uint16).reshape(n, W)
+    assert fnv(oracle, got) == g["gather_fnv"] and hexs(got[0, :8]) == g["gather_row0_head"]
+
+    # configuration 2
+    g = golden["config2"]
+    rows2, table2, slots2 = inputs.config2(oracle)
+    assert fnv(oracle, rows2) == g["rows_fnv"] and fnv(oracle, slots2) == g["slots_fnv"]
+    pool2 = dzeros(table2.size * pb)
+    hip.launch_kv_append_paged(dev(rows2), dev(slots2), pool2, rows2.shape[0], W, PT, table2.size)
+    assert fnv(oracle, back(pool2)) == g["pool_fnv"]
+
+    # configuration 4, small
+    g = golden["config4_small"]
+    rows4, table4, slots4, scores4, k4 = inputs.config4_small(oracle)
+    assert fnv(oracle, rows4) == g["rows_fnv"] and fnv(oracle, scores4) == g["scores_fnv"]
+    assert fnv(oracle, table4) == g["table_fnv"]
+    n_q, nt = scores4.shape
+    pool4 = dzeros(table4.size * pb)
+    hip.launch_kv_append_paged(dev(rows4), dev(slots4), pool4, rows4.shape[0], W, PT, table4.size)
+    assert fnv(oracle, back(pool4)) == g["pool_fnv"]
+    sel = dzeros(n_q * k4 * 4, 0xFF)
+    hip.launch_index_topk_batched(dev(scores4), n_q, nt, None, nt, k4, sel)
+    sel_np = back(sel, np.uint32).reshape(n_q, k4)
+    assert fnv(oracle, sel_np) == g["selected_fnv"]
+    assert [int(v) for v in sel_np[0, :6]] == g["selected_q0_head"]
+    out4 = dzeros(n_q * k4 * W * 2)
+    hip.launch_kv_gather_rows_paged(pool4, dev(table4), sel, None, out4, n_q, k4, table4.shape[1], W, PT,
+                                    table4.size)
+    assert fnv(oracle, back(out4, np.uint16)) == g["gather_rows_fnv"]
