@@ -40,10 +40,16 @@ def parse():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=32768)
-    ap.add_argument("--workload", choices=["decode", "prefill", "dsa", "dsa_scored"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "dsa", "dsa_scored", "attend"], default="decode",
                     help="decode = configuration 3 (the headline line); prefill = configuration 2 "
                          "bulk append; dsa = configuration 4 top-k + sparse gather on synthetic "
-                         "scores; dsa_scored = the same with the scores computed on the device")
+                         "scores; dsa_scored = the same with the scores computed on the device; "
+                         "attend = configuration 3 with the gather replaced by MLA decode "
+                         "attention reading the fp8 pages directly")
+    ap.add_argument("--heads", type=int, default=64, help="attend: query heads")
+    ap.add_argument("--precise", type=int, default=2, choices=[0, 1, 2],
+                    help="attend: 2 = q and softmax weights as bf16 hi+lo (parity mode), "
+                         "1 = q only, 0 = plain bf16")
     ap.add_argument("--tokens", type=int, default=8192, help="prefill: new tokens per step")
     ap.add_argument("--topk", type=int, default=2048)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -77,6 +83,8 @@ def main():
         return bench_prefill(a, torch, hip)
     if a.workload in ("dsa", "dsa_scored"):
         return bench_dsa(a, torch, hip, scored=a.workload == "dsa_scored")
+    if a.workload == "attend":
+        return bench_attend(a, torch, hip)
     L, B, ctx = a.layers, a.batch, a.ctx
     blocks = -(-ctx // PT)
     n_pages = B * blocks
@@ -376,6 +384,107 @@ def bench_dsa(a, torch, hip, scored=False):
                                "cores": cores, "kind": "port",
                                "sample": f"one layer (top-k on {cores} host threads, sparse gather "
                                          f"single-threaded) x{reps} reps; GPU indices and rows checked equal"}
+    print(json.dumps(res), flush=True)
+
+
+def bench_attend(a, torch, hip):
+    """benchmark configuration 3 with the consumer fused in: per layer, append one token per sequence,
+    then MLA decode attention for `heads` query heads over every sequence's full context,
+    straight from the fp8 pages (no bf16 copy of the cache is made)."""
+    L, B, ctx, H = a.layers, a.batch, a.ctx, a.heads
+    KVL, ROPE = 512, 64
+    blocks = -(-ctx // PT)
+    n_pages = B * blocks
+    page_bytes = hip.kv_page_bytes(PT, W)
+    n_tok = B * ctx
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0x5EED0003)
+    rng = np.random.default_rng(0x5EED0003)
+    tables_np = rng.permutation(n_pages).astype(np.int32).reshape(B, blocks)
+    pos = np.arange(ctx)
+    slots_np = np.concatenate([tables_np[s][pos // PT] * PT + pos % PT for s in range(B)]).astype(np.int32)
+    tables, slots_all = torch.from_numpy(tables_np.copy()).cuda(), torch.from_numpy(slots_np).cuda()
+    seq_lens_np = np.full(B, ctx, np.int32)
+    seq_lens = torch.from_numpy(seq_lens_np).cuda()
+    new_slots = torch.from_numpy(slots_np.reshape(B, ctx)[:, -1].copy()).cuda()
+    kv_rows = torch.randn(n_tok, W, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    pools = []
+    for _ in range(L):
+        pool = torch.empty(n_pages * page_bytes, dtype=torch.uint8, device="cuda")
+        hip.launch_kv_append_paged(kv_rows, slots_all, pool, n_tok, W, PT, n_pages)
+        pools.append(pool)
+    del kv_rows
+    new_rows = [torch.randn(B, W, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+                for _ in range(L)]
+    qabs = [torch.randn(B, H, KVL, generator=g, device="cuda", dtype=torch.float32) for _ in range(L)]
+    qrope = [torch.randn(B, H, ROPE, generator=g, device="cuda", dtype=torch.float32) for _ in range(L)]
+    clat = torch.empty(B, H, KVL, dtype=torch.float32, device="cuda")
+    n_scratch = hip.mla_attend_paged_scratch_floats(B, H, ctx)
+    partial = torch.empty(max(n_scratch, 1), dtype=torch.float32, device="cuda")
+    sm_scale = float(W) ** -0.5
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    sh = stream.cuda_stream
+
+    def attend(layer, lens, max_rows, st):
+        hip.launch_mla_attend_paged(qabs[layer], qrope[layer], pools[layer], tables, lens, None, None, B, H,
+                                    max_rows, blocks, KVL, ROPE, PT, n_pages, sm_scale, a.precise, clat,
+                                    partial, None, st)
+
+    def step(events):
+        for layer in range(L):
+            hip.launch_kv_append_paged(new_rows[layer], new_slots, pools[layer], B, W, PT, n_pages, None, sh)
+            bracket(torch, stream, events, "attend", lambda: attend(layer, seq_lens, ctx, sh))
+
+    ms, per = timed(torch, stream, a.steps, a.warmup, step)
+    attend_bytes = n_tok * REC + B * blocks * 4 + B * H * (W + KVL) * 4   # records, table, q in, clat out
+    append_bytes = B * (ROW_IN + 4 + REC)
+    flops = 2.0 * n_tok * H * (W + KVL)
+    res = {"metric": "kv_append_attend_GBps", "value": round(L * (attend_bytes + append_bytes) / (ms * 1e-3) / 1e9, 1),
+           "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 x f32-accumulate",
+           "data": "synthetic",
+           "config": {"workload": "batched decode (benchmark configuration 3 shape) with the cache consumer "
+                                  "fused: append 1 token/seq/layer, then MLA latent attention over every "
+                                  "sequence's full context straight from the fp8 pages",
+                      "layers": L, "batch": B, "ctx": ctx, "heads": H, "page_tokens": PT, "width": W,
+                      "precise": a.precise},
+           "decode_step_kv_ms": round(ms, 4),
+           "tokens_per_s": round(L * n_tok / (ms * 1e-3), 1),
+           "roofline": {"bound": "hbm", "kernel": "mla_attend_paged_kernel",
+                        "achieved": round(attend_bytes / (per["attend"] * 1e-3) / 1e9, 1),
+                        "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                        "frac": round(attend_bytes / (per["attend"] * 1e-3) / HBM_PEAK, 4),
+                        "avg_launch_ms": round(per["attend"], 5), "bytes_per_launch": attend_bytes,
+                        "traffic": None,
+                        "tflops": round(flops / (per["attend"] * 1e-3) / 1e12, 1)}}
+    if not a.no_cpu_baseline:
+        from oracle.kvoracle import oracle as get_oracle
+
+        ora, cores = get_oracle(), max(1, min(16, os.cpu_count() or 1))
+        # bounded sample: the first `cores` sequences cut to 2048 tokens, all heads, layer 0
+        ns, cut = min(B, cores), min(ctx, 2048)
+        lens_cut = np.zeros(B, np.int32)
+        lens_cut[:ns] = cut
+        pool_h = pools[0].cpu().numpy()
+        qa_h, qr_h = qabs[0].cpu().numpy(), qrope[0].cpu().numpy()
+        t0 = time.perf_counter()
+        want = ora.mla_attend_paged(qa_h[:ns], qr_h[:ns], pool_h, tables_np[:ns], lens_cut[:ns], None, None,
+                                    KVL, ROPE, PT, sm_scale, n_threads=cores)
+        spent = time.perf_counter() - t0
+        attend(0, torch.from_numpy(lens_cut).cuda(), ctx, None)
+        torch.cuda.synchronize()
+        got = clat.cpu().numpy()[:ns]
+        err, mx = float(np.abs(got - want).max()), float(np.abs(want).max())
+        bar = {2: 1e-4, 1: 2e-3, 0: 3e-2}[a.precise] * mx
+        if not err <= bar:
+            raise SystemExit(f"bench: GPU attention differs from the CPU oracle: err={err:.3e} max={mx:.3e}")
+        sample_bytes = ns * cut * REC + ns * H * (W + KVL) * 4
+        res["cpu_baseline"] = {"value": round(sample_bytes / spent / 1e9, 4), "unit": "GB/s", "cores": cores,
+                               "kind": "port",
+                               "sample": f"attention of {ns} sequences x {cut} tokens x {H} heads (layer 0, same "
+                                         f"pool) on {cores} host threads; GPU output within {err / mx:.1e} of it",
+                               "tokens_per_s": round(ns * cut / spent, 1)}
     print(json.dumps(res), flush=True)
 
 

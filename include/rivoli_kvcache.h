@@ -149,6 +149,36 @@ int rivoli_index_append_paged(const float* k, const int* slot_mapping, unsigned 
                               int n_tokens, int hd, int page_tokens, int n_pages,
                               unsigned int* bad_slots, void* stream);
 
+/* MLA decode attention in latent space over the PAGED cache — the batched, paged form of
+ * rivoli_mla_attend (crates/backend/kernels/attn.hip:279-308; Rust launch_attend,
+ * crates/backend/src/hip_attn.rs:113-128), consuming the fp8 pages directly instead of a
+ * gathered bf16 copy. For sequence s < n_seqs and head h < H:
+ *   clat[s][h][:] = sum_t softmax_t((qabs[s][h] . L_t + qrope[s][h] . R_t) * scale) * L_t
+ * with L_t = e4m3_to_f32(codes[0:kvl]) * scale_t and R_t = e4m3_to_f32(codes[kvl:kvl+rope]) *
+ * scale_t of the page row. Attended tokens: 0 .. min(seq_lens[s], max_rows)-1 when `rows` is
+ * null (dense); otherwise rows[s*max_rows + j] for j < n_rows[s] (max_rows when n_rows is
+ * null) — the DSA selection, as rivoli_index_topk_batched emits it with k = max_rows.
+ * Tokens whose page id is outside [0, n_pages) are left out of the softmax and counted in
+ * *bad_rows when non-null. A sequence with nothing to attend gets zeros.
+ * `partial` is caller-owned scratch of rivoli_mla_attend_paged_scratch_floats(n_seqs, H,
+ * max_rows) floats (the split-KV partials; may be null when that returns 0). The split plan
+ * is a pure function of (n_seqs, H, max_rows): equal calls give bit-equal results.
+ * `precise`: 2 carries both q and the softmax weights as bf16 hi + lo (~17 bits) through the
+ * matrix cores — the parity mode: results agree with the reference formula far inside its
+ * own bar for this kernel (1e-3 of the largest output + 1e-3, crates/engine/tests/common/
+ * asserts.rs), though not bit for bit; 1 carries only q that way (weights rounded to bf16
+ * once: errors up to ~1e-3 of the SPREAD of the attended rows); 0 rounds q to bf16 once as
+ * well (a score is off by ~2^-10 |q||k|: ordinary bf16 flash-attention numerics).
+ * Guards: 1001 null / non-positive, or a null `partial` when scratch is needed; 1002
+ * n_seqs > 65535; 1004 unless kvl == 512 and rope == 64 (the 576-code page row). */
+size_t rivoli_mla_attend_paged_scratch_floats(int n_seqs, int H, int max_rows);
+int rivoli_mla_attend_paged(const float* qabs, const float* qrope, const unsigned char* pool,
+                            const int* block_table, const int* seq_lens,
+                            const unsigned int* rows, const int* n_rows, int n_seqs, int H,
+                            int max_rows, int max_blocks_per_seq, int kvl, int rope,
+                            int page_tokens, int n_pages, float scale, int precise, float* clat,
+                            float* partial, unsigned int* bad_rows, void* stream);
+
 /* Element codecs as launchers (what formats.hpp:42-57,99-106 and fwd.hip:20-45 are to the
  * reference's kernels), for census tests of the device codecs on arbitrary inputs:
  *   e4m3_encode: out[i] = f32_to_e4m3(x[i])            (rule of crates/core/src/num.rs:128-152)

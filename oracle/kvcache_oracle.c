@@ -416,6 +416,138 @@ void ro_kv_append_paged_mt(const uint16_t* rows, const int32_t* slot_mapping, ui
  * Selection
  * ---------------------------------------------------------------------------------------- */
 
+/* ---- MLA decode attention in latent space ------------------------------------------------
+ * The dense two-pass scalar softmax the reference's flash kernel is checked against:
+ * crates/engine/tests/kernel_attend.rs:201-226 (attend_reference) with
+ * crates/core/src/routing.rs:10-22 (softmax). `lat` is [nr][kvl] and `rk` is [nr][rope], both
+ * already widened to f32 the way the kernel widens them; one running f32 sum per score,
+ * latent terms then roped ones, times `scale`; out[h][i] += p_t * lat[t][i] in token order. */
+void ro_mla_attend_dense(const float* qabs, const float* qrope, const float* lat, const float* rk,
+                         int H, int nr, int kvl, int rope, float scale, float* clat) {
+    float* scores = (float*)malloc(sizeof(float) * (size_t)(nr > 0 ? nr : 1));
+    for (int h = 0; h < H; ++h) {
+        const float* qa = qabs + (size_t)h * kvl;
+        const float* qr = qrope + (size_t)h * rope;
+        float* out = clat + (size_t)h * kvl;
+        for (int i = 0; i < kvl; ++i) out[i] = 0.0f;
+        float mx = -INFINITY;
+        for (int t = 0; t < nr; ++t) {
+            float sum = 0.0f;
+            for (int i = 0; i < kvl; ++i) sum += qa[i] * lat[(size_t)t * kvl + i];
+            for (int d = 0; d < rope; ++d) sum += qr[d] * rk[(size_t)t * rope + d];
+            scores[t] = sum * scale;
+            if (scores[t] > mx) mx = scores[t];
+        }
+        float den = 0.0f;
+        for (int t = 0; t < nr; ++t) {
+            scores[t] = expf(scores[t] - mx);
+            den += scores[t];
+        }
+        if (den > 0.0f)
+            for (int t = 0; t < nr; ++t) scores[t] /= den;
+        for (int t = 0; t < nr; ++t)
+            for (int i = 0; i < kvl; ++i) out[i] += scores[t] * lat[(size_t)t * kvl + i];
+    }
+    free(scores);
+}
+
+/* The reference's cache layout and launcher (crates/backend/kernels/attn.hip:168-183,279-293):
+ * latent e4m3 with one f32 scale per 128 values, roped key bf16, token = rows ? rows[j] : j. */
+int ro_mla_attend(const float* qabs, const float* qrope, const uint8_t* lc8, const float* lscale,
+                  const uint16_t* rc, const uint32_t* rows, int H, int nr, int kvl, int rope,
+                  int n_blocks, float scale, float* clat) {
+    if (H <= 0 || nr <= 0 || kvl <= 0 || rope <= 0 || n_blocks <= 0) return 1001;
+    if (kvl > 512 || kvl % 128) return 1004;
+    float* lat = (float*)malloc(sizeof(float) * (size_t)nr * kvl);
+    float* rk = (float*)malloc(sizeof(float) * (size_t)nr * rope);
+    for (int j = 0; j < nr; ++j) {
+        size_t t = rows ? rows[j] : (size_t)j;
+        for (int i = 0; i < kvl; ++i)
+            lat[(size_t)j * kvl + i] = ro_e4m3_to_f32(lc8[t * kvl + i]) * lscale[t * n_blocks + i / 128];
+        for (int d = 0; d < rope; ++d) rk[(size_t)j * rope + d] = ro_bf16_to_f32(rc[t * rope + d]);
+    }
+    ro_mla_attend_dense(qabs, qrope, lat, rk, H, nr, kvl, rope, scale, clat);
+    free(lat);
+    free(rk);
+    return 0;
+}
+
+/* The paged cache of this build: a token is kvl + rope e4m3 codes under ONE f32 scale, so both
+ * halves widen as e4m3_to_f32(code) * scale. Sequence s attends rows[s*k + j] for
+ * j < n_rows[s] (k when null) if rows is given, else tokens 0..seq_lens[s]-1. */
+static void attend_paged_seq(const float* qabs, const float* qrope, const uint8_t* pool,
+                             const int32_t* block_table, const int32_t* seq_lens,
+                             const uint32_t* rows, const int32_t* n_rows, int k, int s, int H,
+                             int max_blocks_per_seq, int kvl, int rope, int page_tokens,
+                             float scale, float* clat) {
+    const int width = kvl + rope;
+    const size_t page_bytes = ro_kv_page_bytes(page_tokens, width);
+    const int nr = rows ? (n_rows ? n_rows[s] : k) : seq_lens[s];
+    float* out = clat + (size_t)s * H * kvl;
+    if (nr <= 0) {
+        for (size_t i = 0; i < (size_t)H * kvl; ++i) out[i] = 0.0f;
+        return;
+    }
+    float* lat = (float*)malloc(sizeof(float) * (size_t)nr * kvl);
+    float* rk = (float*)malloc(sizeof(float) * (size_t)nr * rope);
+    for (int j = 0; j < nr; ++j) {
+        uint32_t t = rows ? rows[(size_t)s * k + j] : (uint32_t)j;
+        int page = block_table[(size_t)s * max_blocks_per_seq + t / (uint32_t)page_tokens];
+        int off = (int)(t % (uint32_t)page_tokens);
+        const uint8_t* pg = pool + (size_t)page * page_bytes;
+        float scl;
+        memcpy(&scl, pg + (size_t)page_tokens * width + (size_t)off * 4, 4);
+        const uint8_t* codes = pg + (size_t)off * width;
+        for (int i = 0; i < kvl; ++i) lat[(size_t)j * kvl + i] = ro_e4m3_to_f32(codes[i]) * scl;
+        for (int d = 0; d < rope; ++d) rk[(size_t)j * rope + d] = ro_e4m3_to_f32(codes[kvl + d]) * scl;
+    }
+    ro_mla_attend_dense(qabs + (size_t)s * H * kvl, qrope + (size_t)s * H * rope, lat, rk, H, nr,
+                        kvl, rope, scale, out);
+    free(lat);
+    free(rk);
+}
+
+typedef struct {
+    const float *qabs, *qrope;
+    const uint8_t* pool;
+    const int32_t *block_table, *seq_lens;
+    const uint32_t* rows;
+    const int32_t* n_rows;
+    int k, n_seqs, H, max_blocks_per_seq, kvl, rope, page_tokens;
+    float scale;
+    float* clat;
+    int tid, n_threads;
+} attend_job;
+
+static void* attend_worker(void* p) {
+    attend_job* j = (attend_job*)p;
+    for (int s = j->tid; s < j->n_seqs; s += j->n_threads)
+        attend_paged_seq(j->qabs, j->qrope, j->pool, j->block_table, j->seq_lens, j->rows,
+                         j->n_rows, j->k, s, j->H, j->max_blocks_per_seq, j->kvl, j->rope,
+                         j->page_tokens, j->scale, j->clat);
+    return NULL;
+}
+
+void ro_mla_attend_paged(const float* qabs, const float* qrope, const uint8_t* pool,
+                         const int32_t* block_table, const int32_t* seq_lens,
+                         const uint32_t* rows, const int32_t* n_rows, int k, int n_seqs, int H,
+                         int max_blocks_per_seq, int kvl, int rope, int page_tokens, float scale,
+                         float* clat, int n_threads) {
+    if (n_threads < 1) n_threads = 1;
+    if (n_threads > n_seqs) n_threads = n_seqs;
+    pthread_t* th = (pthread_t*)malloc(sizeof(pthread_t) * (size_t)n_threads);
+    attend_job* jobs = (attend_job*)malloc(sizeof(attend_job) * (size_t)n_threads);
+    for (int i = 0; i < n_threads; ++i) {
+        attend_job j = {qabs, qrope, pool, block_table, seq_lens, rows, n_rows, k, n_seqs, H,
+                        max_blocks_per_seq, kvl, rope, page_tokens, scale, clat, i, n_threads};
+        jobs[i] = j;
+        pthread_create(&th[i], NULL, attend_worker, &jobs[i]);
+    }
+    for (int i = 0; i < n_threads; ++i) pthread_join(th[i], NULL);
+    free(jobs);
+    free(th);
+}
+
 /* qsort has no closure argument; selection is only ever run from one thread per array, and
  * the batched form gives each worker its own copy through thread-local storage. */
 static __thread const float* g_scores;

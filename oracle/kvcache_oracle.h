@@ -24,6 +24,11 @@
  *   ro_index_score      float64 restatement within 1e-6 of the scale; the reference test's
  *                       own separation property (head subset [5,0,6,2] vs all heads > 1e-2);
  *                       single-head / all-negative closed forms
+ *   ro_mla_attend*      float64 restatement (numpy) within 1e-5 of the largest output; closed
+ *                       forms (equal scores -> the mean row, one dominant score -> that row,
+ *                       one row -> itself); the paged form against the linear form on the
+ *                       same widened rows. The reference's own expectation for this kernel
+ *                       is computed at test time by this same formula (no stored vectors).
  *   ro_kv_gather_rows   parity unpinned by reference tests (no reference test passes
  *                       rows != null, crates/engine/tests/kernel_attend.rs:114); pinned
  *                       here by gather_rows(rows) == gather_dense()[rows]
@@ -108,6 +113,28 @@ void ro_kv_gather_paged_mt(const uint8_t* pool, const int32_t* block_table,
 void ro_kv_append_paged_mt(const uint16_t* rows, const int32_t* slot_mapping, uint8_t* pool,
                            int n_tokens, int width, int page_tokens, int n_pages,
                            int n_threads);
+
+/* ---- MLA decode attention in latent space: crates/engine/tests/kernel_attend.rs:201-226
+ *      (attend_reference, the dense two-pass softmax the flash kernel is checked against),
+ *      crates/core/src/routing.rs:10-22 (softmax). lat [nr][kvl], rk [nr][rope] are the
+ *      attended rows already widened to f32; clat [H][kvl]. ---- */
+void ro_mla_attend_dense(const float* qabs, const float* qrope, const float* lat, const float* rk,
+                         int H, int nr, int kvl, int rope, float scale, float* clat);
+/* Over the reference's linear slabs (crates/backend/kernels/attn.hip:168-183): e4m3 latent
+ * with one f32 scale per 128 values, bf16 roped key, token = rows ? rows[j] : j. Returns the
+ * launcher's guard code (crates/backend/kernels/attn.hip:284-293). */
+int ro_mla_attend(const float* qabs, const float* qrope, const uint8_t* lc8, const float* lscale,
+                  const uint16_t* rc, const uint32_t* rows, int H, int nr, int kvl, int rope,
+                  int n_blocks, float scale, float* clat);
+/* Over the paged cache (new here): every token is kvl + rope codes under one f32 scale;
+ * sequence s attends its first seq_lens[s] tokens, or rows[s*k + j], j < n_rows[s] (k when
+ * null) when rows is given. qabs [n_seqs][H][kvl], qrope [n_seqs][H][rope], clat like qabs.
+ * Sequences are dealt to n_threads host threads. */
+void ro_mla_attend_paged(const float* qabs, const float* qrope, const uint8_t* pool,
+                         const int32_t* block_table, const int32_t* seq_lens,
+                         const uint32_t* rows, const int32_t* n_rows, int k, int n_seqs, int H,
+                         int max_blocks_per_seq, int kvl, int rope, int page_tokens, float scale,
+                         float* clat, int n_threads);
 
 /* ---- selection: crates/core/src/routing.rs:42-61 then sort_unstable()
  *      (crates/engine/tests/kernel_vector.rs:126-131). Writes min(k, nt) ascending

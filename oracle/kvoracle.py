@@ -64,6 +64,10 @@ class Oracle:
             "ro_kv_gather_paged": (None, [u8p, i32p, i32p, i32p, u16p] + [C.c_int] * 4),
             "ro_kv_gather_paged_mt": (None, [u8p, i32p, i32p, i32p, u16p] + [C.c_int] * 5),
             "ro_kv_gather_rows_paged": (None, [u8p, i32p, u32p, i32p, u16p] + [C.c_int] * 5),
+            "ro_mla_attend_dense": (None, [f32p] * 4 + [C.c_int] * 4 + [C.c_float, f32p]),
+            "ro_mla_attend": (C.c_int, [f32p, f32p, u8p, f32p, u16p, u32p] + [C.c_int] * 5 + [C.c_float, f32p]),
+            "ro_mla_attend_paged": (None, [f32p, f32p, u8p, i32p, i32p, u32p, i32p] + [C.c_int] * 7
+                                    + [C.c_float, f32p, C.c_int]),
             "ro_topk": (C.c_int, [f32p, C.c_int, C.c_int, u32p]),
             "ro_topk_batched": (None, [f32p, C.c_int, C.c_int, i32p, C.c_int, C.c_int, u32p, C.c_int]),
             "ro_fnv1a": (C.c_uint64, [u8p, C.c_size_t]),
@@ -199,6 +203,47 @@ class Oracle:
             None if nr is None else _ptr(nr, C.c_int32), _ptr(out, C.c_uint16), n_q, k,
             max_blocks, width, page_tokens)
         return out
+
+    # ---- attention ----------------------------------------------------------------------
+    def mla_attend_dense(self, qabs, qrope, lat, rk, scale) -> np.ndarray:
+        """qabs [H][kvl], qrope [H][rope], lat [nr][kvl], rk [nr][rope] (all f32) -> clat [H][kvl]."""
+        qabs, qrope, lat, rk = (_c(x, np.float32) for x in (qabs, qrope, lat, rk))
+        (H, kvl), rope, nr = qabs.shape, qrope.shape[1], lat.shape[0]
+        clat = np.zeros((H, kvl), np.float32)
+        self.lib.ro_mla_attend_dense(_ptr(qabs, C.c_float), _ptr(qrope, C.c_float), _ptr(lat, C.c_float),
+                                     _ptr(rk, C.c_float), H, nr, kvl, rope, scale, _ptr(clat, C.c_float))
+        return clat
+
+    def mla_attend(self, qabs, qrope, lc8, lscale, rc, rows, H, nr, kvl, rope, n_blocks, scale):
+        """The reference's linear-slab form. Returns (guard code, clat [H][kvl])."""
+        qabs, qrope = _c(qabs, np.float32), _c(qrope, np.float32)
+        lc8, lscale, rc = _c(lc8, np.uint8), _c(lscale, np.float32), _c(rc, np.uint16)
+        rw = None if rows is None else _c(rows, np.uint32)
+        clat = np.zeros((max(H, 0), max(kvl, 0)), np.float32)
+        code = self.lib.ro_mla_attend(_ptr(qabs, C.c_float), _ptr(qrope, C.c_float), _ptr(lc8, C.c_uint8),
+                                      _ptr(lscale, C.c_float), _ptr(rc, C.c_uint16),
+                                      None if rw is None else _ptr(rw, C.c_uint32), H, nr, kvl, rope,
+                                      n_blocks, scale, _ptr(clat, C.c_float))
+        return int(code), clat
+
+    def mla_attend_paged(self, qabs, qrope, pool, block_table, seq_lens, rows, n_rows, kvl, rope,
+                         page_tokens, scale, n_threads: int = 1) -> np.ndarray:
+        """qabs [n_seqs][H][kvl], qrope [n_seqs][H][rope]; dense when rows is None."""
+        qabs, qrope = _c(qabs, np.float32), _c(qrope, np.float32)
+        block_table = _c(block_table, np.int32)
+        n_seqs, H = qabs.shape[0], qabs.shape[1]
+        lens = None if seq_lens is None else _c(seq_lens, np.int32)
+        rw = None if rows is None else _c(rows, np.uint32)
+        nr = None if n_rows is None else _c(n_rows, np.int32)
+        k = 0 if rw is None else rw.shape[1]
+        clat = np.zeros((n_seqs, H, kvl), np.float32)
+        self.lib.ro_mla_attend_paged(
+            _ptr(qabs, C.c_float), _ptr(qrope, C.c_float), _ptr(pool, C.c_uint8),
+            _ptr(block_table, C.c_int32), None if lens is None else _ptr(lens, C.c_int32),
+            None if rw is None else _ptr(rw, C.c_uint32), None if nr is None else _ptr(nr, C.c_int32),
+            k, n_seqs, H, block_table.shape[1], kvl, rope, page_tokens, scale, _ptr(clat, C.c_float),
+            n_threads)
+        return clat
 
     # ---- selection ----------------------------------------------------------------------
     def topk(self, scores, k: int) -> np.ndarray:

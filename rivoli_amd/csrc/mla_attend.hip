@@ -1,0 +1,532 @@
+// MLA decode attention in latent space, reading the paged fp8 cache directly.
+//
+// For one decoded token per sequence and every head h:
+//
+//     clat_h = sum_t softmax_t((qabs_h . L_t + qrope_h . R_t) * scale) * L_t
+//
+// which is what the reference's mla_latent_attend computes over its linear slabs
+// (crates/backend/kernels/attn.hip:1-17,119-233; combine :235-277). Here a token is one
+// 576-byte row of e4m3 codes (512 latent + 64 rope) with ONE f32 scale, so
+//     L_t = s_t * dec(c_t[0:512]),  R_t = s_t * dec(c_t[512:576]),
+// the per-token scale factors out of both contractions, and the codes themselves (exact in
+// bf16) are what the matrix cores see:
+//     score_t = s_t * scale * (q . dec(c_t)),     clat_h = sum_t (p_t * s_t) * dec(c_t[0:512]).
+// Nothing is materialised: a token costs 580 bytes of HBM traffic instead of the 580 + 1152
+// + 1152 of gather-then-attend.
+//
+// Mapping. A 512-thread workgroup (8 waves, two per SIMD) owns one (sequence, split of the
+// attended rows, block of 64 heads). Waves w and w+4 share heads 16(w&3)..+15 and split the
+// work on them: each takes half of the 576 contraction dims of the scores and half of the
+// 512 output columns. That halves the query registers and the accumulators a wave carries
+// (the whole kernel fits the 256 registers a wave gets at two waves per SIMD, so every MFMA
+// keeps its accumulator in place), and the second wave per SIMD covers the first one's
+// softmax and staging. Tokens move in tiles of 32:
+//   * staging: wave w fetches 4 tokens of the tile (one fully coalesced 512-byte run per
+//     token for the latent, 64 bytes for the rope), converts e4m3 -> bf16 in registers and
+//     writes the tile to LDS twice — row-major [token][dim] for the score contraction (over
+//     dims) and transposed [dim][token] for the value contraction (over tokens); the
+//     register transpose is byte-permutes. The next tile's loads are issued before this
+//     tile's MFMAs; the LDS tile is double-buffered.
+//   * scores: S^T[token][head] = K . Q^T with v_mfma_f32_16x16x32_bf16, A = the tile's rows
+//     from LDS, B = the wave's half of its query heads, resident in registers for the whole
+//     kernel (optionally as bf16 hi + lo, two MFMAs per step, ~17 bits of q). The two
+//     partial sums of a pair meet through LDS; both waves then run the same softmax on the
+//     same numbers. With tokens as the tile's rows a lane ends up holding 8 tokens of ONE
+//     head, which is exactly the A-operand layout of the value MFMA — P never leaves
+//     registers. The tile's token order inside the value contraction is whatever that
+//     layout implies; staging writes the transposed copy in the same order.
+//   * softmax: online, base 2 (log2 e folded into q); the running maximum only moves when a
+//     tile exceeds it by more than 2^8 (the f32 accumulators have the range), so rescaling
+//     the accumulators is rare.
+//   * values: O[head][col] += P . V over the wave's 256 columns, B = the transposed copy.
+// Splits write unnormalised partials (acc, m, l) that mla_attend_combine_kernel merges in
+// ascending split order; the split plan is a pure function of the call's shape, so equal
+// calls give bit-equal results.
+// Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
+#include "codec.hpp"
+
+namespace rk {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kKvl = 512, kRopeW = 64, kRowW = kKvl + kRopeW;
+constexpr int kAttThreads = 512;
+constexpr int kAttWaves = kAttThreads / kWave;
+constexpr int kTile = 32;                  // tokens per LDS tile
+constexpr int kKSteps = kRowW / 32;        // 18 K-steps of the score contraction ...
+constexpr int kKStepsHalf = kKSteps / 2;   // ... 9 per wave of a pair
+constexpr int kColTilesHalf = kKvl / 16 / 2;  // 16 output column tiles per wave of a pair
+constexpr int kKrRowBytes = kRowW * 2 + 16;  // row-major tile: 1152 B of bf16 + 16 B pad
+constexpr int kKrBytes = kTile * kKrRowBytes;
+// transposed tile: a row is one latent column, 32 tokens of bf16 = 64 B = four 16-byte
+// chunks; 16 B of padding after every 8 rows and an XOR of the chunk index with bits 1-2 of
+// the column keep both the staging writes (a lane owns 8 consecutive columns) and the
+// operand reads (16 lanes read 16 consecutive columns) off each other's banks
+constexpr int kVtGroupBytes = 8 * 64 + 16;
+constexpr int kVtBytes = (kKvl / 8) * kVtGroupBytes;
+constexpr int kXchBytes = kAttWaves * kWave * 8 * 4;  // partial scores, 8 f32 per lane
+constexpr int kTableLds = 1024;            // block-table entries staged per workgroup
+constexpr int kAttSmemBytes = 2 * kKrBytes + 2 * kVtBytes + 2 * kTile * 4 + kXchBytes + kTableLds * 4;
+static_assert(kAttSmemBytes <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
+constexpr float kLazyRescale = 8.0f;       // log2 units
+constexpr int kFragAhead = 3;              // score-side operand K-steps in flight (2 fragments each)
+constexpr int kValueAhead = 6;             // value-side operand fragments in flight
+constexpr float kLog2e = 1.4426950408889634f;
+
+// split plan: pure function of the call's shape
+constexpr int kAttTargetGroups = 512;      // two workgroups' worth per CU of a 256-CU part
+constexpr int kAttMinTilesPerSplit = 8;    // below 256 rows a split costs more than it buys
+constexpr int kAttMaxSplits = 64;
+
+struct AttendPlan {
+    int n_splits;
+    int split_rows;  // a multiple of kTile
+};
+
+static inline AttendPlan attend_plan(int n_seqs, int H, int max_rows) {
+    const int head_blocks = (H + 63) / 64;
+    const int tiles = (max_rows + kTile - 1) / kTile;
+    const long long per_split = (long long)n_seqs * head_blocks;
+    int by_grid = (int)((kAttTargetGroups + per_split - 1) / per_split);
+    int by_work = tiles / kAttMinTilesPerSplit;
+    int n = by_grid < by_work ? by_grid : by_work;
+    if (n > kAttMaxSplits) n = kAttMaxSplits;
+    if (n < 1) n = 1;
+    const int tps = (tiles + n - 1) / n;
+    AttendPlan p;
+    p.n_splits = (tiles + tps - 1) / tps;
+    p.split_rows = tps * kTile;
+    return p;
+}
+
+// e4m3 codes -> bf16, exact: four codes (one dword) -> two dwords
+__device__ __forceinline__ void e4m3x4_to_bf16(uint32_t c, uint32_t& lo, uint32_t& hi) {
+    lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c, 1.0f, false));
+    hi = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c, 1.0f, true));
+}
+
+struct AttendArgs {
+    const float* qabs;            // [n_seqs][H][512]
+    const float* qrope;           // [n_seqs][H][64]
+    const uint8_t* pool;
+    const int* block_table;       // [n_seqs][max_blocks]
+    const int* seq_lens;          // dense: attended rows per sequence
+    const unsigned int* rows;     // sparse: [n_seqs][k] token indices (null = dense)
+    const int* n_rows;            // sparse: rows per sequence (null = k)
+    int k;
+    int H, max_blocks, page_tokens, n_pages;
+    size_t page_bytes;
+    float qscale;                 // softmax scale * log2(e)
+    int n_splits, split_rows;
+    float* clat;                  // [n_seqs][H][512]
+    float* part_acc;              // [n_seqs][n_splits][H][512]
+    float* part_ml;               // [n_seqs][n_splits][H][2]
+    unsigned int* bad_rows;
+};
+
+// In the score tile (rows = tokens, 16 per MFMA) a lane of row group g holds rows 4g..4g+3
+// of both 16-token halves, and those 8 values are element j = 4*half + i of the value MFMA's
+// A operand for contraction index 8g + j. Staging wave w owns contraction indices
+// 4w..4w+3 — tile positions 16*(w&1) + 4*(w>>1) + i, four consecutive tokens — which is
+// half of one 16-byte chunk of every transposed row.
+__device__ __forceinline__ int tile_pos_of(int wave, int i) { return 16 * (wave & 1) + 4 * (wave >> 1) + i; }
+
+template <int QSPLIT, int PSPLIT, bool SPARSE>
+__global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const AttendArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t smem[kAttSmemBytes];
+    uint8_t* const kr = smem;
+    uint8_t* const vt = smem + 2 * kKrBytes;
+    float* const sc = reinterpret_cast<float*>(vt + 2 * kVtBytes);  // [2][32], by contraction index
+    f32x4* const xch = reinterpret_cast<f32x4*>(sc + 2 * kTile);    // [8 waves][64 lanes][2]
+    int* const tbl = reinterpret_cast<int*>(xch + kAttWaves * kWave * 2);
+
+    const int split = blockIdx.x, seq = blockIdx.y, hb = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hw = wave & 3;    // which 16 heads of the block
+    const int half = wave >> 2; // which half of the contraction dims / of the output columns
+    const int g = lane >> 4, n16 = lane & 15;
+
+    int n_att;
+    if (SPARSE) n_att = a.n_rows ? min(a.n_rows[seq], a.k) : a.k;
+    else n_att = min(a.seq_lens[seq], a.k);
+    const int r_begin = split * a.split_rows;
+    const int r_end = min(n_att, r_begin + a.split_rows);
+    float* const pml = a.part_ml ? a.part_ml + (((size_t)seq * a.n_splits + split) * a.H) * 2 : nullptr;
+    if (r_begin >= r_end) {
+        // an empty split tells the combine to skip it; a sequence with nothing to attend
+        // gets zeros, like the reference's `l > 0 ? 1/l : 0`
+        if (pml) {
+            for (int h = tid; h < 64; h += kAttThreads)
+                if (hb * 64 + h < a.H) {
+                    pml[(hb * 64 + h) * 2] = -INFINITY;
+                    pml[(hb * 64 + h) * 2 + 1] = 0.0f;
+                }
+        } else {
+            for (int i = tid; i < 64 * kKvl; i += kAttThreads) {
+                const int h = hb * 64 + i / kKvl;
+                if (h < a.H) a.clat[((size_t)seq * a.H + h) * kKvl + (i % kKvl)] = 0.0f;
+            }
+        }
+        return;
+    }
+    const int n_tiles = (r_end - r_begin + kTile - 1) / kTile;
+
+    // ---- block-table slice into LDS -----------------------------------------------------
+    const int* const table_g = a.block_table + (size_t)seq * a.max_blocks;
+    const int tbl_first = SPARSE ? 0 : r_begin / a.page_tokens;
+    const int tbl_last = SPARSE ? a.max_blocks - 1 : min(a.max_blocks - 1, (r_end - 1) / a.page_tokens);
+    const int tbl_count = min(kTableLds, tbl_last - tbl_first + 1);
+    for (int i = tid; i < tbl_count; i += kAttThreads) tbl[i] = table_g[tbl_first + i];
+
+    // ---- this wave's half of its 16 query heads as the B operand, for the whole kernel ---
+    bf16x8 qh[kKStepsHalf], ql[QSPLIT == 2 ? kKStepsHalf : 1];
+    {
+        const int head = hb * 64 + 16 * hw + n16;
+        const bool live = head < a.H;
+        const float* qa = a.qabs + ((size_t)seq * a.H + (live ? head : 0)) * kKvl + 8 * g;
+        const float* qr = a.qrope + ((size_t)seq * a.H + (live ? head : 0)) * kRopeW + 8 * g;
+#pragma unroll
+        for (int j = 0; j < kKStepsHalf; ++j) {
+            const int ks = half * kKStepsHalf + j;  // uniform: 0..8 or 9..17 (16, 17 are the rope)
+            const float4* src = reinterpret_cast<const float4*>(ks < 16 ? qa + 32 * ks : qr + 32 * (ks - 16));
+            float4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
+            if (live) v0 = src[0], v1 = src[1];
+            const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float x = v[i] * a.qscale;
+                const __bf16 hi = (__bf16)x;
+                qh[j][i] = hi;
+                if (QSPLIT == 2) ql[j][i] = (__bf16)(x - (float)hi);
+            }
+        }
+    }
+    __syncthreads();  // table slice visible
+
+    auto table_at = [&](int blk) -> int {
+        const int rel = blk - tbl_first;
+        return (rel >= 0 && rel < tbl_count) ? tbl[rel] : table_g[blk];
+    };
+
+    // Lanes 0..3 resolve the wave's 4 tokens of a tile: row position -> token -> page -> byte
+    // offsets of the code row and of the scale. Offset ~0 marks a token that is not there
+    // (past the end of the split, or its page id outside the pool).
+    constexpr unsigned long long kNone = ~0ull;
+    const unsigned int* const rows_g = SPARSE ? a.rows + (size_t)seq * a.k : nullptr;
+    auto row_token = [&](int tile) -> unsigned int {  // sparse: the row list entry, else the position
+        const int pos = r_begin + tile * kTile + tile_pos_of(wave, lane & 3);
+        if (lane >= 4 || pos >= r_end) return 0xffffffffu;
+        return SPARSE ? rows_g[pos] : (unsigned)pos;
+    };
+    auto resolve = [&](unsigned int tok, unsigned long long& code_off, unsigned long long& scale_off) {
+        code_off = kNone, scale_off = 0;
+        if (tok == 0xffffffffu) return;
+        const unsigned int blk = tok / (unsigned)a.page_tokens;
+        const unsigned int off = tok - blk * (unsigned)a.page_tokens;
+        const int page = blk < (unsigned)a.max_blocks ? table_at((int)blk) : -1;
+        if ((unsigned)page < (unsigned)a.n_pages) {
+            const unsigned long long pbase = (unsigned long long)page * a.page_bytes;
+            code_off = pbase + (unsigned long long)off * kRowW;
+            scale_off = pbase + (unsigned long long)a.page_tokens * kRowW + (unsigned long long)off * 4;
+        } else if (a.bad_rows && hb == 0) {
+            atomicAdd(a.bad_rows, 1u);
+        }
+    };
+
+    u32x2 raw[4];
+    uint32_t raw_rope;
+    float raw_scale;
+    auto issue_loads = [&](unsigned long long code_off, unsigned long long scale_off) {
+        const uint32_t lo = (uint32_t)code_off, hi = (uint32_t)(code_off >> 32);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t blo = __builtin_amdgcn_readlane(lo, i), bhi = __builtin_amdgcn_readlane(hi, i);
+            const unsigned long long b = ((unsigned long long)bhi << 32) | blo;
+            raw[i] = u32x2{0, 0};
+            if (b != kNone) raw[i] = *reinterpret_cast<const u32x2*>(a.pool + b + 8 * lane);
+        }
+        const unsigned long long br = __shfl(code_off, lane >> 4, kWave);
+        raw_rope = 0;
+        if (br != kNone) raw_rope = *reinterpret_cast<const uint32_t*>(a.pool + br + kKvl + 4 * (lane & 15));
+        raw_scale = -1.0f;  // a negative scale marks a token that is not there
+        if (lane < 4 && code_off != kNone) raw_scale = *reinterpret_cast<const float*>(a.pool + scale_off);
+    };
+    auto stage = [&](int buf) {
+        uint8_t* const krb = kr + buf * kKrBytes;
+        uint8_t* const vtb = vt + buf * kVtBytes;
+        uint32_t r[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            e4m3x4_to_bf16(raw[i].x, r[i][0], r[i][1]);
+            e4m3x4_to_bf16(raw[i].y, r[i][2], r[i][3]);
+            *reinterpret_cast<u32x4*>(krb + tile_pos_of(wave, i) * kKrRowBytes + 16 * lane) =
+                u32x4{r[i][0], r[i][1], r[i][2], r[i][3]};
+        }
+#pragma unroll
+        for (int d = 0; d < 8; ++d) {  // column 8*lane + d: the wave's 4 tokens, contraction order
+            const uint32_t sel = (d & 1) ? 0x07060302u : 0x05040100u;
+            u32x2 col;
+            col.x = __builtin_amdgcn_perm(r[1][d >> 1], r[0][d >> 1], sel);
+            col.y = __builtin_amdgcn_perm(r[3][d >> 1], r[2][d >> 1], sel);
+            const int chunk = (wave >> 1) ^ ((d >> 1) & 3);
+            *reinterpret_cast<u32x2*>(vtb + lane * kVtGroupBytes + d * 64 + chunk * 16 + 8 * (wave & 1)) = col;
+        }
+        uint32_t rr0, rr1;
+        e4m3x4_to_bf16(raw_rope, rr0, rr1);
+        *reinterpret_cast<u32x2*>(krb + tile_pos_of(wave, lane >> 4) * kKrRowBytes + kKvl * 2 +
+                                  8 * (lane & 15)) = u32x2{rr0, rr1};
+        if (lane < 4) sc[buf * kTile + 4 * wave + lane] = raw_scale;
+    };
+
+    // ---- prologue: tile 0 staged, tile 1 resolved ---------------------------------------
+    unsigned long long code_off, scale_off;
+    resolve(row_token(0), code_off, scale_off);
+    issue_loads(code_off, scale_off);
+    unsigned int tok_ahead = n_tiles > 1 ? row_token(1) : 0xffffffffu;
+    stage(0);
+    resolve(tok_ahead, code_off, scale_off);
+    __syncthreads();
+
+    f32x4 o[kColTilesHalf];
+#pragma unroll
+    for (int nt = 0; nt < kColTilesHalf; ++nt) o[nt] = f32x4{0, 0, 0, 0};
+    float m_ref = -INFINITY, l_sum = 0.0f;
+    f32x4* const xch_mine = xch + (wave * kWave + lane) * 2;
+    const f32x4* const xch_peer = xch + ((wave ^ 4) * kWave + lane) * 2;
+
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        const int buf = tile & 1;
+        if (tile + 1 < n_tiles) issue_loads(code_off, scale_off);       // tile + 1's bytes
+        tok_ahead = tile + 2 < n_tiles ? row_token(tile + 2) : 0xffffffffu;
+
+        // ---- scores: this wave's half of the dims, S^T[token][head], two 16-token halves --
+        const uint8_t* const krb = kr + buf * kKrBytes + half * (kKStepsHalf * 64);
+        const bf16x8* a0p = reinterpret_cast<const bf16x8*>(krb + n16 * kKrRowBytes + 16 * g);
+        const bf16x8* a1p = reinterpret_cast<const bf16x8*>(krb + (16 + n16) * kKrRowBytes + 16 * g);
+        f32x4 s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0};
+        {
+            // operand fragments run kFragAhead K-steps ahead of the MFMAs that consume them
+            bf16x8 fa0[kFragAhead], fa1[kFragAhead];
+#pragma unroll
+            for (int i = 0; i < kFragAhead; ++i) fa0[i] = a0p[i * 4], fa1[i] = a1p[i * 4];
+#pragma unroll
+            for (int j = 0; j < kKStepsHalf; ++j) {
+                const int slot = j % kFragAhead;
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[slot], qh[j], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[slot], qh[j], s1, 0, 0, 0);
+                if (QSPLIT == 2) {
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[slot], ql[j], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[slot], ql[j], s1, 0, 0, 0);
+                }
+                if (j + kFragAhead < kKStepsHalf)
+                    fa0[slot] = a0p[(j + kFragAhead) * 4], fa1[slot] = a1p[(j + kFragAhead) * 4];
+            }
+        }
+        xch_mine[0] = s0, xch_mine[1] = s1;
+        // the first value-side fragments do not depend on the softmax: fetch them under it
+        const uint8_t* const vtb = vt + buf * kVtBytes;
+        auto vt_frag = [&](int nt) -> bf16x8 {
+            const int c = 16 * (half * kColTilesHalf + nt) + n16;
+            return *reinterpret_cast<const bf16x8*>(vtb + (c >> 3) * kVtGroupBytes + (c & 7) * 64 +
+                                                    ((g ^ ((c >> 1) & 3)) * 16));
+        };
+        bf16x8 fb[kValueAhead];
+#pragma unroll
+        for (int i = 0; i < kValueAhead; ++i) fb[i] = vt_frag(i);
+        __syncthreads();  // both halves of every score are in LDS
+        {
+            const f32x4 p0 = xch_peer[0], p1 = xch_peer[1];
+            s0 += p0, s1 += p1;  // a + b == b + a: the pair works on identical numbers
+        }
+
+        // ---- online softmax over the lane's 8 tokens of head n16 --------------------------
+        const f32x4 sa = *reinterpret_cast<const f32x4*>(sc + buf * kTile + 8 * g);
+        const f32x4 sb = *reinterpret_cast<const f32x4*>(sc + buf * kTile + 8 * g + 4);
+        const float scl[8] = {sa.x, sa.y, sa.z, sa.w, sb.x, sb.y, sb.z, sb.w};
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[i] = scl[i] < 0.0f ? -INFINITY : s0[i] * scl[i];
+            v[4 + i] = scl[4 + i] < 0.0f ? -INFINITY : s1[i] * scl[4 + i];
+        }
+        float tmax = v[0];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) tmax = fmaxf(tmax, v[i]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+        const bool grow = tmax > m_ref + kLazyRescale;  // false while everything is masked
+        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+            const float corr = grow ? __builtin_amdgcn_exp2f(m_ref - tmax) : 1.0f;  // 2^-inf = 0 at first
+            if (grow) m_ref = tmax;
+            l_sum *= corr;
+            float c[4];  // the lane's accumulators are heads 4g+i; corr lives in lanes n16 == head
+#pragma unroll
+            for (int i = 0; i < 4; ++i) c[i] = __shfl(corr, 4 * g + i, kWave);
+#pragma unroll
+            for (int nt = 0; nt < kColTilesHalf; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[nt][i] *= c[i];
+        }
+        const float mu = m_ref == -INFINITY ? 0.0f : m_ref;
+        // The value MFMA sees a_t = bf16(p_t * s_t) (optionally hi + lo). The denominator
+        // sums a_t / s_t, the weights the numerator really carries, so the result is an
+        // exactly normalised average under weights perturbed by their rounding: the error
+        // scales with the spread of the attended rows, not with their magnitude, and
+        // vanishes when one token holds the whole softmax.
+        bf16x8 p, p_lo;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float e = __builtin_amdgcn_exp2f(v[i] - mu);  // masked -> 0
+            const bool there = scl[i] > 0.0f;
+            const float x = e * (there ? scl[i] : 0.0f);
+            const __bf16 w = (__bf16)x;
+            p[i] = w;
+            float carried = (float)w;
+            if (PSPLIT == 2) {
+                const __bf16 w_lo = (__bf16)(x - carried);
+                p_lo[i] = w_lo;
+                carried += (float)w_lo;
+            }
+            l_sum += carried * (there ? __builtin_amdgcn_rcpf(scl[i]) : 0.0f);
+        }
+
+        // ---- values: O[head][col] += P . V over this wave's 256 columns -------------------
+#pragma unroll
+        for (int nt = 0; nt < kColTilesHalf; ++nt) {
+            const int slot = nt % kValueAhead;
+            o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p, fb[slot], o[nt], 0, 0, 0);
+            if (PSPLIT == 2) o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_lo, fb[slot], o[nt], 0, 0, 0);
+            if (nt + kValueAhead < kColTilesHalf) fb[slot] = vt_frag(nt + kValueAhead);
+        }
+
+        // ---- stage tile + 1 into the other buffer, resolve tile + 2 -----------------------
+        if (tile + 1 < n_tiles) stage(buf ^ 1);
+        resolve(tok_ahead, code_off, scale_off);
+        __syncthreads();
+    }
+
+    // ---- epilogue -----------------------------------------------------------------------
+    l_sum += __shfl_xor(l_sum, 16, kWave);
+    l_sum += __shfl_xor(l_sum, 32, kWave);
+    // the lane's accumulators are heads 4g+i; their (m, l) live in lanes with n16 == 4g+i
+    float l_h[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) l_h[i] = __shfl(l_sum, 4 * g + i, kWave);
+    const int head0 = hb * 64 + 16 * hw;
+    const int col0 = half * (kKvl / 2) + n16;
+    if (a.part_acc) {
+        float* const pa = a.part_acc + (((size_t)seq * a.n_splits + split) * a.H) * kKvl;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int head = head0 + 4 * g + i;
+            if (head < a.H) {
+#pragma unroll
+                for (int nt = 0; nt < kColTilesHalf; ++nt) pa[(size_t)head * kKvl + col0 + 16 * nt] = o[nt][i];
+            }
+        }
+        if (half == 0 && g == 0 && head0 + n16 < a.H) {
+            pml[(head0 + n16) * 2] = m_ref;
+            pml[(head0 + n16) * 2 + 1] = l_sum;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int head = head0 + 4 * g + i;
+            const float inv = l_h[i] > 0.0f ? 1.0f / l_h[i] : 0.0f;
+            if (head < a.H) {
+                float* const dst = a.clat + ((size_t)seq * a.H + head) * kKvl;
+#pragma unroll
+                for (int nt = 0; nt < kColTilesHalf; ++nt) dst[col0 + 16 * nt] = o[nt][i] * inv;
+            }
+        }
+    }
+}
+
+// clat[seq][head] = sum_s w_s acc_s / sum_s w_s l_s with w_s = 2^(m_s - max m), splits in
+// ascending order (the reference's combine, crates/backend/kernels/attn.hip:235-277, in
+// base 2). A split whose m is -inf holds no rows and its accumulator is never read.
+__global__ __launch_bounds__(128) void mla_attend_combine_kernel(
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml, int H, int n_splits,
+    float* __restrict__ clat) {
+    const int head = blockIdx.x, seq = blockIdx.y;
+    const float* ml = part_ml + ((size_t)seq * n_splits * H + head) * 2;
+    float m_g = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) m_g = fmaxf(m_g, ml[(size_t)s * H * 2]);
+    float4 sum = {0, 0, 0, 0};
+    float l_g = 0.0f;
+    if (m_g != -INFINITY) {
+        for (int s = 0; s < n_splits; ++s) {
+            const float m_s = ml[(size_t)s * H * 2];
+            if (m_s == -INFINITY) continue;
+            const float w = exp2f(m_s - m_g);
+            l_g += ml[(size_t)s * H * 2 + 1] * w;
+            const float4 v = reinterpret_cast<const float4*>(
+                part_acc + (((size_t)seq * n_splits + s) * H + head) * kKvl)[threadIdx.x];
+            sum.x += v.x * w, sum.y += v.y * w, sum.z += v.z * w, sum.w += v.w * w;
+        }
+    }
+    const float inv = l_g > 0.0f ? 1.0f / l_g : 0.0f;
+    reinterpret_cast<float4*>(clat + ((size_t)seq * H + head) * kKvl)[threadIdx.x] =
+        float4{sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv};
+}
+
+}  // namespace rk
+
+extern "C" size_t rivoli_mla_attend_paged_scratch_floats(int n_seqs, int H, int max_rows) {
+    if (n_seqs <= 0 || H <= 0 || max_rows <= 0) return 0;
+    const rk::AttendPlan p = rk::attend_plan(n_seqs, H, max_rows);
+    if (p.n_splits <= 1) return 0;
+    return (size_t)n_seqs * p.n_splits * H * (rk::kKvl + 2);
+}
+
+extern "C" int rivoli_mla_attend_paged(const float* qabs, const float* qrope,
+                                       const unsigned char* pool, const int* block_table,
+                                       const int* seq_lens, const unsigned int* rows,
+                                       const int* n_rows, int n_seqs, int H, int max_rows,
+                                       int max_blocks_per_seq, int kvl, int rope, int page_tokens,
+                                       int n_pages, float scale, int precise, float* clat,
+                                       float* partial, unsigned int* bad_rows, void* stream) {
+    using namespace rk;
+    if (!qabs || !qrope || !pool || !block_table || !clat) return 1001;
+    if (!rows && !seq_lens) return 1001;
+    if (n_seqs <= 0 || H <= 0 || max_rows <= 0 || max_blocks_per_seq <= 0 || kvl <= 0 || rope <= 0 ||
+        page_tokens <= 0 || n_pages <= 0)
+        return 1001;
+    if (n_seqs > 65535 || H > 64 * 65535) return 1002;
+    if (kvl != kKvl || rope != kRopeW) return 1004;  // the page row is 512 latent + 64 rope codes
+    const AttendPlan plan = attend_plan(n_seqs, H, max_rows);
+    if (plan.n_splits > 1 && !partial) return 1001;
+    AttendArgs a;
+    a.qabs = qabs, a.qrope = qrope, a.pool = pool, a.block_table = block_table;
+    a.seq_lens = seq_lens, a.rows = rows, a.n_rows = n_rows, a.k = max_rows;
+    a.H = H, a.max_blocks = max_blocks_per_seq, a.page_tokens = page_tokens, a.n_pages = n_pages;
+    a.page_bytes = (size_t)page_tokens * kRowW + (size_t)page_tokens * 4;
+    a.qscale = scale * kLog2e;
+    a.n_splits = plan.n_splits, a.split_rows = plan.split_rows;
+    a.clat = clat, a.bad_rows = bad_rows;
+    a.part_acc = plan.n_splits > 1 ? partial : nullptr;
+    a.part_ml = plan.n_splits > 1 ? partial + (size_t)n_seqs * plan.n_splits * H * kKvl : nullptr;
+    const dim3 grid((unsigned)plan.n_splits, (unsigned)n_seqs, (unsigned)((H + 63) / 64));
+    (void)hipGetLastError();
+    hipStream_t st = (hipStream_t)stream;
+#define RK_ATTEND_LAUNCH(Q, P, S) \
+    hipLaunchKernelGGL((mla_attend_paged_kernel<Q, P, S>), grid, dim3(kAttThreads), 0, st, a)
+    if (rows) {
+        if (precise >= 2) RK_ATTEND_LAUNCH(2, 2, true);
+        else if (precise == 1) RK_ATTEND_LAUNCH(2, 1, true);
+        else RK_ATTEND_LAUNCH(1, 1, true);
+    } else {
+        if (precise >= 2) RK_ATTEND_LAUNCH(2, 2, false);
+        else if (precise == 1) RK_ATTEND_LAUNCH(2, 1, false);
+        else RK_ATTEND_LAUNCH(1, 1, false);
+    }
+#undef RK_ATTEND_LAUNCH
+    int rc = launch_status();
+    if (rc != 0 || plan.n_splits <= 1) return rc;
+    hipLaunchKernelGGL(mla_attend_combine_kernel, dim3((unsigned)H, (unsigned)n_seqs), dim3(128), 0, st,
+                       a.part_acc, a.part_ml, H, plan.n_splits, clat);
+    return launch_status();
+}

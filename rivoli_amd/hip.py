@@ -50,6 +50,7 @@ _SIGNATURES = {
     "rivoli_kv_append_paged": [_VP, _VP, _VP, _I, _I, _I, _I, _VP, _VP],
     "rivoli_kv_gather_paged": [_VP] * 5 + [_I] * 5 + [_VP, _VP],
     "rivoli_kv_gather_rows_paged": [_VP] * 5 + [_I] * 6 + [_VP, _VP],
+    "rivoli_mla_attend_paged": [_VP] * 7 + [_I] * 8 + [_F, _I, _VP, _VP, _VP, _VP],
     "rivoli_codec_e4m3_encode": [_VP, _VP, _LL, _VP],
     "rivoli_codec_e4m3_dequant_bf16": [_VP, _F, _VP, _LL, _VP],
     "rivoli_codec_bf16_encode": [_VP, _VP, _LL, _VP],
@@ -64,6 +65,15 @@ def lib() -> C.CDLL:
             raise FileNotFoundError(
                 f"{LIB_PATH} is missing: build it with `python -m rivoli_amd.build` "
                 "(hipcc, gfx950); this package has no CPU fallback")
+        # torch ships its own copy of the HIP runtime. A process must end up with ONE runtime:
+        # if this library were loaded first it would bring in the system copy, torch would
+        # then load its own beside it, and every launch from here would fail with
+        # hipErrorNoDevice (the second runtime never sees the device). So torch, which owns
+        # the device buffers these launchers are handed, is loaded first whenever it exists.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         handle = C.CDLL(LIB_PATH)
         for name, args in _SIGNATURES.items():
             fn = getattr(handle, name)
@@ -71,12 +81,15 @@ def lib() -> C.CDLL:
         for name in ("rivoli_kv_page_bytes", "rivoli_index_topk_workspace_bytes"):
             fn = getattr(handle, name)
             fn.restype, fn.argtypes = C.c_size_t, [_I, _I]
+        fn = handle.rivoli_mla_attend_paged_scratch_floats
+        fn.restype, fn.argtypes = C.c_size_t, [_I, _I, _I]
         _LIB = handle
     return _LIB
 
 
 def exported_symbols() -> list[str]:
-    return sorted(list(_SIGNATURES) + ["rivoli_kv_page_bytes", "rivoli_index_topk_workspace_bytes"])
+    return sorted(list(_SIGNATURES) + ["rivoli_kv_page_bytes", "rivoli_index_topk_workspace_bytes",
+                                       "rivoli_mla_attend_paged_scratch_floats"])
 
 
 def _p(x):
@@ -192,6 +205,21 @@ def launch_index_topk_batched(scores, n_queries, stride, nts, nt, k, rows, works
     ensure_hip_status(lib().rivoli_index_topk_batched(_p(scores), n_queries, stride, _p(nts), nt,
                                                       k, _p(rows), _p(workspace), _s(stream)),
                       "index_topk_batched")
+
+
+# ---- attention over the paged cache -------------------------------------------------------
+
+def mla_attend_paged_scratch_floats(n_seqs: int, H: int, max_rows: int) -> int:
+    return int(lib().rivoli_mla_attend_paged_scratch_floats(n_seqs, H, max_rows))
+
+
+def launch_mla_attend_paged(qabs, qrope, pool, block_table, seq_lens, rows, n_rows, n_seqs, H,
+                            max_rows, max_blocks_per_seq, kvl, rope, page_tokens, n_pages, scale,
+                            precise, clat, partial, bad_rows=None, stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_mla_attend_paged(
+        _p(qabs), _p(qrope), _p(pool), _p(block_table), _p(seq_lens), _p(rows), _p(n_rows), n_seqs,
+        H, max_rows, max_blocks_per_seq, kvl, rope, page_tokens, n_pages, scale, int(precise),
+        _p(clat), _p(partial), _p(bad_rows), _s(stream)), "mla_attend_paged")
 
 
 # ---- element codecs -----------------------------------------------------------------------
