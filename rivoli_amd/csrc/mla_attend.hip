@@ -66,8 +66,8 @@ constexpr int kKrBytes = kTile * kKrRowBytes;
 constexpr int kVtGroupBytes = 8 * 64 + 16;
 constexpr int kVtBytes = (kKvl / 8) * kVtGroupBytes;
 constexpr int kXchBytes = kAttWaves * kWave * 8 * 4;  // partial scores, 8 f32 per lane
-constexpr int kTableLds = 1024;            // block-table entries staged per workgroup
-constexpr int kAttSmemBytes = 2 * kKrBytes + 2 * kVtBytes + 2 * kTile * 4 + kXchBytes + kTableLds * 4;
+constexpr int kTableLds = 960;             // block-table entries staged per workgroup
+constexpr int kAttSmemBytes = 2 * kKrBytes + 2 * kVtBytes + 4 * kTile * 4 + kXchBytes + kTableLds * 4;
 static_assert(kAttSmemBytes <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
 constexpr float kLazyRescale = 8.0f;       // log2 units
 constexpr int kFragAhead = 3;              // score-side operand K-steps in flight (2 fragments each)
@@ -116,6 +116,7 @@ struct AttendArgs {
     const int* n_rows;            // sparse: rows per sequence (null = k)
     int k;
     int H, max_blocks, page_tokens, n_pages;
+    int page_shift;               // log2(page_tokens) when that is a power of two, else -1
     size_t page_bytes;
     float qscale;                 // softmax scale * log2(e)
     int n_splits, split_rows;
@@ -132,13 +133,25 @@ struct AttendArgs {
 // half of one 16-byte chunk of every transposed row.
 __device__ __forceinline__ int tile_pos_of(int wave, int i) { return 16 * (wave & 1) + 4 * (wave >> 1) + i; }
 
-template <int QSPLIT, int PSPLIT, bool SPARSE>
+// MODE: how a tile's tokens are found.
+enum : int {
+    kDense = 0,      // token = row position, any page size: one table lookup per token
+    kSparse = 1,     // token = rows[position]: one list entry and one table lookup per token
+    kDensePaged = 2  // token = row position and page_tokens is a power of two >= the tile: a
+                     // tile lies inside ONE page, so a tile costs one (scalar) table lookup
+};
+
+template <int QSPLIT, int PSPLIT, int MODE>
 __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const AttendArgs a) {
+    constexpr bool SPARSE = MODE == kSparse;
     __shared__ __attribute__((aligned(16))) uint8_t smem[kAttSmemBytes];
     uint8_t* const kr = smem;
     uint8_t* const vt = smem + 2 * kKrBytes;
-    float* const sc = reinterpret_cast<float*>(vt + 2 * kVtBytes);  // [2][32], by contraction index
-    f32x4* const xch = reinterpret_cast<f32x4*>(sc + 2 * kTile);    // [8 waves][64 lanes][2]
+    // per token of a tile, by contraction index: its scale (0 when the token is not there)
+    // and a score bias (0, or -inf when it is not there): score = s * scale + bias
+    float* const sc = reinterpret_cast<float*>(vt + 2 * kVtBytes);  // [2][32] scales, then [2][32] biases
+    float* const sbias = sc + 2 * kTile;
+    f32x4* const xch = reinterpret_cast<f32x4*>(sbias + 2 * kTile);  // [8 waves][64 lanes][2]
     int* const tbl = reinterpret_cast<int*>(xch + kAttWaves * kWave * 2);
 
     const int split = blockIdx.x, seq = blockIdx.y, hb = blockIdx.z;
@@ -211,26 +224,53 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         return (rel >= 0 && rel < tbl_count) ? tbl[rel] : table_g[blk];
     };
 
-    // Lanes 0..3 resolve the wave's 4 tokens of a tile: row position -> token -> page -> byte
-    // offsets of the code row and of the scale. Offset ~0 marks a token that is not there
-    // (past the end of the split, or its page id outside the pool).
+    // ---- where a tile's tokens are ------------------------------------------------------
+    // General form (kDense, kSparse): lanes 0..3 resolve the wave's 4 tokens: row position ->
+    // token -> page -> byte offsets of the code row and of the scale; offset ~0 marks a
+    // token that is not there (past the end of the split, or its page id outside the pool).
+    // kDensePaged: the whole tile is `n_here` consecutive rows of one page starting at
+    // `tile_off`, all wave-uniform.
     constexpr unsigned long long kNone = ~0ull;
+    struct Where {
+        unsigned long long code_off, scale_off;  // per lane (lanes 0..3), general form
+        unsigned long long tile_off, tile_scale_off;  // uniform, kDensePaged
+        int n_here;                                    // uniform, kDensePaged: valid rows in the tile
+    };
     const unsigned int* const rows_g = SPARSE ? a.rows + (size_t)seq * a.k : nullptr;
     auto row_token = [&](int tile) -> unsigned int {  // sparse: the row list entry, else the position
+        if (MODE == kDensePaged) return 0;
         const int pos = r_begin + tile * kTile + tile_pos_of(wave, lane & 3);
         if (lane >= 4 || pos >= r_end) return 0xffffffffu;
         return SPARSE ? rows_g[pos] : (unsigned)pos;
     };
-    auto resolve = [&](unsigned int tok, unsigned long long& code_off, unsigned long long& scale_off) {
-        code_off = kNone, scale_off = 0;
+    auto resolve = [&](int tile, unsigned int tok, Where& w) {
+        if (MODE == kDensePaged) {
+            const int pos0 = r_begin + tile * kTile;  // uniform; the split starts on a tile boundary
+            w.n_here = 0, w.tile_off = 0, w.tile_scale_off = 0;
+            if (pos0 >= r_end) return;
+            const int blk = pos0 >> a.page_shift, off = pos0 & (a.page_tokens - 1);
+            const int page = __builtin_amdgcn_readfirstlane(table_at(blk));
+            const int n = min(kTile, r_end - pos0);
+            if ((unsigned)page < (unsigned)a.n_pages) {
+                w.n_here = n;
+                w.tile_off = (unsigned long long)page * a.page_bytes + (unsigned long long)off * kRowW;
+                w.tile_scale_off = (unsigned long long)page * a.page_bytes +
+                                   (unsigned long long)a.page_tokens * kRowW + (unsigned long long)off * 4;
+            } else if (a.bad_rows && hb == 0 && tid == 0) {
+                atomicAdd(a.bad_rows, (unsigned)n);
+            }
+            return;
+        }
+        w.code_off = kNone, w.scale_off = 0;
         if (tok == 0xffffffffu) return;
-        const unsigned int blk = tok / (unsigned)a.page_tokens;
-        const unsigned int off = tok - blk * (unsigned)a.page_tokens;
+        unsigned int blk, off;
+        if (a.page_shift >= 0) blk = tok >> a.page_shift, off = tok & (unsigned)(a.page_tokens - 1);
+        else blk = tok / (unsigned)a.page_tokens, off = tok - blk * (unsigned)a.page_tokens;
         const int page = blk < (unsigned)a.max_blocks ? table_at((int)blk) : -1;
         if ((unsigned)page < (unsigned)a.n_pages) {
             const unsigned long long pbase = (unsigned long long)page * a.page_bytes;
-            code_off = pbase + (unsigned long long)off * kRowW;
-            scale_off = pbase + (unsigned long long)a.page_tokens * kRowW + (unsigned long long)off * 4;
+            w.code_off = pbase + (unsigned long long)off * kRowW;
+            w.scale_off = pbase + (unsigned long long)a.page_tokens * kRowW + (unsigned long long)off * 4;
         } else if (a.bad_rows && hb == 0) {
             atomicAdd(a.bad_rows, 1u);
         }
@@ -238,9 +278,34 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
 
     u32x2 raw[4];
     uint32_t raw_rope;
-    float raw_scale;
-    auto issue_loads = [&](unsigned long long code_off, unsigned long long scale_off) {
-        const uint32_t lo = (uint32_t)code_off, hi = (uint32_t)(code_off >> 32);
+    float raw_scale, raw_bias;  // lanes 0..3
+    const int my_pos0 = tile_pos_of(wave, 0);  // the wave's 4 tokens are consecutive tile positions
+    auto issue_loads = [&](const Where& w) {
+        if (MODE == kDensePaged) {
+            const uint8_t* const base = a.pool + w.tile_off + (size_t)my_pos0 * kRowW;
+            if (my_pos0 + 3 < w.n_here) {  // the common case: all four rows are there
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    raw[i] = *reinterpret_cast<const u32x2*>(base + i * kRowW + 8 * lane);
+                raw_rope = *reinterpret_cast<const uint32_t*>(base + (lane >> 4) * kRowW + kKvl + 4 * (lane & 15));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    raw[i] = u32x2{0, 0};
+                    if (my_pos0 + i < w.n_here) raw[i] = *reinterpret_cast<const u32x2*>(base + i * kRowW + 8 * lane);
+                }
+                raw_rope = 0;
+                if (my_pos0 + (lane >> 4) < w.n_here)
+                    raw_rope = *reinterpret_cast<const uint32_t*>(base + (lane >> 4) * kRowW + kKvl + 4 * (lane & 15));
+            }
+            raw_scale = 0.0f, raw_bias = -INFINITY;
+            if (lane < 4 && my_pos0 + lane < w.n_here) {
+                raw_scale = *reinterpret_cast<const float*>(a.pool + w.tile_scale_off + (size_t)(my_pos0 + lane) * 4);
+                raw_bias = 0.0f;
+            }
+            return;
+        }
+        const uint32_t lo = (uint32_t)w.code_off, hi = (uint32_t)(w.code_off >> 32);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t blo = __builtin_amdgcn_readlane(lo, i), bhi = __builtin_amdgcn_readlane(hi, i);
@@ -248,11 +313,14 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
             raw[i] = u32x2{0, 0};
             if (b != kNone) raw[i] = *reinterpret_cast<const u32x2*>(a.pool + b + 8 * lane);
         }
-        const unsigned long long br = __shfl(code_off, lane >> 4, kWave);
+        const unsigned long long br = __shfl(w.code_off, lane >> 4, kWave);
         raw_rope = 0;
         if (br != kNone) raw_rope = *reinterpret_cast<const uint32_t*>(a.pool + br + kKvl + 4 * (lane & 15));
-        raw_scale = -1.0f;  // a negative scale marks a token that is not there
-        if (lane < 4 && code_off != kNone) raw_scale = *reinterpret_cast<const float*>(a.pool + scale_off);
+        raw_scale = 0.0f, raw_bias = -INFINITY;
+        if (lane < 4 && w.code_off != kNone) {
+            raw_scale = *reinterpret_cast<const float*>(a.pool + w.scale_off);
+            raw_bias = 0.0f;
+        }
     };
     auto stage = [&](int buf) {
         uint8_t* const krb = kr + buf * kKrBytes;
@@ -262,7 +330,7 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         for (int i = 0; i < 4; ++i) {
             e4m3x4_to_bf16(raw[i].x, r[i][0], r[i][1]);
             e4m3x4_to_bf16(raw[i].y, r[i][2], r[i][3]);
-            *reinterpret_cast<u32x4*>(krb + tile_pos_of(wave, i) * kKrRowBytes + 16 * lane) =
+            *reinterpret_cast<u32x4*>(krb + (my_pos0 + i) * kKrRowBytes + 16 * lane) =
                 u32x4{r[i][0], r[i][1], r[i][2], r[i][3]};
         }
 #pragma unroll
@@ -276,18 +344,24 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         }
         uint32_t rr0, rr1;
         e4m3x4_to_bf16(raw_rope, rr0, rr1);
-        *reinterpret_cast<u32x2*>(krb + tile_pos_of(wave, lane >> 4) * kKrRowBytes + kKvl * 2 +
-                                  8 * (lane & 15)) = u32x2{rr0, rr1};
-        if (lane < 4) sc[buf * kTile + 4 * wave + lane] = raw_scale;
+        *reinterpret_cast<u32x2*>(krb + (my_pos0 + (lane >> 4)) * kKrRowBytes + kKvl * 2 + 8 * (lane & 15)) =
+            u32x2{rr0, rr1};
+        if (lane < 4) {
+            // a scale that is not a positive number cannot come from the append: such a
+            // token is left out like one that is not there
+            const bool ok = raw_scale > 0.0f;
+            sc[buf * kTile + 4 * wave + lane] = ok ? raw_scale : 0.0f;
+            sbias[buf * kTile + 4 * wave + lane] = ok ? raw_bias : -INFINITY;
+        }
     };
 
     // ---- prologue: tile 0 staged, tile 1 resolved ---------------------------------------
-    unsigned long long code_off, scale_off;
-    resolve(row_token(0), code_off, scale_off);
-    issue_loads(code_off, scale_off);
+    Where where;
+    resolve(0, row_token(0), where);
+    issue_loads(where);
     unsigned int tok_ahead = n_tiles > 1 ? row_token(1) : 0xffffffffu;
     stage(0);
-    resolve(tok_ahead, code_off, scale_off);
+    resolve(1, tok_ahead, where);
     __syncthreads();
 
     f32x4 o[kColTilesHalf];
@@ -299,7 +373,7 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
 
     for (int tile = 0; tile < n_tiles; ++tile) {
         const int buf = tile & 1;
-        if (tile + 1 < n_tiles) issue_loads(code_off, scale_off);       // tile + 1's bytes
+        if (tile + 1 < n_tiles) issue_loads(where);       // tile + 1's bytes
         tok_ahead = tile + 2 < n_tiles ? row_token(tile + 2) : 0xffffffffu;
 
         // ---- scores: this wave's half of the dims, S^T[token][head], two 16-token halves --
@@ -326,7 +400,8 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
             }
         }
         xch_mine[0] = s0, xch_mine[1] = s1;
-        // the first value-side fragments do not depend on the softmax: fetch them under it
+        // what does not depend on the other half of the scores is fetched under the barrier:
+        // the first value-side fragments, the tokens' scales and biases
         const uint8_t* const vtb = vt + buf * kVtBytes;
         auto vt_frag = [&](int nt) -> bf16x8 {
             const int c = 16 * (half * kColTilesHalf + nt) + n16;
@@ -336,6 +411,10 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         bf16x8 fb[kValueAhead];
 #pragma unroll
         for (int i = 0; i < kValueAhead; ++i) fb[i] = vt_frag(i);
+        const f32x4 sa = *reinterpret_cast<const f32x4*>(sc + buf * kTile + 8 * g);
+        const f32x4 sb = *reinterpret_cast<const f32x4*>(sc + buf * kTile + 8 * g + 4);
+        const f32x4 ba = *reinterpret_cast<const f32x4*>(sbias + buf * kTile + 8 * g);
+        const f32x4 bb = *reinterpret_cast<const f32x4*>(sbias + buf * kTile + 8 * g + 4);
         __syncthreads();  // both halves of every score are in LDS
         {
             const f32x4 p0 = xch_peer[0], p1 = xch_peer[1];
@@ -343,18 +422,15 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         }
 
         // ---- online softmax over the lane's 8 tokens of head n16 --------------------------
-        const f32x4 sa = *reinterpret_cast<const f32x4*>(sc + buf * kTile + 8 * g);
-        const f32x4 sb = *reinterpret_cast<const f32x4*>(sc + buf * kTile + 8 * g + 4);
         const float scl[8] = {sa.x, sa.y, sa.z, sa.w, sb.x, sb.y, sb.z, sb.w};
+        const float bias[8] = {ba.x, ba.y, ba.z, ba.w, bb.x, bb.y, bb.z, bb.w};
         float v[8];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            v[i] = scl[i] < 0.0f ? -INFINITY : s0[i] * scl[i];
-            v[4 + i] = scl[4 + i] < 0.0f ? -INFINITY : s1[i] * scl[4 + i];
+            v[i] = __builtin_fmaf(s0[i], scl[i], bias[i]);              // -inf where the token is not there
+            v[4 + i] = __builtin_fmaf(s1[i], scl[4 + i], bias[4 + i]);
         }
-        float tmax = v[0];
-#pragma unroll
-        for (int i = 1; i < 8; ++i) tmax = fmaxf(tmax, v[i]);
+        float tmax = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
         const bool grow = tmax > m_ref + kLazyRescale;  // false while everything is masked
@@ -371,26 +447,25 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
                 for (int i = 0; i < 4; ++i) o[nt][i] *= c[i];
         }
         const float mu = m_ref == -INFINITY ? 0.0f : m_ref;
-        // The value MFMA sees a_t = bf16(p_t * s_t) (optionally hi + lo). The denominator
-        // sums a_t / s_t, the weights the numerator really carries, so the result is an
-        // exactly normalised average under weights perturbed by their rounding: the error
-        // scales with the spread of the attended rows, not with their magnitude, and
-        // vanishes when one token holds the whole softmax.
+        // The value MFMA sees a_t = bf16(p_t * s_t), as hi + lo when PSPLIT == 2. Carried
+        // once, the denominator sums a_t / s_t — the weights the numerator really holds — so
+        // the result is an exactly normalised average under weights perturbed by one bf16
+        // rounding each: the error scales with the spread of the attended rows, not their
+        // magnitude, and vanishes when one token holds the whole softmax. Carried as
+        // hi + lo the weights are good to 2^-17 and the denominator sums p_t itself.
         bf16x8 p, p_lo;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const float e = __builtin_amdgcn_exp2f(v[i] - mu);  // masked -> 0
-            const bool there = scl[i] > 0.0f;
-            const float x = e * (there ? scl[i] : 0.0f);
+            const float e = __builtin_amdgcn_exp2f(v[i] - mu);  // not there -> 0
+            const float x = e * scl[i];
             const __bf16 w = (__bf16)x;
             p[i] = w;
-            float carried = (float)w;
             if (PSPLIT == 2) {
-                const __bf16 w_lo = (__bf16)(x - carried);
-                p_lo[i] = w_lo;
-                carried += (float)w_lo;
+                p_lo[i] = (__bf16)(x - (float)w);
+                l_sum += e;
+            } else {
+                l_sum += (float)w * (scl[i] > 0.0f ? __builtin_amdgcn_rcpf(scl[i]) : 0.0f);
             }
-            l_sum += carried * (there ? __builtin_amdgcn_rcpf(scl[i]) : 0.0f);
         }
 
         // ---- values: O[head][col] += P . V over this wave's 256 columns -------------------
@@ -404,7 +479,7 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
 
         // ---- stage tile + 1 into the other buffer, resolve tile + 2 -----------------------
         if (tile + 1 < n_tiles) stage(buf ^ 1);
-        resolve(tok_ahead, code_off, scale_off);
+        resolve(tile + 2, tok_ahead, where);
         __syncthreads();
     }
 
@@ -503,6 +578,7 @@ extern "C" int rivoli_mla_attend_paged(const float* qabs, const float* qrope,
     a.qabs = qabs, a.qrope = qrope, a.pool = pool, a.block_table = block_table;
     a.seq_lens = seq_lens, a.rows = rows, a.n_rows = n_rows, a.k = max_rows;
     a.H = H, a.max_blocks = max_blocks_per_seq, a.page_tokens = page_tokens, a.n_pages = n_pages;
+    a.page_shift = (page_tokens & (page_tokens - 1)) == 0 ? __builtin_ctz((unsigned)page_tokens) : -1;
     a.page_bytes = (size_t)page_tokens * kRowW + (size_t)page_tokens * 4;
     a.qscale = scale * kLog2e;
     a.n_splits = plan.n_splits, a.split_rows = plan.split_rows;
@@ -512,17 +588,18 @@ extern "C" int rivoli_mla_attend_paged(const float* qabs, const float* qrope,
     const dim3 grid((unsigned)plan.n_splits, (unsigned)n_seqs, (unsigned)((H + 63) / 64));
     (void)hipGetLastError();
     hipStream_t st = (hipStream_t)stream;
-#define RK_ATTEND_LAUNCH(Q, P, S) \
-    hipLaunchKernelGGL((mla_attend_paged_kernel<Q, P, S>), grid, dim3(kAttThreads), 0, st, a)
-    if (rows) {
-        if (precise >= 2) RK_ATTEND_LAUNCH(2, 2, true);
-        else if (precise == 1) RK_ATTEND_LAUNCH(2, 1, true);
-        else RK_ATTEND_LAUNCH(1, 1, true);
-    } else {
-        if (precise >= 2) RK_ATTEND_LAUNCH(2, 2, false);
-        else if (precise == 1) RK_ATTEND_LAUNCH(2, 1, false);
-        else RK_ATTEND_LAUNCH(1, 1, false);
-    }
+#define RK_ATTEND_LAUNCH(Q, P, M) \
+    hipLaunchKernelGGL((mla_attend_paged_kernel<Q, P, M>), grid, dim3(kAttThreads), 0, st, a)
+#define RK_ATTEND_MODES(M)                          \
+    do {                                            \
+        if (precise >= 2) RK_ATTEND_LAUNCH(2, 2, M); \
+        else if (precise == 1) RK_ATTEND_LAUNCH(2, 1, M); \
+        else RK_ATTEND_LAUNCH(1, 1, M);             \
+    } while (0)
+    if (rows) RK_ATTEND_MODES(kSparse);
+    else if (a.page_shift >= 0 && page_tokens >= kTile) RK_ATTEND_MODES(kDensePaged);
+    else RK_ATTEND_MODES(kDense);
+#undef RK_ATTEND_MODES
 #undef RK_ATTEND_LAUNCH
     int rc = launch_status();
     if (rc != 0 || plan.n_splits <= 1) return rc;
