@@ -51,6 +51,19 @@ int rivoli_index_topk(const float* scores, int nt, int k, unsigned int* rows);
 int rivoli_hash_rows(const float* x, int n, int stride, unsigned long long i_base,
                      unsigned long long* out, void* stream);
 
+/* Replaces crates/backend/kernels/attn.hip:100-103,279-308 (Rust: attend_scratch_floats and
+ * launch_attend, crates/backend/src/hip_attn.rs:113-128): MLA decode attention for one token
+ * over the LINEAR slabs — clat[h] = sum_t softmax_t((qabs_h . L_t + qrope_h . R_t) * scale) *
+ * L_t with L_t the e4m3 latent times its per-128 f32 scales, R_t the bf16 roped key, token =
+ * rows ? rows[j] : j for j < nr. `partial` is scratch of rivoli_mla_attend_scratch_floats(H,
+ * kvl) floats, or null for a single split. Null stream. Guards as the reference: 1001
+ * non-positive dim; 1002 (kvl + rope) > 1024; 1004 kvl > 512 or kvl % 128. */
+size_t rivoli_mla_attend_scratch_floats(int H, int kvl);
+int rivoli_mla_attend(const float* qabs, const float* qrope, const unsigned char* Lc8,
+                      const float* Lscale, const unsigned short* Rc, const unsigned int* rows, int H,
+                      int nr, int kvl, int rope, int n_blocks, float scale, float* clat,
+                      float* partial);
+
 /* Replaces crates/backend/src/hip.rs:339-342's rivoli_device_sync: hipDeviceSynchronize. */
 int rivoli_device_sync(void);
 

@@ -50,6 +50,7 @@ _SIGNATURES = {
     "rivoli_kv_append_paged": [_VP, _VP, _VP, _I, _I, _I, _I, _VP, _VP],
     "rivoli_kv_gather_paged": [_VP] * 5 + [_I] * 5 + [_VP, _VP],
     "rivoli_kv_gather_rows_paged": [_VP] * 5 + [_I] * 6 + [_VP, _VP],
+    "rivoli_mla_attend": [_VP] * 6 + [_I] * 5 + [_F, _VP, _VP],
     "rivoli_mla_attend_paged": [_VP] * 7 + [_I] * 8 + [_F, _I, _VP, _VP, _VP, _VP],
     "rivoli_codec_e4m3_encode": [_VP, _VP, _LL, _VP],
     "rivoli_codec_e4m3_dequant_bf16": [_VP, _F, _VP, _LL, _VP],
@@ -83,13 +84,16 @@ def lib() -> C.CDLL:
             fn.restype, fn.argtypes = C.c_size_t, [_I, _I]
         fn = handle.rivoli_mla_attend_paged_scratch_floats
         fn.restype, fn.argtypes = C.c_size_t, [_I, _I, _I]
+        fn = handle.rivoli_mla_attend_scratch_floats
+        fn.restype, fn.argtypes = C.c_size_t, [_I, _I]
         _LIB = handle
     return _LIB
 
 
 def exported_symbols() -> list[str]:
     return sorted(list(_SIGNATURES) + ["rivoli_kv_page_bytes", "rivoli_index_topk_workspace_bytes",
-                                       "rivoli_mla_attend_paged_scratch_floats"])
+                                       "rivoli_mla_attend_paged_scratch_floats",
+                                       "rivoli_mla_attend_scratch_floats"])
 
 
 def _p(x):
@@ -205,6 +209,21 @@ def launch_index_topk_batched(scores, n_queries, stride, nts, nt, k, rows, works
     ensure_hip_status(lib().rivoli_index_topk_batched(_p(scores), n_queries, stride, _p(nts), nt,
                                                       k, _p(rows), _p(workspace), _s(stream)),
                       "index_topk_batched")
+
+
+# ---- attention: the reference's single-token launcher over its linear slabs ----------------
+
+def attend_scratch_floats(H: int, kvl: int) -> int:
+    """crates/backend/src/hip_attn.rs: attend_scratch_floats."""
+    return int(lib().rivoli_mla_attend_scratch_floats(H, kvl))
+
+
+def launch_attend(qabs, qrope, lc8, lscale, rc, rows, H, nr, kvl, rope, n_blocks, scale, clat,
+                  partial) -> None:
+    """crates/backend/src/hip_attn.rs:113-128 (launch_attend -> rivoli_mla_attend)."""
+    ensure_hip_status(lib().rivoli_mla_attend(_p(qabs), _p(qrope), _p(lc8), _p(lscale), _p(rc), _p(rows),
+                                              H, nr, kvl, rope, n_blocks, scale, _p(clat), _p(partial)),
+                      "mla_attend")
 
 
 # ---- attention over the paged cache -------------------------------------------------------

@@ -47,6 +47,11 @@ def ref_kernels():
         h.rivoli_append_kv.restype, h.rivoli_append_kv.argtypes = i, [vp] * 5 + [i] * 4
         h.rivoli_index_append.restype, h.rivoli_index_append.argtypes = i, [vp, vp, i, i]
         h.rivoli_index_topk.restype, h.rivoli_index_topk.argtypes = i, [vp, i, i, vp]
+        if hasattr(h, "rivoli_mla_attend"):
+            h.rivoli_mla_attend.restype = i
+            h.rivoli_mla_attend.argtypes = [vp] * 6 + [i] * 5 + [C.c_float, vp, vp]
+            h.rivoli_mla_attend_scratch_floats.restype = C.c_size_t
+            h.rivoli_mla_attend_scratch_floats.argtypes = [i, i]
         h.rivoli_hash_rows.restype = i
         h.rivoli_hash_rows.argtypes = [vp, i, i, C.c_ulonglong, vp, vp]
         _REF = h

@@ -152,3 +152,71 @@ def test_guards():
     assert e.value.code == 1001
     assert hip.mla_attend_paged_scratch_floats(1, 64, 64) == 0
     assert hip.mla_attend_paged_scratch_floats(32, 64, 32768) == 32 * 16 * 64 * 514
+
+
+# ---- the reference's single-token launcher over its linear slabs --------------------------
+
+def run_linear(case, h, nt, kvl, rope, rows=None, scratch=True, launch=None):
+    qabs, qrope, lc8, lscale, rc, nb, scale = case
+    nr = nt if rows is None else rows.size
+    clat = dzeros(h * kvl * 4, 0xFF)
+    part = dzeros(hip.attend_scratch_floats(h, kvl) * 4, 0xFF) if scratch else None
+    args = (dev(qabs), dev(qrope), dev(lc8), dev(lscale), dev(rc), None if rows is None else dev(rows))
+    if launch is None:
+        hip.launch_attend(*args, h, nr, kvl, rope, nb, scale, clat, part)
+    else:
+        rc_ = launch(*[None if a is None else a.data_ptr() for a in args], h, nr, kvl, rope, nb, scale,
+                     clat.data_ptr(), None if part is None else part.data_ptr())
+        assert rc_ == 0
+    return back(clat, np.float32).reshape(h, kvl)
+
+
+def check_linear(got, want, what):
+    """The reference's bar (crates/engine/tests/common/asserts.rs) and, since this launcher
+    computes in f32 like the reference's, a much tighter one."""
+    err, mx = float(np.abs(got.astype(np.float64) - want).max()), float(np.abs(want).max())
+    assert err <= 1e-3 * mx + 1e-3, f"{what}: err={err:.3e} max={mx:.3e}"
+    assert err <= 2e-5 * mx + 1e-7, f"{what}: err={err:.3e} max={mx:.3e} (tight)"
+
+
+@pytest.mark.parametrize("seed,h,nt,kvl,rope", [
+    (0x0A5E1102, 64, 300, 512, 64),      # crates/engine/tests/kernel_attend.rs:270-274
+    (0x5F117BAD, 64, 704, 512, 64),      # :287-297, the split planner's other regimes
+    (0xC1A39ED0, 64, 4608, 512, 64),
+    (0x00C0FFEE, 4, 1, 128, 8),          # :299-307, edges
+    (0xB10CC0DE, 20, 130, 512, 64),
+])
+def test_linear_attend_reference_cases(oracle, seed, h, nt, kvl, rope):
+    from tests.attend_cases import reference_attend_case
+    from tests.gpu_util import ref_kernels
+
+    case = reference_attend_case(oracle, seed, h, nt, kvl, rope)
+    code, want = oracle.mla_attend(*case[:5], None, h, nt, kvl, rope, case[5], case[6])
+    assert code == 0
+    check_linear(run_linear(case, h, nt, kvl, rope), want, "multi-split")
+    check_linear(run_linear(case, h, nt, kvl, rope, scratch=False), want, "single split (null scratch)")
+    ref = ref_kernels()
+    if ref is not None and hasattr(ref, "rivoli_mla_attend"):
+        # the reference's own kernel, compiled for this GPU, agrees with the oracle too
+        check_linear(run_linear(case, h, nt, kvl, rope, launch=ref.rivoli_mla_attend), want, "reference kernel")
+
+
+def test_linear_attend_rows_and_guards(oracle):
+    from tests.attend_cases import reference_attend_case
+
+    h, nt, kvl, rope = 20, 900, 384, 24
+    case = reference_attend_case(oracle, 0x51DE, h, nt, kvl, rope)
+    rows = np.sort(np.random.default_rng(2).choice(nt, 333, replace=False)).astype(np.uint32)
+    code, want = oracle.mla_attend(*case[:5], rows, h, rows.size, kvl, rope, case[5], case[6])
+    assert code == 0
+    check_linear(run_linear(case, h, nt, kvl, rope, rows=rows), want, "row list")
+    # crates/engine/tests/kernel_attend.rs:170-192: kvl over the register cap or off the block size
+    b = dzeros(64 * 1024 * 4)
+    for bad_kvl, code in ((640, 1004), (160, 1004)):
+        with pytest.raises(hip.LaunchError) as e:
+            hip.launch_attend(b, b, b, b, b, None, 8, 16, bad_kvl, 64, bad_kvl // 128 or 1, 1.0, b, b)
+        assert e.value.code == code
+    with pytest.raises(hip.LaunchError) as e:
+        hip.launch_attend(b, b, b, b, b, None, 0, 16, 512, 64, 4, 1.0, b, b)
+    assert e.value.code == 1001
+    assert hip.attend_scratch_floats(64, 512) == 16 * 64 * 514
