@@ -40,10 +40,12 @@ def parse():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=32768)
-    ap.add_argument("--workload", choices=["decode", "prefill", "dsa", "dsa_scored", "attend"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "dsa", "dsa_scored", "dsa_attend", "attend"], default="decode",
                     help="decode = configuration 3 (the headline line); prefill = configuration 2 "
                          "bulk append; dsa = configuration 4 top-k + sparse gather on synthetic "
                          "scores; dsa_scored = the same with the scores computed on the device; "
+                         "dsa_attend = configuration 4 with the sparse gather replaced by MLA decode "
+                         "attention over the selected rows; "
                          "attend = configuration 3 with the gather replaced by MLA decode "
                          "attention reading the fp8 pages directly")
     ap.add_argument("--heads", type=int, default=64, help="attend: query heads")
@@ -81,8 +83,8 @@ def main():
         del src, dst
     if a.workload == "prefill":
         return bench_prefill(a, torch, hip)
-    if a.workload in ("dsa", "dsa_scored"):
-        return bench_dsa(a, torch, hip, scored=a.workload == "dsa_scored")
+    if a.workload in ("dsa", "dsa_scored", "dsa_attend"):
+        return bench_dsa(a, torch, hip, scored=a.workload == "dsa_scored", attend=a.workload == "dsa_attend")
     if a.workload == "attend":
         return bench_attend(a, torch, hip)
     L, B, ctx = a.layers, a.batch, a.ctx
@@ -270,7 +272,7 @@ def bench_prefill(a, torch, hip):
     print(json.dumps(res), flush=True)
 
 
-def bench_dsa(a, torch, hip, scored=False):
+def bench_dsa(a, torch, hip, scored=False, attend=False):
     """benchmark configuration 4: per layer, select the top-k of 65536 indexer scores for each of 16
     queries (ties to the lowest index), then gather + dequantize those rows from fragmented
     pages. One step = all layers."""
@@ -314,6 +316,13 @@ def bench_dsa(a, torch, hip, scored=False):
             scores.append(sc)
     sel = torch.empty(B * k, dtype=torch.int32, device="cuda")
     out = torch.empty(B * k * W, dtype=torch.bfloat16, device="cuda")
+    H = a.heads
+    if attend:
+        qabs = [torch.randn(B, H, 512, generator=g, device="cuda", dtype=torch.float32) for _ in range(L)]
+        qrope = [torch.randn(B, H, 64, generator=g, device="cuda", dtype=torch.float32) for _ in range(L)]
+        clat = torch.empty(B, H, 512, dtype=torch.float32, device="cuda")
+        partial = torch.empty(max(hip.mla_attend_paged_scratch_floats(B, H, k), 1), dtype=torch.float32,
+                              device="cuda")
     ws_topk = torch.zeros(hip.index_topk_workspace_bytes(B, nt), dtype=torch.uint8, device="cuda")
     torch.cuda.synchronize()
     stream = torch.cuda.Stream()
@@ -329,13 +338,22 @@ def bench_dsa(a, torch, hip, scored=False):
             sc_in = score_buf if scored else scores[layer]
             bracket(torch, stream, events, "topk",
                     lambda: hip.launch_index_topk_batched(sc_in, B, nt, None, nt, k, sel, ws_topk, sh))
-            bracket(torch, stream, events, "gather_rows",
-                    lambda: hip.launch_kv_gather_rows_paged(pools[layer], tables, sel, None, out, B, k,
-                                                            blocks, W, PT, n_pages, None, sh))
+            if attend:
+                bracket(torch, stream, events, "attend_rows",
+                        lambda: hip.launch_mla_attend_paged(qabs[layer], qrope[layer], pools[layer], tables, None,
+                                                            sel, None, B, H, k, blocks, 512, 64, PT, n_pages,
+                                                            float(W) ** -0.5, a.precise, clat, partial, None, sh))
+            else:
+                bracket(torch, stream, events, "gather_rows",
+                        lambda: hip.launch_kv_gather_rows_paged(pools[layer], tables, sel, None, out, B, k,
+                                                                blocks, W, PT, n_pages, None, sh))
 
     ms, per = timed(torch, stream, a.steps, a.warmup, step)
     topk_bytes = B * nt * 4 + B * k * 4
     rows_bytes = B * k * (4 + REC + ROW_IN) + B * blocks * 4
+    if attend:  # row list, records and table in, q in, clat out; no bf16 rows are written
+        rows_bytes = B * k * (4 + REC) + B * blocks * 4 + B * H * (W + 512) * 4
+    rows_kernel = "attend_rows" if attend else "gather_rows"
     score_bytes = (B * nt * (HD * 2 + 4) + B * NH * (HD + 1) * 4 + B * blocks * 4) if scored else 0
     layer_bytes = topk_bytes + rows_bytes + score_bytes
     res = {"metric": "kv_dsa_topk_gather_GBps", "value": round(L * layer_bytes / (ms * 1e-3) / 1e9, 2),
@@ -346,11 +364,11 @@ def bench_dsa(a, torch, hip, scored=False):
                       "layers": L, "batch": B, "ctx": nt, "k": k, "width": W, "page_tokens": PT},
            "rows_per_s": round(L * B * k / (ms * 1e-3), 1),
            "kernels_ms": {n: round(v, 5) for n, v in per.items()},
-           "roofline": {"bound": "hbm", "kernel": "kv_gather_rows_kernel",
-                        "achieved": round(rows_bytes / (per["gather_rows"] * 1e-3) / 1e9, 2),
+           "roofline": {"bound": "hbm", "kernel": "mla_attend_paged_kernel" if attend else "kv_gather_rows_kernel",
+                        "achieved": round(rows_bytes / (per[rows_kernel] * 1e-3) / 1e9, 2),
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                        "frac": round(rows_bytes / (per["gather_rows"] * 1e-3) / HBM_PEAK, 5),
-                        "avg_launch_ms": round(per["gather_rows"], 5),
+                        "frac": round(rows_bytes / (per[rows_kernel] * 1e-3) / HBM_PEAK, 5),
+                        "avg_launch_ms": round(per[rows_kernel], 5),
                         "bytes_per_launch": rows_bytes, "traffic": None},
            "topk": {"achieved": round(topk_bytes / (per["topk"] * 1e-3) / 1e9, 2), "unit": "GB/s",
                     "avg_launch_ms": round(per["topk"], 5), "bytes_per_launch": topk_bytes}}
@@ -361,7 +379,12 @@ def bench_dsa(a, torch, hip, scored=False):
                               "unit": "GB/s", "frac": round(score_bytes / (per["score"] * 1e-3) / HBM_PEAK, 4),
                               "avg_launch_ms": round(per["score"], 5), "bytes_per_launch": score_bytes,
                               "tflops": round(B * nt * NH * HD * 2 * 2 / (per["score"] * 1e-3) / 1e12, 1)}
-    if not a.no_cpu_baseline and not scored:
+    if attend:
+        res["metric"] = "kv_dsa_topk_attend_GBps"
+        res["config"]["workload"] = ("DSA sparse path with the consumer fused: top-k, then MLA latent attention "
+                                     "over the selected rows straight from the fp8 pages")
+        res["config"]["heads"], res["config"]["precise"] = H, a.precise
+    if not a.no_cpu_baseline and not scored and not attend:
         from oracle.kvoracle import oracle as get_oracle
 
         ora, cores = get_oracle(), max(1, min(16, os.cpu_count() or 1))

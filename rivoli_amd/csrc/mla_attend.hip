@@ -106,6 +106,21 @@ __device__ __forceinline__ void e4m3x4_to_bf16(uint32_t c, uint32_t& lo, uint32_
     hi = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c, 1.0f, true));
 }
 
+// max / sum of a value over the four 16-lane rows of the wave, in every lane. gfx950's row
+// swaps stay in the vector ALU; the generic cross-lane shuffle goes through the LDS crossbar.
+__device__ __forceinline__ float rows_max(float x) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));  // rows {0,1} and {2,3} paired
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float rows_sum(float x) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 struct AttendArgs {
     const float* qabs;            // [n_seqs][H][512]
     const float* qrope;           // [n_seqs][H][64]
@@ -431,8 +446,7 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
             v[4 + i] = __builtin_fmaf(s1[i], scl[4 + i], bias[4 + i]);
         }
         float tmax = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+        tmax = rows_max(tmax);
         const bool grow = tmax > m_ref + kLazyRescale;  // false while everything is masked
         if (__builtin_amdgcn_ballot_w64(grow) != 0) {
             const float corr = grow ? __builtin_amdgcn_exp2f(m_ref - tmax) : 1.0f;  // 2^-inf = 0 at first
@@ -484,8 +498,7 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
     }
 
     // ---- epilogue -----------------------------------------------------------------------
-    l_sum += __shfl_xor(l_sum, 16, kWave);
-    l_sum += __shfl_xor(l_sum, 32, kWave);
+    l_sum = rows_sum(l_sum);
     // the lane's accumulators are heads 4g+i; their (m, l) live in lanes with n16 == 4g+i
     float l_h[4];
 #pragma unroll
