@@ -75,7 +75,7 @@ constexpr int kValueAhead = 6;             // value-side operand fragments in fl
 constexpr float kLog2e = 1.4426950408889634f;
 
 // split plan: pure function of the call's shape
-constexpr int kAttTargetGroups = 512;      // two workgroups' worth per CU of a 256-CU part
+constexpr int kAttTargetGroups = 256;      // one workgroup per CU of a 256-CU part
 constexpr int kAttMinTilesPerSplit = 8;    // below 256 rows a split costs more than it buys
 constexpr int kAttMaxSplits = 64;
 

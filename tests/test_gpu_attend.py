@@ -151,7 +151,7 @@ def test_guards():
                                     b, None)
     assert e.value.code == 1001
     assert hip.mla_attend_paged_scratch_floats(1, 64, 64) == 0
-    assert hip.mla_attend_paged_scratch_floats(32, 64, 32768) == 32 * 16 * 64 * 514
+    assert hip.mla_attend_paged_scratch_floats(32, 64, 32768) == 32 * 8 * 64 * 514
 
 
 # ---- the reference's single-token launcher over its linear slabs --------------------------
