@@ -94,7 +94,7 @@ __global__ __launch_bounds__(kGatherThreads) void kv_gather_rows_kernel(
     const int width = W ? W : width_rt;
     const int pt = PT ? PT : page_tokens_rt;
     __shared__ unsigned long long s_base[kRowsPerGroup];
-    __shared__ float s_scale[kRowsPerGroup];
+    __shared__ unsigned long long s_scale_at[kRowsPerGroup];
     constexpr unsigned long long kSkip = ~0ull;
 
     const int q = blockIdx.y;
@@ -103,9 +103,12 @@ __global__ __launch_bounds__(kGatherThreads) void kv_gather_rows_kernel(
     if (r0 >= nr) return;
     const int cnt = min(kRowsPerGroup, nr - r0);
 
+    // row index -> page -> where the codes and the scale are. The scale itself is NOT
+    // fetched here: every thread loads its rows' scales together with the codes, so the
+    // chain of dependent memory round trips is row list -> block table -> data, not one
+    // longer.
     if (threadIdx.x < kRowsPerGroup) {
-        unsigned long long base = kSkip;
-        float scale = 0.0f;
+        unsigned long long base = kSkip, scale_at = 0;
         if ((int)threadIdx.x < cnt) {
             const unsigned int tok = rows[(size_t)q * k + r0 + threadIdx.x];
             const unsigned int blk = tok / (unsigned)pt;
@@ -116,14 +119,13 @@ __global__ __launch_bounds__(kGatherThreads) void kv_gather_rows_kernel(
             if ((unsigned)page < (unsigned)n_pages) {
                 const size_t pbase = (size_t)page * page_bytes;
                 base = pbase + (size_t)off * width;
-                scale = *reinterpret_cast<const float*>(pool + pbase + (size_t)pt * width +
-                                                        (size_t)off * 4);
+                scale_at = pbase + (size_t)pt * width + (size_t)off * 4;
             } else if (bad_rows) {
                 atomicAdd(bad_rows, 1u);
             }
         }
         s_base[threadIdx.x] = base;
-        s_scale[threadIdx.x] = scale;
+        s_scale_at[threadIdx.x] = scale_at;
     }
     __syncthreads();
 
@@ -146,7 +148,7 @@ __global__ __launch_bounds__(kGatherThreads) void kv_gather_rows_kernel(
                     live[u] = true;
                     raw[u] = __builtin_nontemporal_load(
                         reinterpret_cast<const u32x2*>(pool + base) + col);
-                    scl[u] = s_scale[r];
+                    scl[u] = *reinterpret_cast<const float*>(pool + s_scale_at[r]);
                 }
             }
         }

@@ -23,10 +23,12 @@
 // softmax and staging. Tokens move in tiles of 32:
 //   * staging: wave w fetches 4 tokens of the tile (one fully coalesced 512-byte run per
 //     token for the latent, 64 bytes for the rope), converts e4m3 -> bf16 in registers and
-//     writes the tile to LDS twice — row-major [token][dim] for the score contraction (over
-//     dims) and transposed [dim][token] for the value contraction (over tokens); the
-//     register transpose is byte-permutes. The next tile's loads are issued before this
-//     tile's MFMAs; the LDS tile is double-buffered.
+//     writes them row-major [token][dim] into LDS, once. The score contraction (over dims)
+//     reads its operands from that tile directly; the value contraction (over tokens)
+//     reads the same tile through gfx950's transposing LDS load (ds_read_b64_tr_b16), so no
+//     second, transposed copy is written. Three tiles rotate: a tile is staged two
+//     iterations before it is consumed and loaded from memory one iteration before that,
+//     which leaves ONE barrier per tile (the one the score exchange needs anyway).
 //   * scores: S^T[token][head] = K . Q^T with v_mfma_f32_16x16x32_bf16, A = the tile's rows
 //     from LDS, B = the wave's half of its query heads, resident in registers for the whole
 //     kernel (optionally as bf16 hi + lo, two MFMAs per step, ~17 bits of q). The two
@@ -34,11 +36,11 @@
 //     same numbers. With tokens as the tile's rows a lane ends up holding 8 tokens of ONE
 //     head, which is exactly the A-operand layout of the value MFMA — P never leaves
 //     registers. The tile's token order inside the value contraction is whatever that
-//     layout implies; staging writes the transposed copy in the same order.
+//     layout implies; the transposing loads address the rows in the same order.
 //   * softmax: online, base 2 (log2 e folded into q); the running maximum only moves when a
 //     tile exceeds it by more than 2^8 (the f32 accumulators have the range), so rescaling
 //     the accumulators is rare.
-//   * values: O[head][col] += P . V over the wave's 256 columns, B = the transposed copy.
+//   * values: O[head][col] += P . V over the wave's 256 columns, B = transposing loads.
 // Splits write unnormalised partials (acc, m, l) that mla_attend_combine_kernel merges in
 // ascending split order; the split plan is a pure function of the call's shape, so equal
 // calls give bit-equal results.
@@ -59,15 +61,10 @@ constexpr int kKStepsHalf = kKSteps / 2;   // ... 9 per wave of a pair
 constexpr int kColTilesHalf = kKvl / 16 / 2;  // 16 output column tiles per wave of a pair
 constexpr int kKrRowBytes = kRowW * 2 + 16;  // row-major tile: 1152 B of bf16 + 16 B pad
 constexpr int kKrBytes = kTile * kKrRowBytes;
-// transposed tile: a row is one latent column, 32 tokens of bf16 = 64 B = four 16-byte
-// chunks; 16 B of padding after every 8 rows and an XOR of the chunk index with bits 1-2 of
-// the column keep both the staging writes (a lane owns 8 consecutive columns) and the
-// operand reads (16 lanes read 16 consecutive columns) off each other's banks
-constexpr int kVtGroupBytes = 8 * 64 + 16;
-constexpr int kVtBytes = (kKvl / 8) * kVtGroupBytes;
-constexpr int kXchBytes = kAttWaves * kWave * 8 * 4;  // partial scores, 8 f32 per lane
-constexpr int kTableLds = 960;             // block-table entries staged per workgroup
-constexpr int kAttSmemBytes = 2 * kKrBytes + 2 * kVtBytes + 4 * kTile * 4 + kXchBytes + kTableLds * 4;
+constexpr int kBufs = 3;                   // LDS tiles in rotation: tile t is staged while t-2 is consumed
+constexpr int kXchBytes = 2 * kAttWaves * kWave * 8 * 4;  // partial scores, 8 f32 per lane, two parities
+constexpr int kTableLds = 1024;            // block-table entries staged per workgroup
+constexpr int kAttSmemBytes = kBufs * kKrBytes + 2 * kBufs * kTile * 4 + kXchBytes + kTableLds * 4;
 static_assert(kAttSmemBytes <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
 constexpr float kLazyRescale = 8.0f;       // log2 units
 constexpr int kFragAhead = 3;              // score-side operand K-steps in flight (2 fragments each)
@@ -144,8 +141,7 @@ struct AttendArgs {
 // In the score tile (rows = tokens, 16 per MFMA) a lane of row group g holds rows 4g..4g+3
 // of both 16-token halves, and those 8 values are element j = 4*half + i of the value MFMA's
 // A operand for contraction index 8g + j. Staging wave w owns contraction indices
-// 4w..4w+3 — tile positions 16*(w&1) + 4*(w>>1) + i, four consecutive tokens — which is
-// half of one 16-byte chunk of every transposed row.
+// 4w..4w+3 — tile positions 16*(w&1) + 4*(w>>1) + i, four consecutive tokens.
 __device__ __forceinline__ int tile_pos_of(int wave, int i) { return 16 * (wave & 1) + 4 * (wave >> 1) + i; }
 
 // MODE: how a tile's tokens are found.
@@ -160,14 +156,13 @@ template <int QSPLIT, int PSPLIT, int MODE>
 __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const AttendArgs a) {
     constexpr bool SPARSE = MODE == kSparse;
     __shared__ __attribute__((aligned(16))) uint8_t smem[kAttSmemBytes];
-    uint8_t* const kr = smem;
-    uint8_t* const vt = smem + 2 * kKrBytes;
+    uint8_t* const kr = smem;  // [kBufs] row-major tiles
     // per token of a tile, by contraction index: its scale (0 when the token is not there)
     // and a score bias (0, or -inf when it is not there): score = s * scale + bias
-    float* const sc = reinterpret_cast<float*>(vt + 2 * kVtBytes);  // [2][32] scales, then [2][32] biases
-    float* const sbias = sc + 2 * kTile;
-    f32x4* const xch = reinterpret_cast<f32x4*>(sbias + 2 * kTile);  // [8 waves][64 lanes][2]
-    int* const tbl = reinterpret_cast<int*>(xch + kAttWaves * kWave * 2);
+    float* const sc = reinterpret_cast<float*>(kr + kBufs * kKrBytes);  // [kBufs][32]
+    float* const sbias = sc + kBufs * kTile;                             // [kBufs][32]
+    f32x4* const xch = reinterpret_cast<f32x4*>(sbias + kBufs * kTile);  // [2 parities][8 waves][64 lanes][2]
+    int* const tbl = reinterpret_cast<int*>(xch + 2 * kAttWaves * kWave * 2);
 
     const int split = blockIdx.x, seq = blockIdx.y, hb = blockIdx.z;
     const int tid = threadIdx.x;
@@ -339,23 +334,12 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
     };
     auto stage = [&](int buf) {
         uint8_t* const krb = kr + buf * kKrBytes;
-        uint8_t* const vtb = vt + buf * kVtBytes;
-        uint32_t r[4][4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            e4m3x4_to_bf16(raw[i].x, r[i][0], r[i][1]);
-            e4m3x4_to_bf16(raw[i].y, r[i][2], r[i][3]);
-            *reinterpret_cast<u32x4*>(krb + (my_pos0 + i) * kKrRowBytes + 16 * lane) =
-                u32x4{r[i][0], r[i][1], r[i][2], r[i][3]};
-        }
-#pragma unroll
-        for (int d = 0; d < 8; ++d) {  // column 8*lane + d: the wave's 4 tokens, contraction order
-            const uint32_t sel = (d & 1) ? 0x07060302u : 0x05040100u;
-            u32x2 col;
-            col.x = __builtin_amdgcn_perm(r[1][d >> 1], r[0][d >> 1], sel);
-            col.y = __builtin_amdgcn_perm(r[3][d >> 1], r[2][d >> 1], sel);
-            const int chunk = (wave >> 1) ^ ((d >> 1) & 3);
-            *reinterpret_cast<u32x2*>(vtb + lane * kVtGroupBytes + d * 64 + chunk * 16 + 8 * (wave & 1)) = col;
+            uint32_t r[4];
+            e4m3x4_to_bf16(raw[i].x, r[0], r[1]);
+            e4m3x4_to_bf16(raw[i].y, r[2], r[3]);
+            *reinterpret_cast<u32x4*>(krb + (my_pos0 + i) * kKrRowBytes + 16 * lane) = u32x4{r[0], r[1], r[2], r[3]};
         }
         uint32_t rr0, rr1;
         e4m3x4_to_bf16(raw_rope, rr0, rr1);
@@ -370,26 +354,36 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         }
     };
 
-    // ---- prologue: tile 0 staged, tile 1 resolved ---------------------------------------
+    // ---- prologue: tiles 0 and 1 staged, tile 2 in registers, tile 3 resolved ------------
     Where where;
     resolve(0, row_token(0), where);
     issue_loads(where);
-    unsigned int tok_ahead = n_tiles > 1 ? row_token(1) : 0xffffffffu;
     stage(0);
-    resolve(1, tok_ahead, where);
+    resolve(1, n_tiles > 1 ? row_token(1) : 0xffffffffu, where);
+    if (n_tiles > 1) {
+        issue_loads(where);
+        stage(1);
+    }
+    resolve(2, n_tiles > 2 ? row_token(2) : 0xffffffffu, where);
+    if (n_tiles > 2) issue_loads(where);
+    resolve(3, n_tiles > 3 ? row_token(3) : 0xffffffffu, where);
     __syncthreads();
 
     f32x4 o[kColTilesHalf];
 #pragma unroll
     for (int nt = 0; nt < kColTilesHalf; ++nt) o[nt] = f32x4{0, 0, 0, 0};
     float m_ref = -INFINITY, l_sum = 0.0f;
-    f32x4* const xch_mine = xch + (wave * kWave + lane) * 2;
-    const f32x4* const xch_peer = xch + ((wave ^ 4) * kWave + lane) * 2;
 
+    // Iteration t: scores of tile t -> exchange -> BARRIER -> softmax, values of tile t ->
+    // stage tile t+2 (in registers since iteration t-1) -> request tile t+3 from memory.
+    // The barrier orders everything that needs ordering: a wave past it knows that every
+    // wave has finished tile t-1 (so its LDS tile, (t+2) mod 3, may be overwritten) and has
+    // staged tile t+1 (which it did before its scores of tile t).
+    int buf = 0;  // t mod 3
     for (int tile = 0; tile < n_tiles; ++tile) {
-        const int buf = tile & 1;
-        if (tile + 1 < n_tiles) issue_loads(where);       // tile + 1's bytes
-        tok_ahead = tile + 2 < n_tiles ? row_token(tile + 2) : 0xffffffffu;
+        const unsigned int tok_ahead = tile + 4 < n_tiles ? row_token(tile + 4) : 0xffffffffu;
+        f32x4* const xch_mine = xch + (((tile & 1) * kAttWaves + wave) * kWave + lane) * 2;
+        const f32x4* const xch_peer = xch + (((tile & 1) * kAttWaves + (wave ^ 4)) * kWave + lane) * 2;
 
         // ---- scores: this wave's half of the dims, S^T[token][head], two 16-token halves --
         const uint8_t* const krb = kr + buf * kKrBytes + half * (kKStepsHalf * 64);
@@ -417,11 +411,21 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         xch_mine[0] = s0, xch_mine[1] = s1;
         // what does not depend on the other half of the scores is fetched under the barrier:
         // the first value-side fragments, the tokens' scales and biases
-        const uint8_t* const vtb = vt + buf * kVtBytes;
+        // value-side operand of column tile nt: for each of the lane's 8 contraction indices
+        // (tokens 4g..4g+3 of both 16-token halves) the value of column 16*nt' + n16. One
+        // transposing load hands a lane element e of the 8-byte chunk that lane
+        // 4e + (n16 >> 2) of its 16-lane row addressed, position n16 & 3 — so lane i
+        // addresses token 4g + (i >> 2), columns 16*nt' + 4*(i & 3) .. +3.
+        const uint8_t* const vrow = kr + buf * kKrBytes + (4 * g + (n16 >> 2)) * kKrRowBytes +
+                                    (half * (kKvl / 2) + 4 * (n16 & 3)) * 2;
         auto vt_frag = [&](int nt) -> bf16x8 {
-            const int c = 16 * (half * kColTilesHalf + nt) + n16;
-            return *reinterpret_cast<const bf16x8*>(vtb + (c >> 3) * kVtGroupBytes + (c & 7) * 64 +
-                                                    ((g ^ ((c >> 1) & 3)) * 16));
+            typedef short s16x4 __attribute__((ext_vector_type(4)));
+            typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow + nt * 32));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow + 16 * kKrRowBytes + nt * 32));
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            return __builtin_bit_cast(bf16x8, both);
         };
         bf16x8 fb[kValueAhead];
 #pragma unroll
@@ -491,10 +495,15 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
             if (nt + kValueAhead < kColTilesHalf) fb[slot] = vt_frag(nt + kValueAhead);
         }
 
-        // ---- stage tile + 1 into the other buffer, resolve tile + 2 -----------------------
-        if (tile + 1 < n_tiles) stage(buf ^ 1);
-        resolve(tile + 2, tok_ahead, where);
-        __syncthreads();
+        // ---- stage tile + 2, request tile + 3, resolve tile + 4 ---------------------------
+        // (the request goes out LAST: resolving reads the block table, and the wait that
+        // read needs would otherwise also wait for the bytes just requested)
+        if (tile + 2 < n_tiles) stage(buf == 0 ? 2 : buf - 1);
+        Where next;
+        resolve(tile + 4, tok_ahead, next);
+        if (tile + 3 < n_tiles) issue_loads(where);
+        where = next;
+        buf = buf == 2 ? 0 : buf + 1;
     }
 
     // ---- epilogue -----------------------------------------------------------------------
