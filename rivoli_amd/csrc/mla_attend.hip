@@ -67,8 +67,6 @@ constexpr int kTableLds = 1024;            // block-table entries staged per wor
 constexpr int kAttSmemBytes = kBufs * kKrBytes + 2 * kBufs * kTile * 4 + kXchBytes + kTableLds * 4;
 static_assert(kAttSmemBytes <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
 constexpr float kLazyRescale = 8.0f;       // log2 units
-constexpr int kFragAhead = 3;              // score-side operand K-steps in flight (2 fragments each)
-constexpr int kValueAhead = 6;             // value-side operand fragments in flight
 constexpr float kLog2e = 1.4426950408889634f;
 
 // split plan: pure function of the call's shape
@@ -155,6 +153,10 @@ enum : int {
 template <int QSPLIT, int PSPLIT, int MODE>
 __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const AttendArgs a) {
     constexpr bool SPARSE = MODE == kSparse;
+    // operand fragments requested together ahead of the MFMAs that consume them: as many
+    // as the register budget of two waves per SIMD (256) leaves room for
+    constexpr int kFragBlock = QSPLIT == 2 ? 3 : 9;   // score side, K-steps (2 fragments each)
+    constexpr int kValueAhead = QSPLIT == 2 ? 4 : 8;  // value side, fragments
     __shared__ __attribute__((aligned(16))) uint8_t smem[kAttSmemBytes];
     uint8_t* const kr = smem;  // [kBufs] row-major tiles
     // per token of a tile, by contraction index: its scale (0 when the token is not there)
@@ -390,23 +392,26 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         const bf16x8* a0p = reinterpret_cast<const bf16x8*>(krb + n16 * kKrRowBytes + 16 * g);
         const bf16x8* a1p = reinterpret_cast<const bf16x8*>(krb + (16 + n16) * kKrRowBytes + 16 * g);
         f32x4 s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0};
-        {
-            // operand fragments run kFragAhead K-steps ahead of the MFMAs that consume them
-            bf16x8 fa0[kFragAhead], fa1[kFragAhead];
+        // The operand fragments of a block of K-steps are all requested before the first MFMA
+        // of the block; left alone the compiler keeps two reads in flight and every pair of
+        // MFMAs then waits out a full LDS round trip.
 #pragma unroll
-            for (int i = 0; i < kFragAhead; ++i) fa0[i] = a0p[i * 4], fa1[i] = a1p[i * 4];
+        for (int j0 = 0; j0 < kKStepsHalf; j0 += kFragBlock) {
+            bf16x8 fa0[kFragBlock], fa1[kFragBlock];
 #pragma unroll
-            for (int j = 0; j < kKStepsHalf; ++j) {
-                const int slot = j % kFragAhead;
-                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[slot], qh[j], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[slot], qh[j], s1, 0, 0, 0);
+            for (int i = 0; i < kFragBlock; ++i) fa0[i] = a0p[(j0 + i) * 4], fa1[i] = a1p[(j0 + i) * 4];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < kFragBlock; ++i) {
+                const int j = j0 + i;
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[i], qh[j], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[i], qh[j], s1, 0, 0, 0);
                 if (QSPLIT == 2) {
-                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[slot], ql[j], s0, 0, 0, 0);
-                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[slot], ql[j], s1, 0, 0, 0);
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[i], ql[j], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[i], ql[j], s1, 0, 0, 0);
                 }
-                if (j + kFragAhead < kKStepsHalf)
-                    fa0[slot] = a0p[(j + kFragAhead) * 4], fa1[slot] = a1p[(j + kFragAhead) * 4];
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
         xch_mine[0] = s0, xch_mine[1] = s1;
         // what does not depend on the other half of the scores is fetched under the barrier:
@@ -430,6 +435,7 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         bf16x8 fb[kValueAhead];
 #pragma unroll
         for (int i = 0; i < kValueAhead; ++i) fb[i] = vt_frag(i);
+        __builtin_amdgcn_sched_barrier(0);
         const f32x4 sa = *reinterpret_cast<const f32x4*>(sc + buf * kTile + 8 * g);
         const f32x4 sb = *reinterpret_cast<const f32x4*>(sc + buf * kTile + 8 * g + 4);
         const f32x4 ba = *reinterpret_cast<const f32x4*>(sbias + buf * kTile + 8 * g);
@@ -488,11 +494,19 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
 
         // ---- values: O[head][col] += P . V over this wave's 256 columns -------------------
 #pragma unroll
-        for (int nt = 0; nt < kColTilesHalf; ++nt) {
-            const int slot = nt % kValueAhead;
-            o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p, fb[slot], o[nt], 0, 0, 0);
-            if (PSPLIT == 2) o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_lo, fb[slot], o[nt], 0, 0, 0);
-            if (nt + kValueAhead < kColTilesHalf) fb[slot] = vt_frag(nt + kValueAhead);
+        for (int n0 = 0; n0 < kColTilesHalf; n0 += kValueAhead) {
+            if (n0 > 0) {
+#pragma unroll
+                for (int i = 0; i < kValueAhead; ++i) fb[i] = vt_frag(n0 + i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < kValueAhead; ++i) {
+                o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p, fb[i], o[n0 + i], 0, 0, 0);
+                if (PSPLIT == 2)
+                    o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_lo, fb[i], o[n0 + i], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
 
         // ---- stage tile + 2, request tile + 3, resolve tile + 4 ---------------------------
