@@ -52,6 +52,9 @@ def parse():
     ap.add_argument("--precise", type=int, default=2, choices=[0, 1, 2],
                     help="attend: 2 = q and softmax weights as bf16 hi+lo (parity mode), "
                          "1 = q only, 0 = plain bf16")
+    ap.add_argument("--ragged", action="store_true",
+                    help="decode / attend: per-sequence context drawn uniformly from [1024, ctx] "
+                         "(configuration 3 as written) instead of every sequence at ctx (its metric point)")
     ap.add_argument("--tokens", type=int, default=8192, help="prefill: new tokens per step")
     ap.add_argument("--topk", type=int, default=2048)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -60,6 +63,13 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     return ap.parse_args()
+
+
+def context_lengths(a, rng):
+    """Every sequence at ctx (the metric point), or ~U[1024, ctx] with --ragged."""
+    if not a.ragged:
+        return np.full(a.batch, a.ctx, np.int32)
+    return rng.integers(min(1024, a.ctx), a.ctx + 1, size=a.batch).astype(np.int32)
 
 
 def main():
@@ -103,11 +113,12 @@ def main():
     slots_np = np.concatenate([tables_np[s][pos // PT] * PT + pos % PT for s in range(B)]).astype(np.int32)
     tables = torch.from_numpy(tables_np.copy()).cuda()
     slots_all = torch.from_numpy(slots_np).cuda()
-    seq_lens_np = np.full(B, ctx, np.int32)
+    seq_lens_np = context_lengths(a, rng)
     cu_np = np.concatenate([[0], np.cumsum(seq_lens_np)]).astype(np.int32)
     seq_lens, cu = torch.from_numpy(seq_lens_np).cuda(), torch.from_numpy(cu_np).cuda()
     # the step's new tokens: the last position of every sequence
-    new_slots = torch.from_numpy(slots_np.reshape(B, ctx)[:, -1].copy()).cuda()
+    new_slots = torch.from_numpy(slots_np.reshape(B, ctx)[np.arange(B), seq_lens_np - 1].copy()).cuda()
+    n_att = int(seq_lens_np.sum())                              # tokens gathered per layer
 
     kv_rows = torch.randn(n_tok, W, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
     pools = []
@@ -152,7 +163,8 @@ def main():
     gather_ms = float(np.mean([e0.elapsed_time(e1) for e0, e1 in events]))
 
     append_bytes = L * B * (ROW_IN + 4 + REC)                   # row + slot in, record out
-    gather_bytes_layer = n_tok * (REC + ROW_IN) + B * blocks * 4  # records + table in, bf16 out
+    table_entries = int((-(-seq_lens_np // PT)).sum())
+    gather_bytes_layer = n_att * (REC + ROW_IN) + table_entries * 4  # records + table in, bf16 out
     step_bytes = append_bytes + L * gather_bytes_layer
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     achieved = gather_bytes_layer / (gather_ms * 1e-3) / 1e9
@@ -165,9 +177,11 @@ def main():
         "config": {"workload": "batched decode (benchmark configuration 3, metric point): append 1 token/"
                                "seq/layer then gather+dequantize every sequence's full context",
                    "layers": L, "batch": B, "ctx": ctx, "page_tokens": PT, "width": W,
-                   "stored": "fp8 e4m3 + 1 f32 scale/token", "out": "bf16"},
+                   "stored": "fp8 e4m3 + 1 f32 scale/token", "out": "bf16",
+                   "contexts": "uniform in [1024, ctx]" if a.ragged else "all at ctx",
+                   "tokens_per_layer": n_att},
         "decode_step_kv_ms": round(ms_per_step, 4),
-        "tokens_per_s": round(L * n_tok / (ms_per_step * 1e-3), 1),
+        "tokens_per_s": round(L * n_att / (ms_per_step * 1e-3), 1),
         "hbm_peak_frac": round(value * 1e9 / HBM_PEAK, 4),
         "roofline": {"bound": "hbm", "kernel": "kv_gather_paged_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": round(achieved * 1e9 / HBM_PEAK, 4),
@@ -175,7 +189,7 @@ def main():
                      # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
                      # this workload, scaled by a known 1 GiB copy (profiles/); it cannot be
                      # read live, so it is only reported for the shape it was measured on
-                     "traffic": 1821500000 if (B, ctx) == (32, 32768) else None},
+                     "traffic": 1821500000 if (B, ctx) == (32, 32768) and not a.ragged else None},
     }
 
     if not a.no_cpu_baseline:
@@ -427,9 +441,10 @@ def bench_attend(a, torch, hip):
     pos = np.arange(ctx)
     slots_np = np.concatenate([tables_np[s][pos // PT] * PT + pos % PT for s in range(B)]).astype(np.int32)
     tables, slots_all = torch.from_numpy(tables_np.copy()).cuda(), torch.from_numpy(slots_np).cuda()
-    seq_lens_np = np.full(B, ctx, np.int32)
+    seq_lens_np = context_lengths(a, rng)
     seq_lens = torch.from_numpy(seq_lens_np).cuda()
-    new_slots = torch.from_numpy(slots_np.reshape(B, ctx)[:, -1].copy()).cuda()
+    new_slots = torch.from_numpy(slots_np.reshape(B, ctx)[np.arange(B), seq_lens_np - 1].copy()).cuda()
+    n_att = int(seq_lens_np.sum())
     kv_rows = torch.randn(n_tok, W, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
     pools = []
     for _ in range(L):
@@ -460,9 +475,10 @@ def bench_attend(a, torch, hip):
             bracket(torch, stream, events, "attend", lambda: attend(layer, seq_lens, ctx, sh))
 
     ms, per = timed(torch, stream, a.steps, a.warmup, step)
-    attend_bytes = n_tok * REC + B * blocks * 4 + B * H * (W + KVL) * 4   # records, table, q in, clat out
+    table_entries = int((-(-seq_lens_np // PT)).sum())
+    attend_bytes = n_att * REC + table_entries * 4 + B * H * (W + KVL) * 4   # records, table, q in, clat out
     append_bytes = B * (ROW_IN + 4 + REC)
-    flops = 2.0 * n_tok * H * (W + KVL)
+    flops = 2.0 * n_att * H * (W + KVL)
     res = {"metric": "kv_append_attend_GBps", "value": round(L * (attend_bytes + append_bytes) / (ms * 1e-3) / 1e9, 1),
            "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 x f32-accumulate",
@@ -471,9 +487,10 @@ def bench_attend(a, torch, hip):
                                   "fused: append 1 token/seq/layer, then MLA latent attention over every "
                                   "sequence's full context straight from the fp8 pages",
                       "layers": L, "batch": B, "ctx": ctx, "heads": H, "page_tokens": PT, "width": W,
-                      "precise": a.precise},
+                      "precise": a.precise, "contexts": "uniform in [1024, ctx]" if a.ragged else "all at ctx",
+                      "tokens_per_layer": n_att},
            "decode_step_kv_ms": round(ms, 4),
-           "tokens_per_s": round(L * n_tok / (ms * 1e-3), 1),
+           "tokens_per_s": round(L * n_att / (ms * 1e-3), 1),
            "roofline": {"bound": "hbm", "kernel": "mla_attend_paged_kernel",
                         "achieved": round(attend_bytes / (per["attend"] * 1e-3) / 1e9, 1),
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
@@ -535,7 +552,7 @@ def cpu_baseline(pool0, tables_np, seq_lens_np, out, budget_s, hip, tables, seq_
     # full-size parity of one layer: GPU gather of the same pool vs the oracle's bytes
     hip.launch_kv_gather_paged(pool0, tables, seq_lens, cu, out, B, blocks, W, PT, n_pages)
     torch.cuda.synchronize()
-    same = bool(np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1, W),
+    same = bool(np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1, W)[:n_tok],
                                out_host))
     if not same:
         raise SystemExit("bench: GPU gather differs from the CPU oracle at full size")
