@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 KVL, ROPE, PT = 512, 64, 64
 
 
-def run_paged(c, max_rows, rows=None, n_rows=None, precise=2, bad=None, use_lens=True):
+def run_paged(c, max_rows, rows=None, n_rows=None, precise=2, bad=None, use_lens=True, pt=PT):
     n_seqs, H = c["qabs"].shape[:2]
     n_scratch = hip.mla_attend_paged_scratch_floats(n_seqs, H, max_rows)
     partial = dzeros(max(n_scratch, 1) * 4, 0xFF)          # NaN-filled: an unwritten partial shows
@@ -28,7 +28,7 @@ def run_paged(c, max_rows, rows=None, n_rows=None, precise=2, bad=None, use_lens
         dev(c["qabs"]), dev(c["qrope"]), dev(c["pool"]), dev(c["table"]),
         dev(c["lens"]) if use_lens else None, None if rows is None else dev(rows),
         None if n_rows is None else dev(n_rows), n_seqs, H, max_rows, c["table"].shape[1], KVL, ROPE,
-        PT, c["n_pages"], c["scale"], precise, clat, partial if n_scratch else None, bad)
+        pt, c["n_pages"], c["scale"], precise, clat, partial if n_scratch else None, bad)
     return back(clat, np.float32).reshape(n_seqs, H, KVL)
 
 
@@ -69,6 +69,24 @@ def test_dense_split_regimes_and_head_counts(oracle, lens, H):
     want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], c["lens"], None, None,
                                    KVL, ROPE, PT, c["scale"], n_threads=8)
     check(run_paged(c, max(lens)), want, 2, f"lens={lens} H={H}")
+
+
+@pytest.mark.parametrize("pt", [16, 48, 128, 4])
+def test_other_page_sizes(oracle, pt):
+    """Pages of 128 tokens keep the one-lookup-per-tile path; 16 (smaller than a tile), 48 (not
+    a power of two) and 4 take the per-token lookup. Dense and row lists."""
+    lens = [700, 33, 1300]
+    c = paged_case(oracle, lens, H=64, seed=700 + pt, page_tokens=pt)
+    want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], c["lens"], None, None,
+                                   KVL, ROPE, pt, c["scale"], n_threads=3)
+    check(run_paged(c, max(lens), pt=pt), want, 2, f"dense, pages of {pt}")
+    k = 300
+    rng = np.random.default_rng(pt)
+    rows = np.stack([np.sort(rng.choice(n, k, replace=n < k)) for n in lens]).astype(np.uint32)
+    n_rows = np.array([300, 20, 257], np.int32)
+    want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], None, rows, n_rows,
+                                   KVL, ROPE, pt, c["scale"], n_threads=3)
+    check(run_paged(c, k, rows=rows, n_rows=n_rows, use_lens=False, pt=pt), want, 2, f"rows, pages of {pt}")
 
 
 def test_peaked_softmax(oracle):
