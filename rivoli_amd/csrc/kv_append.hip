@@ -145,20 +145,22 @@ __global__ __launch_bounds__(kAppendWaves* kWave) void kv_append_paged_token_ker
     const int token =
         __builtin_amdgcn_readfirstlane((int)(blockIdx.x * kAppendWaves + (threadIdx.x >> 6)));
     if (token >= n_tokens) return;
-    const int slot = slot_mapping[token];
-    if (slot < 0) return;  // padding
-    if ((long long)slot >= n_slots) {
-        if (lane == 0 && bad_slots) atomicAdd(bad_slots, 1u);
-        return;
-    }
     const int n_chunks = width >> 3;
     const u32x4* src = reinterpret_cast<const u32x4*>(rows + (size_t)token * width);
 
+    // the row is requested before the slot is looked at: the two fetches overlap instead of
+    // queueing one memory round trip behind the other (a padding token costs a wasted read)
     u32x4 raw[STEPS];
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
         int c = lane + s * kWave;
         raw[s] = c < n_chunks ? __builtin_nontemporal_load(src + c) : u32x4{0, 0, 0, 0};
+    }
+    const int slot = slot_mapping[token];
+    if (slot < 0) return;  // padding
+    if ((long long)slot >= n_slots) {
+        if (lane == 0 && bad_slots) atomicAdd(bad_slots, 1u);
+        return;
     }
     float amax = 0.0f;
 #pragma unroll
