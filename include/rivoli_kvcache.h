@@ -174,8 +174,10 @@ int rivoli_index_append_paged(const float* k, const int* slot_mapping, unsigned 
  * Tokens whose page id is outside [0, n_pages) are left out of the softmax and counted in
  * *bad_rows when non-null. A sequence with nothing to attend gets zeros.
  * `partial` is caller-owned scratch of rivoli_mla_attend_paged_scratch_floats(n_seqs, H,
- * max_rows) floats (the split-KV partials; may be null when that returns 0). The split plan
- * is a pure function of (n_seqs, H, max_rows): equal calls give bit-equal results.
+ * max_rows) floats (the split-KV partials; may be null when that returns 0). When scratch is
+ * used, the 32-token tiles of the whole batch are dealt evenly to the workgroups from the
+ * device-side lengths, so ragged batches keep the GPU full; the plan depends only on
+ * (n_seqs, H, max_rows) and those lengths: equal calls give bit-equal results.
  * `precise`: 2 carries both q and the softmax weights as bf16 hi + lo (~17 bits) through the
  * matrix cores — the parity mode: results agree with the reference formula far inside its
  * own bar for this kernel (1e-3 of the largest output + 1e-3, crates/engine/tests/common/

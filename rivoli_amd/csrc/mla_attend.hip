@@ -14,8 +14,10 @@
 // Nothing is materialised: a token costs 580 bytes of HBM traffic instead of the 580 + 1152
 // + 1152 of gather-then-attend.
 //
-// Mapping. A 512-thread workgroup (8 waves, two per SIMD) owns one (sequence, split of the
-// attended rows, block of 64 heads). Waves w and w+4 share heads 16(w&3)..+15 and split the
+// Mapping. A 512-thread workgroup (8 waves, two per SIMD) owns a block of 64 heads and a run
+// of 32-token tiles: all of one sequence for small calls; otherwise an equal share of the
+// whole batch's tiles, dealt from the device-side lengths, which may cover parts of several
+// sequences (one partial record per part). Waves w and w+4 share heads 16(w&3)..+15 and split the
 // work on them: each takes half of the 576 contraction dims of the scores and half of the
 // 512 output columns. That halves the query registers and the accumulators a wave carries
 // (the whole kernel fits the 256 registers a wave gets at two waves per SIMD, so every MFMA
@@ -41,9 +43,9 @@
 //     tile exceeds it by more than 2^8 (the f32 accumulators have the range), so rescaling
 //     the accumulators is rare.
 //   * values: O[head][col] += P . V over the wave's 256 columns, B = transposing loads.
-// Splits write unnormalised partials (acc, m, l) that mla_attend_combine_kernel merges in
-// ascending split order; the split plan is a pure function of the call's shape, so equal
-// calls give bit-equal results.
+// Parts write unnormalised partials (acc, m, l) that mla_attend_combine_kernel merges in
+// ascending order; the plan is a pure function of the call's shape and of the lengths, so
+// equal calls give bit-equal results.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
 #include "codec.hpp"
 
@@ -51,6 +53,8 @@ namespace rk {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+template <class T>
+using lds_ptr = __attribute__((address_space(3))) T*;
 
 constexpr int kKvl = 512, kRopeW = 64, kRowW = kKvl + kRopeW;
 constexpr int kAttThreads = 512;
@@ -65,18 +69,23 @@ constexpr int kBufs = 3;                   // LDS tiles in rotation: tile t is s
 constexpr int kXchBytes = 2 * kAttWaves * kWave * 8 * 4;  // partial scores, 8 f32 per lane, two parities
 constexpr int kTableLds = 1024;            // block-table entries staged per workgroup
 constexpr int kAttSmemBytes = kBufs * kKrBytes + 2 * kBufs * kTile * 4 + kXchBytes + kTableLds * 4;
-static_assert(kAttSmemBytes <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
+static_assert(kAttSmemBytes + (1024 + 8 + 8) * 4 <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
 constexpr float kLazyRescale = 8.0f;       // log2 units
 constexpr float kLog2e = 1.4426950408889634f;
 
-// split plan: pure function of the call's shape
+// Work plan. `n_splits` is a pure function of the call's shape; with more than one split the
+// attended rows of ALL sequences, in tiles, are dealt evenly to n_seqs * n_splits work items
+// from the device-side lengths (a work item may cover parts of several sequences, a sequence
+// several work items), so ragged batches keep every CU busy.
 constexpr int kAttTargetGroups = 256;      // one workgroup per CU of a 256-CU part
 constexpr int kAttMinTilesPerSplit = 8;    // below 256 rows a split costs more than it buys
 constexpr int kAttMaxSplits = 64;
+constexpr int kDealMaxSeqs = 1024;         // dealing keeps a prefix sum over the sequences in LDS
 
 struct AttendPlan {
     int n_splits;
-    int split_rows;  // a multiple of kTile
+    int n_items;    // work items per head block when dealing (0 = one workgroup per sequence)
+    int n_records;  // partial records when dealing: a (work item, sequence) pair is item + seq
 };
 
 static inline AttendPlan attend_plan(int n_seqs, int H, int max_rows) {
@@ -87,12 +96,21 @@ static inline AttendPlan attend_plan(int n_seqs, int H, int max_rows) {
     int by_work = tiles / kAttMinTilesPerSplit;
     int n = by_grid < by_work ? by_grid : by_work;
     if (n > kAttMaxSplits) n = kAttMaxSplits;
-    if (n < 1) n = 1;
-    const int tps = (tiles + n - 1) / n;
+    if (n < 1 || n_seqs > kDealMaxSeqs) n = 1;
     AttendPlan p;
-    p.n_splits = (tiles + tps - 1) / tps;
-    p.split_rows = tps * kTile;
+    p.n_splits = n;
+    p.n_items = n > 1 ? n * n_seqs : 0;
+    p.n_records = n > 1 ? p.n_items + n_seqs : 0;
     return p;
+}
+
+// The tiles of work item `item` of `n_items` over `total` tiles: [lo, hi).
+__host__ __device__ __forceinline__ long long deal_lo(long long item, long long n_items, long long total) {
+    return item * total / n_items;
+}
+// The work item that holds tile `t` (the largest item whose first tile is <= t).
+__device__ __forceinline__ int deal_item_of(long long t, long long n_items, long long total) {
+    return (int)(((t + 1) * n_items - 1) / total);
 }
 
 // e4m3 codes -> bf16, exact: four codes (one dword) -> two dwords
@@ -129,10 +147,10 @@ struct AttendArgs {
     int page_shift;               // log2(page_tokens) when that is a power of two, else -1
     size_t page_bytes;
     float qscale;                 // softmax scale * log2(e)
-    int n_splits, split_rows;
+    int n_seqs, n_items;          // n_items > 0: tiles are dealt to that many work items
     float* clat;                  // [n_seqs][H][512]
-    float* part_acc;              // [n_seqs][n_splits][H][512]
-    float* part_ml;               // [n_seqs][n_splits][H][2]
+    float* part_acc;              // [n_records][H][512]
+    float* part_ml;               // [n_records][H][2]
     unsigned int* bad_rows;
 };
 
@@ -150,23 +168,30 @@ enum : int {
                      // tile lies inside ONE page, so a tile costs one (scalar) table lookup
 };
 
+// One part of a workgroup's work: rows [r_begin, r_end) of sequence `seq`, heads 64*hb ..+63.
+// `whole`: the part is the whole sequence, so the normalised result goes straight to clat;
+// otherwise the unnormalised accumulators and (m, l) go to the partial record pa / pml.
 template <int QSPLIT, int PSPLIT, int MODE>
-__global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const AttendArgs a) {
+__device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb, int r_begin,
+                                                      int r_end, bool whole, float* pa, float* pml) {
     constexpr bool SPARSE = MODE == kSparse;
     // operand fragments requested together ahead of the MFMAs that consume them: as many
     // as the register budget of two waves per SIMD (256) leaves room for
     constexpr int kFragBlock = QSPLIT == 2 ? 3 : 9;   // score side, K-steps (2 fragments each)
     constexpr int kValueAhead = QSPLIT == 2 ? 4 : 8;  // value side, fragments
     __shared__ __attribute__((aligned(16))) uint8_t smem[kAttSmemBytes];
-    uint8_t* const kr = smem;  // [kBufs] row-major tiles
+    // Every LDS pointer below is typed as such. Left generic, the pointers become loop-carried
+    // once this body sits in the dealing kernel's loop over parts, the compiler can no longer
+    // prove they are LDS, and its fallback (flat addressing) fails in instruction selection.
+    const lds_ptr<uint8_t> kr = (lds_ptr<uint8_t>)smem;  // [kBufs] row-major tiles
     // per token of a tile, by contraction index: its scale (0 when the token is not there)
     // and a score bias (0, or -inf when it is not there): score = s * scale + bias
-    float* const sc = reinterpret_cast<float*>(kr + kBufs * kKrBytes);  // [kBufs][32]
-    float* const sbias = sc + kBufs * kTile;                             // [kBufs][32]
-    f32x4* const xch = reinterpret_cast<f32x4*>(sbias + kBufs * kTile);  // [2 parities][8 waves][64 lanes][2]
-    int* const tbl = reinterpret_cast<int*>(xch + 2 * kAttWaves * kWave * 2);
+    const lds_ptr<float> sc = (lds_ptr<float>)(kr + kBufs * kKrBytes);    // [kBufs][32]
+    const lds_ptr<float> sbias = sc + kBufs * kTile;                       // [kBufs][32]
+    const lds_ptr<f32x4> xch = (lds_ptr<f32x4>)(sbias + kBufs * kTile);    // [2 parities][8 waves][64 lanes][2]
+    const lds_ptr<int> tbl = (lds_ptr<int>)(xch + 2 * kAttWaves * kWave * 2);
 
-    const int split = blockIdx.x, seq = blockIdx.y, hb = blockIdx.z;
+
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -174,29 +199,6 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
     const int half = wave >> 2; // which half of the contraction dims / of the output columns
     const int g = lane >> 4, n16 = lane & 15;
 
-    int n_att;
-    if (SPARSE) n_att = a.n_rows ? min(a.n_rows[seq], a.k) : a.k;
-    else n_att = min(a.seq_lens[seq], a.k);
-    const int r_begin = split * a.split_rows;
-    const int r_end = min(n_att, r_begin + a.split_rows);
-    float* const pml = a.part_ml ? a.part_ml + (((size_t)seq * a.n_splits + split) * a.H) * 2 : nullptr;
-    if (r_begin >= r_end) {
-        // an empty split tells the combine to skip it; a sequence with nothing to attend
-        // gets zeros, like the reference's `l > 0 ? 1/l : 0`
-        if (pml) {
-            for (int h = tid; h < 64; h += kAttThreads)
-                if (hb * 64 + h < a.H) {
-                    pml[(hb * 64 + h) * 2] = -INFINITY;
-                    pml[(hb * 64 + h) * 2 + 1] = 0.0f;
-                }
-        } else {
-            for (int i = tid; i < 64 * kKvl; i += kAttThreads) {
-                const int h = hb * 64 + i / kKvl;
-                if (h < a.H) a.clat[((size_t)seq * a.H + h) * kKvl + (i % kKvl)] = 0.0f;
-            }
-        }
-        return;
-    }
     const int n_tiles = (r_end - r_begin + kTile - 1) / kTile;
 
     // ---- block-table slice into LDS -----------------------------------------------------
@@ -335,17 +337,17 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         }
     };
     auto stage = [&](int buf) {
-        uint8_t* const krb = kr + buf * kKrBytes;
+        const lds_ptr<uint8_t> krb = kr + buf * kKrBytes;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             uint32_t r[4];
             e4m3x4_to_bf16(raw[i].x, r[0], r[1]);
             e4m3x4_to_bf16(raw[i].y, r[2], r[3]);
-            *reinterpret_cast<u32x4*>(krb + (my_pos0 + i) * kKrRowBytes + 16 * lane) = u32x4{r[0], r[1], r[2], r[3]};
+            *(lds_ptr<u32x4>)(krb + (my_pos0 + i) * kKrRowBytes + 16 * lane) = u32x4{r[0], r[1], r[2], r[3]};
         }
         uint32_t rr0, rr1;
         e4m3x4_to_bf16(raw_rope, rr0, rr1);
-        *reinterpret_cast<u32x2*>(krb + (my_pos0 + (lane >> 4)) * kKrRowBytes + kKvl * 2 + 8 * (lane & 15)) =
+        *(lds_ptr<u32x2>)(krb + (my_pos0 + (lane >> 4)) * kKrRowBytes + kKvl * 2 + 8 * (lane & 15)) =
             u32x2{rr0, rr1};
         if (lane < 4) {
             // a scale that is not a positive number cannot come from the append: such a
@@ -384,13 +386,13 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
     int buf = 0;  // t mod 3
     for (int tile = 0; tile < n_tiles; ++tile) {
         const unsigned int tok_ahead = tile + 4 < n_tiles ? row_token(tile + 4) : 0xffffffffu;
-        f32x4* const xch_mine = xch + (((tile & 1) * kAttWaves + wave) * kWave + lane) * 2;
-        const f32x4* const xch_peer = xch + (((tile & 1) * kAttWaves + (wave ^ 4)) * kWave + lane) * 2;
+        const lds_ptr<f32x4> xch_mine = xch + (((tile & 1) * kAttWaves + wave) * kWave + lane) * 2;
+        const lds_ptr<f32x4> xch_peer = xch + (((tile & 1) * kAttWaves + (wave ^ 4)) * kWave + lane) * 2;
 
         // ---- scores: this wave's half of the dims, S^T[token][head], two 16-token halves --
-        const uint8_t* const krb = kr + buf * kKrBytes + half * (kKStepsHalf * 64);
-        const bf16x8* a0p = reinterpret_cast<const bf16x8*>(krb + n16 * kKrRowBytes + 16 * g);
-        const bf16x8* a1p = reinterpret_cast<const bf16x8*>(krb + (16 + n16) * kKrRowBytes + 16 * g);
+        const lds_ptr<uint8_t> krb = kr + buf * kKrBytes + half * (kKStepsHalf * 64);
+        const lds_ptr<bf16x8> a0p = (lds_ptr<bf16x8>)(krb + n16 * kKrRowBytes + 16 * g);
+        const lds_ptr<bf16x8> a1p = (lds_ptr<bf16x8>)(krb + (16 + n16) * kKrRowBytes + 16 * g);
         f32x4 s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0};
         // The operand fragments of a block of K-steps are all requested before the first MFMA
         // of the block; left alone the compiler keeps two reads in flight and every pair of
@@ -421,13 +423,13 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         // transposing load hands a lane element e of the 8-byte chunk that lane
         // 4e + (n16 >> 2) of its 16-lane row addressed, position n16 & 3 — so lane i
         // addresses token 4g + (i >> 2), columns 16*nt' + 4*(i & 3) .. +3.
-        const uint8_t* const vrow = kr + buf * kKrBytes + (4 * g + (n16 >> 2)) * kKrRowBytes +
-                                    (half * (kKvl / 2) + 4 * (n16 & 3)) * 2;
+        const lds_ptr<uint8_t> vrow = kr + buf * kKrBytes + (4 * g + (n16 >> 2)) * kKrRowBytes +
+                                      (half * (kKvl / 2) + 4 * (n16 & 3)) * 2;
         auto vt_frag = [&](int nt) -> bf16x8 {
             typedef short s16x4 __attribute__((ext_vector_type(4)));
-            typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow + nt * 32));
-            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow + 16 * kKrRowBytes + nt * 32));
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr<s16x4>)(vrow + nt * 32));
+            const s16x4 hi =
+                __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr<s16x4>)(vrow + 16 * kKrRowBytes + nt * 32));
             typedef short s16x8 __attribute__((ext_vector_type(8)));
             const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             return __builtin_bit_cast(bf16x8, both);
@@ -436,10 +438,10 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
 #pragma unroll
         for (int i = 0; i < kValueAhead; ++i) fb[i] = vt_frag(i);
         __builtin_amdgcn_sched_barrier(0);
-        const f32x4 sa = *reinterpret_cast<const f32x4*>(sc + buf * kTile + 8 * g);
-        const f32x4 sb = *reinterpret_cast<const f32x4*>(sc + buf * kTile + 8 * g + 4);
-        const f32x4 ba = *reinterpret_cast<const f32x4*>(sbias + buf * kTile + 8 * g);
-        const f32x4 bb = *reinterpret_cast<const f32x4*>(sbias + buf * kTile + 8 * g + 4);
+        const f32x4 sa = *(lds_ptr<f32x4>)(sc + buf * kTile + 8 * g);
+        const f32x4 sb = *(lds_ptr<f32x4>)(sc + buf * kTile + 8 * g + 4);
+        const f32x4 ba = *(lds_ptr<f32x4>)(sbias + buf * kTile + 8 * g);
+        const f32x4 bb = *(lds_ptr<f32x4>)(sbias + buf * kTile + 8 * g + 4);
         __syncthreads();  // both halves of every score are in LDS
         {
             const f32x4 p0 = xch_peer[0], p1 = xch_peer[1];
@@ -528,8 +530,7 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
     for (int i = 0; i < 4; ++i) l_h[i] = __shfl(l_sum, 4 * g + i, kWave);
     const int head0 = hb * 64 + 16 * hw;
     const int col0 = half * (kKvl / 2) + n16;
-    if (a.part_acc) {
-        float* const pa = a.part_acc + (((size_t)seq * a.n_splits + split) * a.H) * kKvl;
+    if (!whole) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int head = head0 + 4 * g + i;
@@ -556,32 +557,151 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
     }
 }
 
-// clat[seq][head] = sum_s w_s acc_s / sum_s w_s l_s with w_s = 2^(m_s - max m), splits in
-// ascending order (the reference's combine, crates/backend/kernels/attn.hip:235-277, in
-// base 2). A split whose m is -inf holds no rows and its accumulator is never read.
+template <int QSPLIT, int PSPLIT, int MODE>
+__global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const AttendArgs a) {
+    __shared__ int pre[kDealMaxSeqs + 8];  // tiles before each sequence, when dealing
+    __shared__ int wave_total[kAttWaves];
+    constexpr bool SPARSE = MODE == kSparse;
+    const int hb = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    auto attended = [&](int s) -> int {
+        if (SPARSE) return a.n_rows ? max(min(a.n_rows[s], a.k), 0) : a.k;
+        return max(min(a.seq_lens[s], a.k), 0);
+    };
+
+    // ---- which rows of which sequences this workgroup attends ------------------------------
+    // One sequence, all of it, when nothing is dealt. Otherwise the tiles [t_lo, t_hi) of the
+    // batch-wide tile sequence: the workgroup walks the sequences that range touches.
+    long long t_lo = 0, t_hi = 0;
+    int seq = blockIdx.y;
+    if (a.n_items > 0) {
+        // inclusive prefix of tiles per sequence, two sequences per thread
+        const int s0 = 2 * tid, s1 = 2 * tid + 1;
+        const int c0 = s0 < a.n_seqs ? (attended(s0) + kTile - 1) / kTile : 0;
+        const int c1 = s1 < a.n_seqs ? (attended(s1) + kTile - 1) / kTile : 0;
+        int run = c0 + c1;
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const int up = __shfl_up(run, off, kWave);
+            if (lane >= off) run += up;
+        }
+        if (lane == kWave - 1) wave_total[wave] = run;
+        __syncthreads();
+        int before = 0;
+        for (int w = 0; w < wave; ++w) before += wave_total[w];
+        run += before;  // tiles of sequences 0 .. s1
+        if (tid == 0) pre[0] = 0;
+        if (s0 < a.n_seqs) pre[s0 + 1] = run - c1;
+        if (s1 < a.n_seqs) pre[s1 + 1] = run;
+        __syncthreads();
+        const long long total = pre[a.n_seqs];
+        t_lo = deal_lo(blockIdx.x, a.n_items, total);
+        t_hi = deal_lo(blockIdx.x + 1, a.n_items, total);
+        if (t_lo >= t_hi) return;
+        // the sequence holding tile t_lo: the last one that starts at or before it
+        int lo = 0, hi = a.n_seqs;  // pre[lo] <= t_lo < pre[hi]
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (pre[mid] <= t_lo) lo = mid;
+            else hi = mid;
+        }
+        seq = lo;
+    }
+
+  for (;; ++seq) {
+    int r_begin = 0, r_end;
+    bool whole = true;                 // the whole sequence is this part: write clat directly
+    float *pa = a.part_acc, *pml = a.part_ml;  // else this part's partial record
+    if (a.n_items > 0) {
+        if (t_lo >= t_hi || seq >= a.n_seqs) break;
+        const long long p0 = pre[seq], p1 = pre[seq + 1];
+        const long long e = t_hi < p1 ? t_hi : p1;
+        if (e <= t_lo) continue;  // a sequence with nothing to attend
+        r_begin = (int)(t_lo - p0) * kTile;
+        r_end = min(attended(seq), (int)(e - p0) * kTile);
+        whole = t_lo == p0 && e == p1;
+        const size_t rec = (size_t)blockIdx.x + seq;  // unique: both only grow along the walk
+        pa = a.part_acc + rec * a.H * kKvl;
+        pml = a.part_ml + rec * a.H * 2;
+        t_lo = e;
+        __syncthreads();  // the previous part is done with the LDS tiles and the prefix reads above
+    } else {
+        r_end = attended(seq);
+        if (r_end <= 0) {
+            // a sequence with nothing to attend gets zeros, like the reference's `l > 0 ? 1/l : 0`
+            for (int i = tid; i < 64 * kKvl; i += kAttThreads) {
+                const int h = hb * 64 + i / kKvl;
+                if (h < a.H) a.clat[((size_t)seq * a.H + h) * kKvl + (i % kKvl)] = 0.0f;
+            }
+            return;
+        }
+    }
+    attend_part<QSPLIT, PSPLIT, MODE>(a, seq, hb, r_begin, r_end, whole, pa, pml);
+    if (a.n_items == 0) break;
+  }  // parts of this workgroup
+}
+
+// Dealt plan: clat[seq][head] = sum_r w_r acc_r / sum_r w_r l_r over the sequence's partial
+// records, w_r = 2^(m_r - max m), in ascending work-item order (the reference's combine,
+// crates/backend/kernels/attn.hip:235-277, in base 2). A sequence that one work item covered
+// whole was written by it directly; one with nothing to attend gets zeros.
 __global__ __launch_bounds__(128) void mla_attend_combine_kernel(
-    const float* __restrict__ part_acc, const float* __restrict__ part_ml, int H, int n_splits,
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml, const int* __restrict__ seq_lens,
+    const int* __restrict__ n_rows, int sparse, int k, int n_seqs, int n_items, int H,
     float* __restrict__ clat) {
+    __shared__ long long s_sum[3][2];  // per wave: tiles before seq, tiles of seq .. end
     const int head = blockIdx.x, seq = blockIdx.y;
-    const float* ml = part_ml + ((size_t)seq * n_splits * H + head) * 2;
+    // tiles before this sequence, of this sequence, and in all
+    long long before = 0, mine = 0, total = 0;
+    for (int s = threadIdx.x; s < n_seqs; s += 128) {
+        int n = sparse ? (n_rows ? min(n_rows[s], k) : k) : min(seq_lens[s], k);
+        n = max(n, 0);
+        const long long t = (n + kTile - 1) / kTile;
+        total += t;
+        if (s < seq) before += t;
+        if (s == seq) mine = t;
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        before += __shfl_xor(before, off, kWave);
+        mine += __shfl_xor(mine, off, kWave);
+        total += __shfl_xor(total, off, kWave);
+    }
+    if ((threadIdx.x & 63) == 0) {
+        s_sum[0][threadIdx.x >> 6] = before;
+        s_sum[1][threadIdx.x >> 6] = mine;
+        s_sum[2][threadIdx.x >> 6] = total;
+    }
+    __syncthreads();
+    before = s_sum[0][0] + s_sum[0][1], mine = s_sum[1][0] + s_sum[1][1], total = s_sum[2][0] + s_sum[2][1];
+    float4* const dst = reinterpret_cast<float4*>(clat + ((size_t)seq * H + head) * kKvl) + threadIdx.x;
+    if (mine == 0) {
+        *dst = float4{0, 0, 0, 0};
+        return;
+    }
+    const int first = deal_item_of(before, n_items, total);
+    const int last = deal_item_of(before + mine - 1, n_items, total);
+    if (first == last) return;  // one work item had the whole sequence and wrote it
     float m_g = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) m_g = fmaxf(m_g, ml[(size_t)s * H * 2]);
+    for (int it = first; it <= last; ++it)
+        m_g = fmaxf(m_g, part_ml[((size_t)(it + seq) * H + head) * 2]);
     float4 sum = {0, 0, 0, 0};
     float l_g = 0.0f;
     if (m_g != -INFINITY) {
-        for (int s = 0; s < n_splits; ++s) {
-            const float m_s = ml[(size_t)s * H * 2];
-            if (m_s == -INFINITY) continue;
-            const float w = exp2f(m_s - m_g);
-            l_g += ml[(size_t)s * H * 2 + 1] * w;
-            const float4 v = reinterpret_cast<const float4*>(
-                part_acc + (((size_t)seq * n_splits + s) * H + head) * kKvl)[threadIdx.x];
+        for (int it = first; it <= last; ++it) {
+            const size_t rec = (size_t)it + seq;
+            const float m_r = part_ml[(rec * H + head) * 2];
+            if (m_r == -INFINITY) continue;
+            const float w = exp2f(m_r - m_g);
+            l_g += part_ml[(rec * H + head) * 2 + 1] * w;
+            const float4 v = reinterpret_cast<const float4*>(part_acc + (rec * H + head) * kKvl)[threadIdx.x];
             sum.x += v.x * w, sum.y += v.y * w, sum.z += v.z * w, sum.w += v.w * w;
         }
     }
     const float inv = l_g > 0.0f ? 1.0f / l_g : 0.0f;
-    reinterpret_cast<float4*>(clat + ((size_t)seq * H + head) * kKvl)[threadIdx.x] =
-        float4{sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv};
+    *dst = float4{sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv};
 }
 
 }  // namespace rk
@@ -589,8 +709,7 @@ __global__ __launch_bounds__(128) void mla_attend_combine_kernel(
 extern "C" size_t rivoli_mla_attend_paged_scratch_floats(int n_seqs, int H, int max_rows) {
     if (n_seqs <= 0 || H <= 0 || max_rows <= 0) return 0;
     const rk::AttendPlan p = rk::attend_plan(n_seqs, H, max_rows);
-    if (p.n_splits <= 1) return 0;
-    return (size_t)n_seqs * p.n_splits * H * (rk::kKvl + 2);
+    return (size_t)p.n_records * H * (rk::kKvl + 2);
 }
 
 extern "C" int rivoli_mla_attend_paged(const float* qabs, const float* qrope,
@@ -617,11 +736,12 @@ extern "C" int rivoli_mla_attend_paged(const float* qabs, const float* qrope,
     a.page_shift = (page_tokens & (page_tokens - 1)) == 0 ? __builtin_ctz((unsigned)page_tokens) : -1;
     a.page_bytes = (size_t)page_tokens * kRowW + (size_t)page_tokens * 4;
     a.qscale = scale * kLog2e;
-    a.n_splits = plan.n_splits, a.split_rows = plan.split_rows;
+    a.n_seqs = n_seqs, a.n_items = plan.n_items;
     a.clat = clat, a.bad_rows = bad_rows;
-    a.part_acc = plan.n_splits > 1 ? partial : nullptr;
-    a.part_ml = plan.n_splits > 1 ? partial + (size_t)n_seqs * plan.n_splits * H * kKvl : nullptr;
-    const dim3 grid((unsigned)plan.n_splits, (unsigned)n_seqs, (unsigned)((H + 63) / 64));
+    a.part_acc = plan.n_items ? partial : nullptr;
+    a.part_ml = plan.n_items ? partial + (size_t)plan.n_records * H * kKvl : nullptr;
+    const dim3 grid(plan.n_items ? (unsigned)plan.n_items : 1u, plan.n_items ? 1u : (unsigned)n_seqs,
+                    (unsigned)((H + 63) / 64));
     (void)hipGetLastError();
     hipStream_t st = (hipStream_t)stream;
 #define RK_ATTEND_LAUNCH(Q, P, M) \
@@ -640,6 +760,7 @@ extern "C" int rivoli_mla_attend_paged(const float* qabs, const float* qrope,
     int rc = launch_status();
     if (rc != 0 || plan.n_splits <= 1) return rc;
     hipLaunchKernelGGL(mla_attend_combine_kernel, dim3((unsigned)H, (unsigned)n_seqs), dim3(128), 0, st,
-                       a.part_acc, a.part_ml, H, plan.n_splits, clat);
+                       a.part_acc, a.part_ml, seq_lens, n_rows, rows ? 1 : 0, max_rows, n_seqs, plan.n_items, H,
+                       clat);
     return launch_status();
 }

@@ -71,6 +71,37 @@ def test_dense_split_regimes_and_head_counts(oracle, lens, H):
     check(run_paged(c, max(lens)), want, 2, f"lens={lens} H={H}")
 
 
+def test_tiles_dealt_across_many_ragged_sequences(oracle):
+    """With more than one split the tiles of the whole batch are dealt evenly to the workgroups
+    from the device-side lengths: a workgroup may walk several sequences (and skip empty
+    ones), a sequence may be shared by several workgroups or owned whole by one."""
+    rng = np.random.default_rng(77)
+    lens = [int(x) for x in rng.integers(0, 2500, size=37)]
+    lens[3], lens[4], lens[5], lens[20], lens[21] = 0, 0, 32, 1, 4096          # a run of empties, tiny ones, a long one
+    lens[36] = 0                                                                # the batch ends on an empty sequence
+    c = paged_case(oracle, lens, H=64, seed=800)
+    assert hip.mla_attend_paged_scratch_floats(len(lens), 64, max(lens)) > 0
+    want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], c["lens"], None, None,
+                                   KVL, ROPE, PT, c["scale"], n_threads=8)
+    got = run_paged(c, max(lens))
+    check(got, want, 2, "dealt, ragged")
+    for s_, n in enumerate(lens):
+        if n == 0:
+            assert not got[s_].any()
+    # the same batch a second time gives the same bits
+    assert np.array_equal(got.view(np.uint32), run_paged(c, max(lens)).view(np.uint32))
+
+
+def test_more_sequences_than_the_dealing_plan_holds(oracle):
+    """Past 1024 sequences the plan goes back to one workgroup per sequence."""
+    lens = [int(x) for x in np.random.default_rng(5).integers(0, 70, size=1100)]
+    c = paged_case(oracle, lens, H=16, seed=900, outlier_frac=0.0)
+    assert hip.mla_attend_paged_scratch_floats(len(lens), 16, 8192) == 0
+    want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], c["lens"], None, None,
+                                   KVL, ROPE, PT, c["scale"], n_threads=8)
+    check(run_paged(c, 8192), want, 2, "1100 sequences", mild=True)
+
+
 @pytest.mark.parametrize("pt", [16, 48, 128, 4])
 def test_other_page_sizes(oracle, pt):
     """Pages of 128 tokens keep the one-lookup-per-tile path; 16 (smaller than a tile), 48 (not
@@ -169,7 +200,7 @@ def test_guards():
                                     b, None)
     assert e.value.code == 1001
     assert hip.mla_attend_paged_scratch_floats(1, 64, 64) == 0
-    assert hip.mla_attend_paged_scratch_floats(32, 64, 32768) == 32 * 8 * 64 * 514
+    assert hip.mla_attend_paged_scratch_floats(32, 64, 32768) == (32 * 8 + 32) * 64 * 514
 
 
 # ---- the reference's single-token launcher over its linear slabs --------------------------
