@@ -6,7 +6,9 @@
  * before anything is launched (1001 non-positive / null argument, 1002 size bound,
  * 1004 divisibility), or -(int)hipError_t from the launch. Launch-only: no allocation, no
  * copy, no synchronisation. Every pointer is a device pointer owned by the caller and must
- * stay live until `stream` (nullptr = the null stream) has drained. Dims cross as int
+ * stay live until `stream` (nullptr = the null stream) has drained. The paged entry points
+ * move 16 bytes per lane: their row, pool, output, query and scratch buffers must be 16-byte
+ * aligned (guard 1004 otherwise). Dims cross as int
  * (the Rust side narrows usize as i32); all byte offsets are formed in 64 bits inside.
  *
  * Paged cache layout ("page"): page_tokens rows of `width` e4m3 codes, then page_tokens f32

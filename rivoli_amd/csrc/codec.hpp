@@ -159,6 +159,10 @@ __device__ __forceinline__ unsigned long long wave_xor(unsigned long long v) {
     return v;
 }
 
+// The vector loads and stores of these kernels are 16 bytes wide: a launcher refuses (1004) a
+// buffer that is not 16-byte aligned rather than let the kernel fault on it.
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
 // Launcher epilogue shared by every entry point: 0 or -(hipError_t).
 inline int launch_status() {
     hipError_t e = hipGetLastError();

@@ -252,7 +252,7 @@ extern "C" int rivoli_kv_append_paged(const unsigned short* rows, const int* slo
     if (!rows || !slot_mapping || !pool) return 1001;
     if (n_tokens <= 0 || width <= 0 || page_tokens <= 0 || n_pages <= 0) return 1001;
     if (width > 1024) return 1002;
-    if ((width % 16) != 0 || (page_tokens % 4) != 0) return 1004;
+    if ((width % 16) != 0 || (page_tokens % 4) != 0 || !aligned16(rows) || !aligned16(pool)) return 1004;
     const size_t page_bytes = rivoli_kv_page_bytes(page_tokens, width);
     const long long n_slots = (long long)n_pages * page_tokens;
     (void)hipGetLastError();

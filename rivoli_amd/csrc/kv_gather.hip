@@ -188,7 +188,7 @@ extern "C" int rivoli_kv_gather_paged(const unsigned char* pool, const int* bloc
     if (n_seqs <= 0 || max_blocks_per_seq <= 0 || width <= 0 || page_tokens <= 0 || n_pages <= 0)
         return 1001;
     if (n_seqs > 65535) return 1002;
-    if (!shape_ok(width, page_tokens)) return 1004;
+    if (!shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
     const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
     (void)hipGetLastError();
     if (width == 576 && page_tokens == 64) {
@@ -224,7 +224,7 @@ extern "C" int rivoli_kv_gather_rows_paged(const unsigned char* pool, const int*
         n_pages <= 0)
         return 1001;
     if (n_queries > 65535) return 1002;
-    if (!shape_ok(width, page_tokens)) return 1004;
+    if (!shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
     const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
     dim3 grid((unsigned)((k + kRowsPerGroup - 1) / kRowsPerGroup), (unsigned)n_queries);
     (void)hipGetLastError();

@@ -727,6 +727,8 @@ extern "C" int rivoli_mla_attend_paged(const float* qabs, const float* qrope,
         return 1001;
     if (n_seqs > 65535 || H > 64 * 65535) return 1002;
     if (kvl != kKvl || rope != kRopeW) return 1004;  // the page row is 512 latent + 64 rope codes
+    if (!aligned16(qabs) || !aligned16(qrope) || !aligned16(pool) || !aligned16(clat) || !aligned16(partial))
+        return 1004;
     const AttendPlan plan = attend_plan(n_seqs, H, max_rows);
     if (plan.n_splits > 1 && !partial) return 1001;
     AttendArgs a;

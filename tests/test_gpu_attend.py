@@ -195,6 +195,9 @@ def test_guards():
         with pytest.raises(hip.LaunchError) as e:
             call(**kw)
         assert e.value.code == code, kw
+    with pytest.raises(hip.LaunchError) as e:          # a query buffer that is not 16-byte aligned
+        hip.launch_mla_attend_paged(b[4:], b, b, b, b, None, None, 1, 64, 64, 1, 512, 64, 64, 1, 1.0, 1, b, b)
+    assert e.value.code == 1004
     with pytest.raises(hip.LaunchError) as e:          # needs scratch, none given
         hip.launch_mla_attend_paged(b, b, b, b, b, None, None, 1, 64, 8192, 128, 512, 64, 64, 128, 1.0, 1,
                                     b, None)
