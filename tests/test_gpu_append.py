@@ -152,6 +152,33 @@ def test_append_rounding_ties_saturation_and_special_rows(oracle):
     assert np.count_nonzero(codes0 & 0x7F) > W // 2
 
 
+def test_append_every_amax_mantissa_against_every_value_below_it(oracle):
+    """The quotient x / scale depends only on the two mantissas and the exponent gap (powers of
+    two are exact), so every bf16 amax mantissa against every bf16 magnitude in the 18 binades
+    below it, both signs, is every quotient the quantizer can meet away from the ends of the
+    f32 range; a few exponents near those ends cover the rest."""
+    amax_bits, span = [], 18 * 128
+    for e in (-118, -60, -9, 0, 8, 61, 120):
+        amax_bits += [((e + 127) << 7) | m for m in range(128)]
+    per = W - 1
+    n_rows_each = -(-(2 * (span + 1)) // per)
+    rows = np.zeros((len(amax_bits) * n_rows_each, W), np.uint16)
+    for i, ab in enumerate(amax_bits):
+        mags = np.arange(max(ab - span, 0), ab + 1, dtype=np.uint16)
+        vals = np.concatenate([mags, mags | 0x8000])
+        block = np.zeros(n_rows_each * per, np.uint16)
+        block[: vals.size] = vals
+        rows[i * n_rows_each:(i + 1) * n_rows_each, 0] = ab
+        rows[i * n_rows_each:(i + 1) * n_rows_each, 1:] = block.reshape(n_rows_each, per)
+    n_pages = -(-rows.shape[0] // PT)
+    slots = np.arange(rows.shape[0], dtype=np.int32)
+    got, want, bad, _ = paged_append_both(oracle, rows, slots, n_pages)
+    assert bad == 0
+    mism = np.flatnonzero(got != want)
+    assert mism.size == 0, [(int(j), hex(got[j]), hex(want[j])) for j in mism[:8]]
+    assert np.unique(want[: PT * W]).size > 200            # nearly every code is produced
+
+
 def test_append_padding_bad_slots_and_guards(oracle):
     rows = make_rows_bf16(6, W, seed=8)
     slots = np.array([5, -1, 128, 2 ** 31 - 1, 64, -7], np.int32)

@@ -59,11 +59,11 @@ def test_dense_ragged_batch(oracle, precise):
 
 
 @pytest.mark.parametrize("lens,H", [([4608], 64), ([5000, 704, 2049], 64), ([1500, 130], 20), ([900], 128),
-                                    ([700, 650], 80)])
+                                    ([700, 650], 80), ([333, 1, 2100], 1), ([40, 777], 4)])
 def test_dense_split_regimes_and_head_counts(oracle, lens, H):
     """Long contexts take several splits and the combine (the reference's own long-context
     shapes, crates/engine/tests/kernel_attend.rs:287-297); H = 20 leaves part of a head block
-    idle, H = 128 and 80 take two head blocks."""
+    idle, H = 128 and 80 take two head blocks, H = 1 and 4 fill a fraction of one matrix tile."""
     c = paged_case(oracle, lens, H=H, seed=200 + H)
     assert hip.mla_attend_paged_scratch_floats(len(lens), H, max(lens)) > 0
     want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], c["lens"], None, None,

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from rivoli_amd import hip
-from tests.gpu_util import back, dev, dzeros
+from tests.gpu_util import back, dev, dzeros, torch_cuda
 from tests.test_oracle_codecs import all_e4m3_values
 
 pytestmark = pytest.mark.gpu
@@ -36,6 +36,23 @@ def test_e4m3_encode_matches_oracle(oracle):
     # the probe really contains the subnormal ties that separate half-away from nearest-even
     q = np.float32(2.0 ** -10)
     assert np.isin(np.array([1, 5, 9, 13], np.float32) * q, x).all()
+
+
+@pytest.mark.parametrize("quarter", range(4))
+def test_e4m3_encode_every_f32_bit_pattern(oracle, quarter):
+    """All 2^32 inputs, a quarter per case, in pieces of 2^26 generated on the device."""
+    torch = torch_cuda()
+    piece = 1 << 26
+    out = dzeros(piece)
+    for k in range(quarter * 16, quarter * 16 + 16):
+        base = k * piece
+        wide = torch.arange(base, base + piece, dtype=torch.int64, device="cuda")
+        bits = torch.where(wide >= 1 << 31, wide - (1 << 32), wide).to(torch.int32)
+        hip.launch_codec_e4m3_encode(bits.view(torch.uint8), out, piece)
+        host = (np.arange(piece, dtype=np.uint32) + np.uint32(base)).view(np.float32)
+        got, want = back(out), oracle.f32_to_e4m3(host)
+        bad = np.flatnonzero(got != want)
+        assert bad.size == 0, [(hex(base + int(i)), hex(got[i]), hex(want[i])) for i in bad[:8]]
 
 
 def test_e4m3_dequant_matches_oracle_for_every_code(oracle):
