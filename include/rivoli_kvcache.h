@@ -196,6 +196,34 @@ int rivoli_mla_attend_paged(const float* qabs, const float* qrope, const unsigne
                             int page_tokens, int n_pages, float scale, int precise, float* clat,
                             float* partial, unsigned int* bad_rows, void* stream);
 
+/* ---- the second cache format: f32 rows holding simulated-fp8 values, a window ring followed
+ * by compressed blocks, and a scored selection of those blocks ---- */
+
+/* Replaces crates/backend/kernels/mla.hip:527-548 (launch_act_quant_f8_prefix,
+ * crates/engine/src/v4/attn.rs:288): the fused quantize-then-dequantize of dims [0, n) of every
+ * row in blocks of `block`: amax = max(1e-4, |x|) over the block, s = 2^ceil(log2(amax/448))
+ * (actquant.hpp:69-81), dst = e4m3_to_f32(rne_e4m3(clamp(src / s, +-448))) * s, nearest even
+ * everywhere (formats.hpp:245-264). Dims [n, row_stride) are not touched. src == dst is the
+ * in-place form. Guards as the reference's: 1001 non-positive or row_stride < n (also null
+ * pointers); 1002 src != dst with n != row_stride (dst rows would be part stale), or more than
+ * 2^32 - 1 elements; 1004 n not a multiple of block. Blocks of 16, 32, 64, 128 or 256 with
+ * 16-byte-aligned rows take the coalesced kernel; anything else a thread-per-block kernel. */
+int rivoli_act_quant_f8_prefix(const float* src, float* dst, int rows, int row_stride, int n,
+                               int block, void* stream);
+
+/* The scored block selection that crates/engine/src/v4/select.rs:153-188 (scored_rows) performs
+ * on the host after a device-to-host copy of the scores, as one launch on the device. scores is
+ * [rows][n_comp] f32 (what launch_index_score_blocks wrote; illegal slots need not be masked).
+ * For query row t: limit = prefill ? min((t + 1) / ratio, n_comp) : n_comp, and the
+ * k = min(index_topk, n_comp) best of the first `limit` scores under f32 total order
+ * (descending; ties to the LOWER block index) are written ascending as block + offset to
+ * out[t*k ..], then -1 out to k columns. Where limit <= k the row is offset .. offset+limit-1
+ * whatever the scores are. The reference takes one query row at decode; here prefill == 0 with
+ * rows > 1 is a batch of decode rows, each over all n_comp blocks.
+ * Guards: 1001 null / non-positive / negative offset; 1002 offset + n_comp overflows int. */
+int rivoli_index_select_blocks(const float* scores, int rows, int n_comp, int ratio,
+                               int index_topk, int prefill, int offset, int* out, void* stream);
+
 /* Element codecs as launchers (what formats.hpp:42-57,99-106 and fwd.hip:20-45 are to the
  * reference's kernels), for census tests of the device codecs on arbitrary inputs:
  *   e4m3_encode: out[i] = f32_to_e4m3(x[i])            (rule of crates/core/src/num.rs:128-152)

@@ -33,7 +33,46 @@ def _c(a, dtype) -> np.ndarray:
     return a
 
 
-class Oracle:
+class _V4Mixin:
+    """The second cache format (v4cache_oracle.h)."""
+
+    def e4m3_encode_rne(self, x) -> np.ndarray:
+        x = _c(x, np.float32)
+        out = np.empty(x.shape, np.uint8)
+        self.lib.ro_e4m3_encode_rne_n(_ptr(x, C.c_float), _ptr(out, C.c_uint8), x.size)
+        return out
+
+    def fast_round_scale(self, amax, max_inv=np.float32(1.0) / np.float32(448.0)) -> np.float32:
+        return np.float32(self.lib.ro_fast_round_scale(float(np.float32(amax)), float(np.float32(max_inv))))
+
+    def act_quant_f8_prefix(self, x, n: int, block: int, inplace: bool = True):
+        """x is [rows, row_stride] f32. Returns (guard code, result); the input is not modified.
+        With inplace=False the source and destination are distinct buffers (n must then cover
+        the row) and the destination starts as NaN-free garbage (0x5a bytes)."""
+        x = _c(x, np.float32)
+        rows, row_stride = x.shape
+        if inplace:
+            dst = x.copy()
+            src = dst
+        else:
+            src, dst = x, np.frombuffer(b"\x5a" * (x.size * 4), np.float32).reshape(x.shape).copy()
+        code = int(self.lib.ro_act_quant_f8_prefix(_ptr(src, C.c_float), _ptr(dst, C.c_float), rows,
+                                                   row_stride, n, block))
+        return code, dst
+
+    def v4_scored_rows(self, scores, ratio: int, index_topk: int, prefill: bool, offset: int):
+        """scores is [rows, n_comp] f32. Returns int32 [rows, min(index_topk, n_comp)]."""
+        scores = _c(scores, np.float32)
+        rows, n_comp = scores.shape
+        k = min(index_topk, n_comp)
+        out = np.empty((rows, k), np.int32)
+        got = int(self.lib.ro_v4_scored_rows(_ptr(scores, C.c_float), rows, n_comp, ratio, index_topk,
+                                             1 if prefill else 0, offset, _ptr(out, C.c_int32)))
+        assert got == k, got
+        return out
+
+
+class Oracle(_V4Mixin):
     def __init__(self, path: str = LIB_PATH):
         if not os.path.exists(path):
             build(with_ref=False)
@@ -73,6 +112,10 @@ class Oracle:
             "ro_fnv1a": (C.c_uint64, [u8p, C.c_size_t]),
             "ro_splitmix_finalize": (C.c_uint64, [C.c_uint64]),
             "ro_xor_fold": (C.c_uint64, [u32p, C.c_size_t, C.c_uint64, C.c_size_t]),
+            "ro_e4m3_encode_rne_n": (None, [f32p, u8p, C.c_size_t]),
+            "ro_fast_round_scale": (C.c_float, [C.c_float, C.c_float]),
+            "ro_act_quant_f8_prefix": (C.c_int, [f32p, f32p] + [C.c_int] * 4),
+            "ro_v4_scored_rows": (C.c_int, [f32p] + [C.c_int] * 6 + [i32p]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(lib, name)

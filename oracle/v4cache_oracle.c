@@ -1,0 +1,146 @@
+/* CPU oracle for the second cache format — TEST INFRASTRUCTURE, NOT PRODUCT.
+ * See v4cache_oracle.h for scope and for what pins each function.
+ * Build: with kvcache_oracle.c into libkvoracle.so (oracle/Makefile). */
+#include "v4cache_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "kvcache_oracle.h"
+
+static inline uint32_t bits_of(float x) {
+    uint32_t b;
+    memcpy(&b, &x, sizeof b);
+    return b;
+}
+static inline float float_of(uint32_t b) {
+    float x;
+    memcpy(&x, &b, sizeof x);
+    return x;
+}
+
+/* numerics.rs:92-94: past the half always up, at the half only off an odd mantissa. */
+static inline int rne_up_f(float rem, float half, int odd) { return rem > half || (rem == half && odd); }
+static inline int rne_up_u(uint32_t rem, uint32_t half, int odd) {
+    return rem > half || (rem == half && odd);
+}
+
+uint8_t ro_e4m3_encode_rne(float x) {
+    if (isnan(x)) return 0x7f;
+    uint8_t sign = signbit(x) ? 0x80 : 0x00;
+    float a = fabsf(x);
+    if (a >= 464.0f) return sign | 0x7e;
+    if (a <= 1.0f / 1024.0f) return sign;
+    uint32_t bits = bits_of(a);
+    int e = (int)((bits >> 23) & 0xff) - 127;
+    if (e < -6) {
+        /* numerics.rs:104-114: value = m * 2^-9; m == 8 promotes to the smallest normal */
+        float scaled = a * 512.0f;
+        float m = floorf(scaled);
+        float rem = scaled - m;
+        if (rne_up_f(rem, 0.5f, ((uint32_t)m & 1u) != 0)) m += 1.0f;
+        uint32_t mi = (uint32_t)m;
+        return mi >= 8 ? (uint8_t)(sign | 0x08) : (uint8_t)(sign | mi);
+    }
+    /* numerics.rs:118-135 */
+    uint32_t mant = bits & 0x007fffffu;
+    uint32_t m3 = mant >> 20;
+    uint32_t rem = mant & 0x000fffffu;
+    if (rne_up_u(rem, 0x00080000u, (m3 & 1u) != 0)) m3 += 1;
+    int exp = e + 7;
+    if (m3 == 8) {
+        m3 = 0;
+        exp += 1;
+    }
+    if (exp >= 15 && m3 >= 7) return sign | 0x7e;
+    return (uint8_t)(sign | (uint8_t)(exp << 3) | (uint8_t)m3);
+}
+
+void ro_e4m3_encode_rne_n(const float* x, uint8_t* out, size_t n) {
+    for (size_t i = 0; i < n; ++i) out[i] = ro_e4m3_encode_rne(x[i]);
+}
+
+float ro_fast_round_scale(float amax, float max_inv) {
+    uint32_t b = bits_of(amax * max_inv);
+    int e = (int)((b >> 23) & 0xff) - 127 + ((b & 0x007fffffu) ? 1 : 0);
+    return float_of((uint32_t)(e + 127) << 23);
+}
+
+int ro_act_quant_f8_prefix(const float* src, float* dst, int rows, int row_stride, int n,
+                           int block) {
+    if (rows <= 0 || n <= 0 || block <= 0 || row_stride < n) return 1001;
+    if (src != dst && n != row_stride) return 1002;
+    if (n % block) return 1004;
+    const float fp8_max = 448.0f, max_inv = 1.0f / 448.0f;
+    for (int r = 0; r < rows; ++r) {
+        for (int b = 0; b < n / block; ++b) {
+            const float* seg = src + (size_t)r * row_stride + (size_t)b * block;
+            float* out = dst + (size_t)r * row_stride + (size_t)b * block;
+            float amax = 1e-4f;
+            /* f32::max keeps the other operand when one is a NaN, quiet or signaling; libm's
+             * fmaxf turns a signaling one into a NaN result, so the compare is spelled out */
+            for (int i = 0; i < block; ++i) {
+                float a = fabsf(seg[i]);
+                if (a > amax) amax = a;
+            }
+            float s = ro_fast_round_scale(amax, max_inv);
+            for (int i = 0; i < block; ++i) {
+                float q = seg[i] / s;
+                /* comparisons, so that a NaN stays a NaN (actquant.hpp:90-99) */
+                q = q < -fp8_max ? -fp8_max : (q > fp8_max ? fp8_max : q);
+                out[i] = ro_e4m3_to_f32(ro_e4m3_encode_rne(q)) * s;
+            }
+        }
+    }
+    return 0;
+}
+
+/* f32::total_cmp's key: the bits as a sign-magnitude integer made two's complement. */
+static inline int32_t total_key(float v) {
+    int32_t b = (int32_t)bits_of(v);
+    return b ^ (int32_t)(((uint32_t)(b >> 31)) >> 1);
+}
+
+typedef struct {
+    int32_t key;
+    int32_t idx;
+} scored_t;
+
+static int by_score_then_index(const void* pa, const void* pb) {
+    const scored_t* a = (const scored_t*)pa;
+    const scored_t* b = (const scored_t*)pb;
+    if (a->key != b->key) return a->key > b->key ? -1 : 1; /* descending score */
+    return a->idx < b->idx ? -1 : (a->idx > b->idx ? 1 : 0);
+}
+static int by_index(const void* pa, const void* pb) {
+    int32_t a = ((const scored_t*)pa)->idx, b = ((const scored_t*)pb)->idx;
+    return a < b ? -1 : (a > b ? 1 : 0);
+}
+
+int ro_v4_scored_rows(const float* scores, int rows, int n_comp, int ratio, int index_topk,
+                      int prefill, int offset, int32_t* out) {
+    if (!scores || !out || rows <= 0 || n_comp <= 0 || ratio <= 0 || index_topk <= 0) return -1;
+    const int k = index_topk < n_comp ? index_topk : n_comp;
+    scored_t* sel = (scored_t*)malloc((size_t)n_comp * sizeof(scored_t));
+    for (int t = 0; t < rows; ++t) {
+        const float* row = scores + (size_t)t * n_comp;
+        int limit = n_comp;
+        if (prefill) {
+            limit = (t + 1) / ratio;
+            if (limit > n_comp) limit = n_comp;
+        }
+        for (int c = 0; c < limit; ++c) {
+            sel[c].key = total_key(row[c]);
+            sel[c].idx = c;
+        }
+        qsort(sel, (size_t)limit, sizeof(scored_t), by_score_then_index);
+        int kept = limit < k ? limit : k;
+        qsort(sel, (size_t)kept, sizeof(scored_t), by_index);
+        int32_t* o = out + (size_t)t * k;
+        for (int j = 0; j < kept; ++j) o[j] = sel[j].idx + offset;
+        for (int j = kept; j < k; ++j) o[j] = -1;
+    }
+    free(sel);
+    return k;
+}

@@ -1,0 +1,68 @@
+/* CPU oracle for the second cache format (window ring + compressed blocks of simulated-fp8
+ * f32 rows) — TEST INFRASTRUCTURE, NOT PRODUCT. Plain-C restatement of the reference's CPU
+ * arithmetic; only tests, the smoke check and the benchmark's CPU-baseline leg may call it.
+ * Paths are relative to the reference tree.
+ *
+ * Pinning status (tests/test_oracle_v4.py):
+ *   ro_e4m3_encode_rne    nearest-value enumeration over the 127 finite magnitudes with ties to
+ *                         the even code (the technique of
+ *                         crates/oracles/tests/v4_oracle_codecs.rs:27-57,103-145) on every
+ *                         code, every midpoint, their neighbours and random points; saturation
+ *                         and NaN KATs of the same test; agreement with ro_f32_to_e4m3
+ *                         everywhere except exact subnormal ties, where the two rules are
+ *                         stated to differ (crates/oracles/src/v4oracle/numerics.rs:60-67)
+ *   ro_fast_round_scale   against ceil(log2) computed exactly (frexp) on powers of two, their
+ *                         neighbours and random values; result is a power of two >= amax/448
+ *                         and < 2 * that
+ *   ro_act_quant_f8_prefix  the reference's own tie fixture restated
+ *                         (crates/engine/tests/kernel_v4_quant.rs:283-343: a 448 pins the
+ *                         scale, multiples and half multiples of 2^-9 in both signs; the data
+ *                         separates RNE from half-away); idempotence; every output is an e4m3
+ *                         value times the block's power-of-two scale; the launcher's guards
+ *                         (crates/backend/kernels/mla.hip:527-541)
+ *   ro_v4_scored_rows     the three reference KATs (crates/engine/src/v4/select.rs:645-747:
+ *                         below the cap the row is offset+0..limit-1 then -1; three-way tie
+ *                         keeps the lower indices; a prefill row cannot take a block that
+ *                         closed after it) and a brute-force sort under f32 total order
+ */
+#ifndef RIVOLI_V4CACHE_ORACLE_H
+#define RIVOLI_V4CACHE_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* crates/oracles/src/v4oracle/numerics.rs:68-139 (device twin f2e4m3_rne,
+ * crates/backend/kernels/formats.hpp:245-264): nearest even everywhere, subnormals included;
+ * |x| >= 464 saturates to 0x7e; |x| <= 2^-10 is signed zero; NaN -> 0x7f. */
+uint8_t ro_e4m3_encode_rne(float x);
+void ro_e4m3_encode_rne_n(const float* x, uint8_t* out, size_t n);
+
+/* numerics.rs:202-218 (device: crates/backend/kernels/actquant.hpp:69-81): 2^ceil(log2(amax *
+ * max_inv)) by exponent-field surgery. */
+float ro_fast_round_scale(float amax, float max_inv);
+
+/* crates/backend/kernels/mla.hip:319-338 and its launcher :527-548 (CPU statement:
+ * numerics.rs:245-285 act_quant_inplace with round_scale = true). For every row r < rows and
+ * block b < n / block: amax = max(1e-4, |src[r*row_stride + b*block + i]|), s =
+ * fast_round_scale(amax, 1/448), dst[..] = decode(encode_rne(clamp(src[..] / s, +-448))) * s.
+ * Dims [n, row_stride) of a row are not touched. Returns the launcher's guard code (0, 1001,
+ * 1002, 1004) and does nothing when it is non-zero. src == dst is the in-place form. */
+int ro_act_quant_f8_prefix(const float* src, float* dst, int rows, int row_stride, int n,
+                           int block);
+
+/* crates/engine/src/v4/select.rs:153-188 scored_rows: for query row t < rows, limit =
+ * prefill ? min((t + 1) / ratio, n_comp) : n_comp; the min(index_topk, n_comp) best of
+ * scores[t*n_comp + 0..limit) under f32 total order (descending; ties to the lower index),
+ * written ascending as index + offset, then -1 out to k = min(index_topk, n_comp) columns.
+ * out is [rows][k]. Returns k, or -1 for a non-positive argument. */
+int ro_v4_scored_rows(const float* scores, int rows, int n_comp, int ratio, int index_topk,
+                      int prefill, int offset, int32_t* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -47,6 +47,19 @@ __device__ __forceinline__ uint32_t topk_key(float v) {
     return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);
 }
 
+// The two orders a selection can run under: the DSA rule above, and IEEE total order
+// (f32::total_cmp: -0.0 strictly below +0.0, NaNs ordered by sign and payload), which the
+// scored block selection of the second cache format uses.
+struct FoldedZeroKey {
+    static __device__ __forceinline__ uint32_t of(float v) { return topk_key(v); }
+};
+struct TotalOrderKey {
+    static __device__ __forceinline__ uint32_t of(float v) {
+        const uint32_t b = __float_as_uint(v);
+        return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);
+    }
+};
+
 __device__ __forceinline__ uint32_t lanes_below(unsigned long long mask) {
     return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
                                      __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
@@ -111,9 +124,11 @@ constexpr int topk_block_lds_words() {
 
 // Shape (1): the whole selection for one query by one workgroup of THREADS threads.
 // ITEMS: keys per lane kept in registers; 0 = re-read the scores on every sweep.
-template <int THREADS, int ITEMS>
+// KEY: the order (FoldedZeroKey or TotalOrderKey); `add` is added to every emitted index.
+template <int THREADS, int ITEMS, class KEY = FoldedZeroKey>
 __device__ __forceinline__ void topk_block(const float* __restrict__ s, int nt, uint32_t kq,
-                                           uint32_t* __restrict__ out, uint32_t* lds) {
+                                           uint32_t* __restrict__ out, uint32_t* lds,
+                                           uint32_t add = 0u) {
     constexpr int WAVES = THREADS / kWave;
     constexpr int TPB = THREADS / kBins;  // threads that share one bin's copies
     static_assert(TPB == 1 || TPB == 4, "256 or 1024 threads");
@@ -146,16 +161,16 @@ __device__ __forceinline__ void topk_block(const float* __restrict__ s, int nt, 
                 key[j] = j < steps ? __float_as_uint(sp[j * kWave]) : 0u;
 #pragma unroll
             for (int j = 0; j < ITEMS; ++j)
-                key[j] = j < steps ? topk_key(__uint_as_float(key[j])) : 0u;
+                key[j] = j < steps ? KEY::of(__uint_as_float(key[j])) : 0u;
         } else {
 #pragma unroll
             for (int j = 0; j < ITEMS; ++j)
-                key[j] = (j * kWave < limit) ? topk_key(sp[j * kWave]) : 0u;
+                key[j] = (j * kWave < limit) ? KEY::of(sp[j * kWave]) : 0u;
         }
     }
     auto key_at = [&](int j) -> uint32_t {
         if constexpr (ITEMS > 0) return key[j];
-        return (j * kWave < limit) ? topk_key(s[seg0 + (long long)j * kWave + lane]) : 0u;
+        return (j * kWave < limit) ? KEY::of(s[seg0 + (long long)j * kWave + lane]) : 0u;
     };
 
     uint32_t pivot = 0u, mask = 0u, need = kq;
@@ -223,7 +238,7 @@ __device__ __forceinline__ void topk_block(const float* __restrict__ s, int nt, 
         // slot < kq holds by construction; the compare keeps a wrong pivot from ever
         // turning into a write outside the caller's buffer
         if ((g || (e && E < need)) && slot < kq)
-            out[slot] = (uint32_t)(seg0 + (long long)j * kWave + lane);
+            out[slot] = (uint32_t)(seg0 + (long long)j * kWave + lane) + add;
         run_gt += (uint32_t)__popcll(mg);
         run_eq += (uint32_t)__popcll(me);
     });
@@ -895,7 +910,68 @@ static int index_topk_launch(const float* scores, int n_queries, int stride, con
     return launch_status();
 }
 
+// ---------------------------------------------------------------------------------------------
+// Scored block selection of the second cache format (crates/engine/src/v4/select.rs:153-188,
+// done on the host there): query row t keeps the min(k, limit_t) best of its first limit_t
+// block scores under IEEE total order, ties to the lower block, and lists them ascending as
+// block + offset, then -1 out to k columns. limit_t = min((t + 1) / ratio, n_comp) at prefill
+// (a block is legal once it has closed), n_comp at decode. Where limit_t <= k the row is the
+// positional fill offset .. offset + limit_t - 1 whatever the scores say.
+// ---------------------------------------------------------------------------------------------
+template <int THREADS, int ITEMS>
+__global__ __launch_bounds__(THREADS) void block_select_kernel(const float* __restrict__ scores,
+                                                               int n_comp, int ratio, int prefill,
+                                                               int k, int offset,
+                                                               int32_t* __restrict__ out) {
+    __shared__ uint32_t lds[topk_block_lds_words<THREADS>()];
+    const int t = blockIdx.x;
+    const int limit = prefill ? min((int)(((long long)t + 1) / ratio), n_comp) : n_comp;
+    int32_t* o = out + (size_t)t * k;
+    if (limit <= k) {
+        for (int i = threadIdx.x; i < k; i += THREADS) o[i] = i < limit ? offset + i : -1;
+        return;
+    }
+    topk_block<THREADS, ITEMS, TotalOrderKey>(scores + (size_t)t * n_comp, limit, (uint32_t)k,
+                                              reinterpret_cast<uint32_t*>(o), lds,
+                                              (uint32_t)offset);
+}
+
+static int block_select_launch(const float* scores, int rows, int n_comp, int ratio,
+                               int index_topk, int prefill, int offset, int* out,
+                               hipStream_t stream) {
+    if (!scores || !out) return 1001;
+    if (rows <= 0 || n_comp <= 0 || ratio <= 0 || index_topk <= 0 || offset < 0) return 1001;
+    if ((long long)offset + n_comp > 0x7fffffffLL) return 1002;
+    const int k = index_topk < n_comp ? index_topk : n_comp;
+    (void)hipGetLastError();
+    const dim3 grid((unsigned)rows);
+#define RK_SELECT(T, I)                                                                       \
+    hipLaunchKernelGGL((block_select_kernel<T, I>), grid, dim3(T), 0, stream, scores, n_comp, \
+                       ratio, prefill ? 1 : 0, k, offset, out)
+    // keys stay in registers while a row fits; small rows take the small workgroup so that a
+    // prefill's thousands of rows share the chip
+    if (n_comp <= 256 * 4)
+        RK_SELECT(256, 4);
+    else if (n_comp <= 256 * 16)
+        RK_SELECT(256, 16);
+    else if (n_comp <= 1024 * 16)
+        RK_SELECT(1024, 16);
+    else if (n_comp <= 1024 * 64)
+        RK_SELECT(1024, 64);
+    else
+        RK_SELECT(1024, 0);
+#undef RK_SELECT
+    return launch_status();
+}
+
 }  // namespace rk
+
+extern "C" int rivoli_index_select_blocks(const float* scores, int rows, int n_comp, int ratio,
+                                          int index_topk, int prefill, int offset, int* out,
+                                          void* stream) {
+    return rk::block_select_launch(scores, rows, n_comp, ratio, index_topk, prefill, offset, out,
+                                   (hipStream_t)stream);
+}
 
 extern "C" size_t rivoli_index_topk_workspace_bytes(int n_queries, int nt) {
     if (n_queries <= 0 || nt <= 0) return 0;

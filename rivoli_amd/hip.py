@@ -52,6 +52,8 @@ _SIGNATURES = {
     "rivoli_kv_gather_rows_paged": [_VP] * 5 + [_I] * 6 + [_VP, _VP],
     "rivoli_mla_attend": [_VP] * 6 + [_I] * 5 + [_F, _VP, _VP],
     "rivoli_mla_attend_paged": [_VP] * 7 + [_I] * 8 + [_F, _I, _VP, _VP, _VP, _VP],
+    "rivoli_act_quant_f8_prefix": [_VP, _VP] + [_I] * 4 + [_VP],
+    "rivoli_index_select_blocks": [_VP] + [_I] * 6 + [_VP, _VP],
     "rivoli_codec_e4m3_encode": [_VP, _VP, _LL, _VP],
     "rivoli_codec_e4m3_dequant_bf16": [_VP, _F, _VP, _LL, _VP],
     "rivoli_codec_bf16_encode": [_VP, _VP, _LL, _VP],
@@ -239,6 +241,24 @@ def launch_mla_attend_paged(qabs, qrope, pool, block_table, seq_lens, rows, n_ro
         _p(qabs), _p(qrope), _p(pool), _p(block_table), _p(seq_lens), _p(rows), _p(n_rows), n_seqs,
         H, max_rows, max_blocks_per_seq, kvl, rope, page_tokens, n_pages, scale, int(precise),
         _p(clat), _p(partial), _p(bad_rows), _s(stream)), "mla_attend_paged")
+
+
+# ---- the second cache format: simulated-fp8 rows, scored block selection -------------------
+
+def launch_act_quant_f8_prefix(src, dst, rows, row_stride, n, block, stream=NULL_STREAM) -> None:
+    """crates/backend/src/hip_attn.rs launch_act_quant_f8_prefix: quantize-dequantize dims
+    [0, n) of every row in blocks of `block`; src may be dst."""
+    ensure_hip_status(lib().rivoli_act_quant_f8_prefix(_p(src), _p(dst), rows, row_stride, n, block,
+                                                       _s(stream)), "act_quant_f8_prefix")
+
+
+def launch_index_select_blocks(scores, rows, n_comp, ratio, index_topk, prefill, offset, out,
+                               stream=NULL_STREAM) -> None:
+    """crates/engine/src/v4/select.rs scored_rows on the device: out is int32
+    [rows][min(index_topk, n_comp)]."""
+    ensure_hip_status(lib().rivoli_index_select_blocks(_p(scores), rows, n_comp, ratio, index_topk,
+                                                       1 if prefill else 0, offset, _p(out),
+                                                       _s(stream)), "index_select_blocks")
 
 
 # ---- element codecs -----------------------------------------------------------------------
