@@ -40,14 +40,19 @@ def parse():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=32768)
-    ap.add_argument("--workload", choices=["decode", "prefill", "dsa", "dsa_scored", "dsa_attend", "attend"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "dsa", "dsa_scored", "dsa_attend", "attend", "v4"],
+                    default="decode",
                     help="decode = configuration 3 (the headline line); prefill = configuration 2 "
                          "bulk append; dsa = configuration 4 top-k + sparse gather on synthetic "
                          "scores; dsa_scored = the same with the scores computed on the device; "
                          "dsa_attend = configuration 4 with the sparse gather replaced by MLA decode "
                          "attention over the selected rows; "
                          "attend = configuration 3 with the gather replaced by MLA decode "
-                         "attention reading the fp8 pages directly")
+                         "attention reading the fp8 pages directly; "
+                         "v4 = the second cache format's prefill ops: block-64 quantize-dequantize "
+                         "of `tokens` f32 cache rows, then the scored block selection for every "
+                         "query row (ratio 4, cap --index-topk)")
+    ap.add_argument("--index-topk", type=int, default=512, help="v4: blocks kept per query row")
     ap.add_argument("--heads", type=int, default=64, help="attend: query heads")
     ap.add_argument("--precise", type=int, default=2, choices=[0, 1, 2],
                     help="attend: 2 = q and softmax weights as bf16 hi+lo (parity mode), "
@@ -97,6 +102,8 @@ def main():
         return bench_dsa(a, torch, hip, scored=a.workload == "dsa_scored", attend=a.workload == "dsa_attend")
     if a.workload == "attend":
         return bench_attend(a, torch, hip)
+    if a.workload == "v4":
+        return bench_v4(a, torch, hip)
     L, B, ctx = a.layers, a.batch, a.ctx
     blocks = -(-ctx // PT)
     n_pages = B * blocks
@@ -283,6 +290,82 @@ def bench_prefill(a, torch, hip):
                                "cores": cores, "kind": "port",
                                "sample": f"the same {n}-token append x{reps} reps, {cores} host "
                                          "threads; GPU pool bytes checked equal"}
+    print(json.dumps(res), flush=True)
+
+
+def bench_v4(a, torch, hip):
+    """The second cache format at prefill: `tokens` new f32 cache rows of 512 dims are quantized
+    and dequantized in place over their first 448 dims at block 64 (the rotated tail keeps its
+    precision), and every query row selects its best `index_topk` closed blocks (ratio 4) from
+    its row of the [tokens, tokens / 4] score matrix."""
+    n, hd, nq, blk, ratio = a.tokens, 512, 448, 64, 4
+    n_comp, cap, offset = n // ratio, a.index_topk, 128
+    k = min(cap, n_comp)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0x5EED0006)
+    fresh = torch.randn(n, hd, generator=g, device="cuda", dtype=torch.float32)
+    hit = torch.rand(n, generator=g, device="cuda") < 0.01
+    fresh[hit] *= 200.0
+    kv = fresh.clone()
+    scores = torch.randn(n, n_comp, generator=g, device="cuda", dtype=torch.float32)
+    sel = torch.empty(n, k, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.Stream()
+    sh = stream.cuda_stream
+
+    def step(events):
+        bracket(torch, stream, events, "quant",
+                lambda: hip.launch_act_quant_f8_prefix(kv, kv, n, hd, nq, blk, sh))
+        bracket(torch, stream, events, "select",
+                lambda: hip.launch_index_select_blocks(scores, n, n_comp, ratio, cap, True, offset, sel, sh))
+
+    ms, per = timed(torch, stream, a.steps, a.warmup, step)
+    limit = np.minimum((np.arange(n) + 1) // ratio, n_comp)
+    quant_bytes = n * nq * 8                                       # f32 in, f32 out
+    select_bytes = int(limit[limit > k].sum()) * 4 + n * k * 4     # ranked rows' legal scores in, rows out
+    dom = "select" if per["select"] >= per["quant"] else "quant"
+    dom_bytes = select_bytes if dom == "select" else quant_bytes
+    res = {"metric": "v4_cache_quant_select_GBps",
+           "value": round((quant_bytes + select_bytes) / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+           "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+           "data": "synthetic",
+           "config": {"workload": "second cache format, prefill: block-64 quantize-dequantize of the new "
+                                  "cache rows, then scored block selection per query row",
+                      "tokens": n, "head_dim": hd, "quantized_dims": nq, "block": blk, "ratio": ratio,
+                      "n_comp": n_comp, "index_topk": cap},
+           "tokens_per_s": round(n / (ms * 1e-3), 1),
+           "kernels": {"act_quant_kernel": {"avg_launch_ms": round(per["quant"], 5), "bytes_per_launch": quant_bytes,
+                                            "GBps": round(quant_bytes / (per["quant"] * 1e-3) / 1e9, 1)},
+                       "block_select_kernel": {"avg_launch_ms": round(per["select"], 5),
+                                               "bytes_per_launch": select_bytes,
+                                               "GBps": round(select_bytes / (per["select"] * 1e-3) / 1e9, 1)}},
+           "roofline": {"bound": "hbm", "kernel": "block_select_kernel" if dom == "select" else "act_quant_kernel",
+                        "achieved": round(dom_bytes / (per[dom] * 1e-3) / 1e9, 1), "peak": HBM_PEAK / 1e9,
+                        "unit": "GB/s", "frac": round(dom_bytes / (per[dom] * 1e-3) / HBM_PEAK, 4),
+                        "avg_launch_ms": round(per[dom], 5), "bytes_per_launch": dom_bytes, "traffic": None}}
+    if not a.no_cpu_baseline:
+        from oracle.kvoracle import oracle as get_oracle
+
+        ora = get_oracle()
+        # bounded sample: the first rows of the same inputs, one host thread; the sample doubles
+        # as a parity check of both kernels
+        nr = min(n, 2048)
+        x_h, s_h = fresh[:nr].cpu().numpy(), scores[:nr].cpu().numpy()
+        t0 = time.perf_counter()
+        code, want_kv = ora.act_quant_f8_prefix(x_h, nq, blk)
+        want_sel = ora.v4_scored_rows(s_h, ratio, cap, True, offset)
+        spent = time.perf_counter() - t0
+        got_kv, got_sel = kv[:nr].cpu().numpy(), sel[:nr].cpu().numpy()
+        if code != 0 or not np.array_equal(got_kv.view(np.uint32), want_kv.view(np.uint32)):
+            raise SystemExit("bench: GPU quantize-dequantize differs from the CPU oracle")
+        if not np.array_equal(got_sel, want_sel):
+            raise SystemExit("bench: GPU block selection differs from the CPU oracle")
+        sample_bytes = nr * nq * 8 + int(limit[:nr][limit[:nr] > k].sum()) * 4 + nr * k * 4
+        res["cpu_baseline"] = {"value": round(sample_bytes / spent / 1e9, 3), "unit": "GB/s", "cores": 1,
+                               "kind": "port",
+                               "sample": f"the first {nr} rows of the same inputs through the oracle's "
+                                         "act_quant and scored_rows, one host thread; GPU results "
+                                         "checked equal"}
     print(json.dumps(res), flush=True)
 
 

@@ -918,6 +918,153 @@ static int index_topk_launch(const float* scores, int n_queries, int stride, con
 // (a block is legal once it has closed), n_comp at decode. Where limit_t <= k the row is the
 // positional fill offset .. offset + limit_t - 1 whatever the scores say.
 // ---------------------------------------------------------------------------------------------
+//
+// A prefill asks for thousands of short selections at once (a row has at most n_comp scores,
+// a few thousand), the opposite of the one long query topk_block is built for: its LDS
+// histograms cost more to clear and fold than such a row costs to read. select_bisect keeps a
+// row's keys in registers (a wave owns a contiguous run, 64 per step) and finds the k-th
+// largest key by bisection on its bits, most significant first: count the keys >= candidate
+// (a compare and an add per key, one cross-lane sum per step), keep the bit when at least k
+// remain. A count of exactly k ends the search early — that candidate already separates the
+// selection — which on distinct scores happens after ~log2(spread / spacing) bits, about half
+// of the 32. No LDS traffic besides one word per wave per step when a row spans several waves.
+template <int WAVES, int ITEMS, class KEY>
+__device__ __forceinline__ void select_bisect(const float* __restrict__ s, int nt, uint32_t kq,
+                                              uint32_t* __restrict__ out, uint32_t* lds,
+                                              uint32_t add) {
+    // requires 1 <= kq < nt <= WAVES * 64 * ITEMS
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int per_wave = ((nt + WAVES * kWave - 1) / (WAVES * kWave)) * kWave;
+    const int steps = per_wave / kWave;
+    const int seg0 = wave * per_wave;
+    const int rem = nt - seg0;
+    const int limit = (rem < per_wave ? rem : per_wave) - lane;  // element j exists iff j*64 < limit
+
+    uint32_t key[ITEMS];
+    {
+        const float* sp = s + seg0 + lane;
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j)
+            key[j] = j * kWave < limit ? KEY::of(sp[j * kWave]) : 0u;
+    }
+    // keys >= cand over the whole row, cand >= 1 (so the zero keys of absent elements never
+    // count). `turn` alternates the LDS slots so that one barrier per call is enough.
+    auto count_ge = [&](uint32_t cand, int turn) -> uint32_t {
+        // absent elements hold key 0 < cand, so only whole groups of 8 steps past the row's end
+        // are skipped (one scalar branch per group instead of one per key)
+        uint32_t c = 0;
+#pragma unroll
+        for (int j0 = 0; j0 < ITEMS; j0 += 8) {
+            if (j0 < steps) {
+#pragma unroll
+                for (int j = j0; j < j0 + 8 && j < ITEMS; ++j)
+                    c += (uint32_t)__popcll(__ballot(key[j] >= cand));
+            }
+        }
+        if constexpr (WAVES > 1) {
+            uint32_t* slot = lds + (turn & 1) * WAVES;
+            if (lane == 0) slot[wave] = c;
+            __syncthreads();
+            c = 0;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) c += slot[w];
+        }
+        return c;
+    };
+
+    // T: select key > T, and the first `need` (in index order) of key == T
+    uint32_t p = 0, T = 0, need = 0;
+    bool exact = false;
+    for (int b = 31; b >= 0; --b) {
+        const uint32_t cand = p | (1u << b);
+        const uint32_t c = count_ge(cand, b);
+        if (c >= kq) p = cand;
+        if (c == kq) {
+            exact = true;
+            T = cand - 1u;
+            break;
+        }
+    }
+    if (!exact) {
+        // p is the k-th largest key: count(key >= p) > kq > count(key > p)
+        T = p;
+        const uint32_t above = p == 0xffffffffu ? 0u : count_ge(p + 1u, 1);  // bit 0 used slot 0
+        need = kq - above;
+    }
+
+    uint32_t cnt_gt = 0, cnt_eq = 0;
+    if constexpr (WAVES > 1) {
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            const bool live = j * kWave < limit;
+            cnt_gt += live && key[j] > T ? 1u : 0u;
+            cnt_eq += live && key[j] == T ? 1u : 0u;
+        }
+    }
+    uint32_t run_gt = 0, run_eq = 0;
+    if constexpr (WAVES > 1) {
+        const uint32_t gt_total = wave_sum(cnt_gt), eq_total = wave_sum(cnt_eq);
+        uint32_t* s_gt = lds + 2 * WAVES;
+        uint32_t* s_eq = s_gt + WAVES;
+        if (lane == 0) {
+            s_gt[wave] = gt_total;
+            s_eq[wave] = eq_total;
+        }
+        __syncthreads();
+        for (int w = 0; w < wave; ++w) {
+            run_gt += s_gt[w];
+            run_eq += s_eq[w];
+        }
+    }
+#pragma unroll
+    for (int j0 = 0; j0 < ITEMS; j0 += 8) {
+        if (j0 >= steps) break;
+#pragma unroll
+        for (int j = j0; j < j0 + 8 && j < ITEMS; ++j) {
+            const bool live = j * kWave < limit;
+            const bool g = live && key[j] > T;
+            const bool e = live && key[j] == T;
+            const unsigned long long mg = __ballot(g), me = __ballot(e);
+            const uint32_t G = run_gt + lanes_below(mg);
+            const uint32_t E = run_eq + lanes_below(me);
+            const uint32_t slot = G + (E < need ? E : need);
+            // slot < kq holds by construction; the compare keeps a wrong threshold from ever
+            // turning into a write outside the caller's buffer
+            if ((g || (e && E < need)) && slot < kq)
+                out[slot] = (uint32_t)(seg0 + j * kWave + lane) + add;
+            run_gt += (uint32_t)__popcll(mg);
+            run_eq += (uint32_t)__popcll(me);
+        }
+    }
+}
+
+// The limit of query row t, and the rows that need no ranking (everything legal is kept).
+__device__ __forceinline__ int select_row_limit(int t, int n_comp, int ratio, int prefill) {
+    return prefill ? min((int)(((long long)t + 1) / ratio), n_comp) : n_comp;
+}
+template <int THREADS>
+__device__ __forceinline__ bool select_positional(int32_t* o, int limit, int k, int offset) {
+    if (limit > k) return false;
+    for (int i = threadIdx.x; i < k; i += THREADS) o[i] = i < limit ? offset + i : -1;
+    return true;
+}
+
+template <int WAVES, int ITEMS>
+__global__ __launch_bounds__(WAVES* kWave) void block_select_bisect_kernel(
+    const float* __restrict__ scores, int n_comp, int ratio, int prefill, int k, int offset,
+    int32_t* __restrict__ out) {
+    __shared__ uint32_t lds[4 * WAVES];
+    const int t = blockIdx.x;
+    const int limit = select_row_limit(t, n_comp, ratio, prefill);
+    int32_t* o = out + (size_t)t * k;
+    if (select_positional<WAVES * kWave>(o, limit, k, offset)) return;
+    select_bisect<WAVES, ITEMS, TotalOrderKey>(scores + (size_t)t * n_comp, limit, (uint32_t)k,
+                                               reinterpret_cast<uint32_t*>(o), lds,
+                                               (uint32_t)offset);
+}
+
+// Rows too long for the register form: the single-query radix select, one workgroup per row.
 template <int THREADS, int ITEMS>
 __global__ __launch_bounds__(THREADS) void block_select_kernel(const float* __restrict__ scores,
                                                                int n_comp, int ratio, int prefill,
@@ -925,12 +1072,9 @@ __global__ __launch_bounds__(THREADS) void block_select_kernel(const float* __re
                                                                int32_t* __restrict__ out) {
     __shared__ uint32_t lds[topk_block_lds_words<THREADS>()];
     const int t = blockIdx.x;
-    const int limit = prefill ? min((int)(((long long)t + 1) / ratio), n_comp) : n_comp;
+    const int limit = select_row_limit(t, n_comp, ratio, prefill);
     int32_t* o = out + (size_t)t * k;
-    if (limit <= k) {
-        for (int i = threadIdx.x; i < k; i += THREADS) o[i] = i < limit ? offset + i : -1;
-        return;
-    }
+    if (select_positional<THREADS>(o, limit, k, offset)) return;
     topk_block<THREADS, ITEMS, TotalOrderKey>(scores + (size_t)t * n_comp, limit, (uint32_t)k,
                                               reinterpret_cast<uint32_t*>(o), lds,
                                               (uint32_t)offset);
@@ -945,21 +1089,30 @@ static int block_select_launch(const float* scores, int rows, int n_comp, int ra
     const int k = index_topk < n_comp ? index_topk : n_comp;
     (void)hipGetLastError();
     const dim3 grid((unsigned)rows);
+#define RK_BISECT(WV, I)                                                                     \
+    hipLaunchKernelGGL((block_select_bisect_kernel<WV, I>), grid, dim3(WV* kWave), 0, stream, \
+                       scores, n_comp, ratio, prefill ? 1 : 0, k, offset, out)
 #define RK_SELECT(T, I)                                                                       \
     hipLaunchKernelGGL((block_select_kernel<T, I>), grid, dim3(T), 0, stream, scores, n_comp, \
                        ratio, prefill ? 1 : 0, k, offset, out)
-    // keys stay in registers while a row fits; small rows take the small workgroup so that a
-    // prefill's thousands of rows share the chip
-    if (n_comp <= 256 * 4)
-        RK_SELECT(256, 4);
-    else if (n_comp <= 256 * 16)
-        RK_SELECT(256, 16);
-    else if (n_comp <= 1024 * 16)
-        RK_SELECT(1024, 16);
+    // up to 32 keys per lane; a row takes as few waves as hold it
+    if (n_comp <= 64 * 8)
+        RK_BISECT(1, 8);
+    else if (n_comp <= 64 * 32)
+        RK_BISECT(1, 32);
+    else if (n_comp <= 128 * 32)
+        RK_BISECT(2, 32);
+    else if (n_comp <= 256 * 32)
+        RK_BISECT(4, 32);
+    else if (n_comp <= 512 * 32)
+        RK_BISECT(8, 32);
+    else if (n_comp <= 1024 * 32)
+        RK_BISECT(16, 32);
     else if (n_comp <= 1024 * 64)
         RK_SELECT(1024, 64);
     else
         RK_SELECT(1024, 0);
+#undef RK_BISECT
 #undef RK_SELECT
     return launch_status();
 }
