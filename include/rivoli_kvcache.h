@@ -224,6 +224,55 @@ int rivoli_act_quant_f8_prefix(const float* src, float* dst, int rows, int row_s
 int rivoli_index_select_blocks(const float* scores, int rows, int n_comp, int ratio,
                                int index_topk, int prefill, int offset, int* out, void* stream);
 
+/* The compressor's pooling stage (crates/backend/kernels/kvcompress.hip; Rust rows
+ * launch_kv_compress_deposit / _prefill / _decode, crates/backend/src/hip_attn.rs:547-605).
+ * The two structs cross the boundary by pointer, as in the reference (kvcompress.hip:40-48,
+ * :63-67; crates/engine/src/v4/kvcompress.rs GeomAbi / Finish are the same repr(C) layouts). */
+typedef struct rivoli_comp_geom {
+    int ratio; /* positions pooled into one compressed row */
+    int coff;  /* 1 + overlap; overlapping windows exist at ratio 4 only */
+    int d;     /* the compressor's head width */
+    int cd;    /* coff * d: width of the kv / score projections and of an ape row */
+    int ents;  /* coff * ratio: entries in one pooling window, at most 128 */
+    int rd;    /* the last rd dims of a pooled row are rotated */
+    float eps; /* RMSNorm epsilon */
+} rivoli_comp_geom;
+typedef struct rivoli_comp_finish {
+    const float* norm;  /* [d] the compressor's own RMSNorm weight */
+    const float* freqs; /* [positions][rd] (cos, sin) pairs of the COMPRESSED rotation table */
+    float* out;         /* [nblk][d] at prefill, one row at decode */
+} rivoli_comp_finish;
+
+/* Replaces kvcompress.hip:419-437. kv, score: [s][cd] f32 (this call's projections); ape:
+ * [ratio][cd]; the states: [coff*ratio][cd], a sequence starting with kv_state zeroed and
+ * score_state -inf. A prefill of s tokens (slot0 = 0) stores its last complete block as the
+ * next block's overlap half (overlapping layers) and its s % ratio trailing rows; a decode
+ * step (s = 1) stores its row at slot0 = start_pos % ratio. score_state gets score + the ape
+ * row of the position within its block. Launch it on every call, also when nothing is emitted.
+ * Codes: 1000 null geometry; the geometry guard 1001 (ranges), 1002 (rd), 1003 (cd / ents not
+ * the derived values), 1004 (ents > 128), 1010 (overlap and ratio disagree); 1001 null buffer;
+ * 1005 s <= 0; 1008 slot0 out of range. */
+int rivoli_kv_compress_deposit(const float* kv, const float* score, const float* ape,
+                               float* kv_state, float* score_state, const rivoli_comp_geom* p,
+                               int s, int slot0, void* stream);
+
+/* Replaces kvcompress.hip:439-456. For block b < nblk: per feature, softmax over the window's
+ * entries of score + ape and the weighted sum of kv (on overlapping layers the window is the
+ * previous block's rows, dims [0, d), then the block's own rows, dims [d, 2d); block 0's first
+ * half is masked); then bf16 store, RMSNorm (f32 statistic, weight after the scale) with its
+ * bf16 store, rotation of adjacent pairs of the last rd dims at position b * ratio, bf16 store;
+ * out[b][d] holds bf16 values in f32. Codes as above, plus 1002 d > 8192, 1006 nblk <= 0. */
+int rivoli_kv_compress_prefill(const float* kv, const float* score, const float* ape,
+                               const rivoli_comp_finish* f, const rivoli_comp_geom* p, int nblk,
+                               void* stream);
+
+/* Replaces kvcompress.hip:458-478. Pools the completed window out of the state into f->out[d]
+ * (rotated at the block's first position, (start_pos / ratio) * ratio), then slides the window
+ * on overlapping layers. One workgroup. Codes as above, plus 1007 start_pos <= 0 and 1009 when
+ * start_pos + 1 is not a multiple of ratio. */
+int rivoli_kv_compress_decode(float* kv_state, float* score_state, const rivoli_comp_finish* f,
+                              const rivoli_comp_geom* p, int start_pos, void* stream);
+
 /* Element codecs as launchers (what formats.hpp:42-57,99-106 and fwd.hip:20-45 are to the
  * reference's kernels), for census tests of the device codecs on arbitrary inputs:
  *   e4m3_encode: out[i] = f32_to_e4m3(x[i])            (rule of crates/core/src/num.rs:128-152)

@@ -33,6 +33,18 @@ def _c(a, dtype) -> np.ndarray:
     return a
 
 
+class CompGeom(C.Structure):
+    """crates/backend/kernels/kvcompress.hip:40-48, by value the layout both sides share."""
+    _fields_ = [("ratio", C.c_int), ("coff", C.c_int), ("d", C.c_int), ("cd", C.c_int),
+                ("ents", C.c_int), ("rd", C.c_int), ("eps", C.c_float)]
+
+    @classmethod
+    def attention(cls, ratio: int, d: int = 512, rd: int = 64, eps: float = 1e-6) -> "CompGeom":
+        """The attention compressor's geometry: overlapping windows at ratio 4 only."""
+        coff = 2 if ratio == 4 else 1
+        return cls(ratio, coff, d, coff * d, coff * ratio, rd, eps)
+
+
 class _V4Mixin:
     """The second cache format (v4cache_oracle.h)."""
 
@@ -59,6 +71,36 @@ class _V4Mixin:
         code = int(self.lib.ro_act_quant_f8_prefix(_ptr(src, C.c_float), _ptr(dst, C.c_float), rows,
                                                    row_stride, n, block))
         return code, dst
+
+    def compress_guard(self, geom: CompGeom) -> int:
+        return int(self.lib.ro_compress_guard(C.byref(geom)))
+
+    def kv_compress_deposit(self, kv, score, ape, kv_state, score_state, geom: CompGeom, s: int,
+                            slot0: int) -> int:
+        """The two states are float32 arrays updated in place."""
+        kv, score, ape = _c(kv, np.float32), _c(score, np.float32), _c(ape, np.float32)
+        return int(self.lib.ro_kv_compress_deposit(
+            _ptr(kv, C.c_float), _ptr(score, C.c_float), _ptr(ape, C.c_float),
+            _ptr(kv_state, C.c_float), _ptr(score_state, C.c_float), C.byref(geom), s, slot0))
+
+    def kv_compress_prefill(self, kv, score, ape, norm, freqs, geom: CompGeom, nblk: int):
+        """Returns (code, out[nblk, d])."""
+        kv, score, ape = _c(kv, np.float32), _c(score, np.float32), _c(ape, np.float32)
+        norm, freqs = _c(norm, np.float32), _c(freqs, np.float32)
+        out = np.zeros((max(nblk, 1), geom.d), np.float32)
+        code = int(self.lib.ro_kv_compress_prefill(
+            _ptr(kv, C.c_float), _ptr(score, C.c_float), _ptr(ape, C.c_float), _ptr(norm, C.c_float),
+            _ptr(freqs, C.c_float), _ptr(out, C.c_float), C.byref(geom), nblk))
+        return code, out[:max(nblk, 0)]
+
+    def kv_compress_decode(self, kv_state, score_state, norm, freqs, geom: CompGeom, start_pos: int):
+        """Returns (code, out[d]); the states are updated in place (the window slides)."""
+        norm, freqs = _c(norm, np.float32), _c(freqs, np.float32)
+        out = np.zeros(geom.d, np.float32)
+        code = int(self.lib.ro_kv_compress_decode(
+            _ptr(kv_state, C.c_float), _ptr(score_state, C.c_float), _ptr(norm, C.c_float),
+            _ptr(freqs, C.c_float), _ptr(out, C.c_float), C.byref(geom), start_pos))
+        return code, out
 
     def v4_scored_rows(self, scores, ratio: int, index_topk: int, prefill: bool, offset: int):
         """scores is [rows, n_comp] f32. Returns int32 [rows, min(index_topk, n_comp)]."""
@@ -116,6 +158,10 @@ class Oracle(_V4Mixin):
             "ro_fast_round_scale": (C.c_float, [C.c_float, C.c_float]),
             "ro_act_quant_f8_prefix": (C.c_int, [f32p, f32p] + [C.c_int] * 4),
             "ro_v4_scored_rows": (C.c_int, [f32p] + [C.c_int] * 6 + [i32p]),
+            "ro_compress_guard": (C.c_int, [C.POINTER(CompGeom)]),
+            "ro_kv_compress_deposit": (C.c_int, [f32p] * 5 + [C.POINTER(CompGeom), C.c_int, C.c_int]),
+            "ro_kv_compress_prefill": (C.c_int, [f32p] * 6 + [C.POINTER(CompGeom), C.c_int]),
+            "ro_kv_compress_decode": (C.c_int, [f32p] * 5 + [C.POINTER(CompGeom), C.c_int]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(lib, name)

@@ -144,3 +144,158 @@ int ro_v4_scored_rows(const float* scores, int rows, int n_comp, int ratio, int 
     free(sel);
     return k;
 }
+
+/* ------------------------------------------------------------------------------------------
+ * The compressor's pooling stage
+ * ---------------------------------------------------------------------------------------- */
+
+static inline float round_bf16(float x) { return ro_bf16_to_f32(ro_f32_to_bf16(x)); }
+
+int ro_compress_guard(const ro_comp_geom* p) {
+    if (p->ratio <= 1 || p->d <= 0 || p->rd <= 0 || p->coff < 1 || p->coff > 2) return 1001;
+    if (p->rd > p->d || (p->rd & 1)) return 1002;
+    if (p->cd != p->coff * p->d || p->ents != p->coff * p->ratio) return 1003;
+    if (p->ents > 128) return 1004;
+    if ((p->coff == 2) != (p->ratio == 4)) return 1010;
+    return 0;
+}
+
+int ro_kv_compress_deposit(const float* kv, const float* score, const float* ape, float* kv_state,
+                           float* score_state, const ro_comp_geom* p, int s, int slot0) {
+    if (!p) return 1000;
+    int g = ro_compress_guard(p);
+    if (g) return g;
+    if (s <= 0) return 1005;
+    if (slot0 < 0 || slot0 + s % p->ratio > p->ratio) return 1008;
+    const int remainder = s % p->ratio, cutoff = s - remainder;
+    const int overlap = p->coff == 2;
+    const int state_off = overlap ? p->ratio : 0;
+    const size_t cd = (size_t)p->cd;
+    if (overlap && cutoff >= p->ratio) {
+        /* the last complete block is also the next block's overlap half */
+        for (size_t i = 0; i < (size_t)p->ratio * cd; ++i) {
+            size_t src = (size_t)(cutoff - p->ratio) * cd + i;
+            kv_state[i] = kv[src];
+            score_state[i] = score[src] + ape[i];
+        }
+    }
+    for (size_t i = 0; i < (size_t)remainder * cd; ++i) {
+        size_t src = (size_t)cutoff * cd + i;
+        size_t dst = (size_t)(state_off + slot0) * cd + i;
+        kv_state[dst] = kv[src];
+        score_state[dst] = score[src] + ape[(size_t)slot0 * cd + i]; /* the slot WITHIN its block */
+    }
+    return 0;
+}
+
+/* kvcompress.hip:117-150: softmax over the entries of one feature, then the weighted sum; a
+ * null score pointer is a masked entry; a null ape table means it is already in the score. */
+static void pool_row(const float* const* kvp, const float* const* scp, const float* const* apep,
+                     int ents, int d, float* outrow) {
+    for (int e = 0; e < d; ++e) {
+        float mx = -INFINITY;
+        for (int j = 0; j < ents; ++j) {
+            if (!scp[j]) continue;
+            mx = fmaxf(mx, scp[j][e] + (apep ? apep[j][e] : 0.0f));
+        }
+        if (!isfinite(mx)) {
+            outrow[e] = 0.0f;
+            continue;
+        }
+        float sum = 0.0f;
+        for (int j = 0; j < ents; ++j) {
+            if (!scp[j]) continue;
+            sum += expf(scp[j][e] + (apep ? apep[j][e] : 0.0f) - mx);
+        }
+        float acc = 0.0f;
+        for (int j = 0; j < ents; ++j) {
+            if (!scp[j]) continue;
+            acc += kvp[j][e] * (expf(scp[j][e] + (apep ? apep[j][e] : 0.0f) - mx) / sum);
+        }
+        outrow[e] = acc;
+    }
+}
+
+/* kvcompress.hip:176-203: bf16 store, RMSNorm (f32 statistic, weight after the scale, bf16
+ * store), adjacent-pair rotation of the last rd dims at `pos`, bf16 store. */
+static void finish_row(float* row, const float* norm, const float* freqs, int pos,
+                       const ro_comp_geom* p) {
+    const int d = p->d, rd = p->rd;
+    for (int e = 0; e < d; ++e) row[e] = round_bf16(row[e]);
+    float ss = 0.0f;
+    for (int e = 0; e < d; ++e) ss += row[e] * row[e];
+    const float rs = 1.0f / sqrtf(ss / (float)d + p->eps);
+    for (int e = 0; e < d; ++e) row[e] = round_bf16(norm[e] * (row[e] * rs));
+    const float* t = freqs + (size_t)pos * rd;
+    float* seg = row + (d - rd);
+    for (int i = 0; i < rd / 2; ++i) {
+        float c = t[2 * i], s = t[2 * i + 1];
+        float a = seg[2 * i], b = seg[2 * i + 1];
+        seg[2 * i] = a * c - b * s;
+        seg[2 * i + 1] = a * s + b * c;
+    }
+    for (int e = 0; e < d; ++e) row[e] = round_bf16(row[e]);
+}
+
+int ro_kv_compress_prefill(const float* kv, const float* score, const float* ape,
+                           const float* norm, const float* freqs, float* out,
+                           const ro_comp_geom* p, int nblk) {
+    if (!p || !norm || !freqs || !out) return 1000;
+    int g = ro_compress_guard(p);
+    if (g) return g;
+    if (nblk <= 0) return 1006;
+    const int overlap = p->coff == 2;
+    const float* kvp[128];
+    const float* scp[128];
+    const float* apep[128];
+    for (int b = 0; b < nblk; ++b) {
+        for (int j = 0; j < p->ents; ++j) {
+            int sblk, src_j, half;
+            if (!overlap) {
+                sblk = b, src_j = j, half = 0;
+            } else if (j >= p->ratio) {
+                sblk = b, src_j = j - p->ratio, half = p->d; /* the block's own rows, "normal" half */
+            } else if (b > 0) {
+                sblk = b - 1, src_j = j, half = 0; /* the previous block's rows, "overlap" half */
+            } else {
+                kvp[j] = scp[j] = apep[j] = NULL; /* block 0 has no previous block */
+                continue;
+            }
+            size_t src = (size_t)(sblk * p->ratio + src_j) * p->cd + half;
+            kvp[j] = kv + src;
+            scp[j] = score + src;
+            apep[j] = ape + (size_t)src_j * p->cd + half;
+        }
+        float* row = out + (size_t)b * p->d;
+        pool_row(kvp, scp, apep, p->ents, p->d, row);
+        finish_row(row, norm, freqs, b * p->ratio, p);
+    }
+    return 0;
+}
+
+int ro_kv_compress_decode(float* kv_state, float* score_state, const float* norm,
+                          const float* freqs, float* out, const ro_comp_geom* p, int start_pos) {
+    if (!p || !norm || !freqs || !out) return 1000;
+    int g = ro_compress_guard(p);
+    if (g) return g;
+    if (start_pos <= 0) return 1007;
+    if ((start_pos + 1) % p->ratio != 0) return 1009;
+    const int overlap = p->coff == 2;
+    const float* kvp[128];
+    const float* scp[128];
+    for (int j = 0; j < p->ents; ++j) {
+        int half = (overlap && j >= p->ratio) ? p->d : 0;
+        kvp[j] = kv_state + (size_t)j * p->cd + half;
+        scp[j] = score_state + (size_t)j * p->cd + half;
+    }
+    pool_row(kvp, scp, NULL, p->ents, p->d, out);
+    finish_row(out, norm, freqs, (start_pos / p->ratio) * p->ratio, p);
+    if (overlap) {
+        size_t n = (size_t)p->ratio * p->cd;
+        for (size_t i = 0; i < n; ++i) {
+            kv_state[i] = kv_state[n + i];
+            score_state[i] = score_state[n + i];
+        }
+    }
+    return 0;
+}

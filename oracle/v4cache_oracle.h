@@ -20,6 +20,17 @@
  *                         separates RNE from half-away); idempotence; every output is an e4m3
  *                         value times the block's power-of-two scale; the launcher's guards
  *                         (crates/backend/kernels/mla.hip:527-541)
+ *   ro_kv_compress_*      closed forms of the pooling (equal scores -> the mean of the window;
+ *                         one dominant score -> that entry; block 0's masked overlap half);
+ *                         the overlap index map against a literal overlap_transform tensor
+ *                         and a float64 softmax (numpy); norm and rotation against float64 /
+ *                         complex arithmetic; and the reference's state machine as an
+ *                         invariant: a prefill of s tokens followed by single-token decode
+ *                         steps emits bit for bit the blocks of one longer prefill
+ *                         (crates/oracles/src/v4oracle/compress.rs:62-199 computes both arms
+ *                         with the same per-feature fold). The reference's expectation for
+ *                         these kernels is computed at test time from seeded weights
+ *                         (crates/engine/tests/kernel_v4_compress.rs); it stores no vectors.
  *   ro_v4_scored_rows     the three reference KATs (crates/engine/src/v4/select.rs:645-747:
  *                         below the cap the row is offset+0..limit-1 then -1; three-way tie
  *                         keeps the lower indices; a prefill row cannot take a block that
@@ -61,6 +72,40 @@ int ro_act_quant_f8_prefix(const float* src, float* dst, int rows, int row_strid
  * out is [rows][k]. Returns k, or -1 for a non-positive argument. */
 int ro_v4_scored_rows(const float* scores, int rows, int n_comp, int ratio, int index_topk,
                       int prefill, int offset, int32_t* out);
+
+/* ---- the compressor's pooling stage: crates/backend/kernels/kvcompress.hip:103-384 and its
+ * launchers :386-478; CPU statement crates/oracles/src/v4oracle/compress.rs:42-199 with
+ * rmsnorm / rope_row / softmax_strided of forward.rs:353-383,427-456,557-580 ---- */
+
+/* kvcompress.hip:40-48. cd = coff * d and ents = coff * ratio are derived and checked. */
+typedef struct {
+    int ratio;
+    int coff;
+    int d;
+    int cd;
+    int ents;
+    int rd;
+    float eps;
+} ro_comp_geom;
+
+/* The launchers' shared guard (kvcompress.hip:386-405): 0, 1001, 1002, 1003, 1004 or 1010. */
+int ro_compress_guard(const ro_comp_geom* p);
+
+/* kvcompress.hip:227-262 + :419-437. kv, score: [s][cd]; ape: [ratio][cd]; the two states:
+ * [coff * ratio][cd]. Returns the launcher's code (1000, the guard's, 1005, 1008, or 0). */
+int ro_kv_compress_deposit(const float* kv, const float* score, const float* ape, float* kv_state,
+                           float* score_state, const ro_comp_geom* p, int s, int slot0);
+
+/* kvcompress.hip:278-319 + :439-456: nblk pooled, normed and rotated rows into out[nblk][d].
+ * norm: [d]; freqs: [positions][rd] as (cos, sin) pairs. Code 1000 / guard / 1006 / 0. */
+int ro_kv_compress_prefill(const float* kv, const float* score, const float* ape,
+                           const float* norm, const float* freqs, float* out,
+                           const ro_comp_geom* p, int nblk);
+
+/* kvcompress.hip:332-382 + :458-478: pool the completed window out of the state into out[d],
+ * then slide the window when overlapping. Code 1000 / guard / 1007 / 1009 / 0. */
+int ro_kv_compress_decode(float* kv_state, float* score_state, const float* norm,
+                          const float* freqs, float* out, const ro_comp_geom* p, int start_pos);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,386 @@
+// The pooling stage of the second cache format's compressor: `ratio` consecutive positions
+// become one compressed cache row (crates/backend/kernels/kvcompress.hip:103-384, launchers
+// :386-478; CPU statement crates/oracles/src/v4oracle/compress.rs:42-199). Three launches, the
+// reference's signatures:
+//   deposit  writes the trailing partial window (prefill) or this step's row (decode) into the
+//            per-sequence state, the position-in-block embedding added to the scores;
+//   prefill  one output row per complete block: per feature a softmax over the window's
+//            entries (2 * ratio of them on overlapping layers: the previous block's rows
+//            contribute their first d dims, the block's own rows their last d; block 0's
+//            missing half is masked) and the weighted sum; then the bf16 store, RMSNorm with its
+//            bf16 store, and the adjacent-pair rotation of the last rd dims at the block's
+//            FIRST position, stored as bf16 values in f32;
+//   decode   the same out of the state once a window completes, then the window slides.
+// The projections that produce kv / score (two GEMMs) and the block quantization that follows
+// (act_quant.hip) are separate launches, as in the reference.
+//
+// Shape here: a workgroup per output row; a lane owns 4 consecutive features (16-byte loads,
+// coalesced across the wave). Windows of up to 16 entries are fetched once, all loads in
+// flight together, and every pass of the softmax runs from registers (the reference re-reads
+// each entry three times and evaluates expf twice per element). Wider windows stream three
+// times, one feature per lane with four times the lanes, out of L2. The row then stays in
+// LDS through norm and rotation. HBM traffic is the window once plus the row once.
+#include "codec.hpp"
+#include "rivoli_kvcache.h"
+
+// the rotation's a*c - b*s is two products and a subtraction in the reference's arithmetic
+#pragma clang fp contract(off)
+
+namespace rk {
+
+typedef rivoli_comp_geom CompGeom;
+typedef rivoli_comp_finish CompFinish;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kCompEntsMax = 128;   // the reference's bound on a pooling window
+constexpr int kCompRegEnts = 16;    // windows up to this many entries live in registers
+constexpr int kCompMaxD = 8192;     // one row in LDS
+
+__device__ __forceinline__ float rbf16(float x) {
+    return __uint_as_float((uint32_t)f32_to_bf16(x) << 16);
+}
+
+// Where entry j of a window lives: null score = masked.
+struct Entry {
+    const float* kv;
+    const float* sc;
+    const float* ape;  // null: already in the score
+};
+
+// Prefill's overlap_transform as an index map (kvcompress.hip:264-309).
+__device__ __forceinline__ Entry prefill_entry(const float* kv, const float* score,
+                                               const float* ape, const CompGeom& p, int b, int j) {
+    int sblk = b, src_j = j, half = 0;
+    if (p.coff == 2) {
+        if (j >= p.ratio) {
+            src_j = j - p.ratio;
+            half = p.d;
+        } else if (b > 0) {
+            sblk = b - 1;
+        } else {
+            return Entry{nullptr, nullptr, nullptr};
+        }
+    }
+    const size_t src = (size_t)(sblk * p.ratio + src_j) * p.cd + half;
+    return Entry{kv + src, score + src, ape + (size_t)src_j * p.cd + half};
+}
+// Decode reads the state: low slots their overlap half, high slots their normal half
+// (kvcompress.hip:340-349).
+__device__ __forceinline__ Entry state_entry(const float* kv_state, const float* score_state,
+                                             const CompGeom& p, int j) {
+    const int half = (p.coff == 2 && j >= p.ratio) ? p.d : 0;
+    const size_t src = (size_t)j * p.cd + half;
+    return Entry{kv_state + src, score_state + src, nullptr};
+}
+
+// Softmax over the entries of VEC features starting at e, then the weighted sum
+// (kvcompress.hip:117-150), from registers.
+template <int VEC, class GetEntry>
+__device__ __forceinline__ void pool_registers(GetEntry&& entry, int ents, int e, float (&out)[VEC]) {
+    float v[kCompRegEnts][VEC], k[kCompRegEnts][VEC];
+    bool live[kCompRegEnts];
+#pragma unroll
+    for (int j = 0; j < kCompRegEnts; ++j) {
+        live[j] = false;
+        if (j < ents) {
+            const Entry en = entry(j);
+            live[j] = en.sc != nullptr;
+            if (live[j]) {
+                if constexpr (VEC == 4) {
+                    const f32x4 s4 = *reinterpret_cast<const f32x4*>(en.sc + e);
+                    const f32x4 k4 = *reinterpret_cast<const f32x4*>(en.kv + e);
+                    f32x4 a4 = {0, 0, 0, 0};
+                    if (en.ape) a4 = *reinterpret_cast<const f32x4*>(en.ape + e);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        v[j][i] = en.ape ? s4[i] + a4[i] : s4[i] + 0.0f;
+                        k[j][i] = k4[i];
+                    }
+                } else {
+                    v[j][0] = en.sc[e] + (en.ape ? en.ape[e] : 0.0f);
+                    k[j][0] = en.kv[e];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < kCompRegEnts; ++j)
+            if (j < ents && live[j]) mx = fmaxf(mx, v[j][i]);
+        if (!isfinite(mx)) {  // every entry masked: a zero row, as the CPU statement has it
+            out[i] = 0.0f;
+            continue;
+        }
+        float ex[kCompRegEnts], sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kCompRegEnts; ++j) {
+            if (j < ents && live[j]) {
+                ex[j] = expf(v[j][i] - mx);
+                sum += ex[j];
+            }
+        }
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kCompRegEnts; ++j)
+            if (j < ents && live[j]) acc += k[j][i] * (ex[j] / sum);
+        out[i] = acc;
+    }
+}
+
+// The same for wide windows: three sweeps over memory, one feature.
+template <class GetEntry>
+__device__ __forceinline__ float pool_streamed(GetEntry&& entry, int ents, int e) {
+    float mx = -INFINITY;
+    for (int j = 0; j < ents; ++j) {
+        const Entry en = entry(j);
+        if (!en.sc) continue;
+        mx = fmaxf(mx, en.sc[e] + (en.ape ? en.ape[e] : 0.0f));
+    }
+    if (!isfinite(mx)) return 0.0f;
+    float sum = 0.0f;
+    for (int j = 0; j < ents; ++j) {
+        const Entry en = entry(j);
+        if (!en.sc) continue;
+        sum += expf(en.sc[e] + (en.ape ? en.ape[e] : 0.0f) - mx);
+    }
+    float acc = 0.0f;
+    for (int j = 0; j < ents; ++j) {
+        const Entry en = entry(j);
+        if (!en.sc) continue;
+        acc += en.kv[e] * (expf(en.sc[e] + (en.ape ? en.ape[e] : 0.0f) - mx) / sum);
+    }
+    return acc;
+}
+
+// Sum over the workgroup; red holds one word per wave. Every thread must call it.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int waves = (blockDim.x + kWave - 1) / kWave;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float t = 0.0f;
+    for (int w = 0; w < waves; ++w) t += red[w];
+    return t;
+}
+
+// Pool one row into LDS, finish it there (kvcompress.hip:176-203) and write it out.
+// VEC == 4 requires d % 4 == 0 and 16-byte-aligned rows.
+template <int VEC, bool REG, class GetEntry>
+__device__ __forceinline__ void compress_row(GetEntry&& entry, const CompFinish& f, float* out_row,
+                                             int pos, const CompGeom& p, float* row, float* red) {
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    float ss = 0.0f;
+    for (int e = tid * VEC; e < p.d; e += nthr * VEC) {
+        float pooled[VEC];
+        static_assert(VEC == 1 || VEC == 4, "one feature or four");
+        if constexpr (REG) {
+            pool_registers<VEC>(entry, p.ents, e, pooled);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) pooled[i] = pool_streamed(entry, p.ents, e + i);
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const float r = rbf16(pooled[i]);  // the bf16 store before the norm
+            row[e + i] = r;
+            ss += r * r;
+        }
+    }
+    // 1/sqrt, not a reciprocal-square-root approximation: the factor multiplies the whole row
+    const float rs = 1.0f / sqrtf(block_sum(ss, red) / (float)p.d + p.eps);
+    for (int e = tid * VEC; e < p.d; e += nthr * VEC) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) row[e + i] = rbf16(f.norm[e + i] * (row[e + i] * rs));
+    }
+    __syncthreads();
+    const float* t = f.freqs + (size_t)pos * p.rd;
+    float* seg = row + (p.d - p.rd);
+    for (int i = tid; i < p.rd / 2; i += nthr) {
+        const float c = t[2 * i], s = t[2 * i + 1];
+        const float a = seg[2 * i], b = seg[2 * i + 1];
+        seg[2 * i] = rbf16(a * c - b * s);
+        seg[2 * i + 1] = rbf16(a * s + b * c);
+    }
+    __syncthreads();
+    // the closing bf16 store is the identity on the dims the rotation did not touch
+    for (int e = tid * VEC; e < p.d; e += nthr * VEC) {
+        if constexpr (VEC == 4) {
+            *reinterpret_cast<f32x4*>(out_row + e) = *reinterpret_cast<const f32x4*>(row + e);
+        } else {
+            out_row[e] = row[e];
+        }
+    }
+}
+
+// REG: the window (<= 16 entries) is held in registers, which wants a small workgroup; wide
+// windows stream and want many lanes.
+template <int VEC, bool REG>
+__global__ __launch_bounds__(REG ? 256 : 1024) void kv_compress_prefill_kernel(const float* __restrict__ kv,
+                                           const float* __restrict__ score,
+                                           const float* __restrict__ ape, CompFinish f,
+                                           CompGeom p) {
+    extern __shared__ float lds[];
+    float* row = lds;
+    float* red = lds + p.d;
+    const int b = blockIdx.x;
+    auto entry = [&](int j) { return prefill_entry(kv, score, ape, p, b, j); };
+    compress_row<VEC, REG>(entry, f, f.out + (size_t)b * p.d, b * p.ratio, p, row, red);
+}
+
+// One workgroup: its barriers order the pooling's reads against the window slide.
+template <int VEC, bool REG>
+__global__ __launch_bounds__(REG ? 256 : 1024) void kv_compress_decode_kernel(float* kv_state, float* score_state, CompFinish f,
+                                          CompGeom p, int start_pos) {
+    extern __shared__ float lds[];
+    float* row = lds;
+    float* red = lds + p.d;
+    auto entry = [&](int j) { return state_entry(kv_state, score_state, p, j); };
+    // the block's first absolute position, not its index (kvcompress.hip:360-371)
+    compress_row<VEC, REG>(entry, f, f.out, (start_pos / p.ratio) * p.ratio, p, row, red);
+    __syncthreads();
+    if (p.coff == 2) {
+        // this block's normal half becomes the next block's overlap half
+        const size_t n = (size_t)p.ratio * p.cd;
+        for (size_t i = threadIdx.x; i < n; i += blockDim.x) {
+            kv_state[i] = kv_state[n + i];
+            score_state[i] = score_state[n + i];
+        }
+    }
+}
+
+// kvcompress.hip:227-262, both phases: a prefill of s tokens starts at slot 0, a decode step
+// deposits its one row at slot0 = start_pos % ratio.
+__global__ void kv_compress_deposit_kernel(const float* __restrict__ kv,
+                                           const float* __restrict__ score,
+                                           const float* __restrict__ ape,
+                                           float* __restrict__ kv_state,
+                                           float* __restrict__ score_state, CompGeom p, int s,
+                                           int slot0) {
+    const int remainder = s % p.ratio, cutoff = s - remainder;
+    const bool overlap = p.coff == 2;
+    const int state_off = overlap ? p.ratio : 0;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (overlap && cutoff >= p.ratio) {
+        const size_t n = (size_t)p.ratio * p.cd, src0 = (size_t)(cutoff - p.ratio) * p.cd;
+        for (size_t i = tid; i < n; i += stride) {
+            kv_state[i] = kv[src0 + i];
+            score_state[i] = score[src0 + i] + ape[i];
+        }
+    }
+    if (remainder > 0) {
+        const size_t n = (size_t)remainder * p.cd, src0 = (size_t)cutoff * p.cd;
+        const size_t dst0 = (size_t)(state_off + slot0) * p.cd, ape0 = (size_t)slot0 * p.cd;
+        for (size_t i = tid; i < n; i += stride) {
+            kv_state[dst0 + i] = kv[src0 + i];
+            score_state[dst0 + i] = score[src0 + i] + ape[ape0 + i];
+        }
+    }
+}
+
+// kvcompress.hip:386-405.
+static int compress_guard(const CompGeom& p) {
+    if (p.ratio <= 1 || p.d <= 0 || p.rd <= 0 || p.coff < 1 || p.coff > 2) return 1001;
+    if (p.rd > p.d || (p.rd & 1)) return 1002;
+    if (p.cd != p.coff * p.d || p.ents != p.coff * p.ratio) return 1003;
+    if (p.ents > kCompEntsMax) return 1004;
+    if ((p.coff == 2) != (p.ratio == 4)) return 1010;  // overlap is ratio 4 and nothing else
+    return 0;
+}
+
+struct RowLaunch {
+    bool vec, reg;
+    unsigned threads;
+    size_t lds;
+};
+static RowLaunch row_launch(const CompGeom& p, bool aligned) {
+    RowLaunch r;
+    r.reg = p.ents <= kCompRegEnts;
+    // registers hold a short window for four features per lane; a wide one streams, one
+    // feature per lane, so that more lanes share the latency
+    r.vec = r.reg && aligned && p.d % 4 == 0;
+    const int per_lane = r.vec ? 4 : 1, cap = r.reg ? 256 : 1024;
+    const int threads = ((p.d + per_lane - 1) / per_lane + kWave - 1) / kWave * kWave;
+    r.threads = (unsigned)(threads > cap ? cap : threads);
+    r.lds = ((size_t)p.d + 16) * sizeof(float);
+    return r;
+}
+
+// One of the three instantiations in use: <4, registers>, <1, registers>, <1, streamed>.
+#define RK_COMPRESS_DISPATCH(KERNEL, GRID, R, STREAM, ...)                                        \
+    do {                                                                                          \
+        if ((R).vec)                                                                              \
+            hipLaunchKernelGGL((KERNEL<4, true>), GRID, dim3((R).threads), (R).lds, STREAM,       \
+                               __VA_ARGS__);                                                      \
+        else if ((R).reg)                                                                         \
+            hipLaunchKernelGGL((KERNEL<1, true>), GRID, dim3((R).threads), (R).lds, STREAM,       \
+                               __VA_ARGS__);                                                      \
+        else                                                                                      \
+            hipLaunchKernelGGL((KERNEL<1, false>), GRID, dim3((R).threads), (R).lds, STREAM,      \
+                               __VA_ARGS__);                                                      \
+    } while (0)
+
+}  // namespace rk
+
+extern "C" int rivoli_kv_compress_deposit(const float* kv, const float* score, const float* ape,
+                                          float* kv_state, float* score_state,
+                                          const rivoli_comp_geom* pp, int s, int slot0,
+                                          void* stream) {
+    if (!pp) return 1000;
+    const rk::CompGeom p = *pp;
+    if (int g = rk::compress_guard(p)) return g;
+    if (!kv || !score || !ape || !kv_state || !score_state) return 1001;
+    if (s <= 0) return 1005;
+    if (slot0 < 0 || slot0 + s % p.ratio > p.ratio) return 1008;
+    (void)hipGetLastError();
+    const int rem = s % p.ratio;
+    const size_t n = (size_t)(p.ratio > rem ? p.ratio : rem) * p.cd;
+    hipLaunchKernelGGL(rk::kv_compress_deposit_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256),
+                       0, (hipStream_t)stream, kv, score, ape, kv_state, score_state, p, s, slot0);
+    return rk::launch_status();
+}
+
+extern "C" int rivoli_kv_compress_prefill(const float* kv, const float* score, const float* ape,
+                                          const rivoli_comp_finish* ff, const rivoli_comp_geom* pp,
+                                          int nblk, void* stream) {
+    if (!pp || !ff) return 1000;
+    const rk::CompGeom p = *pp;
+    if (int g = rk::compress_guard(p)) return g;
+    if (!kv || !score || !ape || !ff->norm || !ff->freqs || !ff->out) return 1001;
+    if (p.d > rk::kCompMaxD) return 1002;
+    // refused, not a silent success: the caller believed a block would be emitted
+    if (nblk <= 0) return 1006;
+    const bool aligned = rk::aligned16(kv) && rk::aligned16(score) && rk::aligned16(ape) &&
+                         rk::aligned16(ff->out);
+    const rk::RowLaunch r = rk::row_launch(p, aligned);
+    (void)hipGetLastError();
+    RK_COMPRESS_DISPATCH(rk::kv_compress_prefill_kernel, dim3((unsigned)nblk), r, (hipStream_t)stream,
+                         kv, score, ape, *ff, p);
+    return rk::launch_status();
+}
+
+extern "C" int rivoli_kv_compress_decode(float* kv_state, float* score_state,
+                                         const rivoli_comp_finish* ff, const rivoli_comp_geom* pp,
+                                         int start_pos, void* stream) {
+    if (!pp || !ff) return 1000;
+    const rk::CompGeom p = *pp;
+    if (int g = rk::compress_guard(p)) return g;
+    if (!kv_state || !score_state || !ff->norm || !ff->freqs || !ff->out) return 1001;
+    if (p.d > rk::kCompMaxD) return 1002;
+    if (start_pos <= 0) return 1007;  // position 0 is the prefill path
+    // only a position that COMPLETES a block may pool: a half-filled window still gives
+    // finite, plausible numbers
+    if ((start_pos + 1) % p.ratio != 0) return 1009;
+    const bool aligned = rk::aligned16(kv_state) && rk::aligned16(score_state) &&
+                         rk::aligned16(ff->out);
+    const rk::RowLaunch r = rk::row_launch(p, aligned);
+    (void)hipGetLastError();
+    RK_COMPRESS_DISPATCH(rk::kv_compress_decode_kernel, dim3(1), r, (hipStream_t)stream, kv_state,
+                         score_state, *ff, p, start_pos);
+    return rk::launch_status();
+}

@@ -54,6 +54,9 @@ _SIGNATURES = {
     "rivoli_mla_attend_paged": [_VP] * 7 + [_I] * 8 + [_F, _I, _VP, _VP, _VP, _VP],
     "rivoli_act_quant_f8_prefix": [_VP, _VP] + [_I] * 4 + [_VP],
     "rivoli_index_select_blocks": [_VP] + [_I] * 6 + [_VP, _VP],
+    "rivoli_kv_compress_deposit": [_VP] * 6 + [_I, _I, _VP],
+    "rivoli_kv_compress_prefill": [_VP] * 5 + [_I, _VP],
+    "rivoli_kv_compress_decode": [_VP] * 4 + [_I, _VP],
     "rivoli_codec_e4m3_encode": [_VP, _VP, _LL, _VP],
     "rivoli_codec_e4m3_dequant_bf16": [_VP, _F, _VP, _LL, _VP],
     "rivoli_codec_bf16_encode": [_VP, _VP, _LL, _VP],
@@ -259,6 +262,52 @@ def launch_index_select_blocks(scores, rows, n_comp, ratio, index_topk, prefill,
     ensure_hip_status(lib().rivoli_index_select_blocks(_p(scores), rows, n_comp, ratio, index_topk,
                                                        1 if prefill else 0, offset, _p(out),
                                                        _s(stream)), "index_select_blocks")
+
+
+class CompGeom(C.Structure):
+    """rivoli_comp_geom (crates/engine/src/v4/kvcompress.rs GeomAbi): only `build` derives the
+    dependent fields, so a stale cd / ents cannot be handed over."""
+    _fields_ = [("ratio", C.c_int), ("coff", C.c_int), ("d", C.c_int), ("cd", C.c_int),
+                ("ents", C.c_int), ("rd", C.c_int), ("eps", C.c_float)]
+
+    @classmethod
+    def build(cls, ratio: int, d: int, rd: int, eps: float) -> "CompGeom":
+        coff = 2 if ratio == 4 else 1        # overlapping windows exist at ratio 4 only
+        return cls(ratio, coff, d, coff * d, coff * ratio, rd, eps)
+
+
+class CompFinish(C.Structure):
+    """rivoli_comp_finish: device pointers of the norm weight, the compressed rotation table
+    and the output rows."""
+    _fields_ = [("norm", C.c_void_p), ("freqs", C.c_void_p), ("out", C.c_void_p)]
+
+    @classmethod
+    def of(cls, norm, freqs, out) -> "CompFinish":
+        return cls(_p(norm), _p(freqs), _p(out))
+
+
+def _ref_or_null(struct):
+    return None if struct is None else C.byref(struct)
+
+
+def launch_kv_compress_deposit(kv, score, ape, kv_state, score_state, geom, s, slot0,
+                               stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_kv_compress_deposit(
+        _p(kv), _p(score), _p(ape), _p(kv_state), _p(score_state), _ref_or_null(geom), s, slot0,
+        _s(stream)), "kv_compress_deposit")
+
+
+def launch_kv_compress_prefill(kv, score, ape, finish, geom, nblk, stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_kv_compress_prefill(
+        _p(kv), _p(score), _p(ape), _ref_or_null(finish), _ref_or_null(geom), nblk, _s(stream)),
+        "kv_compress_prefill")
+
+
+def launch_kv_compress_decode(kv_state, score_state, finish, geom, start_pos,
+                              stream=NULL_STREAM) -> None:
+    ensure_hip_status(lib().rivoli_kv_compress_decode(
+        _p(kv_state), _p(score_state), _ref_or_null(finish), _ref_or_null(geom), start_pos,
+        _s(stream)), "kv_compress_decode")
 
 
 # ---- element codecs -----------------------------------------------------------------------

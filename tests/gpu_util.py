@@ -55,6 +55,13 @@ def ref_kernels():
         if hasattr(h, "rivoli_act_quant_f8_prefix"):
             h.rivoli_act_quant_f8_prefix.restype = i
             h.rivoli_act_quant_f8_prefix.argtypes = [vp, vp] + [i] * 4 + [vp]
+        if hasattr(h, "rivoli_kv_compress_prefill"):
+            h.rivoli_kv_compress_deposit.restype = i
+            h.rivoli_kv_compress_deposit.argtypes = [vp] * 6 + [i, i, vp]
+            h.rivoli_kv_compress_prefill.restype = i
+            h.rivoli_kv_compress_prefill.argtypes = [vp] * 5 + [i, vp]
+            h.rivoli_kv_compress_decode.restype = i
+            h.rivoli_kv_compress_decode.argtypes = [vp] * 4 + [i, vp]
         h.rivoli_hash_rows.restype = i
         h.rivoli_hash_rows.argtypes = [vp, i, i, C.c_ulonglong, vp, vp]
         _REF = h

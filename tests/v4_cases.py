@@ -1,0 +1,65 @@
+"""Inputs and independent restatements for the second cache format's compressor tests."""
+import numpy as np
+
+from oracle.kvoracle import CompGeom
+
+
+def compress_inputs(geom: CompGeom, s: int, seed: int, positions: int = 0):
+    """Projected kv / gate scores for s tokens, the position-in-block embedding, the norm weight
+    and a rotation table of (cos, sin) pairs for `positions` positions (at least s)."""
+    rng = np.random.default_rng(seed)
+    kv = rng.standard_normal((s, geom.cd)).astype(np.float32)
+    score = (rng.standard_normal((s, geom.cd)) * 2.0).astype(np.float32)
+    ape = rng.standard_normal((geom.ratio, geom.cd)).astype(np.float32)
+    norm = (1.0 + 0.1 * rng.standard_normal(geom.d)).astype(np.float32)
+    n_pos = max(positions, s, 1)
+    inv = 160000.0 ** (-np.arange(geom.rd // 2, dtype=np.float64) * 2.0 / geom.rd)
+    ang = np.arange(n_pos, dtype=np.float64)[:, None] * inv[None, :]
+    freqs = np.stack([np.cos(ang), np.sin(ang)], axis=-1).reshape(n_pos, geom.rd).astype(np.float32)
+    return kv, score, ape, norm, freqs
+
+
+def bf16_gap(oracle, a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """Distance in bf16 codes under a monotone ordering (crates/engine/tests/v4_compressor/
+    metric.rs: 0 is bit-identical, 1 is adjacent representable values)."""
+    def ordered(x):
+        c = oracle.f32_to_bf16(np.ascontiguousarray(x, np.float32)).astype(np.int64)
+        return np.where(c & 0x8000, -(c & 0x7FFF), c)
+    return np.abs(ordered(a) - ordered(b))
+
+
+def literal_pooling(geom: CompGeom, kv, score, ape, nblk: int) -> np.ndarray:
+    """model.py's own order of operations in float64: add the position embedding to the scores,
+    materialise overlap_transform's [nblk, ents, d] tensors (zero / -inf where block 0 has no
+    previous block), softmax over the entry axis, weighted sum."""
+    r, d, cd = geom.ratio, geom.d, geom.cd
+    kv64 = kv[: nblk * r].astype(np.float64).reshape(nblk, r, cd)
+    sc64 = (score[: nblk * r].astype(np.float32).reshape(nblk, r, cd) + ape[None, :, :]).astype(np.float64)
+    if geom.coff == 2:
+        kb = np.zeros((nblk, 2 * r, d))
+        sb = np.full((nblk, 2 * r, d), -np.inf)
+        kb[:, r:] = kv64[:, :, d:]
+        sb[:, r:] = sc64[:, :, d:]
+        kb[1:, :r] = kv64[:-1, :, :d]
+        sb[1:, :r] = sc64[:-1, :, :d]
+    else:
+        kb, sb = kv64, sc64
+    w = np.exp(sb - sb.max(axis=1, keepdims=True))
+    w /= w.sum(axis=1, keepdims=True)
+    return (kb * w).sum(axis=1)
+
+
+def literal_finish(oracle, geom: CompGeom, pooled, norm, freqs, first_pos: int) -> np.ndarray:
+    """bf16 store, RMSNorm in float64 with the bf16 store, complex rotation of the last rd dims
+    at each block's first position, bf16 store."""
+    rb = lambda x: oracle.e4m3_to_f32(np.zeros(0, np.uint8)) if x.size == 0 else \
+        (oracle.f32_to_bf16(x.astype(np.float32)).astype(np.uint32) << 16).view(np.float32)
+    d, rd, r = geom.d, geom.rd, geom.ratio
+    x = rb(pooled).astype(np.float64)
+    rs = 1.0 / np.sqrt((x * x).mean(axis=1, keepdims=True) + np.float64(np.float32(geom.eps)))
+    x = rb(norm.astype(np.float64)[None, :] * (x * rs)).astype(np.float64)
+    pos = first_pos + np.arange(x.shape[0]) * r
+    t = freqs[pos].astype(np.float64).reshape(-1, rd // 2, 2)
+    z = (x[:, d - rd::2] + 1j * x[:, d - rd + 1::2]) * (t[:, :, 0] + 1j * t[:, :, 1])
+    x[:, d - rd::2], x[:, d - rd + 1::2] = z.real, z.imag
+    return rb(x)
