@@ -293,6 +293,12 @@ def bench_prefill(a, torch, hip):
     print(json.dumps(res), flush=True)
 
 
+def ordered_bf16(ora, x):
+    """bf16 codes under a monotone ordering, for code-distance comparisons."""
+    c = ora.f32_to_bf16(np.ascontiguousarray(x, np.float32)).astype(np.int64)
+    return np.where(c & 0x8000, -(c & 0x7FFF), c)
+
+
 def bench_v4(a, torch, hip):
     """The second cache format at prefill: `tokens` new f32 cache rows of 512 dims are quantized
     and dequantized in place over their first 448 dims at block 64 (the rotated tail keeps its
@@ -312,7 +318,22 @@ def bench_v4(a, torch, hip):
     stream = torch.cuda.Stream()
     sh = stream.cuda_stream
 
+    # the attention compressor at ratio 4 (overlapping windows): the projections' outputs for the
+    # same tokens, pooled into n / 4 compressed rows
+    geom = hip.CompGeom.build(ratio, hd, hd - nq, 1e-6)
+    c_kv = torch.randn(n, geom.cd, generator=g, device="cuda", dtype=torch.float32)
+    c_score = torch.randn(n, geom.cd, generator=g, device="cuda", dtype=torch.float32) * 2.0
+    c_ape = torch.randn(ratio, geom.cd, generator=g, device="cuda", dtype=torch.float32)
+    c_norm = 1.0 + 0.1 * torch.randn(hd, generator=g, device="cuda", dtype=torch.float32)
+    inv = 160000.0 ** (-torch.arange(geom.rd // 2, device="cuda", dtype=torch.float64) * 2.0 / geom.rd)
+    ang = torch.arange(n, device="cuda", dtype=torch.float64)[:, None] * inv[None, :]
+    c_freqs = torch.stack([torch.cos(ang), torch.sin(ang)], dim=-1).reshape(n, geom.rd).float().contiguous()
+    c_out = torch.empty(n_comp, hd, dtype=torch.float32, device="cuda")
+    c_fin = hip.CompFinish.of(c_norm, c_freqs, c_out)
+
     def step(events):
+        bracket(torch, stream, events, "compress",
+                lambda: hip.launch_kv_compress_prefill(c_kv, c_score, c_ape, c_fin, geom, n_comp, sh))
         bracket(torch, stream, events, "quant",
                 lambda: hip.launch_act_quant_f8_prefix(kv, kv, n, hd, nq, blk, sh))
         bracket(torch, stream, events, "select",
@@ -322,24 +343,31 @@ def bench_v4(a, torch, hip):
     limit = np.minimum((np.arange(n) + 1) // ratio, n_comp)
     quant_bytes = n * nq * 8                                       # f32 in, f32 out
     select_bytes = int(limit[limit > k].sum()) * 4 + n * k * 4     # ranked rows' legal scores in, rows out
-    dom = "select" if per["select"] >= per["quant"] else "quant"
-    dom_bytes = select_bytes if dom == "select" else quant_bytes
-    res = {"metric": "v4_cache_quant_select_GBps",
-           "value": round((quant_bytes + select_bytes) / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+    compress_bytes = 2 * n * geom.cd * 4 + n_comp * hd * 4         # kv + score windows in, rows out
+    names = {"select": ("block_select_kernel", select_bytes), "quant": ("act_quant_kernel", quant_bytes),
+             "compress": ("kv_compress_prefill_kernel", compress_bytes)}
+    dom = max(names, key=lambda k_: per[k_])
+    dom_bytes = names[dom][1]
+    res = {"metric": "v4_cache_compress_quant_select_GBps",
+           "value": round((compress_bytes + quant_bytes + select_bytes) / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
            "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
            "data": "synthetic",
-           "config": {"workload": "second cache format, prefill: block-64 quantize-dequantize of the new "
-                                  "cache rows, then scored block selection per query row",
+           "config": {"workload": "second cache format, prefill: pooling of the tokens into compressed rows "
+                                  "(ratio 4, overlapping windows), block-64 quantize-dequantize of the "
+                                  "new cache rows, scored block selection per query row",
                       "tokens": n, "head_dim": hd, "quantized_dims": nq, "block": blk, "ratio": ratio,
                       "n_comp": n_comp, "index_topk": cap},
            "tokens_per_s": round(n / (ms * 1e-3), 1),
-           "kernels": {"act_quant_kernel": {"avg_launch_ms": round(per["quant"], 5), "bytes_per_launch": quant_bytes,
+           "kernels": {"kv_compress_prefill_kernel": {"avg_launch_ms": round(per["compress"], 5),
+                                                      "bytes_per_launch": compress_bytes,
+                                                      "GBps": round(compress_bytes / (per["compress"] * 1e-3) / 1e9, 1)},
+                       "act_quant_kernel": {"avg_launch_ms": round(per["quant"], 5), "bytes_per_launch": quant_bytes,
                                             "GBps": round(quant_bytes / (per["quant"] * 1e-3) / 1e9, 1)},
                        "block_select_kernel": {"avg_launch_ms": round(per["select"], 5),
                                                "bytes_per_launch": select_bytes,
                                                "GBps": round(select_bytes / (per["select"] * 1e-3) / 1e9, 1)}},
-           "roofline": {"bound": "hbm", "kernel": "block_select_kernel" if dom == "select" else "act_quant_kernel",
+           "roofline": {"bound": "hbm", "kernel": names[dom][0],
                         "achieved": round(dom_bytes / (per[dom] * 1e-3) / 1e9, 1), "peak": HBM_PEAK / 1e9,
                         "unit": "GB/s", "frac": round(dom_bytes / (per[dom] * 1e-3) / HBM_PEAK, 4),
                         "avg_launch_ms": round(per[dom], 5), "bytes_per_launch": dom_bytes, "traffic": None}}
@@ -354,18 +382,36 @@ def bench_v4(a, torch, hip):
         t0 = time.perf_counter()
         code, want_kv = ora.act_quant_f8_prefix(x_h, nq, blk)
         want_sel = ora.v4_scored_rows(s_h, ratio, cap, True, offset)
+        from oracle.kvoracle import CompGeom as OracleGeom
+
+        og = OracleGeom.attention(ratio, hd, hd - nq)
+        code_c, want_c = ora.kv_compress_prefill(c_kv[:nr].cpu().numpy(), c_score[:nr].cpu().numpy(),
+                                                 c_ape.cpu().numpy(), c_norm.cpu().numpy(),
+                                                 c_freqs[:nr].cpu().numpy(), og, nr // ratio)
         spent = time.perf_counter() - t0
         got_kv, got_sel = kv[:nr].cpu().numpy(), sel[:nr].cpu().numpy()
         if code != 0 or not np.array_equal(got_kv.view(np.uint32), want_kv.view(np.uint32)):
             raise SystemExit("bench: GPU quantize-dequantize differs from the CPU oracle")
         if not np.array_equal(got_sel, want_sel):
             raise SystemExit("bench: GPU block selection differs from the CPU oracle")
-        sample_bytes = nr * nq * 8 + int(limit[:nr][limit[:nr] > k].sum()) * 4 + nr * k * 4
+        got_c = c_out[: nr // ratio].cpu().numpy()
+        gap = np.abs(ordered_bf16(ora, got_c) - ordered_bf16(ora, want_c))
+        # a value that cancelled to almost nothing against its row carries the terms' absolute
+        # error, which is many codes of the small result: those are compared absolutely, to
+        # 2^-14 of the row's largest value (2^-8 in the rotated tail)
+        top = np.abs(want_c).max(axis=1, keepdims=True)
+        near = np.abs(got_c - want_c) <= top * np.where((np.arange(hd) >= nq)[None, :], 2.0 ** -8, 2.0 ** -14)
+        gap = np.where(near, np.minimum(gap, 2), gap)
+        if code_c != 0 or gap.max() > 2 or np.mean(gap > 0) > 0.01:
+            raise SystemExit(f"bench: GPU compressor pooling is more than 2 bf16 codes from the CPU oracle "
+                             f"(code {code_c}, max gap {gap.max()}, differing {np.mean(gap > 0):.4f})")
+        sample_bytes = (nr * nq * 8 + int(limit[:nr][limit[:nr] > k].sum()) * 4 + nr * k * 4
+                        + 2 * nr * geom.cd * 4 + (nr // ratio) * hd * 4)
         res["cpu_baseline"] = {"value": round(sample_bytes / spent / 1e9, 3), "unit": "GB/s", "cores": 1,
                                "kind": "port",
                                "sample": f"the first {nr} rows of the same inputs through the oracle's "
-                                         "act_quant and scored_rows, one host thread; GPU results "
-                                         "checked equal"}
+                                         "compressor pooling, act_quant and scored_rows, one host thread; "
+                                         "GPU results checked (pooling within 2 bf16 codes, the others equal)"}
     print(json.dumps(res), flush=True)
 
 

@@ -75,12 +75,13 @@ __device__ __forceinline__ Entry state_entry(const float* kv_state, const float*
 
 // Softmax over the entries of VEC features starting at e, then the weighted sum
 // (kvcompress.hip:117-150), from registers.
-template <int VEC, class GetEntry>
+template <int VEC, int SLOTS, class GetEntry>
 __device__ __forceinline__ void pool_registers(GetEntry&& entry, int ents, int e, float (&out)[VEC]) {
-    float v[kCompRegEnts][VEC], k[kCompRegEnts][VEC];
-    bool live[kCompRegEnts];
+    static_assert(SLOTS <= kCompRegEnts, "register windows are short");
+    float v[SLOTS][VEC], k[SLOTS][VEC];
+    bool live[SLOTS];
 #pragma unroll
-    for (int j = 0; j < kCompRegEnts; ++j) {
+    for (int j = 0; j < SLOTS; ++j) {
         live[j] = false;
         if (j < ents) {
             const Entry en = entry(j);
@@ -107,15 +108,15 @@ __device__ __forceinline__ void pool_registers(GetEntry&& entry, int ents, int e
     for (int i = 0; i < VEC; ++i) {
         float mx = -INFINITY;
 #pragma unroll
-        for (int j = 0; j < kCompRegEnts; ++j)
+        for (int j = 0; j < SLOTS; ++j)
             if (j < ents && live[j]) mx = fmaxf(mx, v[j][i]);
         if (!isfinite(mx)) {  // every entry masked: a zero row, as the CPU statement has it
             out[i] = 0.0f;
             continue;
         }
-        float ex[kCompRegEnts], sum = 0.0f;
+        float ex[SLOTS], sum = 0.0f;
 #pragma unroll
-        for (int j = 0; j < kCompRegEnts; ++j) {
+        for (int j = 0; j < SLOTS; ++j) {
             if (j < ents && live[j]) {
                 ex[j] = expf(v[j][i] - mx);
                 sum += ex[j];
@@ -123,7 +124,7 @@ __device__ __forceinline__ void pool_registers(GetEntry&& entry, int ents, int e
         }
         float acc = 0.0f;
 #pragma unroll
-        for (int j = 0; j < kCompRegEnts; ++j)
+        for (int j = 0; j < SLOTS; ++j)
             if (j < ents && live[j]) acc += k[j][i] * (ex[j] / sum);
         out[i] = acc;
     }
@@ -170,7 +171,8 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 
 // Pool one row into LDS, finish it there (kvcompress.hip:176-203) and write it out.
 // VEC == 4 requires d % 4 == 0 and 16-byte-aligned rows.
-template <int VEC, bool REG, class GetEntry>
+// SLOTS: 8 or 16 = the window is held in that many register slots; 0 = streamed.
+template <int VEC, int SLOTS, class GetEntry>
 __device__ __forceinline__ void compress_row(GetEntry&& entry, const CompFinish& f, float* out_row,
                                              int pos, const CompGeom& p, float* row, float* red) {
     const int tid = threadIdx.x, nthr = blockDim.x;
@@ -178,8 +180,8 @@ __device__ __forceinline__ void compress_row(GetEntry&& entry, const CompFinish&
     for (int e = tid * VEC; e < p.d; e += nthr * VEC) {
         float pooled[VEC];
         static_assert(VEC == 1 || VEC == 4, "one feature or four");
-        if constexpr (REG) {
-            pool_registers<VEC>(entry, p.ents, e, pooled);
+        if constexpr (SLOTS > 0) {
+            pool_registers<VEC, SLOTS>(entry, p.ents, e, pooled);
         } else {
 #pragma unroll
             for (int i = 0; i < VEC; ++i) pooled[i] = pool_streamed(entry, p.ents, e + i);
@@ -217,10 +219,9 @@ __device__ __forceinline__ void compress_row(GetEntry&& entry, const CompFinish&
     }
 }
 
-// REG: the window (<= 16 entries) is held in registers, which wants a small workgroup; wide
-// windows stream and want many lanes.
-template <int VEC, bool REG>
-__global__ __launch_bounds__(REG ? 256 : 1024) void kv_compress_prefill_kernel(const float* __restrict__ kv,
+// A window held in registers wants a small workgroup; wide windows stream and want many lanes.
+template <int VEC, int SLOTS>
+__global__ __launch_bounds__(SLOTS ? 256 : 1024) void kv_compress_prefill_kernel(const float* __restrict__ kv,
                                            const float* __restrict__ score,
                                            const float* __restrict__ ape, CompFinish f,
                                            CompGeom p) {
@@ -229,19 +230,19 @@ __global__ __launch_bounds__(REG ? 256 : 1024) void kv_compress_prefill_kernel(c
     float* red = lds + p.d;
     const int b = blockIdx.x;
     auto entry = [&](int j) { return prefill_entry(kv, score, ape, p, b, j); };
-    compress_row<VEC, REG>(entry, f, f.out + (size_t)b * p.d, b * p.ratio, p, row, red);
+    compress_row<VEC, SLOTS>(entry, f, f.out + (size_t)b * p.d, b * p.ratio, p, row, red);
 }
 
 // One workgroup: its barriers order the pooling's reads against the window slide.
-template <int VEC, bool REG>
-__global__ __launch_bounds__(REG ? 256 : 1024) void kv_compress_decode_kernel(float* kv_state, float* score_state, CompFinish f,
+template <int VEC, int SLOTS>
+__global__ __launch_bounds__(SLOTS ? 256 : 1024) void kv_compress_decode_kernel(float* kv_state, float* score_state, CompFinish f,
                                           CompGeom p, int start_pos) {
     extern __shared__ float lds[];
     float* row = lds;
     float* red = lds + p.d;
     auto entry = [&](int j) { return state_entry(kv_state, score_state, p, j); };
     // the block's first absolute position, not its index (kvcompress.hip:360-371)
-    compress_row<VEC, REG>(entry, f, f.out, (start_pos / p.ratio) * p.ratio, p, row, red);
+    compress_row<VEC, SLOTS>(entry, f, f.out, (start_pos / p.ratio) * p.ratio, p, row, red);
     __syncthreads();
     if (p.coff == 2) {
         // this block's normal half becomes the next block's overlap half
@@ -311,17 +312,21 @@ static RowLaunch row_launch(const CompGeom& p, bool aligned) {
     return r;
 }
 
-// One of the three instantiations in use: <4, registers>, <1, registers>, <1, streamed>.
-#define RK_COMPRESS_DISPATCH(KERNEL, GRID, R, STREAM, ...)                                        \
+// The instantiations in use: four features per lane with 8 or 16 register slots, one feature
+// per lane with 16, one feature per lane streamed.
+#define RK_COMPRESS_DISPATCH(KERNEL, GRID, R, ENTS, STREAM, ...)                                  \
     do {                                                                                          \
-        if ((R).vec)                                                                              \
-            hipLaunchKernelGGL((KERNEL<4, true>), GRID, dim3((R).threads), (R).lds, STREAM,       \
+        if ((R).vec && (ENTS) <= 8)                                                               \
+            hipLaunchKernelGGL((KERNEL<4, 8>), GRID, dim3((R).threads), (R).lds, STREAM,          \
+                               __VA_ARGS__);                                                      \
+        else if ((R).vec)                                                                         \
+            hipLaunchKernelGGL((KERNEL<4, 16>), GRID, dim3((R).threads), (R).lds, STREAM,         \
                                __VA_ARGS__);                                                      \
         else if ((R).reg)                                                                         \
-            hipLaunchKernelGGL((KERNEL<1, true>), GRID, dim3((R).threads), (R).lds, STREAM,       \
+            hipLaunchKernelGGL((KERNEL<1, 16>), GRID, dim3((R).threads), (R).lds, STREAM,         \
                                __VA_ARGS__);                                                      \
         else                                                                                      \
-            hipLaunchKernelGGL((KERNEL<1, false>), GRID, dim3((R).threads), (R).lds, STREAM,      \
+            hipLaunchKernelGGL((KERNEL<1, 0>), GRID, dim3((R).threads), (R).lds, STREAM,          \
                                __VA_ARGS__);                                                      \
     } while (0)
 
@@ -359,8 +364,8 @@ extern "C" int rivoli_kv_compress_prefill(const float* kv, const float* score, c
                          rk::aligned16(ff->out);
     const rk::RowLaunch r = rk::row_launch(p, aligned);
     (void)hipGetLastError();
-    RK_COMPRESS_DISPATCH(rk::kv_compress_prefill_kernel, dim3((unsigned)nblk), r, (hipStream_t)stream,
-                         kv, score, ape, *ff, p);
+    RK_COMPRESS_DISPATCH(rk::kv_compress_prefill_kernel, dim3((unsigned)nblk), r, p.ents,
+                         (hipStream_t)stream, kv, score, ape, *ff, p);
     return rk::launch_status();
 }
 
@@ -380,7 +385,7 @@ extern "C" int rivoli_kv_compress_decode(float* kv_state, float* score_state,
                          rk::aligned16(ff->out);
     const rk::RowLaunch r = rk::row_launch(p, aligned);
     (void)hipGetLastError();
-    RK_COMPRESS_DISPATCH(rk::kv_compress_decode_kernel, dim3(1), r, (hipStream_t)stream, kv_state,
-                         score_state, *ff, p, start_pos);
+    RK_COMPRESS_DISPATCH(rk::kv_compress_decode_kernel, dim3(1), r, p.ents, (hipStream_t)stream,
+                         kv_state, score_state, *ff, p, start_pos);
     return rk::launch_status();
 }

@@ -1,7 +1,8 @@
 """The compressor's pooling stage on the device against the CPU oracle. The deposit is copies
 and one add: bit-exact. Pooling, norm and rotation go through expf and a block reduction, so
 the bar is the reference's own for these kernels: at most 2 bf16 codes apart
-(crates/engine/tests/v4_compressor/metric.rs, CLEAN_ULP = 2), with almost every element equal."""
+(crates/engine/tests/v4_compressor/metric.rs, CLEAN_ULP = 2), with almost every element equal;
+values that cancelled to almost nothing are compared absolutely (tests/v4_cases.py)."""
 import ctypes as C
 
 import numpy as np
@@ -10,7 +11,7 @@ import pytest
 from oracle.kvoracle import CompGeom as OracleGeom
 from rivoli_amd import hip
 from tests.gpu_util import back, dev, dzeros, ref_kernels
-from tests.v4_cases import bf16_gap, compress_inputs
+from tests.v4_cases import compress_gap, compress_inputs
 
 pytestmark = pytest.mark.gpu
 CLEAN_ULP = 2
@@ -38,8 +39,8 @@ def device_prefill(hg, kv, score, ape, norm, freqs, nblk, launch=None):
     return back(out, np.float32).reshape(nblk, hg.d)
 
 
-def assert_clean(oracle, got, want, what):
-    gap = bf16_gap(oracle, got, want)
+def assert_clean(oracle, got, want, what, rd):
+    gap = compress_gap(oracle, got, want, rd)
     assert gap.max() <= CLEAN_ULP and np.mean(gap > 0) < 0.01, (what, int(gap.max()), float(np.mean(gap > 0)))
 
 
@@ -55,12 +56,12 @@ def test_prefill_matches_oracle(oracle, ratio, d, rd, s):
     code, want = oracle.kv_compress_prefill(kv, score, ape, norm, freqs, og, nblk)
     assert code == 0
     got = device_prefill(hg, kv, score, ape, norm, freqs, nblk)
-    assert_clean(oracle, got, want, f"ratio {ratio} d {d}")
+    assert_clean(oracle, got, want, f"ratio {ratio} d {d}", rd)
     ref = ref_kernels()
     if ref is not None and hasattr(ref, "rivoli_kv_compress_prefill") and d <= 1024:
         # the reference's own kernel, compiled for this GPU, agrees with the oracle too
         theirs = device_prefill(hg, kv, score, ape, norm, freqs, nblk, launch=ref.rivoli_kv_compress_prefill)
-        assert_clean(oracle, theirs, want, f"reference kernel, ratio {ratio} d {d}")
+        assert_clean(oracle, theirs, want, f"reference kernel, ratio {ratio} d {d}", rd)
 
 
 def test_masked_and_peaked_windows(oracle):
@@ -72,7 +73,7 @@ def test_masked_and_peaked_windows(oracle):
     code, want = oracle.kv_compress_prefill(kv, score, ape, norm, freqs, og, 16)
     got = device_prefill(hg, kv, score, ape, norm, freqs, 16)
     assert code == 0 and np.isfinite(want).all()
-    assert_clean(oracle, got, want, "masked / peaked")
+    assert_clean(oracle, got, want, "masked / peaked", 64)
 
 
 @pytest.mark.parametrize("ratio,d,rd,s,s0", [(4, 512, 64, 45, 14), (4, 64, 16, 30, 2), (128, 512, 64, 400, 130),
@@ -114,7 +115,7 @@ def test_deposit_and_decode_follow_the_state_machine(oracle, ratio, d, rd, s, s0
             want_blocks.append(w)
             check_states(f"after the block at {pos}")     # the slide is bit-exact too
     blocks, want_blocks = np.array(blocks), np.array(want_blocks)
-    assert_clean(oracle, blocks, want_blocks, "stepped blocks")
+    assert_clean(oracle, blocks, want_blocks, "stepped blocks", rd)
     whole = device_prefill(hg, kv, score, ape, norm, freqs, s // ratio)
     assert np.array_equal(blocks.view(np.uint32), whole.view(np.uint32))
 

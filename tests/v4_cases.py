@@ -63,3 +63,17 @@ def literal_finish(oracle, geom: CompGeom, pooled, norm, freqs, first_pos: int) 
     z = (x[:, d - rd::2] + 1j * x[:, d - rd + 1::2]) * (t[:, :, 0] + 1j * t[:, :, 1])
     x[:, d - rd::2], x[:, d - rd + 1::2] = z.real, z.imag
     return rb(x)
+
+
+def compress_gap(oracle, got: np.ndarray, want: np.ndarray, rd: int) -> np.ndarray:
+    """bf16 code distance between two sets of compressed rows, with the two places where a code
+    distance says nothing taken out: a value that is tiny against its row because the weighted
+    sum (or the rotation's a*c - b*s) cancelled carries an absolute error of the terms' size,
+    which is many codes of the small result. Such elements count as equal when they agree to
+    2^-14 of the row's largest value (2^-8 in the rotated tail, where a one-code difference of
+    an input passes straight through)."""
+    gap = bf16_gap(oracle, got, want)
+    top = np.abs(want).max(axis=1, keepdims=True)
+    tail = (np.arange(got.shape[1]) >= got.shape[1] - rd)[None, :]
+    near = np.abs(got - want) <= top * np.where(tail, 2.0 ** -8, 2.0 ** -14)
+    return np.where(near, np.minimum(gap, 2), gap)
