@@ -97,6 +97,53 @@ def build_cases(oracle) -> dict:
                           "table_fnv": fnv(oracle, table4), "pool_fnv": fnv(oracle, pool4),
                           "selected_fnv": fnv(oracle, sel4), "selected_q0_head": [int(v) for v in sel4[0, :6]],
                           "gather_rows_fnv": fnv(oracle, out4)}
+    g.update(second_format_cases(oracle))
+    return g
+
+
+def second_format_inputs(oracle):
+    """Seeded inputs of the second cache format's cases, from the reference tests' own
+    generator (crates/engine/tests/common/reference.rs:141-162)."""
+    from oracle.kvoracle import CompGeom
+
+    lcg = oracle.lcg(0x5EED0006)
+    rows = (lcg.fill(24 * 512) * np.float32(2.0)).reshape(24, 512)
+    rows[3, 64:128] = 0.0                                   # an all-zero block: the amax floor
+    rows[5] *= np.float32(200.0)
+    scores = lcg.fill(24 * 40).reshape(24, 40)
+    scores[:, ::5] = np.float32(0.25)                       # ties
+    geom = CompGeom.attention(4, 64, 16)
+    kv, score = lcg.fill(16 * geom.cd).reshape(16, geom.cd), lcg.fill(16 * geom.cd).reshape(16, geom.cd)
+    ape, norm = lcg.fill(4 * geom.cd).reshape(4, geom.cd), np.float32(1.0) + np.float32(0.1) * lcg.fill(geom.d)
+    ang = np.arange(16, dtype=np.float64)[:, None] * (10000.0 ** (-np.arange(8) / 8.0))[None, :]
+    freqs = np.stack([np.cos(ang), np.sin(ang)], axis=-1).reshape(16, 16).astype(np.float32)
+    return rows, scores, (geom, kv, score, ape, norm, freqs)
+
+
+def second_format_cases(oracle) -> dict:
+    from tests.test_oracle_v4 import reference_tie_block
+
+    rows, scores, (geom, kv, score, ape, norm, freqs) = second_format_inputs(oracle)
+    g = {}
+    # the reference's tie fixture (crates/engine/tests/kernel_v4_quant.rs:283-296), in full
+    code, tie = oracle.act_quant_f8_prefix(reference_tie_block()[None, :], 64, 64)
+    assert code == 0
+    g["act_quant_tie_block_u32"] = hexs(tie.view(np.uint32))
+    code, q = oracle.act_quant_f8_prefix(rows, 448, 64)
+    assert code == 0
+    g["act_quant_rows"] = {"rows_fnv": fnv(oracle, rows), "fnv": fnv(oracle, q),
+                           "row0_head_u32": hexs(q[0, :8].view(np.uint32))}
+    sel_p = oracle.v4_scored_rows(scores, 4, 4, True, 128)
+    sel_d = oracle.v4_scored_rows(scores, 4, 6, False, 128)
+    g["scored_rows"] = {"scores_fnv": fnv(oracle, scores), "prefill_fnv": fnv(oracle, sel_p),
+                        "prefill_row23": [int(v) for v in sel_p[23]], "prefill_row9": [int(v) for v in sel_p[9]],
+                        "decode_fnv": fnv(oracle, sel_d), "decode_row0": [int(v) for v in sel_d[0]]}
+    # the compressor pooling: a small overlapping case in full (the device matches it to within
+    # two bf16 codes, not bit for bit)
+    code, out = oracle.kv_compress_prefill(kv, score, ape, norm, freqs, geom, 4)
+    assert code == 0
+    g["compress_prefill_ratio4"] = {"kv_fnv": fnv(oracle, kv), "score_fnv": fnv(oracle, score),
+                                    "out_u32": hexs(out.view(np.uint32))}
     return g
 
 
@@ -105,7 +152,9 @@ def main() -> None:
     rc = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "not gpu",
                          os.path.join(ROOT, "tests", "test_oracle_codecs.py"),
                          os.path.join(ROOT, "tests", "test_oracle_quant.py"),
-                         os.path.join(ROOT, "tests", "test_oracle_topk_hash.py")], cwd=ROOT).returncode
+                         os.path.join(ROOT, "tests", "test_oracle_topk_hash.py"),
+                         os.path.join(ROOT, "tests", "test_oracle_v4.py"),
+                         os.path.join(ROOT, "tests", "test_oracle_v4_compress.py")], cwd=ROOT).returncode
     if rc != 0:
         sys.exit("the oracle does not pass its known-answer tests: no vectors written")
     from oracle.kvoracle import oracle as get_oracle

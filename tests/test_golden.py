@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from tests.golden import inputs
-from tests.golden.make_golden import OUT, PT, W, build_cases, fnv, hexs
+from tests.golden.make_golden import OUT, PT, W, build_cases, fnv, hexs, second_format_inputs
 from tests.test_oracle_quant import fixture_a99e
 from tests.topk_cases import reference_topk_cases
 
@@ -37,6 +37,14 @@ def test_golden_known_values(golden):
     assert golden["subnormal_tie_codes"] == [1, 3, 5, 7, 8]
     assert golden["index_topk_cases"]["k > nt (wrapper clamp)"]["n"] == 500
     assert golden["index_topk_cases"]["ReLU-sparse (prefix answer)"]["head"] == [0, 1, 2, 3, 4, 5]
+    # second cache format: the tie block's 448 survives, its half quanta went to the even side
+    # (crates/engine/tests/kernel_v4_quant.rs:283-343); a prefill row of the selection is the
+    # positional fill while its limit is within the cap (crates/engine/src/v4/select.rs:645-676)
+    tie = np.frombuffer(bytes.fromhex(golden["act_quant_tie_block_u32"]), np.uint32).view(np.float32)
+    q = 2.0 ** -9
+    assert tie[0] == 448.0 and (tie[[2, 4, 6, 8, 10]] / q).tolist() == [-0.0, -2.0, -2.0, -4.0, -4.0]
+    assert golden["scored_rows"]["prefill_row9"] == [128, 129, -1, -1]
+    assert sorted(golden["scored_rows"]["prefill_row23"]) == golden["scored_rows"]["prefill_row23"]
 
 
 @pytest.mark.gpu
@@ -121,3 +129,40 @@ def test_device_reproduces_golden(oracle, golden):
     hip.launch_kv_gather_rows_paged(pool4, dev(table4), sel, None, out4, n_q, k4, table4.shape[1], W, PT,
                                     table4.size)
     assert fnv(oracle, back(out4, np.uint16)) == g["gather_rows_fnv"]
+
+
+@pytest.mark.gpu
+def test_device_reproduces_second_format_golden(oracle, golden):
+    from rivoli_amd import hip
+    from tests.gpu_util import back, dev, dzeros
+    from tests.test_oracle_v4 import reference_tie_block
+    from tests.v4_cases import compress_gap
+
+    rows, scores, (geom, kv, score, ape, norm, freqs) = second_format_inputs(oracle)
+    tie = dev(reference_tie_block())
+    hip.launch_act_quant_f8_prefix(tie, tie, 1, 64, 64, 64)
+    assert hexs(back(tie, np.uint32)) == golden["act_quant_tie_block_u32"]
+    g = golden["act_quant_rows"]
+    assert fnv(oracle, rows) == g["rows_fnv"]
+    rows_d = dev(rows)
+    hip.launch_act_quant_f8_prefix(rows_d, rows_d, 24, 512, 448, 64)
+    got = back(rows_d, np.uint32).reshape(24, 512)
+    assert fnv(oracle, got) == g["fnv"] and hexs(got[0, :8]) == g["row0_head_u32"]
+
+    g = golden["scored_rows"]
+    assert fnv(oracle, scores) == g["scores_fnv"]
+    for prefill, cap, key, row, idx in ((True, 4, "prefill_fnv", "prefill_row23", 23),
+                                        (False, 6, "decode_fnv", "decode_row0", 0)):
+        out = dzeros(24 * cap * 4, 0xEE)
+        hip.launch_index_select_blocks(dev(scores), 24, 40, 4, cap, prefill, 128, out)
+        sel = back(out, np.int32).reshape(24, cap)
+        assert fnv(oracle, sel) == g[key] and [int(v) for v in sel[idx]] == g[row]
+
+    g = golden["compress_prefill_ratio4"]
+    assert fnv(oracle, kv) == g["kv_fnv"] and fnv(oracle, score) == g["score_fnv"]
+    out = dzeros(4 * geom.d * 4)
+    norm_d, freqs_d = dev(norm), dev(freqs)
+    hip.launch_kv_compress_prefill(dev(kv), dev(score), dev(ape), hip.CompFinish.of(norm_d, freqs_d, out),
+                                   hip.CompGeom.build(4, 64, 16, 1e-6), 4)
+    want = np.frombuffer(bytes.fromhex(g["out_u32"]), np.uint32).view(np.float32).reshape(4, geom.d)
+    assert compress_gap(oracle, back(out, np.float32).reshape(4, geom.d), want, 16).max() <= 2
