@@ -81,36 +81,44 @@ __device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
 }
 
 // The append quantizer divides by the row scale before encoding: code = rule(RN(x / scl)).
-// A correctly rounded divide costs ~11 instructions, so the fast path multiplies by the
-// correctly rounded reciprocal instead: q' = RN(x * RN(1/scl)) is within 3 ulps of RN(x/scl)
-// (two roundings of 2^-24 relative each against one). The e4m3 code of both is the same
-// unless a rounding tie lies between them; ties sit where the 20 dropped mantissa bits equal
-// 0x80000, so a q' farther than 8 ulps from that pattern, inside the hardware converter's
-// exact domain, is safe to convert directly. Everything else takes the exact divide and the
-// software encoder. Requires scl and 1/scl normal and finite (the caller checks the row).
-__device__ __forceinline__ bool quotient_needs_exact(float q) {
-    const uint32_t b = __float_as_uint(q);
-    const float a = fabsf(q);
-    const bool out_of_domain = !(a >= 0.015625f) && a != 0.0f;  // subnormal band, or NaN
-    const bool near_tie = ((b & 0x000fffffu) - 0x0007fff8u) < 16u;
-    return out_of_domain || near_tie;
-}
+// A correctly rounded divide costs ~11 instructions; the fast path gets the same quotient in
+// three: with y = RN(1 / scl) (one divide per row), q0 = RN(x * y), r = fma(-q0, scl, x) (the
+// exact residual) and q = fma(r, y, q0), q IS RN(x / scl) (Markstein's correction of a
+// reciprocal product). x is a bf16 and scl = RN(amax / 448) with amax a bf16, so the claim
+// depends only on two 8-bit mantissas and the exponent gap: it was checked over all of them in
+// exact rational arithmetic, and the device is checked the same way against the oracle's divide
+// (every amax mantissa against every value below it). It needs the residual to stay a normal
+// number, which row_scale_is_fast guarantees. With the exact quotient in hand, gfx950's
+// v_cvt_pk_fp8_f32 (nearest even everywhere) is the reference's encoder wherever that one is
+// nearest-even too: 2^-6 <= |q| (|q| <= 448 * (1 + 2^-22) always, since |x| <= amax) or q == 0.
+// A chunk with a quotient in the subnormal band (the reference rounds those ties AWAY), or a
+// NaN, takes the divide and the integer encoder.
+__device__ __forceinline__ bool row_scale_is_fast(float scl) { return scl >= 1e-20f && scl <= 1e20f; }
 
 // Eight consecutive bf16 (four dwords) -> eight e4m3 codes (two dwords) under one row scale.
+// The two conditions are folded over the eight quotients as an unsigned minimum and maximum of
+// their bit patterns (no per-element compare, select or mask logic) and tested once:
+//   0 < |q| < 2^-6   <=> min over (|bits| - 1) < 0x3c7fffff      (zero wraps to the top)
+//   NaN              <=> max over |bits| > 0x7f800000
 __device__ __forceinline__ u32x2 quantize8(const uint32_t (&w)[4], float scl, float rinv,
                                            bool row_fast) {
     float x[8], q[8];
-    bool exact = !row_fast;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         x[2 * i] = bf16_lo_to_f32(w[i]);
         x[2 * i + 1] = bf16_hi_to_f32(w[i]);
     }
+    uint32_t low = 0xffffffffu, top = 0u;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        q[i] = x[i] * rinv;
-        exact = exact || quotient_needs_exact(q[i]);
+        const float q0 = x[i] * rinv;
+        // the sign is x's (scl > 0); taking it from x keeps -0.0, which (-0) + (+0) loses
+        q[i] = __builtin_copysignf(__builtin_fmaf(__builtin_fmaf(-q0, scl, x[i]), rinv, q0), x[i]);
+        const uint32_t mag = __float_as_uint(q[i]) & 0x7fffffffu;
+        low = min(low, mag - 1u);
+        top = max(top, mag);
     }
+    const bool exact = !row_fast || low < 0x3c7fffffu || top > 0x7f800000u;
     if (!exact) {
         u32x2 r = {e4m3x4_hw(q[0], q[1], q[2], q[3]), e4m3x4_hw(q[4], q[5], q[6], q[7])};
         return r;

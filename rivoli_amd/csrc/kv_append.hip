@@ -10,9 +10,13 @@
 // way the amax is a max over registers, LDS and wave butterflies — exact and order-free, so
 // it equals the reference's LDS tree bit for bit.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
+#include <type_traits>
+
 #include "codec.hpp"
 
 namespace rk {
+
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kAppendWaves = 4;   // linear-slab kernel: tokens per workgroup
 constexpr int kRowsPerWave = 8;   // paged kernel: tokens per (one-wave) workgroup
@@ -74,20 +78,33 @@ __global__ __launch_bounds__(kWave) void kv_append_paged_kernel(
         s_dst[lane] = dst;
         s_sdst[lane] = sdst;
     }
+    // Row maxima. |bf16| patterns order like the values they encode, so the chunk maxima are
+    // packed 16-bit integer maxima (one AND and one packed max per two elements) and every
+    // later step compares bit patterns. A NaN's pattern sorts above infinity, while the rule's
+    // max ignores NaNs: a row whose maximum comes out a NaN is folded again with float maxima.
+    auto row_maxima = [&](auto as_bits) {
+        constexpr bool kBits = decltype(as_bits)::value;
 #pragma unroll
-    for (int j = 0; j < MAXJ; ++j) {
-        const int c = lane + j * kWave;
-        if (c < n_chunks) {
-            const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
-            float m = 0.0f;
+        for (int j = 0; j < MAXJ; ++j) {
+            const int c = lane + j * kWave;
+            if (c < n_chunks) {
+                const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+                if constexpr (kBits) {
+                    u16x2 m = {0, 0};
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                m = fmaxf(m, fmaxf(fabsf(bf16_lo_to_f32(w[i])), fabsf(bf16_hi_to_f32(w[i]))));
-            s_amax[c] = m;
+                    for (int i = 0; i < 4; ++i)
+                        m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2, w[i] & 0x7fff7fffu));
+                    s_amax[c] = __uint_as_float((uint32_t)max(m.x, m.y) << 16);
+                } else {
+                    float m = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        m = fmaxf(m, fmaxf(fabsf(bf16_lo_to_f32(w[i])), fabsf(bf16_hi_to_f32(w[i]))));
+                    s_amax[c] = m;
+                }
+            }
         }
-    }
-    __syncthreads();
-    {
+        __syncthreads();
         // lane = (row, part): each of a row's 8 lanes folds a slice of its chunk maxima
         const int r = lane >> 3, part = lane & 7;
         const int per = (cpr + 7) >> 3;
@@ -97,18 +114,31 @@ __global__ __launch_bounds__(kWave) void kv_append_paged_kernel(
 #pragma unroll
             for (int i = 0; i < PER_MAX; ++i) {  // independent LDS reads, not a dependent loop
                 const int at = part * per + i;
-                if (i < per && at < cpr) m = fmaxf(m, s_amax[r * cpr + at]);
+                if (i < per && at < cpr) {
+                    const float v = s_amax[r * cpr + at];
+                    m = kBits ? __uint_as_float(max(__float_as_uint(m), __float_as_uint(v))) : fmaxf(m, v);
+                }
             }
         }
-        m = fmaxf(m, __shfl_xor(m, 1, kWave));
-        m = fmaxf(m, __shfl_xor(m, 2, kWave));
-        m = fmaxf(m, __shfl_xor(m, 4, kWave));
+#pragma unroll
+        for (int off = 1; off < 8; off <<= 1) {
+            const float o = __shfl_xor(m, off, kWave);
+            m = kBits ? __uint_as_float(max(__float_as_uint(m), __float_as_uint(o))) : fmaxf(m, o);
+        }
+        return m;
+    };
+    float m = row_maxima(std::true_type{});
+    if (__any(__float_as_uint(m) > 0x7f800000u)) {  // some row holds a NaN
+        __syncthreads();
+        m = row_maxima(std::false_type{});
+    }
+    {
+        const int r = lane >> 3, part = lane & 7;
         if (part == 0 && r < nrows) {
             const float scl = m > 0.0f ? m / 448.0f : 1.0f;
             s_scl[r] = scl;
             s_rinv[r] = 1.0f / scl;
-            // the reciprocal shortcut needs scl and 1/scl comfortably normal and finite
-            s_fast[r] = (scl >= 1e-30f && scl <= 1e30f) ? 1 : 0;
+            s_fast[r] = row_scale_is_fast(scl) ? 1 : 0;
         }
     }
     __syncthreads();
@@ -173,7 +203,7 @@ __global__ __launch_bounds__(kAppendWaves* kWave) void kv_append_paged_token_ker
     amax = wave_max(amax);
     const float scl = amax > 0.0f ? amax / 448.0f : 1.0f;
     const float rinv = 1.0f / scl;
-    const bool row_fast = scl >= 1e-30f && scl <= 1e30f;
+    const bool row_fast = row_scale_is_fast(scl);
 
     const int page = slot / page_tokens;
     const int off = slot - page * page_tokens;

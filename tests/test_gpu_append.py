@@ -123,7 +123,7 @@ def test_config2_prefill_bulk_append_with_outlier_rows(oracle):
 
 
 def test_append_rounding_ties_saturation_and_special_rows(oracle):
-    f32 = np.zeros((16, W), np.float32)
+    f32 = np.zeros((19, W), np.float32)
     q = np.float32(2.0 ** -10)
     # row 0: a 448 pins scale == 1; the rest are multiples and half-multiples of the subnormal
     # quantum in both signs, so exact subnormal ties reach the encoder
@@ -141,11 +141,19 @@ def test_append_rounding_ties_saturation_and_special_rows(oracle):
     f32[6, 17] *= 200.0                                    # one outlier crushes the rest
     f32[7, 5] = 3.0                                        # single non-zero
     f32[8] = np.random.default_rng(4).standard_normal(W) * 200.0   # the x200 outlier-token case
-    f32[9:] = np.random.default_rng(5).standard_normal((7, W)) * np.float32(2.0) ** np.arange(-60, 61, 20)[:, None]
+    f32[9:16] = np.random.default_rng(5).standard_normal((7, W)) * np.float32(2.0) ** np.arange(-60, 61, 20)[:, None]
+    # NaNs do not take part in the row maximum and encode as 0x7f; an infinity makes the scale
+    # infinite (finite values -> 0, the infinity itself -> NaN -> 0x7f)
+    f32[16:19] = np.random.default_rng(6).standard_normal((3, W))
+    f32[16, [3, 200, 575]] = np.nan
+    f32[17, 40] = np.inf
+    f32[18, 7], f32[18, 300] = -np.inf, np.nan
     rows = f32_to_bf16_rne(f32)
-    slots = np.arange(16, dtype=np.int32) * 3
+    slots = np.arange(19, dtype=np.int32) * 3
     got, want, bad, _ = paged_append_both(oracle, rows, slots, 1)
     assert bad == 0 and np.array_equal(got, want)
+    nan_row = want[16 * 3 * W: (16 * 3 + 1) * W]
+    assert (nan_row[[3, 200, 575]] & 0x7F).tolist() == [0x7F] * 3 and (nan_row == 0x7E).any() | (nan_row == 0xFE).any()
     codes0 = want[: W]
     assert {1, 3, 5, 7}.issubset(set(codes0.tolist()))      # half-away results are present
     # anti-vacuity: nearest-even on those ties would have produced a different row
