@@ -95,31 +95,42 @@ __device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
 // NaN, takes the divide and the integer encoder.
 __device__ __forceinline__ bool row_scale_is_fast(float scl) { return scl >= 1e-20f && scl <= 1e20f; }
 
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+// The band test is made on the inputs, where it is a packed 16-bit compare: q < 2^-6 needs
+// |x| < scl * 2^-6, and |bf16| patterns order like their values, so every such x has a pattern
+// <= T = bits(scl * 2^-6) >> 16. A chunk is sent to the exact path when some non-zero |x| has a
+// pattern <= T + 1 (one pattern of slack; the exact path is right for any input). A row whose
+// scale is not fast gets the band 0x10000, which every pattern is below.
+__device__ __forceinline__ uint32_t row_band(float scl) {
+    return row_scale_is_fast(scl) ? (__float_as_uint(scl * 0.015625f) >> 16) + 1u : 0x10000u;
+}
+
 // Eight consecutive bf16 (four dwords) -> eight e4m3 codes (two dwords) under one row scale.
-// The two conditions are folded over the eight quotients as an unsigned minimum and maximum of
-// their bit patterns (no per-element compare, select or mask logic) and tested once:
-//   0 < |q| < 2^-6   <=> min over (|bits| - 1) < 0x3c7fffff      (zero wraps to the top)
-//   NaN              <=> max over |bits| > 0x7f800000
+// Per two elements the test costs an AND, a packed subtract, a packed min and a packed max:
+//   some 0 < |x| pattern <= band - 1   <=> min over (|pattern| - 1, wrapping zero to 0xffff) < band
+//   some NaN                           <=> max over |pattern| > 0x7f80
 __device__ __forceinline__ u32x2 quantize8(const uint32_t (&w)[4], float scl, float rinv,
-                                           bool row_fast) {
+                                           uint32_t band) {
+    u16x2 low = {0xffff, 0xffff}, top = {0, 0};
+    const u16x2 one = {1, 1};
     float x[8], q[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
+        const u16x2 mag = __builtin_bit_cast(u16x2, w[i] & 0x7fff7fffu);
+        low = __builtin_elementwise_min(low, mag - one);
+        top = __builtin_elementwise_max(top, mag);
         x[2 * i] = bf16_lo_to_f32(w[i]);
         x[2 * i + 1] = bf16_hi_to_f32(w[i]);
     }
-    uint32_t low = 0xffffffffu, top = 0u;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const float q0 = x[i] * rinv;
-        // the sign is x's (scl > 0); taking it from x keeps -0.0, which (-0) + (+0) loses
-        q[i] = __builtin_copysignf(__builtin_fmaf(__builtin_fmaf(-q0, scl, x[i]), rinv, q0), x[i]);
-        const uint32_t mag = __float_as_uint(q[i]) & 0x7fffffffu;
-        low = min(low, mag - 1u);
-        top = max(top, mag);
-    }
-    const bool exact = !row_fast || low < 0x3c7fffffu || top > 0x7f800000u;
+    const bool exact = (uint32_t)min(low.x, low.y) < band || max(top.x, top.y) > 0x7f80;
     if (!exact) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float q0 = x[i] * rinv;
+            // q0 - (q0 * scl - x) * rinv: the residual with this sign keeps a -0.0 input -0.0
+            q[i] = __builtin_fmaf(-__builtin_fmaf(q0, scl, -x[i]), rinv, q0);
+        }
         u32x2 r = {e4m3x4_hw(q[0], q[1], q[2], q[3]), e4m3x4_hw(q[4], q[5], q[6], q[7])};
         return r;
     }

@@ -16,8 +16,6 @@
 
 namespace rk {
 
-typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-
 constexpr int kAppendWaves = 4;   // linear-slab kernel: tokens per workgroup
 constexpr int kRowsPerWave = 8;   // paged kernel: tokens per (one-wave) workgroup
 constexpr int kMaxChunksPerRow = 128;  // width <= 1024
@@ -33,7 +31,10 @@ constexpr int kBulkAppendTokens = RIVOLI_BULK_APPEND_TOKENS;
 // that is 8 x 72 = 576 chunks, exactly 9 per lane, so no lane idles and every load is a full
 // 1 KiB wave access. Per-chunk maxima go through LDS to a segmented reduce (8 lanes per row),
 // which is exact and order-free like the reference's LDS tree; one lane per row derives the
-// scale, its reciprocal and the row's destination. Codes leave as 8-byte stores.
+// scale, its reciprocal and the row's destination. Codes leave as 8-byte nontemporal stores
+// (nothing here is read again; measured 6 % faster than plain stores). With the arithmetic
+// hidden (a variant that skips it runs no faster), the kernel moves its 2:1 read:write mix at
+// the rate this part gives any such copy.
 // CPR = chunks per row at compile time (0 = runtime, up to 128).
 template <int CPR>
 __global__ __launch_bounds__(kWave) void kv_append_paged_kernel(
@@ -44,8 +45,7 @@ __global__ __launch_bounds__(kWave) void kv_append_paged_kernel(
                              : kRowsPerWave * kMaxChunksPerRow / kWave;
     constexpr unsigned long long kSkip = ~0ull;
     __shared__ float s_amax[kRowsPerWave * (CPR ? CPR : kMaxChunksPerRow)];
-    __shared__ float s_scl[kRowsPerWave], s_rinv[kRowsPerWave];
-    __shared__ int s_fast[kRowsPerWave];
+    __shared__ u32x4 s_row[kRowsPerWave];  // scale, its reciprocal, the exact-path band (bits)
     __shared__ unsigned long long s_dst[kRowsPerWave], s_sdst[kRowsPerWave];
 
     const int cpr = CPR ? CPR : width >> 3;
@@ -136,9 +136,8 @@ __global__ __launch_bounds__(kWave) void kv_append_paged_kernel(
         const int r = lane >> 3, part = lane & 7;
         if (part == 0 && r < nrows) {
             const float scl = m > 0.0f ? m / 448.0f : 1.0f;
-            s_scl[r] = scl;
-            s_rinv[r] = 1.0f / scl;
-            s_fast[r] = row_scale_is_fast(scl) ? 1 : 0;
+            const u32x4 row = {__float_as_uint(scl), __float_as_uint(1.0f / scl), row_band(scl), 0u};
+            s_row[r] = row;
         }
     }
     __syncthreads();
@@ -150,14 +149,15 @@ __global__ __launch_bounds__(kWave) void kv_append_paged_kernel(
             const unsigned long long dst = s_dst[r];
             if (dst != kSkip) {
                 const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
-                reinterpret_cast<u32x2*>(pool + dst)[col] =
-                    quantize8(w, s_scl[r], s_rinv[r], s_fast[r] != 0);
+                const u32x4 row = s_row[r];
+                __builtin_nontemporal_store(quantize8(w, __uint_as_float(row.x), __uint_as_float(row.y), row.z),
+                                            reinterpret_cast<u32x2*>(pool + dst) + col);
             }
         }
     }
     // the scales last: a global store ahead of a barrier would make the barrier wait for it
     if (lane < nrows && s_dst[lane] != kSkip)
-        *reinterpret_cast<float*>(pool + s_sdst[lane]) = s_scl[lane];
+        *reinterpret_cast<float*>(pool + s_sdst[lane]) = __uint_as_float(s_row[lane].x);
 }
 
 // Paged append, low-latency form for small batches (decode steps, short prefill chunks): one
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(kAppendWaves* kWave) void kv_append_paged_token_ker
     amax = wave_max(amax);
     const float scl = amax > 0.0f ? amax / 448.0f : 1.0f;
     const float rinv = 1.0f / scl;
-    const bool row_fast = row_scale_is_fast(scl);
+    const uint32_t band = row_band(scl);
 
     const int page = slot / page_tokens;
     const int off = slot - page * page_tokens;
@@ -214,7 +214,7 @@ __global__ __launch_bounds__(kAppendWaves* kWave) void kv_append_paged_token_ker
         int c = lane + s * kWave;
         if (c < n_chunks) {
             const uint32_t w[4] = {raw[s].x, raw[s].y, raw[s].z, raw[s].w};
-            dst[c] = quantize8(w, scl, rinv, row_fast);
+            dst[c] = quantize8(w, scl, rinv, band);
         }
     }
     if (lane == 0)
