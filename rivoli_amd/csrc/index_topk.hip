@@ -920,19 +920,32 @@ static int index_topk_launch(const float* scores, int n_queries, int stride, con
 // ---------------------------------------------------------------------------------------------
 //
 // A prefill asks for thousands of short selections at once (a row has at most n_comp scores,
-// a few thousand), the opposite of the one long query topk_block is built for: its LDS
-// histograms cost more to clear and fold than such a row costs to read. select_bisect keeps a
-// row's keys in registers (a wave owns a contiguous run, 64 per step) and finds the k-th
-// largest key by bisection on its bits, most significant first: count the keys >= candidate
-// (a compare and an add per key, one cross-lane sum per step), keep the bit when at least k
-// remain. A count of exactly k ends the search early — that candidate already separates the
-// selection — which on distinct scores happens after ~log2(spread / spacing) bits, about half
-// of the 32. No LDS traffic besides one word per wave per step when a row spans several waves.
+// a few thousand), the opposite of the one long query topk_block is built for: its replicated
+// LDS histograms cost more to clear and fold than such a row costs to read. select_bisect
+// keeps a row's keys in registers (a wave owns a contiguous run, 64 per step) and finds the
+// k-th largest key in two stages. The top 10 bits (sign, exponent, first mantissa bit) come
+// from one plain 1024-bin LDS histogram, one atomic per key, walked from the top by one wave.
+// The other 22 bits are found by bisection, most significant first — count the keys >=
+// candidate, keep the bit when enough remain, stop as soon as a count is exactly what is
+// needed (on distinct scores after ~log2(spread / spacing) bits) — over the members of the
+// pivot bin only: they are listed in LDS (over the histogram, which is no longer needed) and
+// one wave bisects them from its registers, a handful per lane. A bin too full to list (heavy
+// ties) is bisected over all the keys instead. The selection is then emitted in index order
+// by ballots and prefix counts.
+//
+constexpr int kSelBits = 10;               // key bits resolved by the histogram
+constexpr int kSelBins = 1 << kSelBits;
+constexpr int kSelLow = 32 - kSelBits;
+constexpr int kSelCand = 1024;             // pivot-bin members listed in LDS
+constexpr int kSelMisc = 4 * 16 + 8;       // per-wave slots (up to 16 waves) and the pivot record
+constexpr int kSelLdsWords = kSelMisc + (kSelBins > kSelCand ? kSelBins : kSelCand);
+
 template <int WAVES, int ITEMS, class KEY>
 __device__ __forceinline__ void select_bisect(const float* __restrict__ s, int nt, uint32_t kq,
                                               uint32_t* __restrict__ out, uint32_t* lds,
                                               uint32_t add) {
-    // requires 1 <= kq < nt <= WAVES * 64 * ITEMS
+    // requires 1 <= kq < nt <= WAVES * 64 * ITEMS; lds holds kSelLdsWords words
+    for (int i = threadIdx.x; i < kSelBins; i += WAVES * kWave) lds[kSelMisc + i] = 0u;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int per_wave = ((nt + WAVES * kWave - 1) / (WAVES * kWave)) * kWave;
@@ -948,6 +961,7 @@ __device__ __forceinline__ void select_bisect(const float* __restrict__ s, int n
         for (int j = 0; j < ITEMS; ++j)
             key[j] = j * kWave < limit ? KEY::of(sp[j * kWave]) : 0u;
     }
+    __syncthreads();  // the histogram is clear
     // keys >= cand over the whole row, cand >= 1 (so the zero keys of absent elements never
     // count). `turn` alternates the LDS slots so that one barrier per call is enough.
     auto count_ge = [&](uint32_t cand, int turn) -> uint32_t {
@@ -973,24 +987,146 @@ __device__ __forceinline__ void select_bisect(const float* __restrict__ s, int n
         return c;
     };
 
-    // T: select key > T, and the first `need` (in index order) of key == T
-    uint32_t p = 0, T = 0, need = 0;
-    bool exact = false;
-    for (int b = 31; b >= 0; --b) {
-        const uint32_t cand = p | (1u << b);
-        const uint32_t c = count_ge(cand, b);
-        if (c >= kq) p = cand;
-        if (c == kq) {
-            exact = true;
-            T = cand - 1u;
-            break;
+    // ---- the top kSelBits of the k-th largest key, by one LDS histogram -----------------------
+    // (sign, exponent and the first mantissa bit of a score): one atomic per key instead of a
+    // bisection step per bit. s_hist was cleared and a barrier passed before this point.
+    uint32_t* s_hist = lds + kSelMisc;
+    uint32_t* s_cand = s_hist;  // the list reuses the histogram once the pivot bin is known
+    uint32_t* s_pv = lds + 4 * WAVES;  // [0] pivot bin, [1] keys in higher bins, [2] keys in it, [3] list fill
+#pragma unroll
+    for (int j0 = 0; j0 < ITEMS; j0 += 8) {
+        if (j0 >= steps) break;
+#pragma unroll
+        for (int j = j0; j < j0 + 8 && j < ITEMS; ++j)
+            if (j * kWave < limit) atomicAdd(&s_hist[key[j] >> kSelLow], 1u);
+    }
+    __syncthreads();
+    if (wave == 0) {
+        // a lane owns 16 consecutive bins; suffix sums over the lanes find the lane where the
+        // running count from the top reaches kq, which then walks its own bins
+        uint32_t c[kSelBins / kWave], mine = 0;
+#pragma unroll
+        for (int i = 0; i < kSelBins / kWave; ++i) {
+            c[i] = s_hist[lane * (kSelBins / kWave) + i];
+            mine += c[i];
+        }
+        uint32_t suffix = mine;  // inclusive of this lane, over lanes >= lane
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const uint32_t v = __shfl_down(suffix, off, kWave);
+            if (lane + off < kWave) suffix += v;
+        }
+        const uint32_t above_lane = suffix - mine;
+        if (above_lane < kq && kq <= suffix) {
+            uint32_t acc = above_lane;
+            int i = kSelBins / kWave - 1;
+            for (; i > 0; --i) {
+                if (acc + c[i] >= kq) break;
+                acc += c[i];
+            }
+            s_pv[0] = (uint32_t)(lane * (kSelBins / kWave) + i);
+            s_pv[1] = acc;
+            s_pv[2] = c[i];
+            s_pv[3] = 0u;
         }
     }
-    if (!exact) {
-        // p is the k-th largest key: count(key >= p) > kq > count(key > p)
-        T = p;
-        const uint32_t above = p == 0xffffffffu ? 0u : count_ge(p + 1u, 1);  // bit 0 used slot 0
-        need = kq - above;
+    __syncthreads();
+    const uint32_t pbin = s_pv[0], above_bin = s_pv[1], in_bin = s_pv[2];
+    const uint32_t need_in_bin = kq - above_bin;  // 1 <= need_in_bin <= in_bin
+
+    // T: select key > T, and the first `need` (in index order) of key == T
+    uint32_t T = 0, need = 0;
+    if (need_in_bin == in_bin) {
+        T = (pbin << kSelLow) - 1u;  // the whole bin is selected (pbin == 0 would need every key: kq < nt)
+    } else if (in_bin <= (uint32_t)kSelCand) {
+        // ---- the other bits among the bin's members only: they are listed (any order) in LDS
+        // and one wave bisects them from registers
+        uint32_t fill = 0;  // where this wave's members start in the list
+        if constexpr (WAVES > 1) {
+            uint32_t mine = 0;
+#pragma unroll
+            for (int j0 = 0; j0 < ITEMS; j0 += 8) {
+                if (j0 >= steps) break;
+#pragma unroll
+                for (int j = j0; j < j0 + 8 && j < ITEMS; ++j)
+                    mine += (uint32_t)__popcll(__ballot(j * kWave < limit && (key[j] >> kSelLow) == pbin));
+            }
+            uint32_t* s_cnt = lds;  // the count_ge slots are idle here
+            if (lane == 0) s_cnt[wave] = mine;
+            __syncthreads();
+            for (int w = 0; w < wave; ++w) fill += s_cnt[w];
+        }
+#pragma unroll
+        for (int j0 = 0; j0 < ITEMS; j0 += 8) {
+            if (j0 >= steps) break;
+#pragma unroll
+            for (int j = j0; j < j0 + 8 && j < ITEMS; ++j) {
+                const bool is = j * kWave < limit && (key[j] >> kSelLow) == pbin;
+                const unsigned long long m = __ballot(is);
+                if (is) s_cand[fill + lanes_below(m)] = key[j];
+                fill += (uint32_t)__popcll(m);
+            }
+        }
+        __syncthreads();
+        if (wave == 0) {
+            constexpr int CP = kSelCand / kWave;
+            uint32_t ck[CP];
+            const int csteps = ((int)in_bin + kWave - 1) / kWave;
+#pragma unroll
+            for (int i = 0; i < CP; ++i) ck[i] = (i * kWave + lane) < (int)in_bin ? s_cand[i * kWave + lane] : 0u;
+            auto cand_ge = [&](uint32_t cand) -> uint32_t {  // cand >= 1
+                uint32_t c = 0;
+#pragma unroll
+                for (int i = 0; i < CP; ++i)
+                    if (i < csteps) c += (uint32_t)__popcll(__ballot(ck[i] >= cand));
+                return c;
+            };
+            uint32_t p = pbin << kSelLow, t = 0, nd = 0;
+            bool exact = false;
+            for (int b = kSelLow - 1; b >= 0; --b) {
+                const uint32_t cand = p | (1u << b);
+                const uint32_t c = cand_ge(cand);
+                if (c >= need_in_bin) p = cand;
+                if (c == need_in_bin) {
+                    exact = true;
+                    t = cand - 1u;
+                    break;
+                }
+            }
+            if (!exact) {
+                // p is the need_in_bin-th largest member: members >= p outnumber it, members > p do not
+                t = p;
+                const uint32_t higher = (p & ((1u << kSelLow) - 1u)) == ((1u << kSelLow) - 1u) ? 0u : cand_ge(p + 1u);
+                nd = need_in_bin - higher;
+            }
+            if (lane == 0) {
+                s_pv[0] = t;
+                s_pv[1] = nd;
+            }
+        }
+        __syncthreads();
+        T = s_pv[0];
+        need = s_pv[1];
+    } else {
+        // ---- a bin too full to list (heavy ties): bisect its bits over all the keys
+        uint32_t p = pbin << kSelLow;
+        bool exact = false;
+        for (int b = kSelLow - 1; b >= 0; --b) {
+            const uint32_t cand = p | (1u << b);
+            const uint32_t c = count_ge(cand, b);
+            if (c >= kq) p = cand;
+            if (c == kq) {
+                exact = true;
+                T = cand - 1u;
+                break;
+            }
+        }
+        if (!exact) {
+            // p is the k-th largest key: count(key >= p) > kq > count(key > p)
+            T = p;
+            const uint32_t above = p == 0xffffffffu ? 0u : count_ge(p + 1u, 1);  // bit 0 used slot 0
+            need = kq - above;
+        }
     }
 
     uint32_t cnt_gt = 0, cnt_eq = 0;
@@ -1027,14 +1163,19 @@ __device__ __forceinline__ void select_bisect(const float* __restrict__ s, int n
             const bool e = live && key[j] == T;
             const unsigned long long mg = __ballot(g), me = __ballot(e);
             const uint32_t G = run_gt + lanes_below(mg);
-            const uint32_t E = run_eq + lanes_below(me);
-            const uint32_t slot = G + (E < need ? E : need);
             // slot < kq holds by construction; the compare keeps a wrong threshold from ever
             // turning into a write outside the caller's buffer
-            if ((g || (e && E < need)) && slot < kq)
-                out[slot] = (uint32_t)(seg0 + j * kWave + lane) + add;
+            if (me == 0ull) {  // no key equal to the threshold in this step: the usual case
+                const uint32_t slot = G + (run_eq < need ? run_eq : need);
+                if (g && slot < kq) out[slot] = (uint32_t)(seg0 + j * kWave + lane) + add;
+            } else {
+                const uint32_t E = run_eq + lanes_below(me);
+                const uint32_t slot = G + (E < need ? E : need);
+                if ((g || (e && E < need)) && slot < kq)
+                    out[slot] = (uint32_t)(seg0 + j * kWave + lane) + add;
+                run_eq += (uint32_t)__popcll(me);
+            }
             run_gt += (uint32_t)__popcll(mg);
-            run_eq += (uint32_t)__popcll(me);
         }
     }
 }
@@ -1054,7 +1195,7 @@ template <int WAVES, int ITEMS>
 __global__ __launch_bounds__(WAVES* kWave) void block_select_bisect_kernel(
     const float* __restrict__ scores, int n_comp, int ratio, int prefill, int k, int offset,
     int32_t* __restrict__ out) {
-    __shared__ uint32_t lds[4 * WAVES];
+    __shared__ uint32_t lds[kSelLdsWords];
     const int t = blockIdx.x;
     const int limit = select_row_limit(t, n_comp, ratio, prefill);
     int32_t* o = out + (size_t)t * k;
