@@ -1,7 +1,6 @@
 """Pins the oracle's element codecs against the reference's own known-answer tests and against
 checks that share no line with the encoder (nearest-value brute force, closed forms)."""
 import numpy as np
-import pytest
 
 
 def all_e4m3_values():
