@@ -206,17 +206,26 @@ def main():
 
 
 def timed(torch, stream, steps, warmup, step):
-    """Warm up, then time `steps` calls of step(events) with HIP events on `stream`."""
+    """Warm up, time `steps` calls of step(None) with one HIP event pair around all of them (the
+    step time), then run the same `steps` calls again as step(events) with every kernel
+    bracketed by its own event pair (the per-kernel times). The two passes are separate because
+    an event pair per launch keeps the launches of a short step from queueing ahead of the
+    device: the bracketed pass of the configuration 4 step takes 2.9 ms where the plain one
+    takes 2.1 ms."""
     for _ in range(warmup):
         step(None)
     stream.synchronize()
     torch.cuda.synchronize()
     t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    events = {}
     t0.record(stream)
     for _ in range(steps):
-        step(events)
+        step(None)
     t1.record(stream)
+    stream.synchronize()
+    torch.cuda.synchronize()
+    events = {}
+    for _ in range(steps):
+        step(events)
     stream.synchronize()
     torch.cuda.synchronize()
     per_kernel = {k: float(np.mean([a.elapsed_time(b) for a, b in v])) for k, v in events.items()}
