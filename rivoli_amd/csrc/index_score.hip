@@ -34,14 +34,21 @@ constexpr int kScoreBlocks = 16;     // 32-token blocks per wave
 constexpr int kScoreTokensPerGroup = kScoreWaves * kScoreBlocks * 32;
 constexpr int kScoreRowPad = 8;      // bf16 of padding per staged query row
 
-// RB = 32-head row blocks (1 or 2).
-template <int RB>
+// RB = 32-head row blocks (1 or 2). HD = the head dimension at compile time (128, the shipped
+// one) or 0 for the runtime value: with it the chunk-to-row divisions are shifts (with a runtime
+// width they were two thirds of the kernel's vector instructions), the K loop has a constant
+// trip count, and the head halves of the query's operand fragments (the same for every block
+// of tokens) are read from LDS once and kept in registers instead of being re-read per block:
+// two of every five LDS reads of the runtime form. Keeping the remainder halves as well leaves
+// room for one wave per SIMD and is no faster; neither is a second block in flight per wave.
+template <int RB, int HD>
 __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
     const float* __restrict__ q, const float* __restrict__ w,
     const uint16_t* __restrict__ kpool, const int* __restrict__ block_table,
     const int* __restrict__ nts, const unsigned int* __restrict__ heads, int max_blocks_per_seq,
-    int stride, int nt_all, int nh, int nact, int hd, int page_tokens, int n_pages, float wscale,
+    int stride, int nt_all, int nh, int nact, int hd_rt, int page_tokens, int n_pages, float wscale,
     float dscale, float* __restrict__ scores) {
+    const int hd = HD ? HD : hd_rt;
     __shared__ __attribute__((aligned(16))) uint16_t s_qh[RB * 32][kScoreMaxHd + kScoreRowPad];
     __shared__ __attribute__((aligned(16))) uint16_t s_ql[RB * 32][kScoreMaxHd + kScoreRowPad];
     __shared__ float s_w[RB * 32];
@@ -95,6 +102,15 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
     const int col = lane & 31;        // the lane's token within a block / head within a row block
     const int khalf = (lane >> 5) * 8;  // which 8 of each 16-wide K-step this lane carries
     const int ksteps = hd >> 4;
+    constexpr int KS = HD ? HD / 16 : 1;
+    bf16x8 qh[RB][KS];
+    if constexpr (HD != 0) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int s = 0; s < KS; ++s)
+                qh[rb][s] = *reinterpret_cast<const bf16x8*>(&s_qh[rb * 32 + col][khalf + 16 * s]);
+    }
     // accumulator element v of a lane is head row 8*(v/4) + 4*(lane/32) + v%4, token `col`:
     // the lane's 16 (32) head weights are fixed for the whole kernel, so they sit in registers
     float wv[RB][16];
@@ -167,8 +183,11 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
                 const bf16x8 kb = *reinterpret_cast<const bf16x8*>(&tile[col][khalf + 16 * s]);
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb) {
-                    const bf16x8 ah =
-                        *reinterpret_cast<const bf16x8*>(&s_qh[rb * 32 + col][khalf + 16 * s]);
+                    bf16x8 ah;
+                    if constexpr (HD != 0)
+                        ah = qh[rb][s];
+                    else
+                        ah = *reinterpret_cast<const bf16x8*>(&s_qh[rb * 32 + col][khalf + 16 * s]);
                     const bf16x8 al =
                         *reinterpret_cast<const bf16x8*>(&s_ql[rb * 32 + col][khalf + 16 * s]);
                     acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, kb, acc[rb], 0, 0, 0);
@@ -225,14 +244,16 @@ static int index_score_launch(const float* q, const float* w, const unsigned sho
     dim3 grid((unsigned)((nt + kScoreTokensPerGroup - 1) / kScoreTokensPerGroup),
               (unsigned)n_queries);
     (void)hipGetLastError();
-    if (nact <= 32)
-        hipLaunchKernelGGL(index_score_kernel<1>, grid, dim3(kScoreThreads), 0, stream, q, w, kpool,
-                           block_table, nts, heads, max_blocks_per_seq, stride, nt, nh, nact, hd,
-                           page_tokens, n_pages, wscale, dscale, scores);
-    else
-        hipLaunchKernelGGL(index_score_kernel<2>, grid, dim3(kScoreThreads), 0, stream, q, w, kpool,
-                           block_table, nts, heads, max_blocks_per_seq, stride, nt, nh, nact, hd,
-                           page_tokens, n_pages, wscale, dscale, scores);
+#define RK_SCORE(RBV, HDV)                                                                      \
+    hipLaunchKernelGGL((index_score_kernel<RBV, HDV>), grid, dim3(kScoreThreads), 0, stream, q, w, \
+                       kpool, block_table, nts, heads, max_blocks_per_seq, stride, nt, nh, nact,  \
+                       hd, page_tokens, n_pages, wscale, dscale, scores)
+    if (hd == 128) {
+        if (nact <= 32) RK_SCORE(1, 128); else RK_SCORE(2, 128);
+    } else {
+        if (nact <= 32) RK_SCORE(1, 0); else RK_SCORE(2, 0);
+    }
+#undef RK_SCORE
     return launch_status();
 }
 
