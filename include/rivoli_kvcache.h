@@ -224,6 +224,41 @@ int rivoli_act_quant_f8_prefix(const float* src, float* dst, int rows, int row_s
 int rivoli_index_select_blocks(const float* scores, int rows, int n_comp, int ratio,
                                int index_topk, int prefill, int offset, int* out, void* stream);
 
+/* Selection rectangles (crates/engine/src/v4/select.rs:334-488, Sel::shape / Sel::gather /
+ * Sel::gather_scored, which the reference fills on the host and uploads per call): one row per
+ * query, [window columns | compressed columns], -1 for a masked cell; the index-list attention
+ * below reads it as is. The phase is start_pos == 0 (prefill: seqlen rows, values are absolute
+ * positions, the last `win` up to the query's own) or not (decode: one row, values are ring
+ * slots oldest first, slot p % win holding position p; slots not yet written are -1).
+ * Compressed columns are block + offset with offset = seqlen at prefill and win at decode
+ * (select.rs:268-270); at prefill query t may read block c only if c < (t + 1) / ratio.
+ * ratio == 0 is a layer without a compressor, ratio == 4 the class with an indexer
+ * (crates/engine/src/v4/geometry.rs:86-92,128-130).
+ * rivoli_sel_shape is pure host arithmetic: rows, and cols = window columns (min(seqlen, win) at
+ * prefill, win at decode) + (start_pos + rows) / ratio. rivoli_sel_gather fills that rectangle
+ * with the positional rule (every closed block). rivoli_sel_gather_scored fills the window
+ * columns and then the k = min(index_topk, n_comp) columns of rivoli_index_select_blocks over
+ * scores [rows][n_comp]; *cols_out (host, optional) receives window columns + k.
+ * Guards: 1001 null / win <= 0 / seqlen <= 0 / negative arguments (gather_scored: ratio == 0,
+ * nothing to rank); 1002 more than 65535 query rows; 1005 decode with seqlen != 1
+ * (select.rs:78-86); 1006 positional selection on the indexed class with more closed blocks
+ * than index_topk (select.rs:363-383: the scored form is how that is answered). */
+int rivoli_sel_shape(int win, int ratio, int index_topk, int seqlen, int start_pos, int* rows,
+                     int* cols);
+int rivoli_sel_gather(int win, int ratio, int index_topk, int seqlen, int start_pos, int* out,
+                      void* stream);
+int rivoli_sel_gather_scored(const float* scores, int n_comp, int win, int ratio, int index_topk,
+                             int seqlen, int start_pos, int* out, int* cols_out, void* stream);
+
+/* Replaces the device copies of crates/engine/src/v4/attn.rs:343-378 (write_ring) with one
+ * launch: cache is the layer's [win][hd] f32 ring, kv the step's rows ([seqlen][hd] at prefill,
+ * one row at decode). Decode writes slot start_pos % win; a prompt seeds slot t % win with
+ * position t for its last min(seqlen, win) positions. kv and cache must not overlap.
+ * Guards: 1001, 1005 as above. Which buffer the attention then indexes is the caller's rule
+ * (the prompt's own rows at prefill, the cache at decode). */
+int rivoli_kv_ring_write(const float* kv, float* cache, int win, int hd, int seqlen,
+                         int start_pos, void* stream);
+
 /* The compressor's pooling stage (crates/backend/kernels/kvcompress.hip; Rust rows
  * launch_kv_compress_deposit / _prefill / _decode, crates/backend/src/hip_attn.rs:547-605).
  * The two structs cross the boundary by pointer, as in the reference (kvcompress.hip:40-48,

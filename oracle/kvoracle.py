@@ -114,6 +114,57 @@ class _V4Mixin:
         return out
 
 
+    def sel_shape(self, win: int, ratio: int, index_topk: int, seqlen: int, start_pos: int):
+        """(code, rows, cols) of a positional selection rectangle."""
+        rows, cols = C.c_int(0), C.c_int(0)
+        code = int(self.lib.ro_sel_shape(win, ratio, index_topk, seqlen, start_pos, C.byref(rows),
+                                         C.byref(cols)))
+        return code, rows.value, cols.value
+
+    def sel_gather(self, win: int, ratio: int, index_topk: int, seqlen: int, start_pos: int):
+        """(code, int32 [rows, cols]) — window columns then the positional compressed columns."""
+        code, rows, cols = self.sel_shape(win, ratio, index_topk, seqlen, start_pos)
+        if code:
+            return code, None
+        out = np.full((rows, cols), -7, np.int32)
+        code = int(self.lib.ro_sel_gather(win, ratio, index_topk, seqlen, start_pos, _ptr(out, C.c_int32)))
+        return code, out
+
+    def sel_gather_scored(self, scores, win: int, ratio: int, index_topk: int, seqlen: int, start_pos: int):
+        """scores is [rows, n_comp] f32 (n_comp may be 0). (code, int32 [rows, cols])."""
+        scores = _c(scores, np.float32)
+        rows, n_comp = scores.shape
+        win_cols = min(seqlen, win) if start_pos == 0 else win
+        out = np.full((max(rows, 1), win_cols + min(index_topk, n_comp)), -7, np.int32)
+        cols = C.c_int(0)
+        code = int(self.lib.ro_sel_gather_scored(_ptr(scores, C.c_float) if n_comp else None, n_comp, win, ratio,
+                                                 index_topk, seqlen, start_pos, _ptr(out, C.c_int32),
+                                                 C.byref(cols)))
+        assert code or cols.value == out.shape[1]
+        return code, (None if code else out)
+
+    def ring_write(self, kv, cache, win: int, seqlen: int, start_pos: int) -> int:
+        """Updates cache ([win, hd] f32) in place from kv ([rows, hd] f32)."""
+        kv = _c(kv, np.float32)
+        assert cache.dtype == np.float32 and cache.flags.c_contiguous and cache.shape == (win, kv.shape[1])
+        return int(self.lib.ro_ring_write(_ptr(kv, C.c_float), _ptr(cache, C.c_float), win, kv.shape[1], seqlen,
+                                          start_pos))
+
+    def sparse_attn(self, q, kv, sink, idxs, scale: float) -> np.ndarray:
+        """q [m, h, d], kv [rows, d], sink [h], idxs int32 [m, topk] -> o [m, h, d] (bf16-valued f32)."""
+        q, kv, sink = _c(q, np.float32), _c(kv, np.float32), _c(sink, np.float32)
+        idxs = _c(idxs, np.int32)
+        m, h, d = q.shape
+        assert idxs.shape[0] == m and kv.shape[1] == d and sink.shape == (h,)
+        assert idxs.max(initial=-1) < kv.shape[0]
+        o = np.empty((m, h, d), np.float32)
+        code = int(self.lib.ro_sparse_attn(_ptr(q, C.c_float), _ptr(kv, C.c_float), _ptr(sink, C.c_float),
+                                           _ptr(idxs, C.c_int32), m, h, d, idxs.shape[1], scale,
+                                           _ptr(o, C.c_float)))
+        assert code == 0, code
+        return o
+
+
 class Oracle(_V4Mixin):
     def __init__(self, path: str = LIB_PATH):
         if not os.path.exists(path):
@@ -158,6 +209,11 @@ class Oracle(_V4Mixin):
             "ro_fast_round_scale": (C.c_float, [C.c_float, C.c_float]),
             "ro_act_quant_f8_prefix": (C.c_int, [f32p, f32p] + [C.c_int] * 4),
             "ro_v4_scored_rows": (C.c_int, [f32p] + [C.c_int] * 6 + [i32p]),
+            "ro_sel_shape": (C.c_int, [C.c_int] * 5 + [C.POINTER(C.c_int)] * 2),
+            "ro_sel_gather": (C.c_int, [C.c_int] * 5 + [i32p]),
+            "ro_sel_gather_scored": (C.c_int, [f32p] + [C.c_int] * 6 + [i32p, C.POINTER(C.c_int)]),
+            "ro_ring_write": (C.c_int, [f32p, f32p] + [C.c_int] * 4),
+            "ro_sparse_attn": (C.c_int, [f32p, f32p, f32p, i32p] + [C.c_int] * 4 + [C.c_float, f32p]),
             "ro_compress_guard": (C.c_int, [C.POINTER(CompGeom)]),
             "ro_kv_compress_deposit": (C.c_int, [f32p] * 5 + [C.POINTER(CompGeom), C.c_int, C.c_int]),
             "ro_kv_compress_prefill": (C.c_int, [f32p] * 6 + [C.POINTER(CompGeom), C.c_int]),

@@ -145,11 +145,155 @@ int ro_v4_scored_rows(const float* scores, int rows, int n_comp, int ratio, int 
     return k;
 }
 
+static inline float round_bf16(float x) { return ro_bf16_to_f32(ro_f32_to_bf16(x)); }
+
+/* ------------------------------------------------------------------------------------------
+ * Selection rectangles, the ring write, the index-list attention
+ * ---------------------------------------------------------------------------------------- */
+
+int ro_sel_shape(int win, int ratio, int index_topk, int seqlen, int start_pos, int* rows,
+                 int* cols) {
+    if (win <= 0 || seqlen <= 0 || start_pos < 0 || ratio < 0 || index_topk < 0) return 1001;
+    const int prefill = start_pos == 0;
+    if (!prefill && seqlen != 1) return 1005;
+    const int q = prefill ? seqlen : 1;
+    const int win_cols = prefill ? (seqlen < win ? seqlen : win) : win;
+    int n_comp = 0;
+    if (ratio > 0) {
+        n_comp = (start_pos + q) / ratio;
+        if (ratio == 4 && n_comp > index_topk) return 1006;
+    }
+    if (rows) *rows = q;
+    if (cols) *cols = win_cols + n_comp;
+    return 0;
+}
+
+/* one window cell: select.rs:195-216 */
+static int32_t window_cell(int win, int seqlen, int start_pos, int t, int j) {
+    if (start_pos == 0) {
+        int first = t - (win - 1);
+        if (first < 0) first = 0;
+        const int v = first + j;
+        return v <= t ? v : -1;
+    }
+    if (start_pos >= win - 1) return (start_pos % win + 1 + j) % win;
+    (void)seqlen;
+    return j <= start_pos ? j : -1;
+}
+
+static void window_fill(int win, int seqlen, int start_pos, int q, int win_cols, int cols,
+                        int32_t* out) {
+    for (int t = 0; t < q; ++t)
+        for (int j = 0; j < win_cols; ++j)
+            out[(size_t)t * cols + j] = window_cell(win, seqlen, start_pos, t, j);
+}
+
+int ro_sel_gather(int win, int ratio, int index_topk, int seqlen, int start_pos, int32_t* out) {
+    int q, cols;
+    const int code = ro_sel_shape(win, ratio, index_topk, seqlen, start_pos, &q, &cols);
+    if (code) return code;
+    if (!out) return 1001;
+    const int prefill = start_pos == 0;
+    const int win_cols = prefill ? (seqlen < win ? seqlen : win) : win;
+    const int offset = prefill ? seqlen : win;
+    window_fill(win, seqlen, start_pos, q, win_cols, cols, out);
+    for (int t = 0; t < q; ++t)
+        for (int c = 0; c < cols - win_cols; ++c) {
+            const int legal = prefill ? c < (t + 1) / ratio : 1;
+            out[(size_t)t * cols + win_cols + c] = legal ? c + offset : -1;
+        }
+    return 0;
+}
+
+int ro_sel_gather_scored(const float* scores, int n_comp, int win, int ratio, int index_topk,
+                         int seqlen, int start_pos, int32_t* out, int* cols_out) {
+    if (win <= 0 || seqlen <= 0 || start_pos < 0 || ratio <= 0 || index_topk < 0 || n_comp < 0)
+        return 1001;
+    const int prefill = start_pos == 0;
+    if (!prefill && seqlen != 1) return 1005;
+    if (!out || (n_comp > 0 && !scores)) return 1001;
+    const int q = prefill ? seqlen : 1;
+    const int win_cols = prefill ? (seqlen < win ? seqlen : win) : win;
+    const int k = index_topk < n_comp ? index_topk : n_comp;
+    const int cols = win_cols + k;
+    if (cols_out) *cols_out = cols;
+    window_fill(win, seqlen, start_pos, q, win_cols, cols, out);
+    if (k > 0) {
+        int32_t* comp = (int32_t*)malloc((size_t)q * k * sizeof(int32_t));
+        ro_v4_scored_rows(scores, q, n_comp, ratio, index_topk, prefill, prefill ? seqlen : win,
+                          comp);
+        for (int t = 0; t < q; ++t)
+            memcpy(out + (size_t)t * cols + win_cols, comp + (size_t)t * k, (size_t)k * 4);
+        free(comp);
+    }
+    return 0;
+}
+
+int ro_ring_write(const float* kv, float* cache, int win, int hd, int seqlen, int start_pos) {
+    if (!kv || !cache || win <= 0 || hd <= 0 || seqlen <= 0 || start_pos < 0) return 1001;
+    if (start_pos != 0 && seqlen != 1) return 1005;
+    const size_t row = (size_t)hd * sizeof(float);
+    if (start_pos != 0) {
+        memcpy(cache + (size_t)(start_pos % win) * hd, kv, row);
+        return 0;
+    }
+    if (seqlen <= win) {
+        memcpy(cache, kv, (size_t)seqlen * row);
+        return 0;
+    }
+    const int cut = seqlen % win;
+    memcpy(cache + (size_t)cut * hd, kv + (size_t)(seqlen - win) * hd, (size_t)(win - cut) * row);
+    if (cut > 0) memcpy(cache, kv + (size_t)(seqlen - cut) * hd, (size_t)cut * row);
+    return 0;
+}
+
+int ro_sparse_attn(const float* q, const float* kv, const float* sink, const int32_t* idxs, int m,
+                   int h, int d, int topk, float scale, float* o) {
+    if (!q || !kv || !sink || !idxs || !o || m <= 0 || h <= 0 || d <= 0 || topk <= 0) return 1001;
+    float* logits = (float*)malloc((size_t)topk * sizeof(float));
+    float* acc = (float*)malloc((size_t)d * sizeof(float));
+    for (int t = 0; t < m; ++t) {
+        const int32_t* ix = idxs + (size_t)t * topk;
+        for (int hh = 0; hh < h; ++hh) {
+            const float* qh = q + ((size_t)t * h + hh) * d;
+            float* dst = o + ((size_t)t * h + hh) * d;
+            float mx = -INFINITY;
+            for (int j = 0; j < topk; ++j) {
+                logits[j] = -INFINITY;
+                if (ix[j] < 0) continue;
+                const float* k = kv + (size_t)ix[j] * d;
+                float a = 0.0f;
+                for (int i = 0; i < d; ++i) a += qh[i] * k[i];
+                const float l = a * scale;
+                if (l > mx) mx = l; /* f32::max: a NaN logit loses */
+                logits[j] = l;
+            }
+            if (!isfinite(mx)) {
+                for (int i = 0; i < d; ++i) dst[i] = NAN;
+                continue;
+            }
+            float sum = 0.0f;
+            for (int i = 0; i < d; ++i) acc[i] = 0.0f;
+            for (int j = 0; j < topk; ++j) {
+                if (ix[j] < 0) continue;
+                const float e = expf(logits[j] - mx);
+                sum += e;
+                const float* k = kv + (size_t)ix[j] * d;
+                for (int i = 0; i < d; ++i) acc[i] += e * k[i];
+            }
+            sum += expf(sink[hh] - mx);
+            for (int i = 0; i < d; ++i) dst[i] = round_bf16(acc[i] / sum);
+        }
+    }
+    free(logits);
+    free(acc);
+    return 0;
+}
+
 /* ------------------------------------------------------------------------------------------
  * The compressor's pooling stage
  * ---------------------------------------------------------------------------------------- */
 
-static inline float round_bf16(float x) { return ro_bf16_to_f32(ro_f32_to_bf16(x)); }
 
 int ro_compress_guard(const ro_comp_geom* p) {
     if (p->ratio <= 1 || p->d <= 0 || p->rd <= 0 || p->coff < 1 || p->coff > 2) return 1001;

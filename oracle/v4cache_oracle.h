@@ -35,6 +35,22 @@
  *                         below the cap the row is offset+0..limit-1 then -1; three-way tie
  *                         keeps the lower indices; a prefill row cannot take a block that
  *                         closed after it) and a brute-force sort under f32 total order
+ *   ro_sel_shape / ro_sel_gather / ro_sel_gather_scored
+ *                         the reference's own unit cases (select.rs:514-808: multi-row decode
+ *                         refused; full ring read oldest first; ring not yet full padded; the
+ *                         prefill causal rule for blocks; the indexed layer's cap; below the
+ *                         cap the scored fill equals the positional one byte for byte; the
+ *                         rectangle shapes of five layer/phase cases) and a literal per-cell
+ *                         restatement in Python
+ *   ro_ring_write         the three arms of crates/engine/src/v4/attn.rs:343-378 against the
+ *                         rule "slot t % win holds position t" for every live position
+ *   ro_sparse_attn        closed forms (one live slot -> the row over 1 + exp(sink - logit);
+ *                         equal rows -> that row times the softmax mass; sink = -inf -> the
+ *                         plain softmax average), a float64 numpy softmax on random cases,
+ *                         masked slots never dereferenced, a fully masked query -> NaN
+ *                         (crates/backend/kernels/attn.hip:344-351). The reference's goldens
+ *                         for this kernel are captured at test time from its frozen model
+ *                         oracle (crates/engine/tests/kernel_v4_attend.rs); it stores none.
  */
 #ifndef RIVOLI_V4CACHE_ORACLE_H
 #define RIVOLI_V4CACHE_ORACLE_H
@@ -72,6 +88,40 @@ int ro_act_quant_f8_prefix(const float* src, float* dst, int rows, int row_strid
  * out is [rows][k]. Returns k, or -1 for a non-positive argument. */
 int ro_v4_scored_rows(const float* scores, int rows, int n_comp, int ratio, int index_topk,
                       int prefill, int offset, int32_t* out);
+
+/* crates/engine/src/v4/select.rs:334-400 (Sel::shape, Sel::n_comp): rows = seqlen at prefill
+ * (start_pos == 0), 1 at decode; cols = window columns (min(seqlen, win) at prefill, win at
+ * decode) + compressed columns ((start_pos + rows) / ratio; none when ratio == 0). Returns 0, or
+ * 1001 (win <= 0, seqlen <= 0, negative start_pos / ratio / index_topk), 1005 (decode with
+ * seqlen != 1: select.rs:78-86), 1006 (ratio == 4, the indexed class of geometry.rs:86-92,
+ * 128-130, with more live blocks than index_topk: the positional rule refuses, select.rs:363-383). */
+int ro_sel_shape(int win, int ratio, int index_topk, int seqlen, int start_pos, int* rows,
+                 int* cols);
+/* select.rs:395-408 Sel::gather = window_rows (:195-216) ‖ compressed_rows (:224-241) at
+ * compress_offset (:268-270), row-major [rows][cols] with -1 for masked cells. Returns
+ * ro_sel_shape's code and writes nothing when it is non-zero. */
+int ro_sel_gather(int win, int ratio, int index_topk, int seqlen, int start_pos, int32_t* out);
+/* select.rs:418-434 Sel::gather_scored over scored_rows(scores [rows][n_comp]) : the same window
+ * fill, then the min(index_topk, n_comp) scored columns. cols_out receives the row width.
+ * Returns 0, 1001 (as above, or ratio == 0: a scored selection needs a compressor), 1005. */
+int ro_sel_gather_scored(const float* scores, int n_comp, int win, int ratio, int index_topk,
+                         int seqlen, int start_pos, int32_t* out, int* cols_out);
+
+/* crates/engine/src/v4/attn.rs:343-378 write_ring: decode copies kv row 0 into slot
+ * start_pos % win; a prompt of s <= win rows seeds slots [0, s); a longer one seeds every slot
+ * with the last win positions, position t in slot t % win. cache is [win][hd]. Returns 0 or
+ * 1001 / 1005 as ro_sel_shape. */
+int ro_ring_write(const float* kv, float* cache, int win, int hd, int seqlen, int start_pos);
+
+/* crates/oracles/src/v4oracle/attention.rs:118-193 sparse_attn / attn_head (device twin
+ * gather_attn_shared_kv, crates/backend/kernels/attn.hip:358-443): for query t < m and head
+ * hh < h, over the slots j < topk with idxs[t*topk + j] >= 0 in ascending j:
+ * logit = (sum_i q[i] * kv[idx][i], ascending i) * scale; mx their maximum;
+ * e = expf(logit - mx); sum += e; acc[i] += e * kv[idx][i]; then sum += expf(sink[hh] - mx)
+ * and o = bf16_round(acc[i] / sum). A query with no live slot gets NaN (the device kernel's
+ * rule; the reference's CPU oracle asserts instead). o is [m][h][d]. Returns 0 or 1001. */
+int ro_sparse_attn(const float* q, const float* kv, const float* sink, const int32_t* idxs, int m,
+                   int h, int d, int topk, float scale, float* o);
 
 /* ---- the compressor's pooling stage: crates/backend/kernels/kvcompress.hip:103-384 and its
  * launchers :386-478; CPU statement crates/oracles/src/v4oracle/compress.rs:42-199 with

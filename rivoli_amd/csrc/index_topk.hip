@@ -1194,11 +1194,11 @@ __device__ __forceinline__ bool select_positional(int32_t* o, int limit, int k, 
 template <int WAVES, int ITEMS>
 __global__ __launch_bounds__(WAVES* kWave) void block_select_bisect_kernel(
     const float* __restrict__ scores, int n_comp, int ratio, int prefill, int k, int offset,
-    int32_t* __restrict__ out) {
+    int32_t* __restrict__ out, int out_stride) {
     __shared__ uint32_t lds[kSelLdsWords];
     const int t = blockIdx.x;
     const int limit = select_row_limit(t, n_comp, ratio, prefill);
-    int32_t* o = out + (size_t)t * k;
+    int32_t* o = out + (size_t)t * out_stride;
     if (select_positional<WAVES * kWave>(o, limit, k, offset)) return;
     select_bisect<WAVES, ITEMS, TotalOrderKey>(scores + (size_t)t * n_comp, limit, (uint32_t)k,
                                                reinterpret_cast<uint32_t*>(o), lds,
@@ -1210,32 +1210,36 @@ template <int THREADS, int ITEMS>
 __global__ __launch_bounds__(THREADS) void block_select_kernel(const float* __restrict__ scores,
                                                                int n_comp, int ratio, int prefill,
                                                                int k, int offset,
-                                                               int32_t* __restrict__ out) {
+                                                               int32_t* __restrict__ out,
+                                                               int out_stride) {
     __shared__ uint32_t lds[topk_block_lds_words<THREADS>()];
     const int t = blockIdx.x;
     const int limit = select_row_limit(t, n_comp, ratio, prefill);
-    int32_t* o = out + (size_t)t * k;
+    int32_t* o = out + (size_t)t * out_stride;
     if (select_positional<THREADS>(o, limit, k, offset)) return;
     topk_block<THREADS, ITEMS, TotalOrderKey>(scores + (size_t)t * n_comp, limit, (uint32_t)k,
                                               reinterpret_cast<uint32_t*>(o), lds,
                                               (uint32_t)offset);
 }
 
+// `out_stride` (>= k) is the distance between the rows of `out`: k for a bare selection, the
+// rectangle's width when the selection is the tail of a [window | compressed] row.
 static int block_select_launch(const float* scores, int rows, int n_comp, int ratio,
-                               int index_topk, int prefill, int offset, int* out,
+                               int index_topk, int prefill, int offset, int* out, int out_stride,
                                hipStream_t stream) {
     if (!scores || !out) return 1001;
     if (rows <= 0 || n_comp <= 0 || ratio <= 0 || index_topk <= 0 || offset < 0) return 1001;
     if ((long long)offset + n_comp > 0x7fffffffLL) return 1002;
     const int k = index_topk < n_comp ? index_topk : n_comp;
+    if (out_stride < k) return 1001;
     (void)hipGetLastError();
     const dim3 grid((unsigned)rows);
 #define RK_BISECT(WV, I)                                                                     \
     hipLaunchKernelGGL((block_select_bisect_kernel<WV, I>), grid, dim3(WV* kWave), 0, stream, \
-                       scores, n_comp, ratio, prefill ? 1 : 0, k, offset, out)
+                       scores, n_comp, ratio, prefill ? 1 : 0, k, offset, out, out_stride)
 #define RK_SELECT(T, I)                                                                       \
     hipLaunchKernelGGL((block_select_kernel<T, I>), grid, dim3(T), 0, stream, scores, n_comp, \
-                       ratio, prefill ? 1 : 0, k, offset, out)
+                       ratio, prefill ? 1 : 0, k, offset, out, out_stride)
     // up to 32 keys per lane; a row takes as few waves as hold it
     if (n_comp <= 64 * 8)
         RK_BISECT(1, 8);
@@ -1258,13 +1262,107 @@ static int block_select_launch(const float* scores, int rows, int n_comp, int ra
     return launch_status();
 }
 
+// ---- selection rectangles: [window columns | compressed columns] per query row --------------
+// crates/engine/src/v4/select.rs:334-400. The phase is start_pos == 0 (prefill: one row per
+// prompt position, values are absolute positions) or not (decode: one row, values are ring
+// slots). ratio == 4 is the class with an indexer (geometry.rs:86-92,128-130).
+struct SelShape {
+    int code, rows, win_cols, n_comp, offset;
+};
+static SelShape sel_shape(int win, int ratio, int seqlen, int start_pos) {
+    SelShape s = {0, 0, 0, 0, 0};
+    if (win <= 0 || seqlen <= 0 || start_pos < 0 || ratio < 0) return s.code = 1001, s;
+    const bool prefill = start_pos == 0;
+    if (!prefill && seqlen != 1) return s.code = 1005, s;
+    s.rows = prefill ? seqlen : 1;
+    s.win_cols = prefill ? (seqlen < win ? seqlen : win) : win;
+    s.n_comp = ratio > 0 ? (int)(((long long)start_pos + s.rows) / ratio) : 0;
+    s.offset = prefill ? seqlen : win;  // compress_offset, select.rs:268-270
+    return s;
+}
+
+// One thread per cell of the first `win_cols + n_pos` columns of a `cols`-wide row: the window
+// rule (select.rs:195-216), then the positional block rule (:224-241) for n_pos columns.
+__global__ __launch_bounds__(256) void sel_fill_kernel(int win, int ratio, int seqlen,
+                                                       int start_pos, int win_cols, int n_pos,
+                                                       int offset, int cols,
+                                                       int32_t* __restrict__ out) {
+    const int j = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
+    if (j >= win_cols + n_pos) return;
+    int v;
+    if (j < win_cols) {
+        if (start_pos == 0) {
+            const int first = t > win - 1 ? t - (win - 1) : 0;
+            v = first + j <= t ? first + j : -1;
+        } else if (start_pos >= win - 1) {
+            v = (start_pos % win + 1 + j) % win;  // oldest first, from just past the newest slot
+        } else {
+            v = j <= start_pos ? j : -1;
+        }
+    } else {
+        const int c = j - win_cols;
+        v = (start_pos != 0 || c < (t + 1) / ratio) ? c + offset : -1;
+    }
+    out[(size_t)t * cols + j] = v;
+}
+
+static int sel_fill_launch(const SelShape& s, int win, int ratio, int seqlen, int start_pos,
+                           int n_pos, int cols, int* out, hipStream_t stream) {
+    (void)hipGetLastError();
+    const dim3 grid((unsigned)((s.win_cols + n_pos + 255) / 256), (unsigned)s.rows);
+    if (s.rows > 65535) return 1002;
+    hipLaunchKernelGGL(sel_fill_kernel, grid, dim3(256), 0, stream, win, ratio, seqlen, start_pos,
+                       s.win_cols, n_pos, s.offset, cols, out);
+    return launch_status();
+}
+
 }  // namespace rk
+
+extern "C" int rivoli_sel_shape(int win, int ratio, int index_topk, int seqlen, int start_pos,
+                                int* rows, int* cols) {
+    if (index_topk < 0) return 1001;
+    const rk::SelShape s = rk::sel_shape(win, ratio, seqlen, start_pos);
+    if (s.code) return s.code;
+    if (ratio == 4 && s.n_comp > index_topk) return 1006;
+    if (rows) *rows = s.rows;
+    if (cols) *cols = s.win_cols + s.n_comp;
+    return 0;
+}
+
+extern "C" int rivoli_sel_gather(int win, int ratio, int index_topk, int seqlen, int start_pos,
+                                 int* out, void* stream) {
+    int rows, cols;
+    const int code = rivoli_sel_shape(win, ratio, index_topk, seqlen, start_pos, &rows, &cols);
+    if (code) return code;
+    if (!out) return 1001;
+    const rk::SelShape s = rk::sel_shape(win, ratio, seqlen, start_pos);
+    return rk::sel_fill_launch(s, win, ratio, seqlen, start_pos, s.n_comp, cols, out,
+                               (hipStream_t)stream);
+}
+
+extern "C" int rivoli_sel_gather_scored(const float* scores, int n_comp, int win, int ratio,
+                                        int index_topk, int seqlen, int start_pos, int* out,
+                                        int* cols_out, void* stream) {
+    if (ratio <= 0 || index_topk < 0 || n_comp < 0) return 1001;
+    const rk::SelShape s = rk::sel_shape(win, ratio, seqlen, start_pos);
+    if (s.code) return s.code;
+    if (!out || (n_comp > 0 && !scores)) return 1001;
+    const int k = index_topk < n_comp ? index_topk : n_comp;
+    const int cols = s.win_cols + k;
+    if (cols_out) *cols_out = cols;
+    const int code = rk::sel_fill_launch(s, win, ratio, seqlen, start_pos, 0, cols, out,
+                                         (hipStream_t)stream);
+    if (code || k == 0) return code;
+    return rk::block_select_launch(scores, s.rows, n_comp, ratio, index_topk, start_pos == 0,
+                                   s.offset, out + s.win_cols, cols, (hipStream_t)stream);
+}
 
 extern "C" int rivoli_index_select_blocks(const float* scores, int rows, int n_comp, int ratio,
                                           int index_topk, int prefill, int offset, int* out,
                                           void* stream) {
+    const int k = index_topk < n_comp ? index_topk : n_comp;
     return rk::block_select_launch(scores, rows, n_comp, ratio, index_topk, prefill, offset, out,
-                                   (hipStream_t)stream);
+                                   k, (hipStream_t)stream);
 }
 
 extern "C" size_t rivoli_index_topk_workspace_bytes(int n_queries, int nt) {

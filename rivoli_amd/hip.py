@@ -54,6 +54,10 @@ _SIGNATURES = {
     "rivoli_mla_attend_paged": [_VP] * 7 + [_I] * 8 + [_F, _I, _VP, _VP, _VP, _VP],
     "rivoli_act_quant_f8_prefix": [_VP, _VP] + [_I] * 4 + [_VP],
     "rivoli_index_select_blocks": [_VP] + [_I] * 6 + [_VP, _VP],
+    "rivoli_sel_shape": [_I] * 5 + [_VP, _VP],
+    "rivoli_sel_gather": [_I] * 5 + [_VP, _VP],
+    "rivoli_sel_gather_scored": [_VP] + [_I] * 6 + [_VP, _VP, _VP],
+    "rivoli_kv_ring_write": [_VP, _VP] + [_I] * 4 + [_VP],
     "rivoli_kv_compress_deposit": [_VP] * 6 + [_I, _I, _VP],
     "rivoli_kv_compress_prefill": [_VP] * 5 + [_I, _VP],
     "rivoli_kv_compress_decode": [_VP] * 4 + [_I, _VP],
@@ -262,6 +266,39 @@ def launch_index_select_blocks(scores, rows, n_comp, ratio, index_topk, prefill,
     ensure_hip_status(lib().rivoli_index_select_blocks(_p(scores), rows, n_comp, ratio, index_topk,
                                                        1 if prefill else 0, offset, _p(out),
                                                        _s(stream)), "index_select_blocks")
+
+
+def sel_shape(win, ratio, index_topk, seqlen, start_pos):
+    """crates/engine/src/v4/select.rs Sel::shape: (rows, cols) of the positional rectangle;
+    raises LaunchError with the guard code where the reference refuses."""
+    rows, cols = C.c_int(0), C.c_int(0)
+    ensure_hip_status(lib().rivoli_sel_shape(win, ratio, index_topk, seqlen, start_pos, C.byref(rows),
+                                             C.byref(cols)), "sel_shape")
+    return rows.value, cols.value
+
+
+def launch_sel_gather(win, ratio, index_topk, seqlen, start_pos, out, stream=NULL_STREAM):
+    """Sel::gather on the device: out is int32 [rows][cols] of sel_shape. Returns (rows, cols)."""
+    shape = sel_shape(win, ratio, index_topk, seqlen, start_pos)
+    ensure_hip_status(lib().rivoli_sel_gather(win, ratio, index_topk, seqlen, start_pos, _p(out), _s(stream)),
+                      "sel_gather")
+    return shape
+
+
+def launch_sel_gather_scored(scores, n_comp, win, ratio, index_topk, seqlen, start_pos, out,
+                             stream=NULL_STREAM):
+    """Sel::gather_scored over scored_rows on the device. Returns (rows, cols)."""
+    cols = C.c_int(0)
+    ensure_hip_status(lib().rivoli_sel_gather_scored(_p(scores), n_comp, win, ratio, index_topk, seqlen,
+                                                     start_pos, _p(out), C.byref(cols), _s(stream)),
+                      "sel_gather_scored")
+    return (seqlen if start_pos == 0 else 1), cols.value
+
+
+def launch_kv_ring_write(kv, cache, win, hd, seqlen, start_pos, stream=NULL_STREAM) -> None:
+    """crates/engine/src/v4/attn.rs write_ring as one launch."""
+    ensure_hip_status(lib().rivoli_kv_ring_write(_p(kv), _p(cache), win, hd, seqlen, start_pos, _s(stream)),
+                      "kv_ring_write")
 
 
 class CompGeom(C.Structure):

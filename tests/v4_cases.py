@@ -77,3 +77,49 @@ def compress_gap(oracle, got: np.ndarray, want: np.ndarray, rd: int) -> np.ndarr
     tail = (np.arange(got.shape[1]) >= got.shape[1] - rd)[None, :]
     near = np.abs(got - want) <= top * np.where(tail, 2.0 ** -8, 2.0 ** -14)
     return np.where(near, np.minimum(gap, 2), gap)
+
+
+def literal_sel_gather(win, ratio, seqlen, start_pos):
+    """One selection rectangle cell by cell from the rule as the reference words it
+    (crates/engine/src/v4/select.rs:195-241): at prefill the last `win` absolute positions up
+    to the query's own; at decode the ring's slots oldest first, slot p % win holding position
+    p; then every compressed block that has closed, shifted past the window region."""
+    prefill = start_pos == 0
+    rows = seqlen if prefill else 1
+    out = []
+    for t in range(rows):
+        if prefill:
+            width = min(seqlen, win)
+            live = list(range(max(0, t - win + 1), t + 1))
+            if t >= win - 1:
+                row = live
+            else:
+                row = [v if v <= t else -1 for v in range(width)]
+        else:
+            positions = list(range(max(0, start_pos - win + 1), start_pos + 1))   # oldest first
+            row = [p % win for p in positions] + [-1] * (win - len(positions))
+        if ratio:
+            if prefill:
+                closed = (t + 1) // ratio
+                row += [seqlen + c if c < closed else -1 for c in range(seqlen // ratio)]
+            else:
+                row += [win + c for c in range((start_pos + 1) // ratio)]
+        out.append(row)
+    return np.array(out, np.int32).reshape(rows, -1)
+
+
+def sparse_attn_f64(q, kv, sink, idxs, scale):
+    """The index-list attention in float64 with a library softmax shape: masked slots (-1) out,
+    the sink in the denominator only (crates/backend/kernels/attn.hip:333-343)."""
+    q, kv, sink = np.asarray(q, np.float64), np.asarray(kv, np.float64), np.asarray(sink, np.float64)
+    m, h, d = q.shape
+    out = np.empty((m, h, d))
+    for t in range(m):
+        live = [int(i) for i in idxs[t] if i >= 0]
+        rows = kv[live]
+        for hh in range(h):
+            logit = rows @ q[t, hh] * float(np.float32(scale))
+            mx = logit.max()
+            e = np.exp(logit - mx)
+            out[t, hh] = (e @ rows) / (e.sum() + np.exp(sink[hh] - mx))
+    return out
