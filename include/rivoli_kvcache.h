@@ -259,6 +259,33 @@ int rivoli_sel_gather_scored(const float* scores, int n_comp, int win, int ratio
 int rivoli_kv_ring_write(const float* kv, float* cache, int win, int hd, int seqlen,
                          int start_pos, void* stream);
 
+/* Replaces crates/backend/kernels/attn.hip:446-465 (rivoli_gather_attn_shared_kv; Rust row
+ * launch_gather_attn_shared_kv, caller crates/engine/src/v4/attn.rs:304-330), same signature:
+ * multi-query attention with one d-wide row serving as key and value for all h heads, over
+ * the explicit index list idxs [m][topk] into kv [rows][d] (-1 masks a slot, which is then
+ * never dereferenced); sink [h] joins the softmax denominator only, exp(sink - max) after the
+ * running-max shift (attn.hip:333-343); a query with no live slot gets NaN (attn.hip:344-351);
+ * o [m][h][d] is the quotient rounded to bf16, stored as f32. q is [m][h][d] f32.
+ * d == 512 with 16-byte-aligned q / kv / o takes the matrix-core kernel, which reads a query's
+ * rows once for all heads and rounds kv to bf16 on the way in — exact for cache rows, which are
+ * fp8-simulated or bf16-rounded values (crates/engine/src/v4/attn.rs:288, kvcompress.hip) — and
+ * carries q as bf16 hi + lo; any topk. Other shapes take a workgroup per (query, head) under the
+ * reference launcher's limits. Parity bar: the reference's for this kernel, 1/128 of the largest
+ * expected element (crates/engine/tests/kernel_v4_attend.rs:97-106, ATTEND_TOL).
+ * Guards: 1001 null / non-positive; 1002 d > 1024 or m > 65535 on the plain path; 1006 (d + topk)
+ * floats of LDS past 64 KiB on the plain path.
+ * _bounded: the same with n_kv = rows of kv (an index at or past it is treated as masked instead
+ * of read) and `precise` as in rivoli_mla_attend_paged: 2 = q and the softmax weights as
+ * bf16 hi + lo (what the plain name uses), 1 = q hi + lo, 0 = single bf16 (exact products when q
+ * is bf16-valued, as the model's is after its rotary), 3 = the plain f32 kernel at any width (for
+ * kv rows that are not bf16 values and must not be rounded). */
+int rivoli_gather_attn_shared_kv(const float* q, const float* kv, const float* sink,
+                                 const int* idxs, int m, int h, int d, int topk, float scale,
+                                 float* o, void* stream);
+int rivoli_gather_attn_shared_kv_bounded(const float* q, const float* kv, const float* sink,
+                                         const int* idxs, int m, int h, int d, int topk, int n_kv,
+                                         float scale, int precise, float* o, void* stream);
+
 /* The compressor's pooling stage (crates/backend/kernels/kvcompress.hip; Rust rows
  * launch_kv_compress_deposit / _prefill / _decode, crates/backend/src/hip_attn.rs:547-605).
  * The two structs cross the boundary by pointer, as in the reference (kvcompress.hip:40-48,

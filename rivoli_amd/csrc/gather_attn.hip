@@ -1,0 +1,426 @@
+// Attention over an explicit index list into ONE f32 buffer whose rows are key and value at
+// once, for every head of a query (multi-query attention with K = V): the consumer of the
+// second cache format's [ring | compressed] rows.
+//
+//     o[t][h] = bf16( sum_j p_j * kv[idx[t][j]] ),
+//     p_j = exp(l_j - mx) / (sum_j exp(l_j - mx) + exp(sink[h] - mx)),  l_j = scale * q[t][h] . kv[idx[t][j]]
+//
+// over the slots with idx >= 0 (-1 masks a slot; it is never dereferenced). The sink is part
+// of the denominator only. A query with no live slot gets NaN. This is the reference's
+// gather_attn_shared_kv (crates/backend/kernels/attn.hip:325-443, launcher :446-465), which
+// runs one workgroup per (query, head): every head re-reads the query's rows (64 times at 64
+// heads) and each thread walks a whole row for its logit.
+//
+// Here a query's rows are read ONCE for all heads. For d = 512 a 512-thread workgroup (8 waves)
+// owns a query and a block of 64 heads; waves w and w+4 share heads 16(w&3)..+15 and split the
+// 512 contraction dims of the scores and the 512 output columns between them. Slots move in
+// tiles of 32: wave w fetches the 4 rows of its tile positions (2 KiB each, fully coalesced),
+// rounds them to bf16 (exact for cache rows, which are fp8-simulated or bf16-rounded values;
+// other inputs lose bits below the 8th of the mantissa) and writes them row-major into LDS
+// once. Scores S^T[slot][head] = K . Q^T run on v_mfma_f32_16x16x32_bf16 with the tile's rows
+// as A and the wave's query heads as B, resident in registers as bf16 hi (+ lo: ~17 bits of
+// q; the softmax scale is applied to the scores, so a bf16-valued q is exact in hi alone);
+// the two halves of a pair meet through LDS. With slots as the tile's rows a lane ends
+// up with 8 slots of ONE head, which is the A layout of the value MFMA, so P never leaves
+// registers; the value operand is the same LDS tile through the transposing load
+// (ds_read_b64_tr_b16). Online softmax in base 2 with a lazily moved reference maximum; three
+// LDS tiles rotate so one barrier per tile suffices. Other widths take a plain kernel: one
+// workgroup per (query, head), a wave per logit, threads over output dims.
+// Launch-only; see include/rivoli_kvcache.h for the contract.
+#include "attend_common.hpp"
+
+namespace rk {
+
+constexpr int kGaD = 512;
+constexpr int kGaThreads = 512;
+constexpr int kGaWaves = kGaThreads / kWave;
+constexpr int kGaTile = 32;                       // slots per LDS tile
+constexpr int kGaKStepsHalf = kGaD / 32 / 2;      // 8 K-steps of the score contraction per wave of a pair
+constexpr int kGaColTilesHalf = kGaD / 16 / 2;    // 16 output column tiles per wave of a pair
+constexpr int kGaRowBytes = kGaD * 2 + 16;        // row-major tile: 1024 B of bf16 + 16 B pad
+constexpr int kGaTileBytes = kGaTile * kGaRowBytes;
+constexpr int kGaBufs = 3;
+constexpr int kGaXchBytes = 2 * kGaWaves * kWave * 8 * 4;
+constexpr int kGaSmemBytes = kGaBufs * kGaTileBytes + kGaBufs * kGaTile * 4 + kGaXchBytes;
+static_assert(kGaSmemBytes <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
+
+struct GatherAttnArgs {
+    const float* q;      // [m][h][512]
+    const float* kv;     // [rows][512]
+    const float* sink;   // [h]
+    const int* idxs;     // [m][topk]
+    int h, topk;
+    int n_kv;            // rows of kv; an index at or past it is treated as masked
+    float qscale;        // softmax scale * log2(e)
+    float* o;            // [m][h][512]
+};
+
+template <int QSPLIT, int PSPLIT>
+__global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const GatherAttnArgs a) {
+    constexpr int kFragBlock = QSPLIT == 2 ? 2 : 4;   // score side, K-steps requested together
+    constexpr int kValueAhead = QSPLIT == 2 ? 4 : 8;  // value side, fragments requested together
+    __shared__ __attribute__((aligned(16))) uint8_t smem[kGaSmemBytes];
+    const lds_ptr<uint8_t> kr = (lds_ptr<uint8_t>)smem;                     // [kGaBufs] row-major tiles
+    const lds_ptr<float> sbias = (lds_ptr<float>)(kr + kGaBufs * kGaTileBytes);  // [kGaBufs][32]: 0 or -inf
+    const lds_ptr<f32x4> xch = (lds_ptr<f32x4>)(sbias + kGaBufs * kGaTile);  // [2 parities][8 waves][64 lanes][2]
+
+    const size_t t = blockIdx.x;
+    const int hb = blockIdx.y;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hw = wave & 3;     // which 16 heads of the block
+    const int half = wave >> 2;  // which half of the contraction dims / of the output columns
+    const int g = lane >> 4, n16 = lane & 15;
+    const int n_tiles = (a.topk + kGaTile - 1) / kGaTile;
+    const int* const ix = a.idxs + t * a.topk;
+
+    // ---- this wave's half of its 16 query heads as the B operand, for the whole kernel ---
+    bf16x8 qh[kGaKStepsHalf], ql[QSPLIT == 2 ? kGaKStepsHalf : 1];
+    {
+        const int head = hb * 64 + 16 * hw + n16;
+        const bool live = head < a.h;
+        const float* qa = a.q + (t * a.h + (live ? head : 0)) * kGaD + half * (kGaD / 2) + 8 * g;
+#pragma unroll
+        for (int j = 0; j < kGaKStepsHalf; ++j) {
+            const float4* src = reinterpret_cast<const float4*>(qa + 32 * j);
+            float4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
+            if (live) v0 = src[0], v1 = src[1];
+            const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float x = v[i];  // unscaled: a bf16-valued q stays exact in its hi part
+                const __bf16 hi = (__bf16)x;
+                qh[j][i] = hi;
+                if (QSPLIT == 2) ql[j][i] = (__bf16)(x - (float)hi);
+            }
+        }
+    }
+
+    // ---- a tile's slots: lanes 0..3 hold the wave's 4 list entries ------------------------
+    const int my_pos0 = tile_pos_of(wave, 0);  // the wave's 4 slots are consecutive tile positions
+    auto list_entry = [&](int tile) -> int {
+        const int pos = tile * kGaTile + my_pos0 + (lane & 3);
+        if (lane >= 4 || pos >= a.topk) return -1;
+        const int p = ix[pos];
+        return (unsigned)p < (unsigned)a.n_kv ? p : -1;
+    };
+    float4 raw[4][2];
+    float raw_bias;  // lanes 0..3
+    auto issue_loads = [&](int entry) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int p = __builtin_amdgcn_readlane(entry, i);
+            raw[i][0] = float4{0, 0, 0, 0}, raw[i][1] = float4{0, 0, 0, 0};
+            if (p >= 0) {
+                const float4* src = reinterpret_cast<const float4*>(a.kv + (size_t)p * kGaD) + 2 * lane;
+                raw[i][0] = src[0], raw[i][1] = src[1];
+            }
+        }
+        raw_bias = entry >= 0 ? 0.0f : -INFINITY;
+    };
+    auto pack2 = [](float lo, float hi) -> uint32_t {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        const bf16x2 p = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, p);
+    };
+    auto stage = [&](int buf) {
+        const lds_ptr<uint8_t> krb = kr + buf * kGaTileBytes;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const u32x4 r = {pack2(raw[i][0].x, raw[i][0].y), pack2(raw[i][0].z, raw[i][0].w),
+                             pack2(raw[i][1].x, raw[i][1].y), pack2(raw[i][1].z, raw[i][1].w)};
+            *(lds_ptr<u32x4>)(krb + (my_pos0 + i) * kGaRowBytes + 16 * lane) = r;
+        }
+        if (lane < 4) sbias[buf * kGaTile + 4 * wave + lane] = raw_bias;
+    };
+
+    // ---- prologue: tiles 0 and 1 staged, tile 2 in registers, tile 3's entries fetched ----
+    issue_loads(list_entry(0));
+    stage(0);
+    if (n_tiles > 1) {
+        issue_loads(list_entry(1));
+        stage(1);
+    }
+    if (n_tiles > 2) issue_loads(list_entry(2));
+    int entry_next = n_tiles > 3 ? list_entry(3) : -1;
+    __syncthreads();
+
+    f32x4 o[kGaColTilesHalf];
+#pragma unroll
+    for (int nt = 0; nt < kGaColTilesHalf; ++nt) o[nt] = f32x4{0, 0, 0, 0};
+    float m_ref = -INFINITY, l_sum = 0.0f;
+
+    // Iteration t: scores of tile t -> exchange -> BARRIER -> softmax, values of tile t ->
+    // stage tile t+2 (in registers since iteration t-1) -> request tile t+3 from memory.
+    // A wave past the barrier knows that every wave has finished tile t-1 (so its LDS tile,
+    // (t+2) mod 3, may be overwritten) and has staged tile t+1.
+    int buf = 0;  // tile mod 3
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        const int entry_ahead = tile + 4 < n_tiles ? list_entry(tile + 4) : -1;
+        const lds_ptr<f32x4> xch_mine = xch + (((tile & 1) * kGaWaves + wave) * kWave + lane) * 2;
+        const lds_ptr<f32x4> xch_peer = xch + (((tile & 1) * kGaWaves + (wave ^ 4)) * kWave + lane) * 2;
+
+        // ---- scores: this wave's half of the dims, S^T[slot][head], two 16-slot halves ----
+        const lds_ptr<uint8_t> krb = kr + buf * kGaTileBytes + half * (kGaKStepsHalf * 64);
+        const lds_ptr<bf16x8> a0p = (lds_ptr<bf16x8>)(krb + n16 * kGaRowBytes + 16 * g);
+        const lds_ptr<bf16x8> a1p = (lds_ptr<bf16x8>)(krb + (16 + n16) * kGaRowBytes + 16 * g);
+        f32x4 s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0};
+#pragma unroll
+        for (int j0 = 0; j0 < kGaKStepsHalf; j0 += kFragBlock) {
+            bf16x8 fa0[kFragBlock], fa1[kFragBlock];
+#pragma unroll
+            for (int i = 0; i < kFragBlock; ++i) fa0[i] = a0p[(j0 + i) * 4], fa1[i] = a1p[(j0 + i) * 4];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < kFragBlock; ++i) {
+                const int j = j0 + i;
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[i], qh[j], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[i], qh[j], s1, 0, 0, 0);
+                if (QSPLIT == 2) {
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[i], ql[j], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[i], ql[j], s1, 0, 0, 0);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        xch_mine[0] = s0, xch_mine[1] = s1;
+        // value-side operand of column tile nt: for each of the lane's 8 contraction indices
+        // (slots 4g..4g+3 of both 16-slot halves) the value of column 16*nt' + n16. One
+        // transposing load hands a lane element e of the 8-byte chunk that lane
+        // 4e + (n16 >> 2) of its 16-lane row addressed, position n16 & 3 — so lane i
+        // addresses slot 4g + (i >> 2), columns 16*nt' + 4*(i & 3) .. +3.
+        const lds_ptr<uint8_t> vrow = kr + buf * kGaTileBytes + (4 * g + (n16 >> 2)) * kGaRowBytes +
+                                      (half * (kGaD / 2) + 4 * (n16 & 3)) * 2;
+        auto vt_frag = [&](int nt) -> bf16x8 {
+            typedef short s16x4 __attribute__((ext_vector_type(4)));
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr<s16x4>)(vrow + nt * 32));
+            const s16x4 hi =
+                __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr<s16x4>)(vrow + 16 * kGaRowBytes + nt * 32));
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            return __builtin_bit_cast(bf16x8, both);
+        };
+        bf16x8 fb[kValueAhead];
+#pragma unroll
+        for (int i = 0; i < kValueAhead; ++i) fb[i] = vt_frag(i);
+        __builtin_amdgcn_sched_barrier(0);
+        const f32x4 ba = *(lds_ptr<f32x4>)(sbias + buf * kGaTile + 8 * g);
+        const f32x4 bb = *(lds_ptr<f32x4>)(sbias + buf * kGaTile + 8 * g + 4);
+        __syncthreads();  // both halves of every score are in LDS
+        {
+            const f32x4 p0 = xch_peer[0], p1 = xch_peer[1];
+            s0 += p0, s1 += p1;  // a + b == b + a: the pair works on identical numbers
+        }
+
+        // ---- online softmax over the lane's 8 slots of head n16 ---------------------------
+        const float bias[8] = {ba.x, ba.y, ba.z, ba.w, bb.x, bb.y, bb.z, bb.w};
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[i] = __builtin_fmaf(s0[i], a.qscale, bias[i]);  // -inf where the slot is masked
+            v[4 + i] = __builtin_fmaf(s1[i], a.qscale, bias[4 + i]);
+        }
+        float tmax = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
+        tmax = rows_max(tmax);
+        const bool grow = tmax > m_ref + kLazyRescale;  // false while everything is masked
+        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+            const float corr = grow ? __builtin_amdgcn_exp2f(m_ref - tmax) : 1.0f;  // 2^-inf = 0 at first
+            if (grow) m_ref = tmax;
+            l_sum *= corr;
+            float c[4];  // the lane's accumulators are heads 4g+i; corr lives in lanes n16 == head
+#pragma unroll
+            for (int i = 0; i < 4; ++i) c[i] = __shfl(corr, 4 * g + i, kWave);
+#pragma unroll
+            for (int nt = 0; nt < kGaColTilesHalf; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[nt][i] *= c[i];
+        }
+        const float mu = m_ref == -INFINITY ? 0.0f : m_ref;
+        // The value MFMA sees bf16(p_j), as hi + lo when PSPLIT == 2. Carried once, the
+        // denominator sums the rounded weights — the ones the numerator really holds — so the
+        // result is an exactly normalised average under weights perturbed by one bf16
+        // rounding each.
+        bf16x8 p, p_lo;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float e = __builtin_amdgcn_exp2f(v[i] - mu);  // masked -> 0
+            const __bf16 w = (__bf16)e;
+            p[i] = w;
+            if (PSPLIT == 2) {
+                p_lo[i] = (__bf16)(e - (float)w);
+                l_sum += e;
+            } else {
+                l_sum += (float)w;
+            }
+        }
+
+        // ---- values: O[head][col] += P . V over this wave's 256 columns -------------------
+#pragma unroll
+        for (int n0 = 0; n0 < kGaColTilesHalf; n0 += kValueAhead) {
+            if (n0 > 0) {
+#pragma unroll
+                for (int i = 0; i < kValueAhead; ++i) fb[i] = vt_frag(n0 + i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < kValueAhead; ++i) {
+                o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p, fb[i], o[n0 + i], 0, 0, 0);
+                if (PSPLIT == 2)
+                    o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_lo, fb[i], o[n0 + i], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        // ---- stage tile + 2, request tile + 3 ---------------------------------------------
+        if (tile + 2 < n_tiles) stage(buf == 0 ? 2 : buf - 1);
+        if (tile + 3 < n_tiles) issue_loads(entry_next);
+        entry_next = entry_ahead;
+        buf = buf == 2 ? 0 : buf + 1;
+    }
+
+    // ---- epilogue: the sink joins the denominator, the quotient is rounded to bf16 ---------
+    l_sum = rows_sum(l_sum);
+    {
+        const int head = hb * 64 + 16 * hw + n16;
+        const float sk = head < a.h ? a.sink[head] : 0.0f;
+        // the slots' weights are 2^(l2 - m_ref), so the sink's is 2^(sink * log2 e - m_ref);
+        // nothing live: m_ref is still -inf and the query's output is NaN
+        l_sum = m_ref == -INFINITY ? NAN : l_sum + exp2f(sk * kLog2e - m_ref);
+    }
+    // the lane's accumulators are heads 4g+i; their denominators live in lanes with n16 == 4g+i
+    float l_h[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) l_h[i] = __shfl(l_sum, 4 * g + i, kWave);
+    const int head0 = hb * 64 + 16 * hw;
+    const int col0 = half * (kGaD / 2) + n16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int head = head0 + 4 * g + i;
+        if (head < a.h) {
+            float* const dst = a.o + (t * a.h + head) * kGaD;
+#pragma unroll
+            for (int nt = 0; nt < kGaColTilesHalf; ++nt)
+                dst[col0 + 16 * nt] = (float)(__bf16)(o[nt][i] / l_h[i]);
+        }
+    }
+}
+
+// Any width: one workgroup of 4 waves per (query, head). Logits: a wave per slot, lanes over
+// dims; then the two-pass softmax of the reference over the logits in LDS; values: threads
+// over output dims, slots ascending.
+constexpr int kGaPlainThreads = 256;
+constexpr int kGaPlainAcc = 4;  // output dims per thread: d <= 1024
+
+__global__ __launch_bounds__(kGaPlainThreads) void gather_attn_plain_kernel(
+    const float* __restrict__ q, const float* __restrict__ kv, const float* __restrict__ sink,
+    const int* __restrict__ idxs, int h, int d, int topk, int n_kv, float scale,
+    float* __restrict__ o) {
+    extern __shared__ float ga_lds[];
+    float* qs = ga_lds;      // [d]
+    float* lg = ga_lds + d;  // [topk] logits, then weights
+    __shared__ float red[kGaPlainThreads / kWave];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int head = blockIdx.x;
+    const size_t t = blockIdx.y;
+    const float* qrow = q + (t * h + head) * d;
+    const int* ix = idxs + t * topk;
+    for (int i = tid; i < d; i += kGaPlainThreads) qs[i] = qrow[i];
+    __syncthreads();
+
+    float mx = -INFINITY;
+    for (int j = wave; j < topk; j += kGaPlainThreads / kWave) {
+        const int p = ix[j];
+        float l = -INFINITY;
+        if ((unsigned)p < (unsigned)n_kv) {
+            const float* kr = kv + (size_t)p * d;
+            float acc = 0.0f;
+            for (int i = lane; i < d; i += kWave) acc += qs[i] * kr[i];
+            for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+            l = acc * scale;
+        }
+        if (lane == 0) lg[j] = l;
+        mx = fmaxf(mx, l);
+    }
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+
+    float ps = 0.0f;
+    for (int j = tid; j < topk; j += kGaPlainThreads) {
+        const float l = lg[j];
+        const float e = l == -INFINITY ? 0.0f : expf(l - mx);
+        lg[j] = e;
+        ps += e;
+    }
+    for (int off = 32; off > 0; off >>= 1) ps += __shfl_xor(ps, off, kWave);
+    if (lane == 0) red[wave] = ps;
+    __syncthreads();
+    const float denom = isfinite(mx) ? (red[0] + red[1]) + (red[2] + red[3]) + expf(sink[head] - mx) : NAN;
+
+    float acc[kGaPlainAcc];
+#pragma unroll
+    for (int c = 0; c < kGaPlainAcc; ++c) acc[c] = 0.0f;
+    for (int j = 0; j < topk; ++j) {
+        const float e = lg[j];
+        if (e == 0.0f) continue;  // masked, or a weight that underflowed: adds nothing either way
+        const float* kr = kv + (size_t)ix[j] * d;
+#pragma unroll
+        for (int c = 0; c < kGaPlainAcc; ++c) {
+            const int i = tid + c * kGaPlainThreads;
+            if (i < d) acc[c] += e * kr[i];
+        }
+    }
+    float* orow = o + (t * h + head) * d;
+#pragma unroll
+    for (int c = 0; c < kGaPlainAcc; ++c) {
+        const int i = tid + c * kGaPlainThreads;
+        if (i < d) orow[i] = (float)(__bf16)(acc[c] / denom);
+    }
+}
+
+static int gather_attn_launch(const float* q, const float* kv, const float* sink, const int* idxs,
+                              int m, int h, int d, int topk, int n_kv, float scale, int precise,
+                              float* o, hipStream_t stream) {
+    if (!q || !kv || !sink || !idxs || !o) return 1001;
+    if (m <= 0 || h <= 0 || d <= 0 || topk <= 0 || n_kv <= 0) return 1001;
+    (void)hipGetLastError();
+    if (precise < 3 && d == kGaD && aligned16(q) && aligned16(kv) && aligned16(o) && (h + 63) / 64 <= 65535) {
+        GatherAttnArgs a;
+        a.q = q, a.kv = kv, a.sink = sink, a.idxs = idxs;
+        a.h = h, a.topk = topk, a.n_kv = n_kv, a.qscale = scale * kLog2e, a.o = o;
+        const dim3 grid((unsigned)m, (unsigned)((h + 63) / 64));
+        if (precise >= 2)
+            hipLaunchKernelGGL((gather_attn_d512_kernel<2, 2>), grid, dim3(kGaThreads), 0, stream, a);
+        else if (precise == 1)
+            hipLaunchKernelGGL((gather_attn_d512_kernel<2, 1>), grid, dim3(kGaThreads), 0, stream, a);
+        else
+            hipLaunchKernelGGL((gather_attn_d512_kernel<1, 1>), grid, dim3(kGaThreads), 0, stream, a);
+        return launch_status();
+    }
+    // the plain kernel keeps the reference launcher's limits (attn.hip:450-458)
+    if (d > kGaPlainThreads * kGaPlainAcc || m > 65535) return 1002;
+    const size_t lds = ((size_t)d + (size_t)topk) * sizeof(float);
+    if (lds + sizeof(float) * (kGaPlainThreads + 2) > 65536) return 1006;
+    hipLaunchKernelGGL(gather_attn_plain_kernel, dim3((unsigned)h, (unsigned)m), dim3(kGaPlainThreads),
+                       (unsigned)lds, stream, q, kv, sink, idxs, h, d, topk, n_kv, scale, o);
+    return launch_status();
+}
+
+}  // namespace rk
+
+extern "C" int rivoli_gather_attn_shared_kv(const float* q, const float* kv, const float* sink,
+                                            const int* idxs, int m, int h, int d, int topk,
+                                            float scale, float* o, void* stream) {
+    return rk::gather_attn_launch(q, kv, sink, idxs, m, h, d, topk, 0x7fffffff, scale, 2, o,
+                                  (hipStream_t)stream);
+}
+
+extern "C" int rivoli_gather_attn_shared_kv_bounded(const float* q, const float* kv,
+                                                    const float* sink, const int* idxs, int m,
+                                                    int h, int d, int topk, int n_kv, float scale,
+                                                    int precise, float* o, void* stream) {
+    return rk::gather_attn_launch(q, kv, sink, idxs, m, h, d, topk, n_kv, scale, precise, o,
+                                  (hipStream_t)stream);
+}

@@ -47,14 +47,9 @@
 // ascending order; the plan is a pure function of the call's shape and of the lengths, so
 // equal calls give bit-equal results.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
-#include "codec.hpp"
+#include "attend_common.hpp"
 
 namespace rk {
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-template <class T>
-using lds_ptr = __attribute__((address_space(3))) T*;
 
 constexpr int kKvl = 512, kRopeW = 64, kRowW = kKvl + kRopeW;
 constexpr int kAttThreads = 512;
@@ -70,8 +65,6 @@ constexpr int kXchBytes = 2 * kAttWaves * kWave * 8 * 4;  // partial scores, 8 f
 constexpr int kTableLds = 1024;            // block-table entries staged per workgroup
 constexpr int kAttSmemBytes = kBufs * kKrBytes + 2 * kBufs * kTile * 4 + kXchBytes + kTableLds * 4;
 static_assert(kAttSmemBytes + (1024 + 8 + 8) * 4 <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
-constexpr float kLazyRescale = 8.0f;       // log2 units
-constexpr float kLog2e = 1.4426950408889634f;
 
 // Work plan. `n_splits` is a pure function of the call's shape; with more than one split the
 // attended rows of ALL sequences, in tiles, are dealt evenly to n_seqs * n_splits work items
@@ -119,21 +112,6 @@ __device__ __forceinline__ void e4m3x4_to_bf16(uint32_t c, uint32_t& lo, uint32_
     hi = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c, 1.0f, true));
 }
 
-// max / sum of a value over the four 16-lane rows of the wave, in every lane. gfx950's row
-// swaps stay in the vector ALU; the generic cross-lane shuffle goes through the LDS crossbar.
-__device__ __forceinline__ float rows_max(float x) {
-    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));  // rows {0,1} and {2,3} paired
-    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
-}
-__device__ __forceinline__ float rows_sum(float x) {
-    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
-    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
-}
-
 struct AttendArgs {
     const float* qabs;            // [n_seqs][H][512]
     const float* qrope;           // [n_seqs][H][64]
@@ -153,12 +131,6 @@ struct AttendArgs {
     float* part_ml;               // [n_records][H][2]
     unsigned int* bad_rows;
 };
-
-// In the score tile (rows = tokens, 16 per MFMA) a lane of row group g holds rows 4g..4g+3
-// of both 16-token halves, and those 8 values are element j = 4*half + i of the value MFMA's
-// A operand for contraction index 8g + j. Staging wave w owns contraction indices
-// 4w..4w+3 — tile positions 16*(w&1) + 4*(w>>1) + i, four consecutive tokens.
-__device__ __forceinline__ int tile_pos_of(int wave, int i) { return 16 * (wave & 1) + 4 * (wave >> 1) + i; }
 
 // MODE: how a tile's tokens are found.
 enum : int {

@@ -58,6 +58,8 @@ _SIGNATURES = {
     "rivoli_sel_gather": [_I] * 5 + [_VP, _VP],
     "rivoli_sel_gather_scored": [_VP] + [_I] * 6 + [_VP, _VP, _VP],
     "rivoli_kv_ring_write": [_VP, _VP] + [_I] * 4 + [_VP],
+    "rivoli_gather_attn_shared_kv": [_VP] * 4 + [_I] * 4 + [_F, _VP, _VP],
+    "rivoli_gather_attn_shared_kv_bounded": [_VP] * 4 + [_I] * 5 + [_F, _I, _VP, _VP],
     "rivoli_kv_compress_deposit": [_VP] * 6 + [_I, _I, _VP],
     "rivoli_kv_compress_prefill": [_VP] * 5 + [_I, _VP],
     "rivoli_kv_compress_decode": [_VP] * 4 + [_I, _VP],
@@ -299,6 +301,20 @@ def launch_kv_ring_write(kv, cache, win, hd, seqlen, start_pos, stream=NULL_STRE
     """crates/engine/src/v4/attn.rs write_ring as one launch."""
     ensure_hip_status(lib().rivoli_kv_ring_write(_p(kv), _p(cache), win, hd, seqlen, start_pos, _s(stream)),
                       "kv_ring_write")
+
+
+def launch_gather_attn_shared_kv(q, kv, sink, idxs, m, h, d, topk, scale, o, stream=NULL_STREAM, *,
+                                 n_kv=None, precise=2) -> None:
+    """crates/backend/src/hip_attn.rs launch_gather_attn_shared_kv. With n_kv (rows of kv) the
+    bounded entry point runs: indices at or past it are treated as masked."""
+    if n_kv is None and precise == 2:
+        code = lib().rivoli_gather_attn_shared_kv(_p(q), _p(kv), _p(sink), _p(idxs), m, h, d, topk, scale, _p(o),
+                                                  _s(stream))
+    else:
+        code = lib().rivoli_gather_attn_shared_kv_bounded(_p(q), _p(kv), _p(sink), _p(idxs), m, h, d, topk,
+                                                          0x7fffffff if n_kv is None else n_kv, scale, precise,
+                                                          _p(o), _s(stream))
+    ensure_hip_status(code, "gather_attn_shared_kv")
 
 
 class CompGeom(C.Structure):

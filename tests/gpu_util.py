@@ -52,6 +52,9 @@ def ref_kernels():
             h.rivoli_mla_attend.argtypes = [vp] * 6 + [i] * 5 + [C.c_float, vp, vp]
             h.rivoli_mla_attend_scratch_floats.restype = C.c_size_t
             h.rivoli_mla_attend_scratch_floats.argtypes = [i, i]
+        if hasattr(h, "rivoli_gather_attn_shared_kv"):
+            h.rivoli_gather_attn_shared_kv.restype = i
+            h.rivoli_gather_attn_shared_kv.argtypes = [vp] * 4 + [i] * 4 + [C.c_float, vp, vp]
         if hasattr(h, "rivoli_act_quant_f8_prefix"):
             h.rivoli_act_quant_f8_prefix.restype = i
             h.rivoli_act_quant_f8_prefix.argtypes = [vp, vp] + [i] * 4 + [vp]

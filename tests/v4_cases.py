@@ -123,3 +123,30 @@ def sparse_attn_f64(q, kv, sink, idxs, scale):
             e = np.exp(logit - mx)
             out[t, hh] = (e @ rows) / (e.sum() + np.exp(sink[hh] - mx))
     return out
+
+
+def bf16_round(x):
+    """f32 -> nearest-even bf16 value, as f32 (finite inputs)."""
+    b = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    return (((b + 0x7FFF + ((b >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32).reshape(np.shape(x))
+
+
+def attend_inputs(oracle, m, h, d, rows, seed, cache_like=True, q_scale=1.0):
+    """q [m, h, d], kv [rows, d], sink [h]. cache_like: what the model hands the kernel — q
+    rounded to bf16 after its rotary, kv rows whose first d - 64 dims went through the block-64
+    fp8 quantize-dequantize and whose last 64 are bf16 values
+    (crates/engine/src/v4/attn.rs:272-290); otherwise arbitrary f32."""
+    rng = np.random.default_rng(seed)
+    q = (rng.standard_normal((m, h, d)) * q_scale).astype(np.float32)
+    kv = rng.standard_normal((rows, d)).astype(np.float32)
+    # outlier rows; milder where the kernel will round the rows to bf16 on load, which moves
+    # a logit by ~2^-9 of its size
+    kv[rng.integers(0, rows, max(1, rows // 50))] *= 8.0 if cache_like else 3.0
+    sink = rng.standard_normal(h).astype(np.float32)
+    if cache_like:
+        q, kv = bf16_round(q), bf16_round(kv)
+        n = d - 64 if d > 64 and (d - 64) % 64 == 0 else 0
+        if n:
+            code, kv = oracle.act_quant_f8_prefix(kv, n, 64)
+            assert code == 0
+    return q, kv, sink
