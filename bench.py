@@ -40,7 +40,8 @@ def parse():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=32768)
-    ap.add_argument("--workload", choices=["decode", "prefill", "dsa", "dsa_scored", "dsa_attend", "attend", "v4"],
+    ap.add_argument("--workload", choices=["decode", "prefill", "dsa", "dsa_scored", "dsa_attend", "attend", "v4",
+                                           "v4_attend"],
                     default="decode",
                     help="decode = configuration 3 (the headline line); prefill = configuration 2 "
                          "bulk append; dsa = configuration 4 top-k + sparse gather on synthetic "
@@ -51,10 +52,13 @@ def parse():
                          "attention reading the fp8 pages directly; "
                          "v4 = the second cache format's prefill ops: block-64 quantize-dequantize "
                          "of `tokens` f32 cache rows, then the scored block selection for every "
-                         "query row (ratio 4, cap --index-topk)")
+                         "query row (ratio 4, cap --index-topk); "
+                         "v4_attend = the second cache format's consumer at prefill: ring write, the "
+                         "[window | scored blocks] selection rectangle, and the index-list attention "
+                         "of `tokens` queries x --heads heads over it")
     ap.add_argument("--index-topk", type=int, default=512, help="v4: blocks kept per query row")
     ap.add_argument("--heads", type=int, default=64, help="attend: query heads")
-    ap.add_argument("--precise", type=int, default=2, choices=[0, 1, 2],
+    ap.add_argument("--precise", type=int, default=2, choices=[0, 1, 2, 3],
                     help="attend: 2 = q and softmax weights as bf16 hi+lo (parity mode), "
                          "1 = q only, 0 = plain bf16")
     ap.add_argument("--ragged", action="store_true",
@@ -104,6 +108,8 @@ def main():
         return bench_attend(a, torch, hip)
     if a.workload == "v4":
         return bench_v4(a, torch, hip)
+    if a.workload == "v4_attend":
+        return bench_v4_attend(a, torch, hip)
     L, B, ctx = a.layers, a.batch, a.ctx
     blocks = -(-ctx // PT)
     n_pages = B * blocks
@@ -421,6 +427,89 @@ def bench_v4(a, torch, hip):
                                "sample": f"the first {nr} rows of the same inputs through the oracle's "
                                          "compressor pooling, act_quant and scored_rows, one host thread; "
                                          "GPU results checked (pooling within 2 bf16 codes, the others equal)"}
+    print(json.dumps(res), flush=True)
+
+
+def bench_v4_attend(a, torch, hip):
+    """The second cache format's consumer at prefill, one layer of the indexed class (window 128,
+    ratio 4): the prompt's last 128 rows go into the ring, every query row gets its
+    [window | best index_topk closed blocks] index list, and all heads of every query attend over
+    those rows of the [prompt rows | compressed rows] buffer (key = value = the 512-wide row)."""
+    n, h, d, win, ratio, cap = a.tokens, a.heads, 512, 128, 4, a.index_topk
+    n_comp = n // ratio
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0x5EED0007)
+    # what the model hands over: q rounded to bf16 after its rotary; cache rows quantized and
+    # dequantized over their first 448 dims, bf16 values in the rotated tail
+    q = torch.randn(n, h, d, generator=g, device="cuda", dtype=torch.float32).bfloat16().float()
+    kv = torch.randn(n + n_comp, d, generator=g, device="cuda", dtype=torch.float32).bfloat16().float()
+    hip.launch_act_quant_f8_prefix(kv, kv, n + n_comp, d, 448, 64)
+    sink = torch.randn(h, generator=g, device="cuda", dtype=torch.float32)
+    scores = torch.randn(n, n_comp, generator=g, device="cuda", dtype=torch.float32)
+    cols = min(n, win) + min(cap, n_comp)
+    idx = torch.empty(n, cols, dtype=torch.int32, device="cuda")
+    ring = torch.zeros(win, d, dtype=torch.float32, device="cuda")
+    o = torch.empty(n, h, d, dtype=torch.float32, device="cuda")
+    scale = d ** -0.5
+    stream = torch.cuda.Stream()
+    sh = stream.cuda_stream
+
+    def step(events):
+        bracket(torch, stream, events, "ring", lambda: hip.launch_kv_ring_write(kv, ring, win, d, n, 0, sh))
+        bracket(torch, stream, events, "select",
+                lambda: hip.launch_sel_gather_scored(scores, n_comp, win, ratio, cap, n, 0, idx, sh))
+        bracket(torch, stream, events, "attend",
+                lambda: hip.launch_gather_attn_shared_kv(q, kv, sink, idx, n, h, d, cols, scale, o, sh,
+                                                         precise=a.precise))
+
+    ms, per = timed(torch, stream, a.steps, a.warmup, step)
+    live = int((idx >= 0).sum().item())
+    flops = 4.0 * h * d * live                                    # scores and values, 2 flops per multiply-add
+    hbm_bytes = 2 * n * h * d * 4 + (n + n_comp) * d * 4 + n * cols * 4   # q in, o out, every row once, the lists
+    att = per["attend"] * 1e-3
+    res = {"metric": "v4_gather_attn_TFLOPs", "value": round(flops / (ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+           "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+           "data": "synthetic",
+           "config": {"workload": "second cache format, prefill consumer: ring write, [window | scored blocks] "
+                                  "selection, index-list attention with shared key/value rows",
+                      "tokens": n, "heads": h, "head_dim": d, "window": win, "ratio": ratio, "index_topk": cap,
+                      "slots_per_query": cols, "live_slots": live, "precise": a.precise},
+           "queries_per_s": round(n / (ms * 1e-3), 1),
+           "kernels_ms": {k_: round(v, 5) for k_, v in per.items()},
+           "roofline": {"bound": "mfma", "kernel": "gather_attn_d512_kernel",
+                        "achieved": round(flops / att / 1e12, 2), "peak": 2500.0, "unit": "TFLOP/s",
+                        "frac": round(flops / att / 2.5e15, 4), "avg_launch_ms": round(per["attend"], 5),
+                        "flops_per_launch": flops, "traffic": None,
+                        "hbm": {"bytes_per_launch": hbm_bytes, "achieved_GBps": round(hbm_bytes / att / 1e9, 1),
+                                "frac": round(hbm_bytes / att / HBM_PEAK, 4)}}}
+    if not a.no_cpu_baseline:
+        from oracle.kvoracle import oracle as get_oracle
+
+        ora = get_oracle()
+        # bounded sample: the last queries of the prompt (full index lists), one host thread;
+        # doubles as the parity check, at the reference's bar for this kernel
+        nq = min(n, 48)
+        q_h, idx_h = q[n - nq:].cpu().numpy(), idx[n - nq:].cpu().numpy()
+        kv_h, sink_h = kv.cpu().numpy(), sink.cpu().numpy()
+        t0 = time.perf_counter()
+        want = ora.sparse_attn(q_h, kv_h, sink_h, idx_h, scale)
+        spent = time.perf_counter() - t0
+        got = o[n - nq:].cpu().numpy()
+        err = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+        if not err <= 1.0 / 128.0:
+            raise SystemExit(f"bench: GPU index-list attention is {err:.4g} of the largest element from the CPU "
+                             "oracle (bar 1/128)")
+        want_idx = ora.sel_gather_scored(scores[n - nq:].cpu().numpy() if n == nq else scores.cpu().numpy(), win,
+                                         ratio, cap, n, 0)[1] if n <= 4096 else None
+        if want_idx is not None and not np.array_equal(idx.cpu().numpy(), want_idx):
+            raise SystemExit("bench: GPU selection rectangle differs from the CPU oracle")
+        sample_flops = 4.0 * h * d * int((idx_h >= 0).sum())
+        res["cpu_baseline"] = {"value": round(sample_flops / spent / 1e12, 6), "unit": "TFLOP/s", "cores": 1,
+                               "kind": "port",
+                               "sample": f"the last {nq} queries of the same inputs through the oracle's "
+                                         f"sparse_attn, one host thread; GPU output within {err:.2g} of the "
+                                         "largest element (bar 1/128)"}
     print(json.dumps(res), flush=True)
 
 

@@ -75,28 +75,6 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
     const int n_tiles = (a.topk + kGaTile - 1) / kGaTile;
     const int* const ix = a.idxs + t * a.topk;
 
-    // ---- this wave's half of its 16 query heads as the B operand, for the whole kernel ---
-    bf16x8 qh[kGaKStepsHalf], ql[QSPLIT == 2 ? kGaKStepsHalf : 1];
-    {
-        const int head = hb * 64 + 16 * hw + n16;
-        const bool live = head < a.h;
-        const float* qa = a.q + (t * a.h + (live ? head : 0)) * kGaD + half * (kGaD / 2) + 8 * g;
-#pragma unroll
-        for (int j = 0; j < kGaKStepsHalf; ++j) {
-            const float4* src = reinterpret_cast<const float4*>(qa + 32 * j);
-            float4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
-            if (live) v0 = src[0], v1 = src[1];
-            const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float x = v[i];  // unscaled: a bf16-valued q stays exact in its hi part
-                const __bf16 hi = (__bf16)x;
-                qh[j][i] = hi;
-                if (QSPLIT == 2) ql[j][i] = (__bf16)(x - (float)hi);
-            }
-        }
-    }
-
     // ---- a tile's slots: lanes 0..3 hold the wave's 4 list entries ------------------------
     const int my_pos0 = tile_pos_of(wave, 0);  // the wave's 4 slots are consecutive tile positions
     auto list_entry = [&](int tile) -> int {
@@ -105,45 +83,80 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
         const int p = ix[pos];
         return (unsigned)p < (unsigned)a.n_kv ? p : -1;
     };
-    float4 raw[4][2];
-    float raw_bias;  // lanes 0..3
-    auto issue_loads = [&](int entry) {
+    struct RawTile {
+        float4 row[4][2];
+        float bias;  // lanes 0..3: 0, or -inf for a masked slot
+    };
+    auto issue_loads = [&](RawTile& r, int entry) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int p = __builtin_amdgcn_readlane(entry, i);
-            raw[i][0] = float4{0, 0, 0, 0}, raw[i][1] = float4{0, 0, 0, 0};
+            r.row[i][0] = float4{0, 0, 0, 0}, r.row[i][1] = float4{0, 0, 0, 0};
             if (p >= 0) {
                 const float4* src = reinterpret_cast<const float4*>(a.kv + (size_t)p * kGaD) + 2 * lane;
-                raw[i][0] = src[0], raw[i][1] = src[1];
+                r.row[i][0] = src[0], r.row[i][1] = src[1];
             }
         }
-        raw_bias = entry >= 0 ? 0.0f : -INFINITY;
+        r.bias = entry >= 0 ? 0.0f : -INFINITY;
     };
     auto pack2 = [](float lo, float hi) -> uint32_t {
         typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
         const bf16x2 p = {(__bf16)lo, (__bf16)hi};
         return __builtin_bit_cast(uint32_t, p);
     };
-    auto stage = [&](int buf) {
+    auto stage = [&](const RawTile& r, int buf) {
         const lds_ptr<uint8_t> krb = kr + buf * kGaTileBytes;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const u32x4 r = {pack2(raw[i][0].x, raw[i][0].y), pack2(raw[i][0].z, raw[i][0].w),
-                             pack2(raw[i][1].x, raw[i][1].y), pack2(raw[i][1].z, raw[i][1].w)};
-            *(lds_ptr<u32x4>)(krb + (my_pos0 + i) * kGaRowBytes + 16 * lane) = r;
+            const u32x4 v = {pack2(r.row[i][0].x, r.row[i][0].y), pack2(r.row[i][0].z, r.row[i][0].w),
+                             pack2(r.row[i][1].x, r.row[i][1].y), pack2(r.row[i][1].z, r.row[i][1].w)};
+            *(lds_ptr<u32x4>)(krb + (my_pos0 + i) * kGaRowBytes + 16 * lane) = v;
         }
-        if (lane < 4) sbias[buf * kGaTile + 4 * wave + lane] = raw_bias;
+        if (lane < 4) sbias[buf * kGaTile + 4 * wave + lane] = r.bias;
     };
 
-    // ---- prologue: tiles 0 and 1 staged, tile 2 in registers, tile 3's entries fetched ----
-    issue_loads(list_entry(0));
-    stage(0);
-    if (n_tiles > 1) {
-        issue_loads(list_entry(1));
-        stage(1);
-    }
-    if (n_tiles > 2) issue_loads(list_entry(2));
+    // ---- prologue ------------------------------------------------------------------------
+    // Everything the first tiles need is requested before anything is waited for: the list
+    // entries of tiles 0..3, the query (oldest request, so its wait leaves the rows in
+    // flight), the rows of tiles 0 and 1. Then: query -> B-operand fragments, tiles 0 and 1
+    // staged, tile 2 requested.
+    const int e0 = list_entry(0);
+    const int e1 = n_tiles > 1 ? list_entry(1) : -1;
+    const int e2 = n_tiles > 2 ? list_entry(2) : -1;
     int entry_next = n_tiles > 3 ? list_entry(3) : -1;
+    // this wave's half of its 16 query heads as the B operand, for the whole kernel
+    bf16x8 qh[kGaKStepsHalf], ql[QSPLIT == 2 ? kGaKStepsHalf : 1];
+    RawTile raw;
+    {
+        const int head = hb * 64 + 16 * hw + n16;
+        const bool live = head < a.h;
+        const float* qa = a.q + (t * a.h + (live ? head : 0)) * kGaD + half * (kGaD / 2) + 8 * g;
+        float4 qv[kGaKStepsHalf][2];
+#pragma unroll
+        for (int j = 0; j < kGaKStepsHalf; ++j) {
+            const float4* src = reinterpret_cast<const float4*>(qa + 32 * j);
+            qv[j][0] = float4{0, 0, 0, 0}, qv[j][1] = float4{0, 0, 0, 0};
+            if (live) qv[j][0] = src[0], qv[j][1] = src[1];
+        }
+        RawTile second;
+        issue_loads(raw, e0);
+        if (n_tiles > 1) issue_loads(second, e1);
+#pragma unroll
+        for (int j = 0; j < kGaKStepsHalf; ++j) {
+            const float v[8] = {qv[j][0].x, qv[j][0].y, qv[j][0].z, qv[j][0].w,
+                                qv[j][1].x, qv[j][1].y, qv[j][1].z, qv[j][1].w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float x = v[i];  // unscaled: a bf16-valued q stays exact in its hi part
+                const __bf16 hi = (__bf16)x;
+                qh[j][i] = hi;
+                if (QSPLIT == 2) ql[j][i] = (__bf16)(x - (float)hi);
+            }
+        }
+        stage(raw, 0);
+        if (n_tiles > 1) stage(second, 1);
+    }
+    if (n_tiles > 2) issue_loads(raw, e2);
     __syncthreads();
 
     f32x4 o[kGaColTilesHalf];
@@ -273,8 +286,8 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
         }
 
         // ---- stage tile + 2, request tile + 3 ---------------------------------------------
-        if (tile + 2 < n_tiles) stage(buf == 0 ? 2 : buf - 1);
-        if (tile + 3 < n_tiles) issue_loads(entry_next);
+        if (tile + 2 < n_tiles) stage(raw, buf == 0 ? 2 : buf - 1);
+        if (tile + 3 < n_tiles) issue_loads(raw, entry_next);
         entry_next = entry_ahead;
         buf = buf == 2 ? 0 : buf + 1;
     }
