@@ -483,6 +483,22 @@ def bench_v4_attend(a, torch, hip):
                         "flops_per_launch": flops, "traffic": None,
                         "hbm": {"bytes_per_launch": hbm_bytes, "achieved_GBps": round(hbm_bytes / att / 1e9, 1),
                                 "frac": round(hbm_bytes / att / HBM_PEAK, 4)}}}
+    # the reference's decode shape: ONE query row over the same 640-slot list, with the list
+    # shared among workgroups through a partial buffer, and without
+    part = torch.empty(max(hip.gather_attn_scratch_floats(1, h, d, cols), 4), dtype=torch.float32, device="cuda")
+    o1 = torch.empty(h, d, dtype=torch.float32, device="cuda")
+
+    def decode_step(events):
+        bracket(torch, stream, events, "split",
+                lambda: hip.launch_gather_attn_shared_kv(q[n - 1], kv, sink, idx[n - 1], 1, h, d, cols, scale, o1,
+                                                         sh, precise=a.precise, partial=part))
+        bracket(torch, stream, events, "whole",
+                lambda: hip.launch_gather_attn_shared_kv(q[n - 1], kv, sink, idx[n - 1], 1, h, d, cols, scale, o1,
+                                                         sh, precise=a.precise))
+
+    _, per_decode = timed(torch, stream, 20, 3, decode_step)
+    res["decode_one_query_us"] = {"split_over_slots": round(per_decode["split"] * 1e3, 2),
+                                  "one_workgroup": round(per_decode["whole"] * 1e3, 2)}
     if not a.no_cpu_baseline:
         from oracle.kvoracle import oracle as get_oracle
 

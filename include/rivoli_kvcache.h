@@ -285,6 +285,21 @@ int rivoli_gather_attn_shared_kv(const float* q, const float* kv, const float* s
 int rivoli_gather_attn_shared_kv_bounded(const float* q, const float* kv, const float* sink,
                                          const int* idxs, int m, int h, int d, int topk, int n_kv,
                                          float scale, int precise, float* o, void* stream);
+/* _split: the bounded form with a caller-provided partial buffer, for calls whose queries alone
+ * cannot fill the GPU (decode: the reference drives one query row, crates/engine/src/v4/select.rs:78-86):
+ * a query's list is shared among several workgroups, each writing unnormalised accumulators and
+ * (max, sum) to `partial`, and a second launch merges them in ascending order, adds the sink and
+ * rounds — the scheme of the reference's mla_attend_combine (attn.hip:235-277) applied to this
+ * kernel, which has no such path in the reference. rivoli_gather_attn_scratch_floats is the
+ * pure sizing function (0 = this shape is not split and partial may be null), as
+ * rivoli_mla_attend_scratch_floats is for the latent attention (attn.hip:100-103). The plan is a
+ * function of the shape alone, so equal calls give bit-equal results. 1001 also when the plan
+ * needs `partial` and it is null or not 16-byte aligned. */
+size_t rivoli_gather_attn_scratch_floats(int m, int h, int d, int topk);
+int rivoli_gather_attn_shared_kv_split(const float* q, const float* kv, const float* sink,
+                                       const int* idxs, int m, int h, int d, int topk, int n_kv,
+                                       float scale, int precise, float* o, float* partial,
+                                       void* stream);
 
 /* The compressor's pooling stage (crates/backend/kernels/kvcompress.hip; Rust rows
  * launch_kv_compress_deposit / _prefill / _decode, crates/backend/src/hip_attn.rs:547-605).

@@ -53,7 +53,25 @@ struct GatherAttnArgs {
     int n_kv;            // rows of kv; an index at or past it is treated as masked
     float qscale;        // softmax scale * log2(e)
     float* o;            // [m][h][512]
+    int n_splits;        // > 1: blockIdx.z owns a share of the query's tiles and writes a partial
+    float* part_acc;     // [m][n_splits][h][512] unnormalised accumulators
+    float* part_ml;      // [m][n_splits][h][2] reference maximum (log2 units), sum of weights
 };
+
+// How many workgroups share one query's list: a pure function of the call's shape. Splitting
+// pays when the queries alone cannot fill the part (decode: one query) and a share still
+// holds a couple of tiles.
+constexpr int kGaTargetGroups = 256;
+constexpr int kGaMinTilesPerSplit = 2;
+constexpr int kGaMaxSplits = 32;
+static inline int gather_attn_splits(int m, int h, int topk) {
+    const long long per_split = (long long)m * ((h + 63) / 64);
+    const int tiles = (topk + kGaTile - 1) / kGaTile;
+    long long n = (kGaTargetGroups + per_split - 1) / per_split;
+    if (n > tiles / kGaMinTilesPerSplit) n = tiles / kGaMinTilesPerSplit;
+    if (n > kGaMaxSplits) n = kGaMaxSplits;
+    return n < 2 ? 1 : (int)n;
+}
 
 template <int QSPLIT, int PSPLIT>
 __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const GatherAttnArgs a) {
@@ -72,13 +90,16 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
     const int hw = wave & 3;     // which 16 heads of the block
     const int half = wave >> 2;  // which half of the contraction dims / of the output columns
     const int g = lane >> 4, n16 = lane & 15;
-    const int n_tiles = (a.topk + kGaTile - 1) / kGaTile;
+    const int all_tiles = (a.topk + kGaTile - 1) / kGaTile;
+    const int split = blockIdx.z;
+    const int tile0 = (int)((long long)split * all_tiles / a.n_splits);  // this workgroup's tiles
+    const int n_tiles = (int)((long long)(split + 1) * all_tiles / a.n_splits) - tile0;
     const int* const ix = a.idxs + t * a.topk;
 
     // ---- a tile's slots: lanes 0..3 hold the wave's 4 list entries ------------------------
     const int my_pos0 = tile_pos_of(wave, 0);  // the wave's 4 slots are consecutive tile positions
     auto list_entry = [&](int tile) -> int {
-        const int pos = tile * kGaTile + my_pos0 + (lane & 3);
+        const int pos = (tile0 + tile) * kGaTile + my_pos0 + (lane & 3);
         if (lane >= 4 || pos >= a.topk) return -1;
         const int p = ix[pos];
         return (unsigned)p < (unsigned)a.n_kv ? p : -1;
@@ -294,6 +315,26 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
 
     // ---- epilogue: the sink joins the denominator, the quotient is rounded to bf16 ---------
     l_sum = rows_sum(l_sum);
+    if (a.n_splits > 1) {
+        // a share of the list: unnormalised accumulators and (m, l) for the combine kernel
+        const size_t rec = (t * a.n_splits + split) * a.h;
+        const int head0 = hb * 64 + 16 * hw;
+        const int col0 = half * (kGaD / 2) + n16;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int head = head0 + 4 * g + i;
+            if (head < a.h) {
+                float* const dst = a.part_acc + (rec + head) * kGaD;
+#pragma unroll
+                for (int nt = 0; nt < kGaColTilesHalf; ++nt) dst[col0 + 16 * nt] = o[nt][i];
+            }
+        }
+        if (half == 0 && g == 0 && head0 + n16 < a.h) {
+            a.part_ml[(rec + head0 + n16) * 2] = m_ref;
+            a.part_ml[(rec + head0 + n16) * 2 + 1] = l_sum;
+        }
+        return;
+    }
     {
         const int head = hb * 64 + 16 * hw + n16;
         const float sk = head < a.h ? a.sink[head] : 0.0f;
@@ -317,6 +358,36 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
                 dst[col0 + 16 * nt] = (float)(__bf16)(o[nt][i] / l_h[i]);
         }
     }
+}
+
+// Split plan: o[t][head] = bf16(sum_r w_r acc_r / (sum_r w_r l_r + 2^(sink * log2 e - max m))),
+// w_r = 2^(m_r - max m), over the query's shares in ascending order. Nothing live anywhere: NaN.
+__global__ __launch_bounds__(128) void gather_attn_combine_kernel(
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+    const float* __restrict__ sink, int n_splits, int h, float* __restrict__ o) {
+    const int head = blockIdx.x;
+    const size_t t = blockIdx.y;
+    const size_t rec0 = t * n_splits * h + head;
+    float m_g = -INFINITY;
+    for (int r = 0; r < n_splits; ++r) m_g = fmaxf(m_g, part_ml[(rec0 + (size_t)r * h) * 2]);
+    float4 sum = {0, 0, 0, 0};
+    float l_g = NAN;
+    if (m_g != -INFINITY) {
+        l_g = 0.0f;
+        for (int r = 0; r < n_splits; ++r) {
+            const size_t rec = rec0 + (size_t)r * h;
+            const float m_r = part_ml[rec * 2];
+            if (m_r == -INFINITY) continue;
+            const float w = exp2f(m_r - m_g);
+            l_g += part_ml[rec * 2 + 1] * w;
+            const float4 v = reinterpret_cast<const float4*>(part_acc + rec * kGaD)[threadIdx.x];
+            sum.x += v.x * w, sum.y += v.y * w, sum.z += v.z * w, sum.w += v.w * w;
+        }
+        l_g += exp2f(sink[head] * kLog2e - m_g);
+    }
+    float4* const dst = reinterpret_cast<float4*>(o + (t * h + head) * kGaD) + threadIdx.x;
+    *dst = float4{(float)(__bf16)(sum.x / l_g), (float)(__bf16)(sum.y / l_g), (float)(__bf16)(sum.z / l_g),
+                  (float)(__bf16)(sum.w / l_g)};
 }
 
 // Any width: one workgroup of 4 waves per (query, head). Logits: a wave per slot, lanes over
@@ -395,7 +466,7 @@ __global__ __launch_bounds__(kGaPlainThreads) void gather_attn_plain_kernel(
 
 static int gather_attn_launch(const float* q, const float* kv, const float* sink, const int* idxs,
                               int m, int h, int d, int topk, int n_kv, float scale, int precise,
-                              float* o, hipStream_t stream) {
+                              float* o, float* partial, hipStream_t stream) {
     if (!q || !kv || !sink || !idxs || !o) return 1001;
     if (m <= 0 || h <= 0 || d <= 0 || topk <= 0 || n_kv <= 0) return 1001;
     (void)hipGetLastError();
@@ -403,13 +474,21 @@ static int gather_attn_launch(const float* q, const float* kv, const float* sink
         GatherAttnArgs a;
         a.q = q, a.kv = kv, a.sink = sink, a.idxs = idxs;
         a.h = h, a.topk = topk, a.n_kv = n_kv, a.qscale = scale * kLog2e, a.o = o;
-        const dim3 grid((unsigned)m, (unsigned)((h + 63) / 64));
+        // a caller without a partial buffer gets the one-workgroup-per-query plan
+        a.n_splits = partial && aligned16(partial) ? gather_attn_splits(m, h, topk) : 1;
+        a.part_acc = partial;
+        a.part_ml = partial ? partial + (size_t)m * a.n_splits * h * kGaD : nullptr;
+        const dim3 grid((unsigned)m, (unsigned)((h + 63) / 64), (unsigned)a.n_splits);
         if (precise >= 2)
             hipLaunchKernelGGL((gather_attn_d512_kernel<2, 2>), grid, dim3(kGaThreads), 0, stream, a);
         else if (precise == 1)
             hipLaunchKernelGGL((gather_attn_d512_kernel<2, 1>), grid, dim3(kGaThreads), 0, stream, a);
         else
             hipLaunchKernelGGL((gather_attn_d512_kernel<1, 1>), grid, dim3(kGaThreads), 0, stream, a);
+        const int rc = launch_status();
+        if (rc != 0 || a.n_splits == 1) return rc;  // a split plan has fewer than 256 queries
+        hipLaunchKernelGGL(gather_attn_combine_kernel, dim3((unsigned)h, (unsigned)m), dim3(128), 0, stream,
+                           a.part_acc, a.part_ml, sink, a.n_splits, h, o);
         return launch_status();
     }
     // the plain kernel keeps the reference launcher's limits (attn.hip:450-458)
@@ -426,7 +505,7 @@ static int gather_attn_launch(const float* q, const float* kv, const float* sink
 extern "C" int rivoli_gather_attn_shared_kv(const float* q, const float* kv, const float* sink,
                                             const int* idxs, int m, int h, int d, int topk,
                                             float scale, float* o, void* stream) {
-    return rk::gather_attn_launch(q, kv, sink, idxs, m, h, d, topk, 0x7fffffff, scale, 2, o,
+    return rk::gather_attn_launch(q, kv, sink, idxs, m, h, d, topk, 0x7fffffff, scale, 2, o, nullptr,
                                   (hipStream_t)stream);
 }
 
@@ -434,6 +513,22 @@ extern "C" int rivoli_gather_attn_shared_kv_bounded(const float* q, const float*
                                                     const float* sink, const int* idxs, int m,
                                                     int h, int d, int topk, int n_kv, float scale,
                                                     int precise, float* o, void* stream) {
-    return rk::gather_attn_launch(q, kv, sink, idxs, m, h, d, topk, n_kv, scale, precise, o,
+    return rk::gather_attn_launch(q, kv, sink, idxs, m, h, d, topk, n_kv, scale, precise, o, nullptr,
+                                  (hipStream_t)stream);
+}
+
+extern "C" size_t rivoli_gather_attn_scratch_floats(int m, int h, int d, int topk) {
+    if (m <= 0 || h <= 0 || topk <= 0 || d != rk::kGaD) return 0;
+    const int n = rk::gather_attn_splits(m, h, topk);
+    return n > 1 ? (size_t)m * n * h * (rk::kGaD + 2) : 0;
+}
+
+extern "C" int rivoli_gather_attn_shared_kv_split(const float* q, const float* kv, const float* sink,
+                                                  const int* idxs, int m, int h, int d, int topk,
+                                                  int n_kv, float scale, int precise, float* o,
+                                                  float* partial, void* stream) {
+    if (rivoli_gather_attn_scratch_floats(m, h, d, topk) > 0 && (!partial || !rk::aligned16(partial)))
+        return 1001;
+    return rk::gather_attn_launch(q, kv, sink, idxs, m, h, d, topk, n_kv, scale, precise, o, partial,
                                   (hipStream_t)stream);
 }

@@ -60,6 +60,7 @@ _SIGNATURES = {
     "rivoli_kv_ring_write": [_VP, _VP] + [_I] * 4 + [_VP],
     "rivoli_gather_attn_shared_kv": [_VP] * 4 + [_I] * 4 + [_F, _VP, _VP],
     "rivoli_gather_attn_shared_kv_bounded": [_VP] * 4 + [_I] * 5 + [_F, _I, _VP, _VP],
+    "rivoli_gather_attn_shared_kv_split": [_VP] * 4 + [_I] * 5 + [_F, _I, _VP, _VP, _VP],
     "rivoli_kv_compress_deposit": [_VP] * 6 + [_I, _I, _VP],
     "rivoli_kv_compress_prefill": [_VP] * 5 + [_I, _VP],
     "rivoli_kv_compress_decode": [_VP] * 4 + [_I, _VP],
@@ -97,6 +98,8 @@ def lib() -> C.CDLL:
         fn.restype, fn.argtypes = C.c_size_t, [_I, _I, _I]
         fn = handle.rivoli_mla_attend_scratch_floats
         fn.restype, fn.argtypes = C.c_size_t, [_I, _I]
+        fn = handle.rivoli_gather_attn_scratch_floats
+        fn.restype, fn.argtypes = C.c_size_t, [_I, _I, _I, _I]
         _LIB = handle
     return _LIB
 
@@ -104,7 +107,7 @@ def lib() -> C.CDLL:
 def exported_symbols() -> list[str]:
     return sorted(list(_SIGNATURES) + ["rivoli_kv_page_bytes", "rivoli_index_topk_workspace_bytes",
                                        "rivoli_mla_attend_paged_scratch_floats",
-                                       "rivoli_mla_attend_scratch_floats"])
+                                       "rivoli_mla_attend_scratch_floats", "rivoli_gather_attn_scratch_floats"])
 
 
 def _p(x):
@@ -303,11 +306,21 @@ def launch_kv_ring_write(kv, cache, win, hd, seqlen, start_pos, stream=NULL_STRE
                       "kv_ring_write")
 
 
+def gather_attn_scratch_floats(m, h, d, topk) -> int:
+    """f32 elements of the partial buffer launch_gather_attn_shared_kv(partial=...) needs (0: none)."""
+    return int(lib().rivoli_gather_attn_scratch_floats(m, h, d, topk))
+
+
 def launch_gather_attn_shared_kv(q, kv, sink, idxs, m, h, d, topk, scale, o, stream=NULL_STREAM, *,
-                                 n_kv=None, precise=2) -> None:
+                                 n_kv=None, precise=2, partial=None) -> None:
     """crates/backend/src/hip_attn.rs launch_gather_attn_shared_kv. With n_kv (rows of kv) the
-    bounded entry point runs: indices at or past it are treated as masked."""
-    if n_kv is None and precise == 2:
+    bounded entry point runs: indices at or past it are treated as masked. With partial (a
+    buffer of gather_attn_scratch_floats f32) a query's list may be shared among workgroups."""
+    if partial is not None:
+        code = lib().rivoli_gather_attn_shared_kv_split(_p(q), _p(kv), _p(sink), _p(idxs), m, h, d, topk,
+                                                        0x7fffffff if n_kv is None else n_kv, scale, precise,
+                                                        _p(o), _p(partial), _s(stream))
+    elif n_kv is None and precise == 2:
         code = lib().rivoli_gather_attn_shared_kv(_p(q), _p(kv), _p(sink), _p(idxs), m, h, d, topk, scale, _p(o),
                                                   _s(stream))
     else:

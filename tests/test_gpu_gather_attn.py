@@ -160,6 +160,46 @@ def test_reference_kernel_agrees_with_the_oracle(oracle):
         assert worst_rel(ours, theirs) <= ATTEND_TOL
 
 
+@pytest.mark.parametrize("m,h,topk,precise", [(1, 64, 640, 2), (1, 64, 128, 0), (3, 64, 1000, 2), (2, 128, 333, 1),
+                                              (1, 8, 64, 2), (40, 64, 640, 2)])
+def test_split_plan_matches_oracle_and_the_unsplit_kernel(oracle, m, h, topk, precise):
+    """Decode-shaped calls: a query's list shared among workgroups through the caller's partial
+    buffer. Same bar against the oracle; against the one-workgroup plan the only difference is
+    where the softmax was re-associated."""
+    d, rows = 512, 1500
+    q, kv, sink = attend_inputs(oracle, m, h, d, rows, seed=m + topk)
+    idx = random_lists(np.random.default_rng(topk + 1), m, topk, rows)
+    idx[0, : topk // 2] = -1                                   # whole shares of query 0 masked
+    n = hip.gather_attn_scratch_floats(m, h, d, topk)
+    assert (n > 0) == (m * ((h + 63) // 64) < 256 and topk > 96)
+    partial = dzeros(max(n, 4) * 4, 0xEE)
+    want = oracle.sparse_attn(q, kv, sink, idx, d ** -0.5)
+    got = device_attend(q, kv, sink, idx, d ** -0.5, precise=precise, partial=partial)
+    assert worst_rel(got, want) <= ATTEND_TOL
+    exact = sparse_attn_f64(q, kv, sink, idx, d ** -0.5)
+    assert np.all(np.abs(got - exact) <= 2.0 ** -8 * np.abs(exact) + 2.0 ** -10 * np.abs(exact).max())
+    whole = device_attend(q, kv, sink, idx, d ** -0.5, precise=precise)
+    assert worst_rel(got, whole) <= 2.0 ** -7                  # one bf16 code where a rounding flipped
+    again = device_attend(q, kv, sink, idx, d ** -0.5, precise=precise, partial=partial)
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))      # the plan depends on the shape alone
+    if n > 0:
+        with pytest.raises(hip.LaunchError) as e:
+            hip.launch_gather_attn_shared_kv(dev(q), dev(kv), dev(sink), dev(idx), m, h, d, topk, d ** -0.5,
+                                             dzeros(m * h * d * 4), partial=dzeros(0))
+        assert e.value.code == 1001
+
+
+def test_split_plan_with_a_fully_masked_query(oracle):
+    d, h, rows, topk = 512, 64, 200, 320
+    q, kv, sink = attend_inputs(oracle, 2, h, d, rows, seed=77)
+    idx = random_lists(np.random.default_rng(8), 2, topk, rows)
+    idx[1] = -1
+    partial = dzeros(hip.gather_attn_scratch_floats(2, h, d, topk) * 4)
+    got = device_attend(q, kv, sink, idx, d ** -0.5, partial=partial)
+    want = oracle.sparse_attn(q, kv, sink, idx, d ** -0.5)
+    assert np.isnan(got[1]).all() and worst_rel(got[0], want[0]) <= ATTEND_TOL
+
+
 def test_plain_kernel_on_request_keeps_f32_rows(oracle):
     """precise = 3: rows that are not bf16 values are not rounded, at width 512 too."""
     d, h, m, rows = 512, 8, 2, 64
