@@ -185,21 +185,15 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
     for (int nt = 0; nt < kGaColTilesHalf; ++nt) o[nt] = f32x4{0, 0, 0, 0};
     float m_ref = -INFINITY, l_sum = 0.0f;
 
-    // Iteration t: scores of tile t -> exchange -> BARRIER -> softmax, values of tile t ->
-    // stage tile t+2 (in registers since iteration t-1) -> request tile t+3 from memory.
-    // A wave past the barrier knows that every wave has finished tile t-1 (so its LDS tile,
-    // (t+2) mod 3, may be overwritten) and has staged tile t+1.
-    int buf = 0;  // tile mod 3
-    for (int tile = 0; tile < n_tiles; ++tile) {
-        const int entry_ahead = tile + 4 < n_tiles ? list_entry(tile + 4) : -1;
-        const lds_ptr<f32x4> xch_mine = xch + (((tile & 1) * kGaWaves + wave) * kWave + lane) * 2;
-        const lds_ptr<f32x4> xch_peer = xch + (((tile & 1) * kGaWaves + (wave ^ 4)) * kWave + lane) * 2;
-
-        // ---- scores: this wave's half of the dims, S^T[slot][head], two 16-slot halves ----
-        const lds_ptr<uint8_t> krb = kr + buf * kGaTileBytes + half * (kGaKStepsHalf * 64);
+    // Scores of one staged tile: this wave's half of the dims, S^T[slot][head], two 16-slot
+    // halves. The operand fragments of a block of K-steps are all requested before the first
+    // MFMA of the block; left alone the compiler keeps two reads in flight and every pair of
+    // MFMAs then waits out a full LDS round trip.
+    auto scores_of = [&](int b, f32x4& s0, f32x4& s1) {
+        const lds_ptr<uint8_t> krb = kr + b * kGaTileBytes + half * (kGaKStepsHalf * 64);
         const lds_ptr<bf16x8> a0p = (lds_ptr<bf16x8>)(krb + n16 * kGaRowBytes + 16 * g);
         const lds_ptr<bf16x8> a1p = (lds_ptr<bf16x8>)(krb + (16 + n16) * kGaRowBytes + 16 * g);
-        f32x4 s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0};
+        s0 = f32x4{0, 0, 0, 0}, s1 = f32x4{0, 0, 0, 0};
 #pragma unroll
         for (int j0 = 0; j0 < kGaKStepsHalf; j0 += kFragBlock) {
             bf16x8 fa0[kFragBlock], fa1[kFragBlock];
@@ -218,7 +212,26 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        xch_mine[0] = s0, xch_mine[1] = s1;
+    };
+
+    // Iteration t: BARRIER -> the pair's scores of tile t meet -> scores of tile t+1 go to the
+    // matrix cores -> softmax of tile t (vector ALU, while those run) -> values of tile t ->
+    // this wave's half of the scores of tile t+1 to the exchange -> stage tile t+2 (in registers
+    // since iteration t-1) -> request tile t+3 from memory. A wave past the barrier knows that
+    // every wave has finished tile t-1 (so its LDS tile, (t+2) mod 3, may be overwritten), has
+    // staged tile t+1 and has written its scores of tile t.
+    int buf = 0;  // tile mod 3
+    f32x4 s0, s1;
+    scores_of(0, s0, s1);
+    {
+        const lds_ptr<f32x4> x = xch + ((0 * kGaWaves + wave) * kWave + lane) * 2;
+        x[0] = s0, x[1] = s1;
+    }
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        const int entry_ahead = tile + 4 < n_tiles ? list_entry(tile + 4) : -1;
+        const lds_ptr<f32x4> xch_peer = xch + (((tile & 1) * kGaWaves + (wave ^ 4)) * kWave + lane) * 2;
+        const lds_ptr<f32x4> xch_next = xch + ((((tile + 1) & 1) * kGaWaves + wave) * kWave + lane) * 2;
+        const int buf_next = buf == 2 ? 0 : buf + 1;
         // value-side operand of column tile nt: for each of the lane's 8 contraction indices
         // (slots 4g..4g+3 of both 16-slot halves) the value of column 16*nt' + n16. One
         // transposing load hands a lane element e of the 8-byte chunk that lane
@@ -241,53 +254,62 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
         __builtin_amdgcn_sched_barrier(0);
         const f32x4 ba = *(lds_ptr<f32x4>)(sbias + buf * kGaTile + 8 * g);
         const f32x4 bb = *(lds_ptr<f32x4>)(sbias + buf * kGaTile + 8 * g + 4);
-        __syncthreads();  // both halves of every score are in LDS
+        __syncthreads();  // both halves of every score of this tile are in LDS
         {
             const f32x4 p0 = xch_peer[0], p1 = xch_peer[1];
             s0 += p0, s1 += p1;  // a + b == b + a: the pair works on identical numbers
         }
-
         // ---- online softmax over the lane's 8 slots of head n16 ---------------------------
-        const float bias[8] = {ba.x, ba.y, ba.z, ba.w, bb.x, bb.y, bb.z, bb.w};
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            v[i] = __builtin_fmaf(s0[i], a.qscale, bias[i]);  // -inf where the slot is masked
-            v[4 + i] = __builtin_fmaf(s1[i], a.qscale, bias[4 + i]);
-        }
-        float tmax = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
-        tmax = rows_max(tmax);
-        const bool grow = tmax > m_ref + kLazyRescale;  // false while everything is masked
-        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-            const float corr = grow ? __builtin_amdgcn_exp2f(m_ref - tmax) : 1.0f;  // 2^-inf = 0 at first
-            if (grow) m_ref = tmax;
-            l_sum *= corr;
-            float c[4];  // the lane's accumulators are heads 4g+i; corr lives in lanes n16 == head
-#pragma unroll
-            for (int i = 0; i < 4; ++i) c[i] = __shfl(corr, 4 * g + i, kWave);
-#pragma unroll
-            for (int nt = 0; nt < kGaColTilesHalf; ++nt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) o[nt][i] *= c[i];
-        }
-        const float mu = m_ref == -INFINITY ? 0.0f : m_ref;
-        // The value MFMA sees bf16(p_j), as hi + lo when PSPLIT == 2. Carried once, the
-        // denominator sums the rounded weights — the ones the numerator really holds — so the
-        // result is an exactly normalised average under weights perturbed by one bf16
-        // rounding each.
         bf16x8 p, p_lo;
+        auto softmax_tile = [&]() {
+            const float bias[8] = {ba.x, ba.y, ba.z, ba.w, bb.x, bb.y, bb.z, bb.w};
+            float v[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float e = __builtin_amdgcn_exp2f(v[i] - mu);  // masked -> 0
-            const __bf16 w = (__bf16)e;
-            p[i] = w;
-            if (PSPLIT == 2) {
-                p_lo[i] = (__bf16)(e - (float)w);
-                l_sum += e;
-            } else {
-                l_sum += (float)w;
+            for (int i = 0; i < 4; ++i) {
+                v[i] = __builtin_fmaf(s0[i], a.qscale, bias[i]);  // -inf where the slot is masked
+                v[4 + i] = __builtin_fmaf(s1[i], a.qscale, bias[4 + i]);
             }
-        }
+            float tmax =
+                fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
+            tmax = rows_max(tmax);
+            const bool grow = tmax > m_ref + kLazyRescale;  // false while everything is masked
+            if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+                const float corr = grow ? __builtin_amdgcn_exp2f(m_ref - tmax) : 1.0f;  // 2^-inf = 0 at first
+                if (grow) m_ref = tmax;
+                l_sum *= corr;
+                float c[4];  // the lane's accumulators are heads 4g+i; corr lives in lanes n16 == head
+#pragma unroll
+                for (int i = 0; i < 4; ++i) c[i] = __shfl(corr, 4 * g + i, kWave);
+#pragma unroll
+                for (int nt = 0; nt < kGaColTilesHalf; ++nt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) o[nt][i] *= c[i];
+            }
+            const float mu = m_ref == -INFINITY ? 0.0f : m_ref;
+            // The value MFMA sees bf16(p_j), as hi + lo when PSPLIT == 2. Carried once, the
+            // denominator sums the rounded weights — the ones the numerator really holds — so
+            // the result is an exactly normalised average under weights perturbed by one bf16
+            // rounding each.
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float e = __builtin_amdgcn_exp2f(v[i] - mu);  // masked -> 0
+                const __bf16 w = (__bf16)e;
+                p[i] = w;
+                if (PSPLIT == 2) {
+                    p_lo[i] = (__bf16)(e - (float)w);
+                    l_sum += e;
+                } else {
+                    l_sum += (float)w;
+                }
+            }
+        };
+        // the next tile's scores go to the matrix cores before this tile's softmax occupies
+        // the vector ALU (the two waves of a pair share a SIMD; running them in opposite order
+        // from two copies of the loop measured the same)
+        f32x4 ns0, ns1;
+        const bool more = tile + 1 < n_tiles;
+        if (more) scores_of(buf_next, ns0, ns1);
+        softmax_tile();
 
         // ---- values: O[head][col] += P . V over this wave's 256 columns -------------------
 #pragma unroll
@@ -306,11 +328,15 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
             __builtin_amdgcn_sched_barrier(0);
         }
 
+        if (more) {
+            xch_next[0] = ns0, xch_next[1] = ns1;
+            s0 = ns0, s1 = ns1;
+        }
         // ---- stage tile + 2, request tile + 3 ---------------------------------------------
         if (tile + 2 < n_tiles) stage(raw, buf == 0 ? 2 : buf - 1);
         if (tile + 3 < n_tiles) issue_loads(raw, entry_next);
         entry_next = entry_ahead;
-        buf = buf == 2 ? 0 : buf + 1;
+        buf = buf_next;
     }
 
     // ---- epilogue: the sink joins the denominator, the quotient is rounded to bf16 ---------
