@@ -144,6 +144,46 @@ def second_format_cases(oracle) -> dict:
     assert code == 0
     g["compress_prefill_ratio4"] = {"kv_fnv": fnv(oracle, kv), "score_fnv": fnv(oracle, score),
                                     "out_u32": hexs(out.view(np.uint32))}
+    g.update(consumer_cases(oracle))
+    return g
+
+
+def consumer_inputs(oracle):
+    """Seeded inputs of the selection / ring / attention cases: a 24-token prompt on the indexed
+    class (window 8, ratio 4), 4 heads of width 64; cache rows and q are bf16 values."""
+    lcg = oracle.lcg(0x5EED0008)
+    n, h, d = 24, 4, 64
+    def bf16_values(x):
+        return (oracle.f32_to_bf16(x).astype(np.uint32) << 16).view(np.float32)
+
+    kv = bf16_values(lcg.fill((n + n // 4) * d)).reshape(n + n // 4, d)
+    q = bf16_values(lcg.fill(n * h * d) * np.float32(2.0)).reshape(n, h, d)
+    sink = lcg.fill(h)
+    scores = lcg.fill(n * (n // 4)).reshape(n, n // 4)
+    return n, h, d, kv, q, sink, scores
+
+
+def consumer_cases(oracle) -> dict:
+    n, h, d, kv, q, sink, scores = consumer_inputs(oracle)
+    g = {}
+    code, pos = oracle.sel_gather(8, 4, 512, n, 0)
+    assert code == 0
+    code, dec = oracle.sel_gather(8, 4, 512, 1, 21)
+    assert code == 0
+    code, scored = oracle.sel_gather_scored(scores, 8, 4, 3, n, 0)
+    assert code == 0
+    g["selection_rectangles"] = {"prefill_shape": list(pos.shape), "prefill_fnv": fnv(oracle, pos),
+                                 "prefill_row10": [int(v) for v in pos[10]],
+                                 "decode_row": [int(v) for v in dec[0]],
+                                 "scored_shape": list(scored.shape), "scored_fnv": fnv(oracle, scored),
+                                 "scored_row23": [int(v) for v in scored[23]]}
+    ring = np.zeros((8, d), np.float32)
+    assert oracle.ring_write(kv[:n], ring, 8, n, 0) == 0
+    g["ring_after_prefill_fnv"] = fnv(oracle, ring)
+    out = oracle.sparse_attn(q, kv, sink, scored, d ** -0.5)
+    # the device matches this to the reference's bar (1/128 of the largest element), not bit for bit
+    g["gather_attn"] = {"q_fnv": fnv(oracle, q), "kv_fnv": fnv(oracle, kv),
+                        "row23_head0_u32": hexs(out[23, 0].view(np.uint32)), "out_fnv": fnv(oracle, out)}
     return g
 
 
@@ -154,7 +194,8 @@ def main() -> None:
                          os.path.join(ROOT, "tests", "test_oracle_quant.py"),
                          os.path.join(ROOT, "tests", "test_oracle_topk_hash.py"),
                          os.path.join(ROOT, "tests", "test_oracle_v4.py"),
-                         os.path.join(ROOT, "tests", "test_oracle_v4_compress.py")], cwd=ROOT).returncode
+                         os.path.join(ROOT, "tests", "test_oracle_v4_compress.py"),
+                         os.path.join(ROOT, "tests", "test_oracle_v4_select.py")], cwd=ROOT).returncode
     if rc != 0:
         sys.exit("the oracle does not pass its known-answer tests: no vectors written")
     from oracle.kvoracle import oracle as get_oracle

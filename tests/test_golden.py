@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from tests.golden import inputs
-from tests.golden.make_golden import OUT, PT, W, build_cases, fnv, hexs, second_format_inputs
+from tests.golden.make_golden import OUT, PT, W, build_cases, consumer_inputs, fnv, hexs, second_format_inputs
 from tests.test_oracle_quant import fixture_a99e
 from tests.topk_cases import reference_topk_cases
 
@@ -166,3 +166,49 @@ def test_device_reproduces_second_format_golden(oracle, golden):
                                    hip.CompGeom.build(4, 64, 16, 1e-6), 4)
     want = np.frombuffer(bytes.fromhex(g["out_u32"]), np.uint32).view(np.float32).reshape(4, geom.d)
     assert compress_gap(oracle, back(out, np.float32).reshape(4, geom.d), want, 16).max() <= 2
+
+
+def test_golden_consumer_known_values(golden):
+    """What the reference's own unit cases fix about these vectors
+    (crates/engine/src/v4/select.rs:533-553): a prefill row reads the last `win` positions up to
+    its own, then the blocks that have closed, shifted past the prompt; a decode row reads the
+    full ring oldest first."""
+    g = golden["selection_rectangles"]
+    assert g["prefill_shape"] == [24, 8 + 6]
+    assert g["prefill_row10"] == [3, 4, 5, 6, 7, 8, 9, 10] + [24, 25, -1, -1, -1, -1]
+    assert g["decode_row"] == [6, 7, 0, 1, 2, 3, 4, 5] + [8, 9, 10, 11, 12]
+    assert g["scored_shape"] == [24, 8 + 3] and g["scored_row23"][:8] == list(range(16, 24))
+    assert all(24 <= v < 30 for v in g["scored_row23"][8:]) and g["scored_row23"][8:] == sorted(g["scored_row23"][8:])
+
+
+@pytest.mark.gpu
+def test_device_reproduces_consumer_golden(oracle, golden):
+    from rivoli_amd import hip
+    from tests.gpu_util import back, dev, dzeros
+
+    n, h, d, kv, q, sink, scores = consumer_inputs(oracle)
+    g = golden["selection_rectangles"]
+    rows, cols = g["prefill_shape"]
+    out = dzeros(rows * cols * 4, 0xEE)
+    assert hip.launch_sel_gather(8, 4, 512, n, 0, out) == (rows, cols)
+    pos = back(out, np.int32).reshape(rows, cols)
+    assert fnv(oracle, pos) == g["prefill_fnv"] and [int(v) for v in pos[10]] == g["prefill_row10"]
+    out = dzeros(13 * 4, 0xEE)
+    assert hip.launch_sel_gather(8, 4, 512, 1, 21, out) == (1, 13)
+    assert [int(v) for v in back(out, np.int32)] == g["decode_row"]
+    rows, cols = g["scored_shape"]
+    idx_d = dzeros(rows * cols * 4, 0xEE)
+    assert hip.launch_sel_gather_scored(dev(scores), n // 4, 8, 4, 3, n, 0, idx_d) == (rows, cols)
+    scored = back(idx_d, np.int32).reshape(rows, cols)
+    assert fnv(oracle, scored) == g["scored_fnv"] and [int(v) for v in scored[23]] == g["scored_row23"]
+    ring = dzeros(8 * d * 4)
+    hip.launch_kv_ring_write(dev(kv[:n]), ring, 8, d, n, 0)
+    assert fnv(oracle, back(ring, np.float32).reshape(8, d)) == golden["ring_after_prefill_fnv"]
+    g = golden["gather_attn"]
+    assert fnv(oracle, q) == g["q_fnv"] and fnv(oracle, kv) == g["kv_fnv"]
+    o = dzeros(n * h * d * 4)
+    hip.launch_gather_attn_shared_kv(dev(q), dev(kv), dev(sink), idx_d, n, h, d, cols, d ** -0.5, o)
+    got = back(o, np.float32).reshape(n, h, d)
+    want = np.frombuffer(bytes.fromhex(g["row23_head0_u32"]), np.uint32).view(np.float32)
+    # the reference's bar for this kernel: 1/128 of the largest expected element
+    assert np.max(np.abs(got[23, 0] - want)) <= np.max(np.abs(want)) / 128.0
