@@ -480,7 +480,11 @@ def bench_v4_attend(a, torch, hip):
            "roofline": {"bound": "mfma", "kernel": "gather_attn_d512_kernel",
                         "achieved": round(flops / att / 1e12, 2), "peak": 2500.0, "unit": "TFLOP/s",
                         "frac": round(flops / att / 2.5e15, 4), "avg_launch_ms": round(per["attend"], 5),
-                        "flops_per_launch": flops, "traffic": None,
+                        "flops_per_launch": flops,
+                        # HBM bytes per launch by rocprofv3 FETCH_SIZE + WRITE_SIZE on this workload,
+                        # each scaled by its reading for a known 1 GiB copy (profiles/); it cannot
+                        # be read from inside the process
+                        "traffic": 2917700000 if (n, h, cap) == (8192, 64, 512) else None,
                         "hbm": {"bytes_per_launch": hbm_bytes, "achieved_GBps": round(hbm_bytes / att / 1e9, 1),
                                 "frac": round(hbm_bytes / att / HBM_PEAK, 4)}}}
     # the reference's decode shape: ONE query row over the same 640-slot list, with the list
