@@ -143,6 +143,19 @@ class _V4Mixin:
         assert code or cols.value == out.shape[1]
         return code, (None if code else out)
 
+    @staticmethod
+    def compress_dst(ratio: int, region_base: int, seqlen: int, start_pos: int):
+        """crates/engine/src/v4/select.rs:278-329 restated branch by branch: None when the call
+        emits no block, else (first_row, count). Pinned by the reference's unit cases
+        (select.rs:556-611) in tests/test_oracle_v4_select.py."""
+        if ratio == 0:                                   # LayerKind::Plain: no compressor at all
+            return None
+        prefill = start_pos == 0
+        emits = seqlen >= ratio if prefill else (start_pos + 1) % ratio == 0
+        if not emits:
+            return None
+        return (region_base, seqlen // ratio) if prefill else (region_base + start_pos // ratio, 1)
+
     def ring_write(self, kv, cache, win: int, seqlen: int, start_pos: int) -> int:
         """Updates cache ([win, hd] f32) in place from kv ([rows, hd] f32)."""
         kv = _c(kv, np.float32)

@@ -282,6 +282,25 @@ def sel_shape(win, ratio, index_topk, seqlen, start_pos):
     return rows.value, cols.value
 
 
+def compress_offset(win, seqlen, start_pos):
+    """crates/engine/src/v4/select.rs:268-270: where the compressed region starts in SELECTION
+    space — past the prompt at prefill, past the ring at decode."""
+    return seqlen if start_pos == 0 else win
+
+
+def compress_dst(ratio, region_base, seqlen, start_pos):
+    """crates/engine/src/v4/select.rs:278-329 (should_compress + compress_dst): the
+    (first_row, count) this call's pooled blocks belong at, or None when the call emits none.
+    Prefill emits every complete block from the region's base; decode emits one block on the
+    position that completes it, at region_base + start_pos // ratio — a function of the
+    position, never of how many blocks were emitted before."""
+    if ratio <= 0:
+        return None
+    if start_pos == 0:
+        return (region_base, seqlen // ratio) if seqlen >= ratio else None
+    return (region_base + start_pos // ratio, 1) if (start_pos + 1) % ratio == 0 else None
+
+
 def launch_sel_gather(win, ratio, index_topk, seqlen, start_pos, out, stream=NULL_STREAM):
     """Sel::gather on the device: out is int32 [rows][cols] of sel_shape. Returns (rows, cols)."""
     shape = sel_shape(win, ratio, index_topk, seqlen, start_pos)

@@ -115,6 +115,22 @@ def test_ring_write_puts_position_t_in_slot_t_mod_win(oracle, win, hd, seqlen, s
     assert oracle.ring_write(kv, cache, win, 2, 3) == 1005
 
 
+def test_compress_dst_reference_cases(oracle):
+    """select.rs:556-611: cache space starts at the window, selection space past the prompt; the
+    decode bases coincide; the decode row is a function of the position (3, 7 for positions 15
+    and 31), not a count of blocks emitted (0, 1)."""
+    from rivoli_amd import hip
+
+    for dst, off in ((oracle.compress_dst, hip.compress_offset), (hip.compress_dst, hip.compress_offset)):
+        win, prompt = 128, 16
+        assert dst(4, win, prompt, 0) == (win, 4)
+        assert dst(4, off(win, prompt, 0), prompt, 0) == (prompt, 4)
+        assert dst(4, win, 1, 47) == (win + 11, 1) and dst(4, off(win, 1, 47), 1, 47) == (win + 11, 1)
+        assert [dst(4, 0, 1, pos)[0] for pos in (15, 31)] == [3, 7]
+        assert dst(4, 0, 1, 16) is None and dst(4, 0, 3, 0) is None and dst(0, 0, 50, 0) is None
+        assert dst(128, 128, 1, 127) == (128, 1) and dst(128, 128, 1, 128) is None
+
+
 def test_sparse_attn_closed_forms(oracle):
     rng = np.random.default_rng(3)
     h, d = 3, 16
