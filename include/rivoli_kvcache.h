@@ -240,7 +240,7 @@ int rivoli_index_select_blocks(const float* scores, int rows, int n_comp, int ra
  * columns and then the k = min(index_topk, n_comp) columns of rivoli_index_select_blocks over
  * scores [rows][n_comp]; *cols_out (host, optional) receives window columns + k.
  * Guards: 1001 null / win <= 0 / seqlen <= 0 / negative arguments (gather_scored: ratio == 0,
- * nothing to rank); 1002 more than 65535 query rows; 1005 decode with seqlen != 1
+ * nothing to rank); 1002 more than 16 776 960 columns; 1005 decode with seqlen != 1
  * (select.rs:78-86); 1006 positional selection on the indexed class with more closed blocks
  * than index_topk (select.rs:363-383: the scored form is how that is answered). */
 int rivoli_sel_shape(int win, int ratio, int index_topk, int seqlen, int start_pos, int* rows,

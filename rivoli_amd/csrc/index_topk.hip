@@ -1287,7 +1287,7 @@ __global__ __launch_bounds__(256) void sel_fill_kernel(int win, int ratio, int s
                                                        int start_pos, int win_cols, int n_pos,
                                                        int offset, int cols,
                                                        int32_t* __restrict__ out) {
-    const int j = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
+    const int j = blockIdx.y * 256 + threadIdx.x, t = blockIdx.x;  // rows on x: no 65 535 limit
     if (j >= win_cols + n_pos) return;
     int v;
     if (j < win_cols) {
@@ -1309,8 +1309,8 @@ __global__ __launch_bounds__(256) void sel_fill_kernel(int win, int ratio, int s
 static int sel_fill_launch(const SelShape& s, int win, int ratio, int seqlen, int start_pos,
                            int n_pos, int cols, int* out, hipStream_t stream) {
     (void)hipGetLastError();
-    const dim3 grid((unsigned)((s.win_cols + n_pos + 255) / 256), (unsigned)s.rows);
-    if (s.rows > 65535) return 1002;
+    const dim3 grid((unsigned)s.rows, (unsigned)((s.win_cols + n_pos + 255) / 256));
+    if (grid.y > 65535) return 1002;
     hipLaunchKernelGGL(sel_fill_kernel, grid, dim3(256), 0, stream, win, ratio, seqlen, start_pos,
                        s.win_cols, n_pos, s.offset, cols, out);
     return launch_status();

@@ -24,7 +24,7 @@ def device_gather(win, ratio, topk, seqlen, start):
     (4, 0, 512, 1, 6), (4, 0, 512, 1, 2), (4, 0, 512, 1, 3), (100, 2, 512, 6, 0), (4, 0, 512, 7, 0),
     (8, 0, 512, 5, 0), (8, 0, 512, 1, 9), (8, 4, 512, 12, 0), (8, 4, 512, 1, 19), (8, 128, 512, 1, 300),
     (128, 4, 512, 2048, 0), (128, 128, 512, 3000, 0), (128, 4, 512, 1, 2047), (128, 128, 512, 1, 60000),
-    (128, 0, 512, 700, 0), (1, 4, 512, 9, 0), (300, 4, 512, 1, 100)])
+    (128, 0, 512, 700, 0), (1, 4, 512, 9, 0), (300, 4, 512, 1, 100), (128, 128, 512, 70000, 0)])
 def test_positional_rectangle(oracle, win, ratio, topk, seqlen, start):
     code, want = oracle.sel_gather(win, ratio, topk, seqlen, start)
     assert code == 0
