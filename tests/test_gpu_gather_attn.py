@@ -128,6 +128,25 @@ def test_plain_kernel_matches_oracle(oracle, m, h, d, topk, rows):
     assert np.all(np.abs(got - exact) <= 2.0 ** -8 * np.abs(exact) + 1e-5)
 
 
+def test_random_shapes(oracle):
+    """40 random (queries, heads, width, list length) shapes: both kernels, odd widths, lists
+    shorter and longer than a tile, with and without a partial buffer."""
+    rng = np.random.default_rng(0xA77)
+    for case in range(40):
+        wide = rng.random() < 0.4
+        d = 512 if wide else int(rng.integers(1, 300))
+        h = int(rng.integers(1, 70)) if wide else int(rng.integers(1, 9))
+        m, topk, rows = int(rng.integers(1, 5)), int(rng.integers(1, 200)), int(rng.integers(1, 120))
+        q, kv, sink = attend_inputs(oracle, m, h, d, rows, seed=case, cache_like=wide)
+        idx = random_lists(rng, m, topk, rows)
+        want = oracle.sparse_attn(q, kv, sink, idx, d ** -0.5)
+        partial = None
+        if rng.random() < 0.5:
+            partial = dzeros(max(hip.gather_attn_scratch_floats(m, h, d, topk), 4) * 4)
+        got = device_attend(q, kv, sink, idx, d ** -0.5, partial=partial)
+        assert worst_rel(got, want) <= ATTEND_TOL, (case, m, h, d, topk, rows)
+
+
 def test_window_selection_feeds_the_attention(oracle):
     """The reference's own drive of this kernel (kernel_v4_attend.rs:167-213): a prefill whose
     prompt outruns the window, selection from the engine's rule, rows = the prompt's own kv."""

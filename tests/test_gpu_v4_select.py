@@ -51,6 +51,33 @@ def test_scored_rectangle(oracle, win, ratio, topk, seqlen, start, n_comp):
     assert (raw[want.size:] == np.int32(-286331154)).all()
 
 
+def test_random_rectangles(oracle):
+    """150 random (window, ratio, phase, length) shapes, positional and scored."""
+    rng = np.random.default_rng(0x5E1)
+    for case in range(150):
+        win = int(rng.integers(1, 200))
+        ratio = int(rng.choice([0, 2, 4, 4, 8, 128]))
+        if rng.random() < 0.5:
+            seqlen, start = int(rng.integers(1, 600)), 0
+        else:
+            seqlen, start = 1, int(rng.integers(1, 5000))
+        rows = seqlen if start == 0 else 1
+        if ratio and rng.random() < 0.5:
+            n_comp = (start + rows) // ratio
+            cap = int(rng.integers(1, 40))
+            scores = rng.standard_normal((rows, n_comp)).astype(np.float32).round(1)      # rounded: ties
+            code, want = oracle.sel_gather_scored(scores, win, ratio, cap, seqlen, start)
+            out = dzeros(want.size * 4 + 16, 0xEE)
+            shape = hip.launch_sel_gather_scored(dev(scores) if n_comp else None, n_comp, win, ratio, cap, seqlen,
+                                                 start, out)
+        else:
+            code, want = oracle.sel_gather(win, ratio, 10 ** 6, seqlen, start)
+            out = dzeros(want.size * 4 + 16, 0xEE)
+            shape = hip.launch_sel_gather(win, ratio, 10 ** 6, seqlen, start, out)
+        assert code == 0 and shape == want.shape, (case, win, ratio, seqlen, start)
+        assert np.array_equal(back(out, np.int32)[:want.size].reshape(want.shape), want), (case, win, ratio, seqlen, start)
+
+
 def test_scored_equals_positional_below_the_cap(oracle):
     """select.rs:645-677 on the device, both phases."""
     for seqlen, start in ((1, 19), (12, 0), (1500, 0)):
