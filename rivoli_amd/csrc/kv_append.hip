@@ -22,7 +22,7 @@ constexpr int kMaxChunksPerRow = 128;  // width <= 1024
 // Batches at least this large take the 8-rows-per-wave kernel (throughput); smaller ones the
 // one-wave-per-token kernel (latency). RIVOLI_BULK_APPEND_TOKENS overrides it at build time.
 #ifndef RIVOLI_BULK_APPEND_TOKENS
-#define RIVOLI_BULK_APPEND_TOKENS 32768
+#define RIVOLI_BULK_APPEND_TOKENS 16384
 #endif
 constexpr int kBulkAppendTokens = RIVOLI_BULK_APPEND_TOKENS;
 

@@ -122,7 +122,9 @@ def test_config2_prefill_bulk_append_with_outlier_rows(oracle):
     assert scales.max() / np.median(scales) > 20      # the outlier rows really moved the scale
 
 
-def test_append_rounding_ties_saturation_and_special_rows(oracle):
+def special_rows():
+    """19 rows that meet every branch of the quantizer: subnormal and normal ties, zeros, tiny
+    and huge scales, outliers, NaNs and infinities."""
     f32 = np.zeros((19, W), np.float32)
     q = np.float32(2.0 ** -10)
     # row 0: a 448 pins scale == 1; the rest are multiples and half-multiples of the subnormal
@@ -148,7 +150,11 @@ def test_append_rounding_ties_saturation_and_special_rows(oracle):
     f32[16, [3, 200, 575]] = np.nan
     f32[17, 40] = np.inf
     f32[18, 7], f32[18, 300] = -np.inf, np.nan
-    rows = f32_to_bf16_rne(f32)
+    return f32_to_bf16_rne(f32)
+
+
+def test_append_rounding_ties_saturation_and_special_rows(oracle):
+    rows = special_rows()
     slots = np.arange(19, dtype=np.int32) * 3
     got, want, bad, _ = paged_append_both(oracle, rows, slots, 1)
     assert bad == 0 and np.array_equal(got, want)
@@ -160,11 +166,9 @@ def test_append_rounding_ties_saturation_and_special_rows(oracle):
     assert np.count_nonzero(codes0 & 0x7F) > W // 2
 
 
-def test_append_every_amax_mantissa_against_every_value_below_it(oracle):
-    """The quotient x / scale depends only on the two mantissas and the exponent gap (powers of
-    two are exact), so every bf16 amax mantissa against every bf16 magnitude in the 18 binades
-    below it, both signs, is every quotient the quantizer can meet away from the ends of the
-    f32 range; a few exponents near those ends cover the rest."""
+def census_rows():
+    """Every bf16 amax mantissa (at seven exponents) against every bf16 magnitude in the 18
+    binades below it, both signs; the row's first element is the amax."""
     amax_bits, span = [], 18 * 128
     for e in (-118, -60, -9, 0, 8, 61, 120):
         amax_bits += [((e + 127) << 7) | m for m in range(128)]
@@ -178,6 +182,15 @@ def test_append_every_amax_mantissa_against_every_value_below_it(oracle):
         block[: vals.size] = vals
         rows[i * n_rows_each:(i + 1) * n_rows_each, 0] = ab
         rows[i * n_rows_each:(i + 1) * n_rows_each, 1:] = block.reshape(n_rows_each, per)
+    return rows
+
+
+def test_append_every_amax_mantissa_against_every_value_below_it(oracle):
+    """The quotient x / scale depends only on the two mantissas and the exponent gap (powers of
+    two are exact), so every bf16 amax mantissa against every bf16 magnitude in the 18 binades
+    below it, both signs, is every quotient the quantizer can meet away from the ends of the
+    f32 range; a few exponents near those ends cover the rest."""
+    rows = census_rows()
     n_pages = -(-rows.shape[0] // PT)
     slots = np.arange(rows.shape[0], dtype=np.int32)
     got, want, bad, _ = paged_append_both(oracle, rows, slots, n_pages)
@@ -213,5 +226,42 @@ def test_append_other_widths(oracle):
         want = np.zeros(n_pages * pb, np.uint8)
         oracle.kv_append_paged(rows, slots, want, width, pt, n_pages)
         pool = dzeros(n_pages * pb)
+        hip.launch_kv_append_paged(dev(rows), dev(slots), pool, n, width, pt, n_pages)
+        assert np.array_equal(back(pool), want), (width, pt)
+
+
+def test_large_batch_kernel_on_the_census_and_the_special_rows(oracle):
+    """Batches of 16 384 tokens and more take the eight-rows-per-wave kernel, which has its own
+    row maxima (packed 16-bit integer maxima, float maxima when a row holds a NaN) and its own
+    per-row record: the same census and special rows, interleaved so that NaN rows share a wave
+    with ordinary ones, repeated up to 40 000 tokens into shuffled slots."""
+    base = np.concatenate([special_rows(), census_rows()])
+    base = base[np.random.default_rng(11).permutation(base.shape[0])]
+    rows = np.concatenate([base] * (-(-40000 // base.shape[0])))[:40000]
+    n_pages = -(-rows.shape[0] // PT) + 3
+    slots = np.random.default_rng(12).permutation(n_pages * PT)[:rows.shape[0]].astype(np.int32)
+    page_bytes = oracle.kv_page_bytes(PT, W)
+    want = np.full(n_pages * page_bytes, 0xA5, np.uint8)
+    assert oracle.kv_append_paged(rows, slots, want, W, PT, n_pages, n_threads=8) == 0
+    pool, bad = dzeros(n_pages * page_bytes, 0xA5), dzeros(4)
+    hip.launch_kv_append_paged(dev(rows), dev(slots), pool, slots.size, W, PT, n_pages, bad)
+    got = back(pool)
+    mism = np.flatnonzero(got != want)
+    assert int(back(bad, np.uint32)[0]) == 0 and mism.size == 0, [(int(j), hex(got[j]), hex(want[j])) for j in mism[:8]]
+
+
+def test_large_batch_kernel_other_widths(oracle):
+    """The eight-rows-per-wave kernel's generic-width form, with padding tokens and a batch that
+    is not a multiple of eight."""
+    for width, pt in ((512, 64), (128, 16), (1024, 32), (64, 4), (592, 64)):
+        n = 33001
+        n_pages = -(-n // pt) + 2
+        rows = make_rows_bf16(n, width, seed=width + 1, outlier_frac=0.01, outlier_mul=200.0)
+        slots = np.random.default_rng(width).permutation(n_pages * pt)[:n].astype(np.int32)
+        slots[::97] = -1                                   # padding tokens
+        pb = oracle.kv_page_bytes(pt, width)
+        want = np.full(n_pages * pb, 0x5A, np.uint8)
+        oracle.kv_append_paged(rows, slots, want, width, pt, n_pages, n_threads=8)
+        pool = dzeros(n_pages * pb, 0x5A)
         hip.launch_kv_append_paged(dev(rows), dev(slots), pool, n, width, pt, n_pages)
         assert np.array_equal(back(pool), want), (width, pt)
