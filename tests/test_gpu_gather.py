@@ -169,3 +169,14 @@ def test_sparse_rows_short_lists_and_bad_rows(oracle):
     keep[0, 7] = keep[1, 2] = False
     full = oracle.kv_gather_rows_paged(pool, tables, rows, W, PT)
     assert np.array_equal(got[keep], full[keep])
+
+
+def test_sparse_rows_other_shapes(oracle):
+    """The sparse gather's generic form: other widths and page sizes, unsorted lists."""
+    for width, pt, ctx, k in ((512, 64, 300, 77), (128, 16, 100, 40), (1024, 32, 65, 65), (64, 4, 9, 5)):
+        lens = [ctx, ctx]
+        pool, tables = build_pool(oracle, lens, 64, seed=width + 3, width=width, pt=pt)
+        rows = np.random.default_rng(width).integers(0, ctx, (2, k)).astype(np.uint32)
+        got, bad = gpu_gather_rows(pool, tables, rows, width=width, pt=pt)
+        want = oracle.kv_gather_rows_paged(pool, tables, rows, width, pt)
+        assert bad == 0 and np.array_equal(got, want), (width, pt)

@@ -163,7 +163,9 @@ def adversarial_scores(rows, n_comp, seed):
     (1, 300, 4, 64, False), (40, 9, 4, 3, True), (130, 2, 128, 1, True), (3, 50, 4, 50, False),
     (700, 160, 4, 40, True),                                          # prefill rows of growing limit
     (1, 16384, 4, 2048, False),                                       # a 64K context at ratio 4
-    (5, 3000, 4, 512, False), (2, 70000, 4, 2048, False), (1, 1025, 4, 1024, False)])
+    (5, 3000, 4, 512, False), (2, 70000, 4, 2048, False), (1, 1025, 4, 1024, False),
+    # one case per remaining dispatch width: 4 waves, 16 waves, the 64-keys-per-thread select
+    (2, 6000, 4, 512, False), (2, 20000, 4, 2048, False), (2, 50000, 4, 700, False), (3, 8192, 4, 8000, False)])
 def test_select_matches_oracle(oracle, rows, n_comp, ratio, topk, prefill):
     s = adversarial_scores(rows, n_comp, seed=rows * 131 + n_comp)
     want = oracle.v4_scored_rows(s, ratio, topk, prefill, 4096)
