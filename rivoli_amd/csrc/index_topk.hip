@@ -260,7 +260,6 @@ constexpr int kTopkWaves = kTopkThreads / kWave;
 constexpr int kLeanBits = 10;
 constexpr int kLeanBins = 1 << kLeanBits;  // == kTopkThreads: one thread per bin
 constexpr int kLeanCopies = 8;
-constexpr int kLeanLow = 32 - kLeanBits;
 constexpr int kLeanCap = 12288;  // candidates held in LDS (index + key)
 static_assert(kLeanBins == kTopkThreads, "one thread per bin");
 constexpr int kLeanLdsWords = 2 * kLeanCap + kLeanBins * kLeanCopies + 4 * kTopkWaves + 8;
@@ -1283,10 +1282,9 @@ static SelShape sel_shape(int win, int ratio, int seqlen, int start_pos) {
 
 // One thread per cell of the first `win_cols + n_pos` columns of a `cols`-wide row: the window
 // rule (select.rs:195-216), then the positional block rule (:224-241) for n_pos columns.
-__global__ __launch_bounds__(256) void sel_fill_kernel(int win, int ratio, int seqlen,
-                                                       int start_pos, int win_cols, int n_pos,
-                                                       int offset, int cols,
-                                                       int32_t* __restrict__ out) {
+__global__ __launch_bounds__(256) void sel_fill_kernel(int win, int ratio, int start_pos,
+                                                       int win_cols, int n_pos, int offset,
+                                                       int cols, int32_t* __restrict__ out) {
     const int j = blockIdx.y * 256 + threadIdx.x, t = blockIdx.x;  // rows on x: no 65 535 limit
     if (j >= win_cols + n_pos) return;
     int v;
@@ -1306,13 +1304,13 @@ __global__ __launch_bounds__(256) void sel_fill_kernel(int win, int ratio, int s
     out[(size_t)t * cols + j] = v;
 }
 
-static int sel_fill_launch(const SelShape& s, int win, int ratio, int seqlen, int start_pos,
-                           int n_pos, int cols, int* out, hipStream_t stream) {
+static int sel_fill_launch(const SelShape& s, int win, int ratio, int start_pos, int n_pos,
+                           int cols, int* out, hipStream_t stream) {
     (void)hipGetLastError();
     const dim3 grid((unsigned)s.rows, (unsigned)((s.win_cols + n_pos + 255) / 256));
     if (grid.y > 65535) return 1002;
-    hipLaunchKernelGGL(sel_fill_kernel, grid, dim3(256), 0, stream, win, ratio, seqlen, start_pos,
-                       s.win_cols, n_pos, s.offset, cols, out);
+    hipLaunchKernelGGL(sel_fill_kernel, grid, dim3(256), 0, stream, win, ratio, start_pos, s.win_cols,
+                       n_pos, s.offset, cols, out);
     return launch_status();
 }
 
@@ -1336,8 +1334,7 @@ extern "C" int rivoli_sel_gather(int win, int ratio, int index_topk, int seqlen,
     if (code) return code;
     if (!out) return 1001;
     const rk::SelShape s = rk::sel_shape(win, ratio, seqlen, start_pos);
-    return rk::sel_fill_launch(s, win, ratio, seqlen, start_pos, s.n_comp, cols, out,
-                               (hipStream_t)stream);
+    return rk::sel_fill_launch(s, win, ratio, start_pos, s.n_comp, cols, out, (hipStream_t)stream);
 }
 
 extern "C" int rivoli_sel_gather_scored(const float* scores, int n_comp, int win, int ratio,
@@ -1350,8 +1347,7 @@ extern "C" int rivoli_sel_gather_scored(const float* scores, int n_comp, int win
     const int k = index_topk < n_comp ? index_topk : n_comp;
     const int cols = s.win_cols + k;
     if (cols_out) *cols_out = cols;
-    const int code = rk::sel_fill_launch(s, win, ratio, seqlen, start_pos, 0, cols, out,
-                                         (hipStream_t)stream);
+    const int code = rk::sel_fill_launch(s, win, ratio, start_pos, 0, cols, out, (hipStream_t)stream);
     if (code || k == 0) return code;
     return rk::block_select_launch(scores, s.rows, n_comp, ratio, index_topk, start_pos == 0,
                                    s.offset, out + s.win_cols, cols, (hipStream_t)stream);
