@@ -803,6 +803,13 @@ def cpu_baseline(pool0, tables_np, seq_lens_np, out, budget_s, hip, tables, seq_
         reps += 1
     per_layer_s = spent / reps
     bytes_layer = n_tok * (REC + ROW_IN) + tables_np.size * 4
+    # the same oracle on ONE host thread, over the first sequence only (a bounded sample)
+    one_len = seq_lens_np[:1].copy()
+    one_out = np.empty((int(one_len[0]), W), np.uint16)
+    t0 = time.perf_counter()
+    ora.kv_gather_paged(pool_host, tables_np[:1], one_len, W, PT, n_threads=1, out=one_out)
+    one_s = time.perf_counter() - t0
+    one_bytes = int(one_len[0]) * (REC + ROW_IN)
     # full-size parity of one layer: GPU gather of the same pool vs the oracle's bytes
     hip.launch_kv_gather_paged(pool0, tables, seq_lens, cu, out, B, blocks, W, PT, n_pages)
     torch.cuda.synchronize()
@@ -814,7 +821,9 @@ def cpu_baseline(pool0, tables_np, seq_lens_np, out, budget_s, hip, tables, seq_
             "kind": "port",
             "sample": f"gather+dequantize of one layer ({n_tok} tokens, same pool and block "
                       f"tables) x{reps} reps, {cores} host threads; GPU output checked equal",
-            "tokens_per_s": round(n_tok / per_layer_s, 1)}
+            "tokens_per_s": round(n_tok / per_layer_s, 1),
+            "one_thread": {"value": round(one_bytes / one_s / 1e9, 3), "unit": "GB/s",
+                           "sample": f"the first sequence of the same layer ({int(one_len[0])} tokens), once"}}
 
 
 if __name__ == "__main__":
