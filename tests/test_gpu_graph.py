@@ -85,3 +85,98 @@ def test_decode_step_replays_from_a_graph(oracle):
     sc = np.random.default_rng(602).standard_normal((n_seqs, max_ctx)).astype(np.float32)
     assert np.array_equal(got[2].cpu().numpy().view(np.uint32).reshape(n_seqs, K),
                           oracle.topk_batched(sc, K, nts=now))
+
+
+def test_second_format_decode_step_replays_from_a_graph(oracle):
+    """The second cache format's decode step — quantize the new entry, write it into the ring,
+    deposit into the compressor (and pool the block this position closes), build the
+    [ring | scored blocks] rectangle, attend with the list shared among workgroups — captured
+    once at a position that closes a block and replayed on fresh inputs."""
+    from oracle.kvoracle import CompGeom as OracleGeom
+    from tests.v4_cases import bf16_round, compress_inputs
+
+    torch = torch_cuda()
+    win, ratio, d, rd, heads, cap, pos = 128, 4, 512, 64, 64, 64, 1023      # position 1023 closes block 255
+    n_comp = (pos + 1) // ratio
+    og, hg = OracleGeom.attention(ratio, d, rd), hip.CompGeom.build(ratio, d, rd, 1e-6)
+    rng = np.random.default_rng(5)
+    _, _, ape, norm, freqs = compress_inputs(og, 8, seed=3, positions=pos + 1)
+    cache0 = bf16_round(rng.standard_normal((win + 512, d)).astype(np.float32))
+    cache, state_kv = dev(cache0), dev(rng.standard_normal((og.coff * ratio, og.cd)).astype(np.float32))
+    state_sc = dev(rng.standard_normal((og.coff * ratio, og.cd)).astype(np.float32))
+    ape_d, norm_d, freqs_d, sink = dev(ape), dev(norm), dev(freqs), dev(rng.standard_normal(heads).astype(np.float32))
+    # the step's inputs live in fixed device buffers that the host refills between replays
+    entry = torch.zeros(d * 4, dtype=torch.uint8, device="cuda")
+    ckv = torch.zeros(og.cd * 4, dtype=torch.uint8, device="cuda")
+    csc = torch.zeros(og.cd * 4, dtype=torch.uint8, device="cuda")
+    q = torch.zeros(heads * d * 4, dtype=torch.uint8, device="cuda")
+    scores = torch.zeros(n_comp * 4, dtype=torch.uint8, device="cuda")
+    cols = win + cap
+    idx = torch.zeros(cols * 4, dtype=torch.uint8, device="cuda")
+    o = torch.zeros(heads * d * 4, dtype=torch.uint8, device="cuda")
+    part = torch.zeros(max(hip.gather_attn_scratch_floats(1, heads, d, cols), 4) * 4, dtype=torch.uint8, device="cuda")
+    first, _ = hip.compress_dst(ratio, win, 1, pos)
+    block_row = cache[first * d * 4:(first + 1) * d * 4]                 # the pooled block's home, by position
+    fin = hip.CompFinish.of(norm_d, freqs_d, block_row)
+
+    def step(stream):
+        hip.launch_act_quant_f8_prefix(entry, entry, 1, d, d - rd, 64, stream)
+        hip.launch_kv_ring_write(entry, cache, win, d, 1, pos, stream)
+        hip.launch_kv_compress_deposit(ckv, csc, ape_d, state_kv, state_sc, hg, 1, pos % ratio, stream)
+        hip.launch_kv_compress_decode(state_kv, state_sc, fin, hg, pos, stream)
+        hip.launch_act_quant_f8_prefix(block_row, block_row, 1, d, d - rd, 64, stream)
+        hip.launch_sel_gather_scored(scores, n_comp, win, ratio, cap, 1, pos, idx, stream)
+        hip.launch_gather_attn_shared_kv(q, cache, sink, idx, 1, heads, d, cols, d ** -0.5, o, stream, partial=part)
+
+    def load_inputs(t):
+        r = np.random.default_rng(900 + t)
+        for buf, a in ((entry, bf16_round(r.standard_normal(d).astype(np.float32))),
+                       (ckv, r.standard_normal(og.cd).astype(np.float32)),
+                       (csc, r.standard_normal(og.cd).astype(np.float32)),
+                       (q, bf16_round(r.standard_normal((heads, d)).astype(np.float32))),
+                       (scores, r.standard_normal(n_comp).astype(np.float32))):
+            buf.copy_(dev(a))
+
+    state = (cache, state_kv, state_sc)
+
+    def outputs():
+        torch.cuda.synchronize()
+        return [b.clone() for b in (cache, state_kv, state_sc, idx, o)]
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        load_inputs(0)
+        saved = [b.clone() for b in state]
+        step(stream.cuda_stream)                                   # warm-up outside the capture
+        stream.synchronize()
+        for b, s in zip(state, saved):
+            b.copy_(s)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            step(torch.cuda.current_stream().cuda_stream)
+        for b, s in zip(state, saved):                             # the capture ran nothing; start clean anyway
+            b.copy_(s)
+        for t in range(3):
+            before = [b.clone() for b in state]
+            load_inputs(t)
+            entry_in = entry.clone()
+            for b in (idx, o):
+                b.fill_(0xEE)
+            step(stream.cuda_stream)                               # eager, for the expectation
+            want = outputs()
+            for b, s in zip(state, before):                        # undo the step, then replay it
+                b.copy_(s)
+            entry.copy_(entry_in)
+            for b in (idx, o):
+                b.fill_(0xEE)
+            graph.replay()
+            got = outputs()
+            for name, g, w in zip(("cache", "compressor kv state", "compressor score state", "rectangle", "attention"),
+                                  got, want):
+                assert torch.equal(g, w), (t, name)
+    # and the eager result is the oracle's: the last rectangle against the CPU rule
+    r = np.random.default_rng(902)                                  # load_inputs(2): its scores are the fifth draw
+    for n in (d, og.cd, og.cd, heads * d):
+        r.standard_normal(n)
+    code, want_rect = oracle.sel_gather_scored(r.standard_normal(n_comp).astype(np.float32)[None, :], win, ratio, cap, 1, pos)
+    assert code == 0 and np.array_equal(got[3].cpu().numpy().view(np.int32).reshape(1, cols), want_rect)
