@@ -66,6 +66,9 @@ def parse():
                          "(configuration 3 as written) instead of every sequence at ctx (its metric point)")
     ap.add_argument("--tokens", type=int, default=8192, help="prefill: new tokens per step")
     ap.add_argument("--topk", type=int, default=2048)
+    ap.add_argument("--unfused", action="store_true",
+                    help="dsa / dsa_scored: run the selection and the sparse gather as two separate "
+                         "entry points instead of the one fused call")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (a known-size kernel to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
@@ -593,14 +596,23 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
     stream = torch.cuda.Stream()
     sh = stream.cuda_stream
 
+    fused = not attend and not a.unfused
+
     def step(events):
         for layer in range(L):
             if scored:
+                score = hip.launch_index_score_paged_hist if fused else hip.launch_index_score_paged
+                tail = (ws_topk, sh) if fused else (sh,)
                 bracket(torch, stream, events, "score",
-                        lambda: hip.launch_index_score_paged(
-                            qs[layer], ws[layer], kpools[layer], tables, None, None, B, blocks, nt,
-                            nt, NH, NH, HD, PT, n_pages, HD ** -0.5, 1.0, score_buf, sh))
+                        lambda: score(qs[layer], ws[layer], kpools[layer], tables, None, None, B, blocks, nt,
+                                      nt, NH, NH, HD, PT, n_pages, HD ** -0.5, 1.0, score_buf, *tail))
             sc_in = score_buf if scored else scores[layer]
+            if fused:
+                bracket(torch, stream, events, "select_gather",
+                        lambda: hip.launch_dsa_select_gather_paged(sc_in, B, nt, None, nt, k, sel, ws_topk, scored,
+                                                                   pools[layer], tables, out, blocks, W, PT,
+                                                                   n_pages, None, sh))
+                continue
             bracket(torch, stream, events, "topk",
                     lambda: hip.launch_index_topk_batched(sc_in, B, nt, None, nt, k, sel, ws_topk, sh))
             if attend:
@@ -618,28 +630,33 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
     rows_bytes = B * k * (4 + REC + ROW_IN) + B * blocks * 4
     if attend:  # row list, records and table in, q in, clat out; no bf16 rows are written
         rows_bytes = B * k * (4 + REC) + B * blocks * 4 + B * H * (W + 512) * 4
-    rows_kernel = "attend_rows" if attend else "gather_rows"
+    rows_kernel = "attend_rows" if attend else ("select_gather" if fused else "gather_rows")
     score_bytes = (B * nt * (HD * 2 + 4) + B * NH * (HD + 1) * 4 + B * blocks * 4) if scored else 0
     layer_bytes = topk_bytes + rows_bytes + score_bytes
+    dom_bytes = topk_bytes + rows_bytes if fused else rows_bytes
     res = {"metric": "kv_dsa_topk_gather_GBps", "value": round(L * layer_bytes / (ms * 1e-3) / 1e9, 2),
            "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-           "config": {"workload": "DSA sparse path (benchmark configuration 4): top-k then sparse row gather",
+           "config": {"workload": "DSA sparse path (benchmark configuration 4): top-k then sparse row gather"
+                                  + (", one fused call per layer" if fused else ""),
                       "layers": L, "batch": B, "ctx": nt, "k": k, "width": W, "page_tokens": PT},
            "rows_per_s": round(L * B * k / (ms * 1e-3), 1),
+           "layer_us": round(ms * 1e3 / L, 2), "hbm_peak_frac": round(L * layer_bytes / (ms * 1e-3) / HBM_PEAK, 4),
            "kernels_ms": {n: round(v, 5) for n, v in per.items()},
-           "roofline": {"bound": "hbm", "kernel": "mla_attend_paged_kernel" if attend else "kv_gather_rows_kernel",
-                        "achieved": round(rows_bytes / (per[rows_kernel] * 1e-3) / 1e9, 2),
+           "roofline": {"bound": "hbm",
+                        "kernel": "mla_attend_paged_kernel" if attend else
+                                  ("topk_hist + topk_cand + topk_finish (select and gather)" if fused
+                                   else "kv_gather_rows_kernel"),
+                        "achieved": round(dom_bytes / (per[rows_kernel] * 1e-3) / 1e9, 2),
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                        "frac": round(rows_bytes / (per[rows_kernel] * 1e-3) / HBM_PEAK, 5),
+                        "frac": round(dom_bytes / (per[rows_kernel] * 1e-3) / HBM_PEAK, 5),
                         "avg_launch_ms": round(per[rows_kernel], 5),
-                        "bytes_per_launch": rows_bytes,
-                        # rocprofv3 FETCH_SIZE + WRITE_SIZE of the sparse gather at configuration 4's
-                        # shape, scaled by a known 1 GiB copy (profiles/)
-                        "traffic": 61700000 if (not attend and (B, nt, k) == (16, 65536, 2048)) else None},
-           "topk": {"achieved": round(topk_bytes / (per["topk"] * 1e-3) / 1e9, 2), "unit": "GB/s",
-                    "avg_launch_ms": round(per["topk"], 5), "bytes_per_launch": topk_bytes}}
+                        "bytes_per_launch": dom_bytes,
+                        "traffic": None}}
+    if not fused:
+        res["topk"] = {"achieved": round(topk_bytes / (per["topk"] * 1e-3) / 1e9, 2), "unit": "GB/s",
+                       "avg_launch_ms": round(per["topk"], 5), "bytes_per_launch": topk_bytes}
     if scored:
         res["config"]["workload"] = ("DSA sparse path with device scores: index_score (64 heads x "
                                      "128, paged bf16 keys) -> top-k -> sparse row gather")
@@ -664,8 +681,12 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
             want_rows = ora.kv_gather_rows_paged(pool_h, tables_np, want_sel, W, PT)
             spent += time.perf_counter() - t0
             reps += 1
-        hip.launch_index_topk_batched(scores[0], B, nt, None, nt, k, sel, ws_topk)
-        hip.launch_kv_gather_rows_paged(pools[0], tables, sel, None, out, B, k, blocks, W, PT, n_pages)
+        if fused:
+            hip.launch_dsa_select_gather_paged(scores[0], B, nt, None, nt, k, sel, ws_topk, False, pools[0], tables,
+                                               out, blocks, W, PT, n_pages)
+        else:
+            hip.launch_index_topk_batched(scores[0], B, nt, None, nt, k, sel, ws_topk)
+            hip.launch_kv_gather_rows_paged(pools[0], tables, sel, None, out, B, k, blocks, W, PT, n_pages)
         torch.cuda.synchronize()
         if not np.array_equal(sel.cpu().numpy().view(np.uint32).reshape(B, k), want_sel):
             raise SystemExit("bench: GPU top-k differs from the CPU oracle")

@@ -125,14 +125,35 @@ int rivoli_kv_gather_rows_paged(const unsigned char* pool, const int* block_tabl
  * when nts is null) and writes rows[q*k .. +min(k, nt_q)), ascending. One call for all
  * queries; the selection rule is the single-query one.
  * `workspace` (nullable) lets the call spread every query over many workgroups instead of
- * one: rivoli_index_topk_workspace_bytes(n_queries, nt) bytes of device memory that the
- * caller zero-fills ONCE (hipMemset) before its first use; every call puts back to zero
+ * one (queries longer than 16384 scores; shorter ones stay on one workgroup either way):
+ * rivoli_index_topk_workspace_bytes(n_queries, nt) bytes of 16-byte-aligned device memory that
+ * the caller zero-fills ONCE (hipMemset) before its first use; every call puts back to zero
  * whatever has to start at zero, so it can be reused call after call on one stream (calls
- * that share a workspace must not overlap). With a null workspace each query is selected by a single workgroup.
- * Guards: 1001 null / non-positive; 1002 stride < nt. */
+ * that share a workspace must not overlap, and a workspace serves one (n_queries, nt) shape).
+ * The split form is three launches on the stream and no workgroup waits for another.
+ * Guards: 1001 null / non-positive; 1002 stride < nt; 1004 workspace not 16-byte aligned. */
 size_t rivoli_index_topk_workspace_bytes(int n_queries, int nt);
 int rivoli_index_topk_batched(const float* scores, int n_queries, int stride, const int* nts,
                               int nt, int k, unsigned int* rows, void* workspace, void* stream);
+
+/* The DSA step the reference runs as index_topk followed by an attend over `rows`, with "no
+ * D2H, no host top-k, and no device_sync" between them (crates/backend/src/hip_attn.rs:478-495),
+ * for a consumer that wants the selected rows as bf16: rivoli_index_topk_batched and
+ * rivoli_kv_gather_rows_paged in one call. rows[q*k + j] as the batched top-k writes them, and
+ * out[(q*k + j)*width ..] = the dequantized token rows[q*k + j] of sequence q for
+ * j < min(k, nt_q), through block_table[q]. With a workspace and a split shape the selection's
+ * last launch gathers the rows it has just placed (no separate gather launch, and the gather
+ * is dealt evenly whatever the positions of the selected tokens); otherwise the two kernels
+ * follow each other on the stream. hist_ready != 0: the workspace's histogram was filled by
+ * rivoli_index_score_paged_hist on the same stream with the same (n_queries, nt, nts) — the
+ * selection then skips its first launch (1001 when the shape is not a split one).
+ * Guards: those of the two calls it stands for. */
+int rivoli_dsa_select_gather_paged(const float* scores, int n_queries, int stride, const int* nts,
+                                   int nt, int k, unsigned int* rows, void* workspace,
+                                   int hist_ready, const unsigned char* pool,
+                                   const int* block_table, unsigned short* out,
+                                   int max_blocks_per_seq, int width, int page_tokens, int n_pages,
+                                   unsigned int* bad_rows, void* stream);
 
 /* Replaces crates/backend/kernels/indexer.hip:278-295 (launch_index_score,
  * crates/backend/src/hip_attn.rs:464-476): scores[t] = sum over the active heads h of
@@ -156,6 +177,20 @@ int rivoli_index_score_paged(const float* q, const float* w, const unsigned shor
                              int n_queries, int max_blocks_per_seq, int stride, int nt, int nh,
                              int nact, int hd, int page_tokens, int n_pages, float wscale,
                              float dscale, float* scores, void* stream);
+
+/* rivoli_index_score_paged that also does the first step of the selection that follows it
+ * (the score -> top-k fusion the reference's design aims at, crates/backend/kernels/
+ * indexer.hip:1-13): while a score is still in a register its selection key's top 12 bits are
+ * counted into topk_workspace (the rivoli_index_topk_workspace_bytes(n_queries, nt) buffer the
+ * selection will be handed, zero-filled as described there), so rivoli_dsa_select_gather_paged
+ * (hist_ready = 1) does not sweep the scores for it. For shapes the selection does not split
+ * (nt <= 16384) the workspace is left alone. Guards as rivoli_index_score_paged, plus 1001 for a
+ * null workspace and 1004 for one that is not 16-byte aligned. */
+int rivoli_index_score_paged_hist(const float* q, const float* w, const unsigned short* kpool,
+                                  const int* block_table, const int* nts, const unsigned int* heads,
+                                  int n_queries, int max_blocks_per_seq, int stride, int nt, int nh,
+                                  int nact, int hd, int page_tokens, int n_pages, float wscale,
+                                  float dscale, float* scores, void* topk_workspace, void* stream);
 
 /* Paged form of rivoli_index_append for many tokens: kpool[slot_mapping[t]*hd + i] =
  * bf16(k[t*hd + i]). Negative slots are padding; slots >= n_pages*page_tokens are counted in

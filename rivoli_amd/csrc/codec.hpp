@@ -172,6 +172,36 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
     return v;
 }
+// A workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every global
+// load and store the wave has in flight (a full memory round trip when a store was just issued);
+// where only LDS contents are handed between waves, that wait is pure latency.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Inclusive prefix sum over the 64 lanes on the DPP path: four shifts inside each row of 16
+// lanes, then the two row broadcasts (lane 15 of a row into the next row, lane 31 into the
+// upper half). A step is one ALU instruction; the generic cross-lane shuffle goes through the
+// LDS crossbar and costs an LDS round trip per step.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_or_zero(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+__device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t v) {
+    v += dpp_or_zero<0x111, 0xf>(v);  // row_shr:1
+    v += dpp_or_zero<0x112, 0xf>(v);  // row_shr:2
+    v += dpp_or_zero<0x114, 0xf>(v);  // row_shr:4
+    v += dpp_or_zero<0x118, 0xf>(v);  // row_shr:8
+    v += dpp_or_zero<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+    v += dpp_or_zero<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+// The sum over the wave, as a scalar.
+__device__ __forceinline__ uint32_t wave_total(uint32_t inclusive) {
+    return (uint32_t)__builtin_amdgcn_readlane((int)inclusive, kWave - 1);
+}
 __device__ __forceinline__ unsigned long long wave_xor(unsigned long long v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v ^= __shfl_xor(v, off, kWave);

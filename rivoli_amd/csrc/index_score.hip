@@ -19,7 +19,7 @@
 // A workgroup stages its query once and walks 2048 tokens (4 waves x 16 blocks of 32). The
 // kernel reads hd*2 bytes per token and is bound by that stream, not by the matrix cores.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
-#include "codec.hpp"
+#include "topk_common.hpp"
 
 namespace rk {
 
@@ -47,13 +47,17 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
     const uint16_t* __restrict__ kpool, const int* __restrict__ block_table,
     const int* __restrict__ nts, const unsigned int* __restrict__ heads, int max_blocks_per_seq,
     int stride, int nt_all, int nh, int nact, int hd_rt, int page_tokens, int n_pages, float wscale,
-    float dscale, float* __restrict__ scores) {
+    float dscale, float* __restrict__ scores, uint32_t* __restrict__ topk_ws, size_t ws_stride) {
     const int hd = HD ? HD : hd_rt;
     __shared__ __attribute__((aligned(16))) uint16_t s_qh[RB * 32][kScoreMaxHd + kScoreRowPad];
     __shared__ __attribute__((aligned(16))) uint16_t s_ql[RB * 32][kScoreMaxHd + kScoreRowPad];
     __shared__ float s_w[RB * 32];
     __shared__ __attribute__((aligned(16)))
     uint16_t s_k[kScoreWaves][32][kScoreMaxHd + kScoreRowPad];  // one key tile per wave
+    // With a top-k workspace: the histogram of this workgroup's scores by the top 12 bits of
+    // their selection key, two 16-bit counters per word (a workgroup scores 2048 tokens).
+    __shared__ uint32_t s_hist[kTopBins / 2];
+    static_assert(kScoreTokensPerGroup < 65536, "16-bit histogram counters");
 
     const int qi = blockIdx.y;
     const int nt = nts ? min(nts[qi], nt_all) : nt_all;
@@ -62,6 +66,8 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    if (topk_ws)
+        for (int i = tid; i < kTopBins / 2; i += kScoreThreads) s_hist[i] = 0u;
 
     // ---- stage the active heads: q = hi + lo in bf16, and the per-head weight ----
     // eight consecutive query values per step: two 16-byte loads in, two 16-byte LDS stores out
@@ -201,9 +207,24 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
 #pragma unroll
             for (int v = 0; v < 16; ++v) sum += wv[rb][v] * fmaxf(acc[rb][v] * dscale, 0.0f);
         sum += __shfl_xor(sum, 32, kWave);
-        if (lane < 32 && valid) scores[(size_t)qi * stride + token] = sum;
+        if (lane < 32 && valid) {
+            scores[(size_t)qi * stride + token] = sum;
+            if (topk_ws) {
+                const uint32_t bin = topk_key(sum) >> kLowBits;
+                atomicAdd(&s_hist[bin >> 1], 1u << ((bin & 1u) * 16u));
+            }
+        }
         tb = tb_next;
         rows_ok = rows_next;
+    }
+    if (!topk_ws) return;
+    // the selection's first launch, done here: one global atomic per non-empty bin
+    __syncthreads();
+    uint32_t* wq = topk_ws + (size_t)qi * ws_stride;
+    for (int i = tid; i < kTopBins / 2; i += kScoreThreads) {
+        const uint32_t c = s_hist[i];
+        if (c & 0xffffu) atomicAdd(&wq[2 * i], c & 0xffffu);
+        if (c >> 16) atomicAdd(&wq[2 * i + 1], c >> 16);
     }
 }
 
@@ -235,19 +256,24 @@ static int index_score_launch(const float* q, const float* w, const unsigned sho
                               const int* block_table, const int* nts, const unsigned int* heads,
                               int n_queries, int max_blocks_per_seq, int stride, int nt, int nh,
                               int nact, int hd, int page_tokens, int n_pages, float wscale,
-                              float dscale, float* scores, hipStream_t stream) {
+                              float dscale, float* scores, void* topk_workspace,
+                              hipStream_t stream) {
     if (!q || !w || !kpool || !scores) return 1001;
     if (n_queries <= 0 || nt <= 0 || nh <= 0 || nact <= 0 || nact > nh || hd <= 0) return 1001;
     if (block_table && (max_blocks_per_seq <= 0 || page_tokens <= 0 || n_pages <= 0)) return 1001;
     if (nact > kScoreMaxHeads || hd > kScoreMaxHd || stride < nt || n_queries > 65535) return 1002;
     if ((hd % 16) != 0 || (block_table && (page_tokens % 32) != 0)) return 1004;
+    // the histogram is only wanted where the selection of this shape runs split over the chip
+    if (topk_workspace && !aligned16(topk_workspace)) return 1004;
+    uint32_t* ws = topk_runs_split(n_queries, nt) ? (uint32_t*)topk_workspace : nullptr;
+    const size_t ws_stride = topk_ws_words(topk_segments(nt));
     dim3 grid((unsigned)((nt + kScoreTokensPerGroup - 1) / kScoreTokensPerGroup),
               (unsigned)n_queries);
     (void)hipGetLastError();
 #define RK_SCORE(RBV, HDV)                                                                      \
     hipLaunchKernelGGL((index_score_kernel<RBV, HDV>), grid, dim3(kScoreThreads), 0, stream, q, w, \
                        kpool, block_table, nts, heads, max_blocks_per_seq, stride, nt, nh, nact,  \
-                       hd, page_tokens, n_pages, wscale, dscale, scores)
+                       hd, page_tokens, n_pages, wscale, dscale, scores, ws, ws_stride)
     if (hd == 128) {
         if (nact <= 32) RK_SCORE(1, 128); else RK_SCORE(2, 128);
     } else {
@@ -263,7 +289,7 @@ extern "C" int rivoli_index_score(const float* q, const float* w, const unsigned
                                   const unsigned int* heads, int nt, int nh, int nact, int hd,
                                   float wscale, float dscale, float* scores) {
     return rk::index_score_launch(q, w, kcache, nullptr, nullptr, heads, 1, 0, nt, nt, nh, nact, hd,
-                                  0, 0, wscale, dscale, scores, nullptr);
+                                  0, 0, wscale, dscale, scores, nullptr, nullptr);
 }
 
 extern "C" int rivoli_index_score_paged(const float* q, const float* w,
@@ -275,7 +301,21 @@ extern "C" int rivoli_index_score_paged(const float* q, const float* w,
     if (!block_table) return 1001;
     return rk::index_score_launch(q, w, kpool, block_table, nts, heads, n_queries,
                                   max_blocks_per_seq, stride, nt, nh, nact, hd, page_tokens,
-                                  n_pages, wscale, dscale, scores, (hipStream_t)stream);
+                                  n_pages, wscale, dscale, scores, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int rivoli_index_score_paged_hist(const float* q, const float* w,
+                                             const unsigned short* kpool, const int* block_table,
+                                             const int* nts, const unsigned int* heads,
+                                             int n_queries, int max_blocks_per_seq, int stride,
+                                             int nt, int nh, int nact, int hd, int page_tokens,
+                                             int n_pages, float wscale, float dscale, float* scores,
+                                             void* topk_workspace, void* stream) {
+    if (!block_table || !topk_workspace) return 1001;
+    return rk::index_score_launch(q, w, kpool, block_table, nts, heads, n_queries,
+                                  max_blocks_per_seq, stride, nt, nh, nact, hd, page_tokens,
+                                  n_pages, wscale, dscale, scores, topk_workspace,
+                                  (hipStream_t)stream);
 }
 
 extern "C" int rivoli_index_append_paged(const float* k, const int* slot_mapping,

@@ -19,57 +19,34 @@
 //     waves one short prefix. It needs no scratch memory, so it serves the reference-signature
 //     entry point; but 65536 keys x several sweeps on ONE compute unit is issue-bound.
 //
-// (2) Split across the chip (`topk_hist_kernel` + `topk_select_kernel`), used when the caller
-//     supplies a workspace: every 4096-score segment of every query gets its own workgroup.
-//     Kernel A histograms the top 12 key bits per query in global memory (LDS histogram first,
-//     then one atomic per non-empty bin); the LAST workgroup of a query to finish — decided by
-//     a ticket, never by waiting — walks the histogram for the bin that holds the k-th key.
-//     Kernel B writes, per segment and in index order, the indices whose key is in that bin or
-//     above (at least k of them, typically ~1.5 k); the last workgroup of the query pulls those
-//     candidates into LDS, finishes the radix select on the low 20 bits among the bin's
-//     members, and emits the selection in index order. If the candidates do not fit in LDS
-//     (degenerate score arrays: huge ties) that workgroup runs shape (1) over the query
-//     instead — slower, same answer. The workspace is left zeroed for the next call.
+// (2) Split across the chip, used when the caller supplies a workspace: three launches, no
+//     workgroup ever waits for another, nothing is elected. `topk_hist_kernel`: every
+//     4096-score segment of every query adds the histogram of its keys' top 12 bits to the
+//     query's global histogram (LDS first, then one atomic per non-empty bin) — a producer that
+//     has the scores in registers anyway (the indexer's score kernel) can do this step itself.
+//     `topk_cand_kernel`: every segment re-derives the pivot bin (the one holding the k-th key)
+//     from that histogram, counts its keys in higher bins and lists its keys IN the pivot bin.
+//     `topk_finish_kernel`: a query's selection is dealt to workgroups by OUTPUT position, 128
+//     slots each. Every one of them pulls the query's listed keys (a few thousand) into LDS and
+//     finishes the radix select on the low 20 bits by itself — redundant work on otherwise idle
+//     compute units instead of a hand-over — which gives the exact pivot and, per segment, how
+//     many keys precede; it then re-reads only the segments its slots fall in, emits those
+//     slots in index order and, when asked to, gathers and dequantizes the selected rows from
+//     the fp8 pages straight away: the selection never waits for a separate gather launch and
+//     the gather is balanced whatever the distribution of the selected tokens. A query whose
+//     pivot bin holds more keys than LDS can list (huge ties) finds its pivot by streaming
+//     shape (1)'s radix passes over the whole query in every workgroup — slower, same answer.
+//     The histogram is left zeroed for the next call.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
 #include <type_traits>
 
-#include "codec.hpp"
+#include "gather_common.hpp"
+#include "topk_common.hpp"
 
 namespace rk {
 
 constexpr int kBins = 256;
 constexpr int kCopies = 32;
-
-// Order-preserving f32 -> u32 with -0.0 folded onto +0.0
-// (crates/backend/kernels/indexer.hip:156-159).
-__device__ __forceinline__ uint32_t topk_key(float v) {
-    uint32_t b = (v == 0.0f) ? 0u : __float_as_uint(v);
-    return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);
-}
-
-// The two orders a selection can run under: the DSA rule above, and IEEE total order
-// (f32::total_cmp: -0.0 strictly below +0.0, NaNs ordered by sign and payload), which the
-// scored block selection of the second cache format uses.
-struct FoldedZeroKey {
-    static __device__ __forceinline__ uint32_t of(float v) { return topk_key(v); }
-};
-struct TotalOrderKey {
-    static __device__ __forceinline__ uint32_t of(float v) {
-        const uint32_t b = __float_as_uint(v);
-        return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);
-    }
-};
-
-__device__ __forceinline__ uint32_t lanes_below(unsigned long long mask) {
-    return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
-                                     __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
-}
-
-// A load that other workgroups' writes (made visible by a fence + ticket) are seen by.
-__device__ __forceinline__ uint32_t load_agent(const uint32_t* p) {
-    return __hip_atomic_load(const_cast<uint32_t*>(p), __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_AGENT);
-}
 
 // One sweep over a lane's elements: a compile-time trip count when the keys live in
 // registers (so every key[j] is a register, never scratch), a runtime one when streaming.
@@ -97,14 +74,9 @@ __device__ __forceinline__ void find_pivot_bin(const uint32_t* bins, uint32_t ne
 #pragma unroll
     for (int b = 0; b < 4; ++b) c[b] = bins[lane * 4 + b];
     const uint32_t tot = c[0] + c[1] + c[2] + c[3];
-    uint32_t suffix = tot;
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        uint32_t v = __shfl_down(suffix, off, kWave);
-        if (lane + off < kWave) suffix += v;
-    }
-    const uint32_t above = suffix - tot;
-    if (above < need && need <= suffix) {
+    const uint32_t incl = wave_inclusive_sum(tot);
+    const uint32_t above = wave_total(incl) - incl;  // keys in the bins of higher lanes
+    if (above < need && need <= above + tot) {
         uint32_t acc = above;
         int b = 3;
         for (; b > 0; --b) {
@@ -122,6 +94,59 @@ constexpr int topk_block_lds_words() {
     return kBins * kCopies + kBins + 2 * (THREADS / kWave) + 2;
 }
 
+// The radix passes of shape (1): the k-th largest key of the elements key_at(j) (element j of a
+// lane exists iff j * 64 < limit) and how many keys EQUAL to it the selection takes, found by
+// four 8-bit histogram passes, most significant byte first. Every thread of the workgroup calls
+// it with the same kq; lds holds topk_block_lds_words<THREADS>() words.
+template <int THREADS, int ITEMS, class KeyAt>
+__device__ __forceinline__ void radix_pivot(KeyAt&& key_at, int steps, int limit, uint32_t kq,
+                                            uint32_t* lds, uint32_t* pivot_out,
+                                            uint32_t* need_out) {
+    constexpr int WAVES = THREADS / kWave;
+    constexpr int TPB = THREADS / kBins;  // threads that share one bin's copies
+    static_assert(TPB == 1 || TPB == 4, "256 or 1024 threads");
+    uint32_t* s_hist = lds;
+    uint32_t* s_bins = s_hist + kBins * kCopies;
+    uint32_t* s_pn = s_bins + kBins + 2 * WAVES;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid >> 6;
+
+    uint32_t pivot = 0u, mask = 0u, need = kq;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        for (int i = tid; i < kBins * kCopies; i += THREADS) s_hist[i] = 0u;
+        __syncthreads();
+        sweep<ITEMS>(steps, [&](int j) {
+            const uint32_t u = key_at(j);
+            if (j * kWave < limit && (u & mask) == pivot)
+                atomicAdd(&s_hist[((u >> shift) & 0xffu) * kCopies + (lane & (kCopies - 1))], 1u);
+        });
+        __syncthreads();
+        {
+            // TPB threads per bin, 32/TPB copies each, rotated so a wave spreads over banks
+            constexpr int PER = kCopies / TPB;
+            const int bin = tid / TPB, part = tid % TPB;
+            uint32_t sum = 0;
+#pragma unroll
+            for (int c = 0; c < PER; ++c)
+                sum += s_hist[bin * kCopies + part * PER + ((c + lane) & (PER - 1))];
+            if (TPB == 4) {
+                sum += __shfl_xor(sum, 1, kWave);
+                sum += __shfl_xor(sum, 2, kWave);
+            }
+            if (part == 0) s_bins[bin] = sum;
+        }
+        __syncthreads();
+        if (wave == 0) find_pivot_bin(s_bins, need, s_pn, lane);
+        __syncthreads();
+        pivot |= s_pn[0] << shift;
+        need = s_pn[1];
+        mask |= 0xffu << shift;
+    }
+    *pivot_out = pivot;
+    *need_out = need;
+}
+
 // Shape (1): the whole selection for one query by one workgroup of THREADS threads.
 // ITEMS: keys per lane kept in registers; 0 = re-read the scores on every sweep.
 // KEY: the order (FoldedZeroKey or TotalOrderKey); `add` is added to every emitted index.
@@ -130,13 +155,8 @@ __device__ __forceinline__ void topk_block(const float* __restrict__ s, int nt, 
                                            uint32_t* __restrict__ out, uint32_t* lds,
                                            uint32_t add = 0u) {
     constexpr int WAVES = THREADS / kWave;
-    constexpr int TPB = THREADS / kBins;  // threads that share one bin's copies
-    static_assert(TPB == 1 || TPB == 4, "256 or 1024 threads");
-    uint32_t* s_hist = lds;
-    uint32_t* s_bins = s_hist + kBins * kCopies;
-    uint32_t* s_gt = s_bins + kBins;
+    uint32_t* s_gt = lds + kBins * kCopies + kBins;
     uint32_t* s_eq = s_gt + WAVES;
-    uint32_t* s_pn = s_eq + WAVES;
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -173,37 +193,8 @@ __device__ __forceinline__ void topk_block(const float* __restrict__ s, int nt, 
         return (j * kWave < limit) ? KEY::of(s[seg0 + (long long)j * kWave + lane]) : 0u;
     };
 
-    uint32_t pivot = 0u, mask = 0u, need = kq;
-    for (int shift = 24; shift >= 0; shift -= 8) {
-        for (int i = tid; i < kBins * kCopies; i += THREADS) s_hist[i] = 0u;
-        __syncthreads();
-        sweep<ITEMS>(steps, [&](int j) {
-            const uint32_t u = key_at(j);
-            if (j * kWave < limit && (u & mask) == pivot)
-                atomicAdd(&s_hist[((u >> shift) & 0xffu) * kCopies + (lane & (kCopies - 1))], 1u);
-        });
-        __syncthreads();
-        {
-            // TPB threads per bin, 32/TPB copies each, rotated so a wave spreads over banks
-            constexpr int PER = kCopies / TPB;
-            const int bin = tid / TPB, part = tid % TPB;
-            uint32_t sum = 0;
-#pragma unroll
-            for (int c = 0; c < PER; ++c)
-                sum += s_hist[bin * kCopies + part * PER + ((c + lane) & (PER - 1))];
-            if (TPB == 4) {
-                sum += __shfl_xor(sum, 1, kWave);
-                sum += __shfl_xor(sum, 2, kWave);
-            }
-            if (part == 0) s_bins[bin] = sum;
-        }
-        __syncthreads();
-        if (wave == 0) find_pivot_bin(s_bins, need, s_pn, lane);
-        __syncthreads();
-        pivot |= s_pn[0] << shift;
-        need = s_pn[1];
-        mask |= 0xffu << shift;
-    }
+    uint32_t pivot, need;
+    radix_pivot<THREADS, ITEMS>(key_at, steps, limit, kq, lds, &pivot, &need);
 
     // Per-wave totals of (key > pivot, key == pivot).
     uint32_t cnt_gt = 0, cnt_eq = 0;
@@ -265,18 +256,17 @@ static_assert(kLeanBins == kTopkThreads, "one thread per bin");
 constexpr int kLeanLdsWords = 2 * kLeanCap + kLeanBins * kLeanCopies + 4 * kTopkWaves + 8;
 static_assert(kLeanCap < 65536, "emission packs two counts into 16 bits each");
 
-// Sum over the 16 wave slots of v[w] for w < wave (*before) and over all of them (*all).
-// Lanes 0..15 read one slot each and a 4-step butterfly adds them: a couple of registers and
-// no dependent chain of LDS reads. Every lane of the wave must call it.
+// Sum over the 16 wave slots of v[w] for w < wave (*before) and over all of them (*all):
+// sixteen independent broadcast reads, which pipeline, instead of a chain of shuffles.
+// Every lane of the wave must call it.
 __device__ __forceinline__ void wave_slots_prefix(const uint32_t* v, int wave, uint32_t* before,
                                                   uint32_t* all) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t x = lane < kTopkWaves ? v[lane] : 0u;
-    uint32_t a = x, b = lane < wave ? x : 0u;
+    uint32_t a = 0, b = 0;
 #pragma unroll
-    for (int off = kTopkWaves / 2; off > 0; off >>= 1) {
-        a += __shfl_xor(a, off, kWave);
-        b += __shfl_xor(b, off, kWave);
+    for (int w = 0; w < kTopkWaves; ++w) {
+        const uint32_t x = v[w];
+        a += x;
+        b += w < wave ? x : 0u;
     }
     *all = __builtin_amdgcn_readfirstlane(a);
     *before = __builtin_amdgcn_readfirstlane(b);
@@ -573,324 +563,486 @@ __global__ __launch_bounds__(kTopkThreads) void index_topk_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// Shape (2): a query split over many workgroups.
+// Shape (2): a query split over many workgroups (three launches, see the file header).
 // ---------------------------------------------------------------------------------------------
-constexpr int kSegThreads = 256;
-constexpr int kSegWaves = kSegThreads / kWave;
-constexpr int kSegKeys = 4096;                     // scores per workgroup
-constexpr int kSegItems = kSegKeys / kSegThreads;  // 16 per thread
-constexpr int kTopBits = 12;
-constexpr int kTopBins = 1 << kTopBits;  // global histogram bins per query
-constexpr int kLowBits = 32 - kTopBits;
-constexpr int kCandCap = 8192;  // candidates the finishing workgroup can cache in LDS
-constexpr int kMaxSegs = 1024;  // segment prefix table held in LDS
+constexpr int kCandCap = 8192;    // pivot-bin keys a finishing workgroup can hold in LDS
+constexpr int kSlotsPerGroup = 128;  // output positions per finishing workgroup
+static_assert(kSegKeys == kSplitThreads * 4, "a wave owns 256 consecutive scores of a segment");
+static_assert(kTopBins == kSplitThreads * 4, "a thread owns four consecutive histogram bins");
+static_assert(kMaxSegs <= kSplitThreads, "one segment per thread in the finishing kernel");
+static_assert(kSplitThreads == kTopkThreads, "the 16-slot wave helpers serve both shapes");
 
-// Workspace, u32 words per query: [0,4096) histogram | 4096 ticket A | 4097 ticket B |
-// 4098 pivot bin | 4099 need | [4100, 4100+S) per-segment candidate counts | (pad to 4) |
-// S x 4096 candidate indices.
-constexpr int kWsTicketA = kTopBins, kWsTicketB = kTopBins + 1, kWsPivot = kTopBins + 2,
-              kWsNeed = kTopBins + 3, kWsCounts = kTopBins + 4;
-__host__ __device__ inline size_t topk_ws_cand_offset(int n_segs) {
-    return ((size_t)kWsCounts + (size_t)n_segs + 3) & ~(size_t)3;
-}
-static inline size_t topk_ws_words(int n_segs) {
-    return topk_ws_cand_offset(n_segs) + (size_t)n_segs * kSegKeys;
-}
-
-// A workgroup's 4096 keys: element (j, tid) is index seg*4096 + j*256 + tid.
-__device__ __forceinline__ void load_segment_keys(const float* __restrict__ s, int nt, int seg,
-                                                  uint32_t (&key)[kSegItems], int& limit) {
-    const int base = seg * kSegKeys + (int)threadIdx.x;
-    limit = nt - base;  // element j exists iff j*256 < limit
-    float raw[kSegItems];
+// A wave's 256 consecutive scores of segment `seg` as keys: element j of lane L is index
+// seg * 4096 + wave * 256 + j * 64 + L (so a ballot over element j lists 64 consecutive indices
+// in lane order) and exists iff j * 64 < *limit.
+__device__ __forceinline__ void load_keys4(const float* __restrict__ s, int nt, int seg,
+                                           uint32_t (&key)[4], int* limit) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int base = seg * kSegKeys + wave * (4 * kWave) + lane;
+    *limit = nt - base;
+    float v[4];
 #pragma unroll
-    for (int j = 0; j < kSegItems; ++j) {
-        int i = base + j * kSegThreads;
-        raw[j] = s[i < nt ? i : nt - 1];
-    }
+    for (int j = 0; j < 4; ++j) v[j] = j * kWave < *limit ? s[base + j * kWave] : 0.0f;
 #pragma unroll
-    for (int j = 0; j < kSegItems; ++j) key[j] = topk_key(raw[j]);
+    for (int j = 0; j < 4; ++j) key[j] = topk_key(v[j]);
 }
 
-// Exclusive prefix sum of one value per thread over a 256-thread workgroup, in thread order;
-// *total receives the workgroup sum. tmp holds kSegWaves words. Every thread must call it.
+// The 16 wave slots v[0..16): the sum of those before `wave` (returned) and of all (*all), as
+// scalars. One LDS read and a 16-lane DPP scan; every lane of the wave must call it.
+__device__ __forceinline__ uint32_t wave_slots_before(const uint32_t* v, int wave, uint32_t* all) {
+    const int lane = threadIdx.x & (kWave - 1);
+    uint32_t x = v[lane & (kSplitWaves - 1)];
+    x += dpp_or_zero<0x111, 0xf>(x);
+    x += dpp_or_zero<0x112, 0xf>(x);
+    x += dpp_or_zero<0x114, 0xf>(x);
+    x += dpp_or_zero<0x118, 0xf>(x);
+    *all = (uint32_t)__builtin_amdgcn_readlane((int)x, kSplitWaves - 1);
+    return wave ? (uint32_t)__builtin_amdgcn_readlane((int)x, wave - 1) : 0u;
+}
+
+// Exclusive prefix sum of one value per thread over the 1024-thread workgroup, in thread
+// order; *total receives the workgroup sum. tmp holds 16 words. Every thread must call it.
 __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* tmp,
                                                          uint32_t* total) {
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
-    uint32_t incl = v;
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        uint32_t t = __shfl_up(incl, off, kWave);
-        if (lane >= off) incl += t;
-    }
-    __syncthreads();  // tmp may still be read from a previous use
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t incl = wave_inclusive_sum(v);
+    lds_barrier();  // tmp may still be read from a previous use
     if (lane == kWave - 1) tmp[wave] = incl;
-    __syncthreads();
-    uint32_t before = 0, all = 0;
-#pragma unroll
-    for (int w = 0; w < kSegWaves; ++w) {
-        if (w < wave) before += tmp[w];
-        all += tmp[w];
-    }
-    *total = all;
-    return before + incl - v;
+    lds_barrier();
+    return wave_slots_before(tmp, wave, total) + incl - v;
 }
 
-// True in exactly one workgroup of the n that share `ticket`: the last to arrive. Nobody
-// waits: the others simply leave. Every wave first drains its own stores into L2, then ONE
-// wave publishes the workgroup's writes device-wide (an L2 write-back is expensive, and 256
-// workgroups x 4 waves of them were measured to cost more than the kernel's real work).
-__device__ __forceinline__ bool last_to_arrive(uint32_t* ticket, uint32_t n, uint32_t* s_flag) {
-    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wave's global stores have completed
-    __syncthreads();
-    if (threadIdx.x < kWave) {
-        __threadfence();
-        if (threadIdx.x == 0) *s_flag = atomicAdd(ticket, 1u);
-    }
-    __syncthreads();
-    const bool last = *s_flag == n - 1;
-    if (last) __threadfence();  // the others' writes are visible after the last ticket
-    return last;
-}
-
-__global__ __launch_bounds__(kSegThreads) void topk_hist_kernel(
-    const float* __restrict__ scores, int stride, const int* __restrict__ nts, int nt_all, int k,
+// Launch 1: the per-query histogram of the keys' top 12 bits.
+__global__ __launch_bounds__(kSplitThreads) void topk_hist_kernel(
+    const float* __restrict__ scores, int stride, const int* __restrict__ nts, int nt_all,
     uint32_t* __restrict__ ws, size_t ws_stride) {
     __shared__ uint32_t s_hist[kTopBins];
-    __shared__ uint32_t s_scan[kSegWaves];
-    __shared__ uint32_t s_flag;
     const int q = blockIdx.y, seg = blockIdx.x, tid = threadIdx.x;
     const int nt = nts ? min(nts[q], nt_all) : nt_all;
+    if (seg * kSegKeys >= nt) return;
+    uint32_t key[4];
+    int limit;
+    load_keys4(scores + (size_t)q * stride, nt, seg, key, &limit);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s_hist[tid + i * kSplitThreads] = 0u;
+    lds_barrier();
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        if (j * kWave < limit) atomicAdd(&s_hist[key[j] >> kLowBits], 1u);
+    lds_barrier();
+    flush_top_bins(s_hist, ws + (size_t)q * ws_stride, tid, kSplitThreads);
+}
+
+// Launch 2: the pivot bin from the histogram; this segment's keys above it counted, its keys
+// in it listed (in any order: only their values matter to the pivot).
+__global__ __launch_bounds__(kSplitThreads) void topk_cand_kernel(
+    const float* __restrict__ scores, int stride, const int* __restrict__ nts, int nt_all, int k,
+    uint32_t* __restrict__ ws, size_t ws_stride, int n_segs) {
+    __shared__ uint32_t s_wave[kSplitWaves];
+    __shared__ uint32_t s_pn[2];
+    __shared__ uint32_t s_cnt[2];  // [0] listed, [1] in higher bins
+    const int q = blockIdx.y, seg = blockIdx.x, tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nt = nts ? min(nts[q], nt_all) : nt_all;
     if (nt <= 0) return;
-    const uint32_t kq = (uint32_t)min(k, nt);
     uint32_t* w = ws + (size_t)q * ws_stride;
+    if (seg * kSegKeys >= nt) {  // a segment past this query's end holds nothing
+        if (tid == 0) {
+            w[kWsCounts + seg] = 0u;
+            w[kWsCounts + n_segs + seg] = 0u;
+        }
+        return;
+    }
+    const uint32_t kq = (uint32_t)min(k, nt);
+    if (tid < 2) s_cnt[tid] = s_pn[tid] = 0u;
+    uint32_t key[4];
+    int limit;
+    load_keys4(scores + (size_t)q * stride, nt, seg, key, &limit);  // before the histogram is used
 
-    for (int i = tid; i < kTopBins; i += kSegThreads) s_hist[i] = 0u;
-    __syncthreads();
-    if (seg * kSegKeys < nt) {
-        uint32_t key[kSegItems];
-        int limit;
-        load_segment_keys(scores + (size_t)q * stride, nt, seg, key, limit);
-#pragma unroll
-        for (int j = 0; j < kSegItems; ++j)
-            if (j * kSegThreads < limit) atomicAdd(&s_hist[key[j] >> kLowBits], 1u);
-    }
-    __syncthreads();
-    for (int b = tid; b < kTopBins; b += kSegThreads) {
-        const uint32_t c = s_hist[b];
-        if (c) atomicAdd(&w[b], c);
-    }
-    if (!last_to_arrive(&w[kWsTicketA], gridDim.x, &s_flag)) return;
-
-    // The query's histogram is complete. Thread t owns bins [16t, 16t+16); find the highest
-    // bin b with (count of bins >= b) >= kq.
-    constexpr int OWN = kTopBins / kSegThreads;
-    uint32_t c[OWN], sum = 0;
-#pragma unroll
-    for (int m = 0; m < OWN; ++m) {
-        c[m] = load_agent(&w[tid * OWN + m]);
-        sum += c[m];
-    }
-    uint32_t all = 0;
-    const uint32_t below = block_exclusive_scan(sum, s_scan, &all);
-    const uint32_t above = all - below - sum;  // candidates in bins owned by higher threads
-    if (above < kq && kq <= above + sum) {
+    // thread t owns bins 4t .. 4t+3; the bin b with (keys in bins > b) < kq <= (keys in bins >= b)
+    const u32x4 c4 = reinterpret_cast<const u32x4*>(w)[tid];
+    const uint32_t c[4] = {c4.x, c4.y, c4.z, c4.w};
+    const uint32_t mine = c[0] + c[1] + c[2] + c[3];
+    const uint32_t incl = wave_inclusive_sum(mine);
+    if (lane == kWave - 1) s_wave[wave] = incl;
+    lds_barrier();
+    uint32_t all;
+    const uint32_t lower = wave_slots_before(s_wave, wave, &all) + incl;  // up to this thread
+    const uint32_t above = all - lower;                                    // in the higher bins
+    if (above < kq && kq <= above + mine) {
         uint32_t acc = above;
-        int m = OWN - 1;
+        int m = 3;
         for (; m > 0; --m) {
             if (acc + c[m] >= kq) break;
             acc += c[m];
         }
-        w[kWsPivot] = (uint32_t)(tid * OWN + m);
-        w[kWsNeed] = kq - acc;
+        s_pn[0] = (uint32_t)(tid * 4 + m);
+        s_pn[1] = kq - acc;
     }
-    // leave the histogram and the ticket zeroed for the next call
+    lds_barrier();
+    const uint32_t p12 = s_pn[0];
+
+    uint32_t* list = w + topk_ws_cand_offset(n_segs) + (size_t)seg * kSegKeys;
+    uint32_t higher = 0;
 #pragma unroll
-    for (int m = 0; m < OWN; ++m) w[tid * OWN + m] = 0u;
-    if (tid == 0) w[kWsTicketA] = 0u;
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t bin = key[j] >> kLowBits;
+        const bool live = j * kWave < limit;
+        higher += (uint32_t)__popcll(__ballot(live && bin > p12));
+        const bool is = live && bin == p12;
+        const unsigned long long m = __ballot(is);
+        if (m) {
+            uint32_t base = 0;
+            if (lane == 0) base = atomicAdd(&s_cnt[0], (uint32_t)__popcll(m));
+            base = __builtin_amdgcn_readfirstlane(base);
+            if (is) list[base + lanes_below(m)] = key[j];
+        }
+    }
+    if (lane == 0 && higher) atomicAdd(&s_cnt[1], higher);
+    lds_barrier();
+    if (tid == 0) {
+        w[kWsCounts + seg] = s_cnt[0];
+        w[kWsCounts + n_segs + seg] = s_cnt[1];
+        if (seg == 0) {
+            w[kWsPivot] = p12;
+            w[kWsNeed] = s_pn[1];
+        }
+    }
 }
 
-__global__ __launch_bounds__(kSegThreads) void topk_select_kernel(
+// Launch 3: exact pivot, per-segment prefixes, then this workgroup's output positions — and,
+// with a pool, the rows themselves. W / PT: the page geometry at compile time (0 = runtime).
+// Two things set this kernel's time before the gather starts. Memory round trips: everything
+// the workgroup will need is requested at once, before the first use — the segment counts, the
+// head of every segment's list (a wave per segment, 256 keys, requested before the counts say
+// how many of them exist), the keys of the three segments its output positions most likely
+// fall in, and the query's block-table row. And instruction issue: a vector instruction keeps
+// a SIMD busy for four cycles and the sixteen waves share four SIMDs, so bookkeeping that all
+// threads repeat costs sixteen times what it costs in one wave; scans over the segments run in
+// wave 0 while the others wait at the barrier, and positions come from ballots and scalar
+// popcounts rather than from per-thread prefix sums.
+constexpr int kSpecSegs = kSplitWaves;  // queries of up to 16 segments fetch list heads early
+constexpr int kSpecKeys = 4 * kWave;    // per segment
+template <int W, int PT>
+__global__ __launch_bounds__(kSplitThreads) void topk_finish_kernel(
     const float* __restrict__ scores, int stride, const int* __restrict__ nts, int nt_all, int k,
-    uint32_t* __restrict__ rows, uint32_t* __restrict__ ws, size_t ws_stride) {
-    // the finishing workgroup's candidate cache (indices, keys); the fallback's LDS aliases it
-    __shared__ uint32_t s_mem[2 * kCandCap];
-    __shared__ uint32_t s_pref[kMaxSegs + 1];
-    __shared__ uint32_t s_cnt[kSegItems * kSegWaves];
-    __shared__ uint32_t s_bins[kBins];
-    __shared__ uint32_t s_pn[2];
-    __shared__ uint32_t s_flag;
-    static_assert(topk_block_lds_words<kSegThreads>() <= 2 * kCandCap, "fallback fits the cache");
-    static_assert(kSegItems * kSegWaves == kWave, "one wave scans the (step, wave) counts");
+    uint32_t* __restrict__ rows, uint32_t* __restrict__ ws, size_t ws_stride, int n_segs,
+    const uint8_t* __restrict__ pool, const int* __restrict__ block_table,
+    uint16_t* __restrict__ out, int max_blocks_per_seq, int width_rt, int page_tokens_rt,
+    int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_rows) {
+    // the listed keys; the streaming fallback's histograms alias them
+    __shared__ uint32_t s_key[kCandCap > topk_block_lds_words<kSplitThreads>()
+                                  ? kCandCap
+                                  : topk_block_lds_words<kSplitThreads>()];
+    __shared__ uint32_t s_G[kMaxSegs + 1];   // keys above the pivot in the segments before
+    __shared__ uint32_t s_E[kMaxSegs + 1];   // keys equal to the pivot in the segments before
+    __shared__ uint32_t s_off[kMaxSegs + 1]; // where a segment's listed keys start in s_key
+    __shared__ uint32_t s_bins[3][kBins];    // one histogram per radix pass, cleared up front
+    __shared__ uint32_t s_pn[3][2];
+    __shared__ uint32_t s_wave[2][kSplitWaves];
+    __shared__ int s_span[2];
+    __shared__ int s_table[kSplitThreads];   // the query's block-table row, when it fits
+    __shared__ uint32_t s_tok[kSlotsPerGroup];
+    __shared__ unsigned long long s_base[kSlotsPerGroup];
+    __shared__ unsigned long long s_scale_at[kSlotsPerGroup];
 
-    const int q = blockIdx.y, seg = blockIdx.x, tid = threadIdx.x;
-    const int lane = tid & (kWave - 1), wave = tid >> 6;
-    const int n_segs = gridDim.x;
+    const int q = blockIdx.y, tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nt = nts ? min(nts[q], nt_all) : nt_all;
     if (nt <= 0) return;
     const uint32_t kq = (uint32_t)min(k, nt);
     const float* s = scores + (size_t)q * stride;
     uint32_t* w = ws + (size_t)q * ws_stride;
-    uint32_t* cand = w + topk_ws_cand_offset(n_segs);
+    const uint32_t* lists = w + topk_ws_cand_offset(n_segs);
+
+    // ---- requests ----
     const uint32_t p12 = w[kWsPivot];
-
-    // ---- this segment's candidates (key's top bits >= pivot bin), in index order ----
-    uint32_t key[kSegItems];
-    int limit = 0;
-    if (seg * kSegKeys < nt) {
-        load_segment_keys(s, nt, seg, key, limit);
-    } else {
-#pragma unroll
-        for (int j = 0; j < kSegItems; ++j) key[j] = 0u;
-    }
-    uint32_t rank[kSegItems];
-    bool sel[kSegItems];
-#pragma unroll
-    for (int j = 0; j < kSegItems; ++j) {
-        sel[j] = j * kSegThreads < limit && (key[j] >> kLowBits) >= p12;
-        const unsigned long long m = __ballot(sel[j]);
-        rank[j] = lanes_below(m);
-        if (lane == 0) s_cnt[j * kSegWaves + wave] = (uint32_t)__popcll(m);
-    }
-    __syncthreads();
-    if (wave == 0) {  // exclusive scan of the 64 (step, wave) counts, which is element order
-        const uint32_t v = s_cnt[lane];
-        uint32_t incl = v;
-#pragma unroll
-        for (int off = 1; off < kWave; off <<= 1) {
-            uint32_t t = __shfl_up(incl, off, kWave);
-            if (lane >= off) incl += t;
-        }
-        s_cnt[lane] = incl - v;
-        if (lane == kWave - 1) w[kWsCounts + seg] = incl;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < kSegItems; ++j)
-        if (sel[j])
-            cand[(size_t)seg * kSegKeys + s_cnt[j * kSegWaves + wave] + rank[j]] =
-                (uint32_t)(seg * kSegKeys + j * kSegThreads + tid);
-    if (!last_to_arrive(&w[kWsTicketB], (uint32_t)n_segs, &s_flag)) return;
-
-    // ---- the query's last workgroup finishes the selection ----
-    if (tid == 0) w[kWsTicketB] = 0u;  // left zeroed for the next call
-    uint32_t* out = rows + (size_t)q * k;
-    uint32_t total = 0;
-    bool cached = n_segs <= kMaxSegs;
-    if (cached) {
-        // thread t owns `per` consecutive segments: load their counts at once, scan, publish
-        constexpr int PER_MAX = kMaxSegs / kSegThreads;
-        const int per = (n_segs + kSegThreads - 1) / kSegThreads;
-        uint32_t cnt[PER_MAX], mine = 0;
-#pragma unroll
-        for (int i = 0; i < PER_MAX; ++i) {
-            const int sg = tid * per + i;
-            cnt[i] = (i < per && sg < n_segs) ? load_agent(&w[kWsCounts + sg]) : 0u;
-            mine += cnt[i];
-        }
-        uint32_t acc = block_exclusive_scan(mine, s_cnt, &total);
-#pragma unroll
-        for (int i = 0; i < PER_MAX; ++i) {
-            const int sg = tid * per + i;
-            if (i < per && sg < n_segs) s_pref[sg] = acc;
-            acc += cnt[i];
-        }
-        if (tid == 0) s_pref[n_segs] = total;
-        __syncthreads();
-        cached = total <= (uint32_t)kCandCap;
-    }
-    if (!cached) {
-        // too many candidates to hold (heavy ties): select over the whole query directly
-        topk_block<kSegThreads, 0>(s, nt, kq, out, s_mem);
-        return;
-    }
-    // Pull the candidates into LDS in index order: a group of threads per segment, so no
-    // thread has to search for the segment an output position belongs to.
-    uint32_t* c_idx = s_mem;
-    uint32_t* c_key = s_mem + kCandCap;
-    {
-        const int tps = n_segs < kSegThreads ? kSegThreads / n_segs : 1;  // threads per segment
-        const int groups = kSegThreads / tps;
-        const int sub = tid % tps;
-        for (int sg = tid / tps; sg < n_segs; sg += groups) {
-            const uint32_t base = s_pref[sg], n = s_pref[sg + 1] - base;
-            const uint32_t* src = cand + (size_t)sg * kSegKeys;
-#pragma unroll 4
-            for (uint32_t i = sub; i < n; i += tps) {
-                const uint32_t idx = load_agent(&src[i]);
-                c_idx[base + i] = idx;
-                c_key[base + i] = topk_key(s[idx]);
-            }
-        }
-    }
-    __syncthreads();
-
-    // Radix select on the low 20 bits among the pivot bin's members: 8 + 8 + 4 bits.
     uint32_t need = w[kWsNeed];
-    uint32_t pivot = p12 << kLowBits, mask = ~0u << kLowBits;
-    for (int shift = kLowBits - 8;; shift = shift >= 8 ? shift - 8 : 0) {
-        const uint32_t dmask = (shift == 0 && (kLowBits % 8)) ? (1u << (kLowBits % 8)) - 1u : 0xffu;
-        s_bins[tid] = 0u;
-        __syncthreads();
-        for (uint32_t c = tid; c < total; c += kSegThreads) {
-            const uint32_t u = c_key[c];
-            if ((u & mask) == pivot) atomicAdd(&s_bins[(u >> shift) & dmask], 1u);
-        }
-        __syncthreads();
-        if (wave == 0) find_pivot_bin(s_bins, need, s_pn, lane);
-        __syncthreads();
-        pivot |= s_pn[0] << shift;
-        need = s_pn[1];
-        mask |= dmask << shift;
-        __syncthreads();
-        if (shift == 0) break;
+    uint32_t n_listed = 0, n_higher = 0;
+    if (tid < n_segs) {
+        n_listed = w[kWsCounts + tid];
+        n_higher = w[kWsCounts + n_segs + tid];
     }
+    const bool spec = n_segs <= kSpecSegs;
+    uint32_t head[4] = {0u, 0u, 0u, 0u};
+    if (spec && wave < n_segs) {  // entries past the segment's count are junk and never used
+#pragma unroll
+        for (int i = 0; i < 4; ++i) head[i] = lists[(size_t)wave * kSegKeys + lane + i * kWave];
+    }
+    // output position p of a query with evenly spread winners sits in segment p * S / kq; the
+    // spread is never even, so the neighbours on both sides are requested as well
+    const int guess = min(n_segs - 1, (int)((long long)blockIdx.x * n_segs / (int)gridDim.x));
+    const int g0 = max(guess - 1, 0);
+    uint32_t pkey[3][4];
+    int plimit[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) load_keys4(s, nt, g0 + i, pkey[i], &plimit[i]);
+    const bool table_cached = pool && max_blocks_per_seq <= kSplitThreads;
+    int my_page = -1;
+    if (table_cached && tid < max_blocks_per_seq)
+        my_page = block_table[(size_t)q * max_blocks_per_seq + tid];
 
-    // Ordered emission: 256 candidates per round, running (gt, eq) counts carried across.
-    uint32_t run_gt = 0, run_eq = 0;
-    for (uint32_t c0 = 0; c0 < total; c0 += kSegThreads) {
-        const uint32_t c = c0 + tid;
-        const bool live = c < total;
-        const uint32_t u = live ? c_key[c] : 0u;
-        const bool g = live && u > pivot, e = live && u == pivot;
-        const unsigned long long mg = __ballot(g), me = __ballot(e);
-        if (lane == 0) {
-            s_cnt[wave] = (uint32_t)__popcll(mg);
-            s_cnt[kSegWaves + wave] = (uint32_t)__popcll(me);
-        }
-        __syncthreads();
-        uint32_t G = run_gt + lanes_below(mg), E = run_eq + lanes_below(me);
-        for (int wv = 0; wv < kSegWaves; ++wv) {
-            if (wv < wave) {
-                G += s_cnt[wv];
-                E += s_cnt[kSegWaves + wv];
-            }
-            run_gt += s_cnt[wv];
-            run_eq += s_cnt[kSegWaves + wv];
-        }
-        const uint32_t slot = G + (E < need ? E : need);
-        if ((g || (e && E < need)) && slot < kq) out[slot] = c_idx[c];
-        __syncthreads();
+    if (blockIdx.x == 0)  // the histogram has served: left zeroed for the next call
+        reinterpret_cast<u32x4*>(w)[tid] = u32x4{0u, 0u, 0u, 0u};
+    if (tid < 3 * kBins) (&s_bins[0][0])[tid] = 0u;
+    if (tid == 0) {
+        s_span[0] = n_segs;
+        s_span[1] = -1;
     }
+    if (tid < n_segs) s_G[tid] = n_higher;
+
+    // ---- where each segment's listed keys go in LDS ----
+    if (n_segs <= kWave) {
+        if (wave == 0) {  // one wave, the others go straight to the barrier
+            const uint32_t incl = wave_inclusive_sum(n_listed);
+            if (lane < n_segs) s_off[lane] = incl - n_listed;
+            if (lane == n_segs - 1) s_off[n_segs] = incl;
+        }
+    } else {
+        uint32_t all;
+        const uint32_t my_off = block_exclusive_scan(n_listed, s_wave[0], &all);
+        if (tid < n_segs) s_off[tid] = my_off;
+        if (tid == 0) s_off[n_segs] = all;
+    }
+    lds_barrier();
+    const uint32_t total = s_off[n_segs];
+
+    uint32_t pivot;
+    if (total <= (uint32_t)kCandCap) {
+        // ---- the listed keys into LDS, a wave per segment ----
+        for (int sg = wave; sg < n_segs; sg += kSplitWaves) {
+            const uint32_t base = s_off[sg], n = s_off[sg + 1] - base;
+            const uint32_t* src = lists + (size_t)sg * kSegKeys;
+            uint32_t i0 = 0;
+            if (spec) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if ((uint32_t)(lane + i * kWave) < n) s_key[base + lane + i * kWave] = head[i];
+                i0 = kSpecKeys;
+            }
+            for (uint32_t i = i0 + lane; i < n; i += kWave) s_key[base + i] = src[i];
+        }
+        lds_barrier();
+        // ---- radix select on the low 20 bits among them: 8 + 8 + 4 ----
+        pivot = p12 << kLowBits;
+        uint32_t mask = ~0u << kLowBits;
+#pragma unroll
+        for (int pass = 0; pass < 3; ++pass) {
+            const int shift = pass == 0 ? kLowBits - 8 : (pass == 1 ? kLowBits - 16 : 0);
+            const uint32_t dmask = pass == 2 ? (1u << (kLowBits - 16)) - 1u : 0xffu;
+            for (uint32_t c = tid; c < total; c += kSplitThreads) {
+                const uint32_t u = s_key[c];
+                if ((u & mask) == pivot) atomicAdd(&s_bins[pass][(u >> shift) & dmask], 1u);
+            }
+            lds_barrier();
+            if (wave == 0) find_pivot_bin(s_bins[pass], need, s_pn[pass], lane);
+            lds_barrier();
+            pivot |= s_pn[pass][0] << shift;
+            need = s_pn[pass][1];
+            mask |= dmask << shift;
+        }
+        // ---- per segment: listed keys above / equal to the pivot, a wave per segment ----
+        for (int sg = wave; sg < n_segs; sg += kSplitWaves) {
+            const uint32_t base = s_off[sg], n = s_off[sg + 1] - base;
+            uint32_t cg = 0, ce = 0;
+            for (uint32_t i0 = 0; i0 < n; i0 += kWave) {
+                const uint32_t i = i0 + lane;
+                const uint32_t u = i < n ? s_key[base + i] : 0u;
+                cg += (uint32_t)__popcll(__ballot(i < n && u > pivot));
+                ce += (uint32_t)__popcll(__ballot(i < n && u == pivot));
+            }
+            if (lane == 0) {
+                s_G[sg] += cg;  // on top of the segment's keys in higher bins
+                s_E[sg] = ce;
+            }
+        }
+    } else {
+        // ---- too many keys in the pivot bin to list (huge ties): the radix passes streamed
+        // over the whole query, then one more sweep for the per-segment counts ----
+        const int per_wave = ((nt + kSplitThreads - 1) / kSplitThreads) * kWave;
+        const int steps = per_wave / kWave;
+        const long long seg0 = (long long)wave * per_wave;
+        const long long rem = (long long)nt - seg0;
+        const int limit = (int)(rem < per_wave ? rem : per_wave) - lane;
+        auto key_at = [&](int j) -> uint32_t {
+            return (j * kWave < limit) ? topk_key(s[seg0 + (long long)j * kWave + lane]) : 0u;
+        };
+        radix_pivot<kSplitThreads, 0>(key_at, steps, limit, kq, s_key, &pivot, &need);
+        lds_barrier();
+        if (tid < n_segs) s_G[tid] = s_E[tid] = 0u;
+        lds_barrier();
+        for (int sg = 0; sg * kSegKeys < nt; ++sg) {
+            uint32_t key[4];
+            int lim;
+            load_keys4(s, nt, sg, key, &lim);
+            uint32_t cg = 0, ce = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                cg += (uint32_t)__popcll(__ballot(j * kWave < lim && key[j] > pivot));
+                ce += (uint32_t)__popcll(__ballot(j * kWave < lim && key[j] == pivot));
+            }
+            if (lane == 0) {
+                if (cg) atomicAdd(&s_G[sg], cg);
+                if (ce) atomicAdd(&s_E[sg], ce);
+            }
+        }
+    }
+    lds_barrier();
+
+    // ---- exclusive prefixes over the segments; a key's output position is
+    // (keys above the pivot before it) + min(keys equal to the pivot before it, need) ----
+    if (n_segs <= kWave) {
+        if (wave == 0) {
+            const uint32_t g = lane < n_segs ? s_G[lane] : 0u, e = lane < n_segs ? s_E[lane] : 0u;
+            const uint32_t gi = wave_inclusive_sum(g), ei = wave_inclusive_sum(e);
+            if (lane < n_segs) {
+                s_G[lane] = gi - g;
+                s_E[lane] = ei - e;
+            }
+            if (lane == n_segs - 1) {
+                s_G[n_segs] = gi;
+                s_E[n_segs] = ei;
+            }
+        }
+    } else {
+        const uint32_t g_seg = tid < n_segs ? s_G[tid] : 0u, e_seg = tid < n_segs ? s_E[tid] : 0u;
+        uint32_t all;
+        const uint32_t gp = block_exclusive_scan(g_seg, s_wave[0], &all);
+        const uint32_t ep = block_exclusive_scan(e_seg, s_wave[0], &all);
+        if (tid < n_segs) {
+            s_G[tid] = gp;
+            s_E[tid] = ep;
+        }
+        if (tid == n_segs - 1) {
+            s_G[n_segs] = gp + g_seg;
+            s_E[n_segs] = ep + e_seg;
+        }
+    }
+    lds_barrier();
+    const uint32_t lo = (uint32_t)blockIdx.x * kSlotsPerGroup;
+    if (lo >= kq) return;
+    const uint32_t hi = min(lo + (uint32_t)kSlotsPerGroup, kq);
+    if (tid < n_segs) {  // the segments whose output positions meet [lo, hi)
+        const uint32_t a = s_G[tid] + min(s_E[tid], need);
+        const uint32_t b = s_G[tid + 1] + min(s_E[tid + 1], need);
+        if (a < hi && b > lo) {
+            atomicMin(&s_span[0], tid);
+            atomicMax(&s_span[1], tid);
+        }
+    }
+    if (table_cached && tid < max_blocks_per_seq) s_table[tid] = my_page;
+    lds_barrier();
+    const int sg_first = s_span[0], sg_last = s_span[1];
+    uint32_t* out_rows = rows + (size_t)q * k;
+    // a wave's 256 keys are 256 consecutive indices, element j in lane order: counts and
+    // positions are ballots and scalar popcounts (the segments may be visited in any order)
+    int turn = 0;
+    auto emit = [&](int sg, const uint32_t (&key)[4], int lim) {
+        unsigned long long mg[4], me[4];
+        uint32_t cg = 0, ce = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool live = j * kWave < lim;
+            mg[j] = __ballot(live && key[j] > pivot);
+            me[j] = __ballot(live && key[j] == pivot);
+            cg += (uint32_t)__popcll(mg[j]);
+            ce += (uint32_t)__popcll(me[j]);
+        }
+        if (lane == 0) s_wave[turn][wave] = cg | (ce << 16);  // at most 256 each
+        lds_barrier();
+        uint32_t all;
+        const uint32_t before = wave_slots_before(s_wave[turn], wave, &all);
+        turn ^= 1;
+        uint32_t G = s_G[sg] + (before & 0xffffu), E = s_E[sg] + (before >> 16);
+        const uint32_t idx0 = (uint32_t)(sg * kSegKeys + wave * (4 * kWave) + lane);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if ((mg[j] | me[j]) == 0ull) continue;  // wave-uniform: nothing of these 64 is taken
+            const bool g = (mg[j] >> lane) & 1ull, eq = (me[j] >> lane) & 1ull;
+            const uint32_t Gl = G + lanes_below(mg[j]), El = E + lanes_below(me[j]);
+            const uint32_t slot = Gl + min(El, need);
+            if ((g || (eq && El < need)) && slot >= lo && slot < hi) {
+                out_rows[slot] = idx0 + j * kWave;
+                s_tok[slot - lo] = idx0 + j * kWave;
+            }
+            G += (uint32_t)__popcll(mg[j]);
+            E += (uint32_t)__popcll(me[j]);
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < 3; ++i)  // the segments requested up front, straight from registers
+        if (g0 + i >= sg_first && g0 + i <= sg_last) emit(g0 + i, pkey[i], plimit[i]);
+    for (int sg = sg_first; sg <= sg_last; ++sg) {
+        if (sg >= g0 && sg < g0 + 3) continue;
+        uint32_t key[4];
+        int lim;
+        load_keys4(s, nt, sg, key, &lim);
+        emit(sg, key, lim);
+    }
+    if (!pool) return;
+
+    // ---- the selected rows of [lo, hi): fp8 page rows -> bf16, as the sparse gather does ----
+    lds_barrier();
+    const int width = W ? W : width_rt;
+    const int pt = PT ? PT : page_tokens_rt;
+    const int cnt = (int)(hi - lo);
+    if (tid < cnt &&
+        !resolve_row(s_tok[tid],
+                     table_cached ? s_table : block_table + (size_t)q * max_blocks_per_seq,
+                     max_blocks_per_seq, width, pt, n_pages, page_bytes, bad_rows, &s_base[tid],
+                     &s_scale_at[tid]))
+        s_span[0] = -1;  // the span has served; now the flag "a row is skipped"
+    lds_barrier();
+    constexpr int kUnroll = W ? (kSlotsPerGroup * (W / 8) + kSplitThreads - 1) / kSplitThreads : 4;
+    const bool plain = s_span[0] >= 0 && cnt * (width >> 3) == kSplitThreads * kUnroll;
+    stream_rows<kSplitThreads, kUnroll>(pool, s_base, s_scale_at, cnt, width, plain,
+                                        out + ((size_t)q * k + lo) * width);
 }
 
+struct GatherArgs {  // the page pool a selection gathers from; pool == nullptr: indices only
+    const uint8_t* pool;
+    const int* block_table;
+    uint16_t* out;
+    int max_blocks_per_seq, width, page_tokens, n_pages;
+    unsigned int* bad_rows;
+};
+
 static int index_topk_launch(const float* scores, int n_queries, int stride, const int* nts,
-                             int nt, int k, unsigned int* rows, void* workspace,
-                             hipStream_t stream) {
+                             int nt, int k, unsigned int* rows, void* workspace, bool hist_ready,
+                             const GatherArgs& ga, hipStream_t stream) {
     if (!scores || !rows) return 1001;
     if (n_queries <= 0 || nt <= 0 || k <= 0) return 1001;
     if (stride < nt) return 1002;
     (void)hipGetLastError();
-    const int n_segs = (nt + kSegKeys - 1) / kSegKeys;
-    // A query that fits one workgroup's registers (<= 65536 scores) is fastest there; longer
-    // ones are split over the chip when the caller brought a workspace. 65535 bounds grid.y.
-    if (workspace && nt > kTopkThreads * 64 && n_queries <= 65535) {
+    // A short query is fastest on one workgroup; longer ones are split over the chip when the
+    // caller brought a workspace.
+    if (workspace && topk_runs_split(n_queries, nt)) {
+        const int n_segs = topk_segments(nt);
         const size_t ws_stride = topk_ws_words(n_segs);
-        dim3 grid((unsigned)n_segs, (unsigned)n_queries), block(kSegThreads);
-        hipLaunchKernelGGL(topk_hist_kernel, grid, block, 0, stream, scores, stride, nts, nt, k,
-                           (uint32_t*)workspace, ws_stride);
-        hipLaunchKernelGGL(topk_select_kernel, grid, block, 0, stream, scores, stride, nts, nt, k,
-                           rows, (uint32_t*)workspace, ws_stride);
+        uint32_t* ws = (uint32_t*)workspace;
+        const dim3 seg_grid((unsigned)n_segs, (unsigned)n_queries), block(kSplitThreads);
+        if (!hist_ready)
+            hipLaunchKernelGGL(topk_hist_kernel, seg_grid, block, 0, stream, scores, stride, nts, nt,
+                               ws, ws_stride);
+        hipLaunchKernelGGL(topk_cand_kernel, seg_grid, block, 0, stream, scores, stride, nts, nt, k,
+                           ws, ws_stride, n_segs);
+        const int kmax = k < nt ? k : nt;
+        const dim3 out_grid((unsigned)((kmax + kSlotsPerGroup - 1) / kSlotsPerGroup),
+                            (unsigned)n_queries);
+        const size_t page_bytes = (size_t)ga.page_tokens * ga.width + (size_t)ga.page_tokens * 4;
+        if (ga.pool && ga.width == 576 && ga.page_tokens == 64)
+            hipLaunchKernelGGL((topk_finish_kernel<576, 64>), out_grid, block, 0, stream, scores,
+                               stride, nts, nt, k, rows, ws, ws_stride, n_segs, ga.pool,
+                               ga.block_table, ga.out, ga.max_blocks_per_seq, ga.width,
+                               ga.page_tokens, ga.n_pages, page_bytes, ga.bad_rows);
+        else
+            hipLaunchKernelGGL((topk_finish_kernel<0, 0>), out_grid, block, 0, stream, scores, stride,
+                               nts, nt, k, rows, ws, ws_stride, n_segs, ga.pool, ga.block_table,
+                               ga.out, ga.max_blocks_per_seq, ga.width, ga.page_tokens, ga.n_pages,
+                               page_bytes, ga.bad_rows);
         return launch_status();
     }
     dim3 grid((unsigned)n_queries), block(kTopkThreads);
@@ -1363,17 +1515,49 @@ extern "C" int rivoli_index_select_blocks(const float* scores, int rows, int n_c
 
 extern "C" size_t rivoli_index_topk_workspace_bytes(int n_queries, int nt) {
     if (n_queries <= 0 || nt <= 0) return 0;
-    const int n_segs = (nt + rk::kSegKeys - 1) / rk::kSegKeys;
-    return (size_t)n_queries * rk::topk_ws_words(n_segs) * sizeof(uint32_t);
+    return (size_t)n_queries * rk::topk_ws_words(rk::topk_segments(nt)) * sizeof(uint32_t);
 }
 
 extern "C" int rivoli_index_topk_batched(const float* scores, int n_queries, int stride,
                                          const int* nts, int nt, int k, unsigned int* rows,
                                          void* workspace, void* stream) {
-    return rk::index_topk_launch(scores, n_queries, stride, nts, nt, k, rows, workspace,
+    if (workspace && !rk::aligned16(workspace)) return 1004;
+    const rk::GatherArgs none = {nullptr, nullptr, nullptr, 0, 0, 0, 0, nullptr};
+    return rk::index_topk_launch(scores, n_queries, stride, nts, nt, k, rows, workspace, false, none,
                                  (hipStream_t)stream);
 }
 
 extern "C" int rivoli_index_topk(const float* scores, int nt, int k, unsigned int* rows) {
-    return rk::index_topk_launch(scores, 1, nt, nullptr, nt, k, rows, nullptr, nullptr);
+    const rk::GatherArgs none = {nullptr, nullptr, nullptr, 0, 0, 0, 0, nullptr};
+    return rk::index_topk_launch(scores, 1, nt, nullptr, nt, k, rows, nullptr, false, none, nullptr);
+}
+
+extern "C" int rivoli_dsa_select_gather_paged(const float* scores, int n_queries, int stride,
+                                              const int* nts, int nt, int k, unsigned int* rows,
+                                              void* workspace, int hist_ready,
+                                              const unsigned char* pool, const int* block_table,
+                                              unsigned short* out, int max_blocks_per_seq,
+                                              int width, int page_tokens, int n_pages,
+                                              unsigned int* bad_rows, void* stream) {
+    using namespace rk;
+    if (!pool || !block_table || !out) return 1001;
+    if (max_blocks_per_seq <= 0 || width <= 0 || page_tokens <= 0 || n_pages <= 0) return 1001;
+    if (n_queries > 65535) return 1002;
+    if (!gather_shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
+    if (workspace && !aligned16(workspace)) return 1004;
+    const GatherArgs ga = {pool, block_table, out, max_blocks_per_seq, width, page_tokens, n_pages,
+                           bad_rows};
+    const bool split = workspace && nt > 0 && n_queries > 0 && topk_runs_split(n_queries, nt);
+    if (hist_ready && !split) return 1001;  // nothing could have filled a histogram for this shape
+    if (split)
+        return index_topk_launch(scores, n_queries, stride, nts, nt, k, rows, workspace,
+                                 hist_ready != 0, ga, (hipStream_t)stream);
+    // short queries: one workgroup per query selects, the sparse gather follows on the stream
+    const GatherArgs none = {nullptr, nullptr, nullptr, 0, 0, 0, 0, nullptr};
+    const int code = index_topk_launch(scores, n_queries, stride, nts, nt, k, rows, nullptr, false,
+                                       none, (hipStream_t)stream);
+    if (code) return code;
+    return gather_rows_launch(pool, block_table, rows, nts, out, n_queries, k,
+                                        k < nt ? k : nt, max_blocks_per_seq, width, page_tokens,
+                                        n_pages, bad_rows, stream);
 }

@@ -16,19 +16,12 @@
 // resolved once into LDS (block-table lookup), then the same 8-in/16-out streaming body runs
 // over the 32 x width bytes.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
-#include "codec.hpp"
+#include "gather_common.hpp"
 
 namespace rk {
 
 constexpr int kGatherThreads = 256;
 constexpr int kRowsPerGroup = 32;  // sparse gather: rows resolved per workgroup
-
-__device__ __forceinline__ u32x4 dequant8_bf16(u32x2 codes, float scale) {
-    u32x2 a = dequant4_bf16(codes.x, scale);
-    u32x2 b = dequant4_bf16(codes.y, scale);
-    u32x4 r = {a.x, a.y, b.x, b.y};
-    return r;
-}
 
 // W / PT are the compile-time row width and page size (0 = take the runtime value), so the
 // flagship 576 x 64 shape gets constant divisors and a fully unrolled body. A workgroup owns
@@ -89,75 +82,31 @@ template <int W, int PT, int UNROLL>
 __global__ __launch_bounds__(kGatherThreads) void kv_gather_rows_kernel(
     const uint8_t* __restrict__ pool, const int* __restrict__ block_table,
     const unsigned int* __restrict__ rows, const int* __restrict__ n_rows,
-    uint16_t* __restrict__ out, int k, int max_blocks_per_seq, int width_rt, int page_tokens_rt,
-    int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_rows) {
+    uint16_t* __restrict__ out, int k, int nr_cap, int max_blocks_per_seq, int width_rt,
+    int page_tokens_rt, int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_rows) {
     const int width = W ? W : width_rt;
     const int pt = PT ? PT : page_tokens_rt;
     __shared__ unsigned long long s_base[kRowsPerGroup];
     __shared__ unsigned long long s_scale_at[kRowsPerGroup];
-    constexpr unsigned long long kSkip = ~0ull;
+    __shared__ int s_skipped;
 
     const int q = blockIdx.y;
     const int r0 = (int)blockIdx.x * kRowsPerGroup;
-    const int nr = n_rows ? min(n_rows[q], k) : k;
+    const int nr = n_rows ? min(n_rows[q], nr_cap) : nr_cap;
     if (r0 >= nr) return;
     const int cnt = min(kRowsPerGroup, nr - r0);
 
-    // row index -> page -> where the codes and the scale are. The scale itself is NOT
-    // fetched here: every thread loads its rows' scales together with the codes, so the
-    // chain of dependent memory round trips is row list -> block table -> data, not one
-    // longer.
-    if (threadIdx.x < kRowsPerGroup) {
-        unsigned long long base = kSkip, scale_at = 0;
-        if ((int)threadIdx.x < cnt) {
-            const unsigned int tok = rows[(size_t)q * k + r0 + threadIdx.x];
-            const unsigned int blk = tok / (unsigned)pt;
-            const unsigned int off = tok - blk * (unsigned)pt;
-            int page = -1;
-            if (blk < (unsigned)max_blocks_per_seq)
-                page = block_table[(size_t)q * max_blocks_per_seq + blk];
-            if ((unsigned)page < (unsigned)n_pages) {
-                const size_t pbase = (size_t)page * page_bytes;
-                base = pbase + (size_t)off * width;
-                scale_at = pbase + (size_t)pt * width + (size_t)off * 4;
-            } else if (bad_rows) {
-                atomicAdd(bad_rows, 1u);
-            }
-        }
-        s_base[threadIdx.x] = base;
-        s_scale_at[threadIdx.x] = scale_at;
-    }
+    if (threadIdx.x == 0) s_skipped = 0;
     __syncthreads();
-
-    const int cpr = width >> 3;
-    const int n_chunks = cnt * cpr;
-    u32x4* dst = reinterpret_cast<u32x4*>(out + ((size_t)q * k + r0) * width);
-    for (int cb = threadIdx.x; cb < n_chunks; cb += kGatherThreads * UNROLL) {
-        u32x2 raw[UNROLL];
-        float scl[UNROLL];
-        bool live[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            int c = cb + u * kGatherThreads;
-            live[u] = false;
-            if (c < n_chunks) {
-                int r = c / cpr;
-                int col = c - r * cpr;
-                unsigned long long base = s_base[r];
-                if (base != kSkip) {
-                    live[u] = true;
-                    raw[u] = __builtin_nontemporal_load(
-                        reinterpret_cast<const u32x2*>(pool + base) + col);
-                    scl[u] = *reinterpret_cast<const float*>(pool + s_scale_at[r]);
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            int c = cb + u * kGatherThreads;
-            if (live[u]) __builtin_nontemporal_store(dequant8_bf16(raw[u], scl[u]), dst + c);
-        }
-    }
+    if ((int)threadIdx.x < cnt &&
+        !resolve_row(rows[(size_t)q * k + r0 + threadIdx.x],
+                     block_table + (size_t)q * max_blocks_per_seq, max_blocks_per_seq, width, pt,
+                     n_pages, page_bytes, bad_rows, &s_base[threadIdx.x], &s_scale_at[threadIdx.x]))
+        s_skipped = 1;
+    __syncthreads();
+    const bool plain = !s_skipped && cnt * (width >> 3) == kGatherThreads * UNROLL;
+    stream_rows<kGatherThreads, UNROLL>(pool, s_base, s_scale_at, cnt, width, plain,
+                                        out + ((size_t)q * k + r0) * width);
 }
 
 // out[i] = bf16(e4m3_to_f32(codes[i]) * scale): the dequant body alone, for codec census tests.
@@ -172,10 +121,6 @@ __global__ void e4m3_dequant_bf16_kernel(const uint8_t* __restrict__ codes, floa
     }
 }
 
-static inline bool shape_ok(int width, int page_tokens) {
-    return (width % 16) == 0 && (page_tokens % 4) == 0;
-}
-
 }  // namespace rk
 
 extern "C" int rivoli_kv_gather_paged(const unsigned char* pool, const int* block_table,
@@ -188,7 +133,7 @@ extern "C" int rivoli_kv_gather_paged(const unsigned char* pool, const int* bloc
     if (n_seqs <= 0 || max_blocks_per_seq <= 0 || width <= 0 || page_tokens <= 0 || n_pages <= 0)
         return 1001;
     if (n_seqs > 65535) return 1002;
-    if (!shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
+    if (!gather_shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
     const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
     (void)hipGetLastError();
     if (width == 576 && page_tokens == 64) {
@@ -213,31 +158,40 @@ extern "C" int rivoli_kv_gather_paged(const unsigned char* pool, const int* bloc
     return launch_status();
 }
 
+// Query q gathers its first min(n_rows[q], nr_cap) listed rows (nr_cap when n_rows is null);
+// the lists and the output are k rows apart.
+int rk::gather_rows_launch(const unsigned char* pool, const int* block_table,
+                           const unsigned int* rows, const int* n_rows, unsigned short* out,
+                           int n_queries, int k, int nr_cap, int max_blocks_per_seq, int width,
+                           int page_tokens, int n_pages, unsigned int* bad_rows, void* stream) {
+    if (!pool || !block_table || !rows || !out) return 1001;
+    if (n_queries <= 0 || k <= 0 || nr_cap <= 0 || nr_cap > k || max_blocks_per_seq <= 0 ||
+        width <= 0 || page_tokens <= 0 || n_pages <= 0)
+        return 1001;
+    if (n_queries > 65535) return 1002;
+    if (!gather_shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
+    const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
+    dim3 grid((unsigned)((nr_cap + kRowsPerGroup - 1) / kRowsPerGroup), (unsigned)n_queries);
+    (void)hipGetLastError();
+    if (width == 576 && page_tokens == 64) {
+        hipLaunchKernelGGL((kv_gather_rows_kernel<576, 64, 9>), grid, dim3(kGatherThreads), 0,
+                           (hipStream_t)stream, pool, block_table, rows, n_rows, out, k, nr_cap,
+                           max_blocks_per_seq, width, page_tokens, n_pages, page_bytes, bad_rows);
+    } else {
+        hipLaunchKernelGGL((kv_gather_rows_kernel<0, 0, 4>), grid, dim3(kGatherThreads), 0,
+                           (hipStream_t)stream, pool, block_table, rows, n_rows, out, k, nr_cap,
+                           max_blocks_per_seq, width, page_tokens, n_pages, page_bytes, bad_rows);
+    }
+    return launch_status();
+}
+
 extern "C" int rivoli_kv_gather_rows_paged(const unsigned char* pool, const int* block_table,
                                            const unsigned int* rows, const int* n_rows,
                                            unsigned short* out, int n_queries, int k,
                                            int max_blocks_per_seq, int width, int page_tokens,
                                            int n_pages, unsigned int* bad_rows, void* stream) {
-    using namespace rk;
-    if (!pool || !block_table || !rows || !out) return 1001;
-    if (n_queries <= 0 || k <= 0 || max_blocks_per_seq <= 0 || width <= 0 || page_tokens <= 0 ||
-        n_pages <= 0)
-        return 1001;
-    if (n_queries > 65535) return 1002;
-    if (!shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
-    const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
-    dim3 grid((unsigned)((k + kRowsPerGroup - 1) / kRowsPerGroup), (unsigned)n_queries);
-    (void)hipGetLastError();
-    if (width == 576 && page_tokens == 64) {
-        hipLaunchKernelGGL((kv_gather_rows_kernel<576, 64, 9>), grid, dim3(kGatherThreads), 0,
-                           (hipStream_t)stream, pool, block_table, rows, n_rows, out, k,
-                           max_blocks_per_seq, width, page_tokens, n_pages, page_bytes, bad_rows);
-    } else {
-        hipLaunchKernelGGL((kv_gather_rows_kernel<0, 0, 4>), grid, dim3(kGatherThreads), 0,
-                           (hipStream_t)stream, pool, block_table, rows, n_rows, out, k,
-                           max_blocks_per_seq, width, page_tokens, n_pages, page_bytes, bad_rows);
-    }
-    return launch_status();
+    return rk::gather_rows_launch(pool, block_table, rows, n_rows, out, n_queries, k, k,
+                                  max_blocks_per_seq, width, page_tokens, n_pages, bad_rows, stream);
 }
 
 extern "C" int rivoli_codec_e4m3_dequant_bf16(const unsigned char* codes, float scale,

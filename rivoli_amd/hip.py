@@ -44,6 +44,9 @@ _SIGNATURES = {
     "rivoli_index_topk_batched": [_VP, _I, _I, _VP, _I, _I, _VP, _VP, _VP],
     "rivoli_index_score": [_VP] * 4 + [_I] * 4 + [_F, _F, _VP],
     "rivoli_index_score_paged": [_VP] * 6 + [_I] * 9 + [_F, _F, _VP, _VP],
+    "rivoli_index_score_paged_hist": [_VP] * 6 + [_I] * 9 + [_F, _F, _VP, _VP, _VP],
+    "rivoli_dsa_select_gather_paged": [_VP, _I, _I, _VP, _I, _I, _VP, _VP, _I, _VP, _VP, _VP,
+                                       _I, _I, _I, _I, _VP, _VP],
     "rivoli_index_append_paged": [_VP, _VP, _VP, _I, _I, _I, _I, _VP, _VP],
     "rivoli_hash_rows": [_VP, _I, _I, _ULL, _VP, _VP],
     "rivoli_device_sync": [],
@@ -170,6 +173,16 @@ def launch_index_score_paged(q, w, kpool, block_table, nts, heads, n_queries, ma
         _p(scores), _s(stream)), "index_score_paged")
 
 
+def launch_index_score_paged_hist(q, w, kpool, block_table, nts, heads, n_queries, max_blocks_per_seq,
+                                  stride, nt, nh, nact, hd, page_tokens, n_pages, wscale, dscale,
+                                  scores, topk_workspace, stream=NULL_STREAM) -> None:
+    """index_score_paged that also counts the selection histogram into the top-k workspace."""
+    ensure_hip_status(lib().rivoli_index_score_paged_hist(
+        _p(q), _p(w), _p(kpool), _p(block_table), _p(nts), _p(heads), n_queries,
+        max_blocks_per_seq, stride, nt, nh, nact, hd, page_tokens, n_pages, wscale, dscale,
+        _p(scores), _p(topk_workspace), _s(stream)), "index_score_paged_hist")
+
+
 def launch_index_append_paged(k, slot_mapping, kpool, n_tokens, hd, page_tokens, n_pages,
                               bad_slots=None, stream=NULL_STREAM) -> None:
     ensure_hip_status(lib().rivoli_index_append_paged(_p(k), _p(slot_mapping), _p(kpool), n_tokens,
@@ -223,6 +236,16 @@ def launch_index_topk_batched(scores, n_queries, stride, nts, nt, k, rows, works
     ensure_hip_status(lib().rivoli_index_topk_batched(_p(scores), n_queries, stride, _p(nts), nt,
                                                       k, _p(rows), _p(workspace), _s(stream)),
                       "index_topk_batched")
+
+
+def launch_dsa_select_gather_paged(scores, n_queries, stride, nts, nt, k, rows, workspace, hist_ready,
+                                   pool, block_table, out, max_blocks_per_seq, width, page_tokens,
+                                   n_pages, bad_rows=None, stream=NULL_STREAM) -> None:
+    """Top-k selection and the sparse gather of the selected rows in one call."""
+    ensure_hip_status(lib().rivoli_dsa_select_gather_paged(
+        _p(scores), n_queries, stride, _p(nts), nt, k, _p(rows), _p(workspace), 1 if hist_ready else 0,
+        _p(pool), _p(block_table), _p(out), max_blocks_per_seq, width, page_tokens, n_pages,
+        _p(bad_rows), _s(stream)), "dsa_select_gather_paged")
 
 
 # ---- attention: the reference's single-token launcher over its linear slabs ----------------

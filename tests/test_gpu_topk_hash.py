@@ -60,8 +60,8 @@ def batched_topk(scores, nts, k, split):
         rows = dzeros(n_q * k * 4, 0xFF)
         hip.launch_index_topk_batched(sd, n_q, stride, ntd, stride, k, rows, ws)
         got = back(rows, np.uint32).reshape(n_q, k)
-    if split:   # the histogram and both tickets are back to zero
-        assert not back(ws, np.uint32).reshape(n_q, -1)[:, :4098].any()
+    if split:   # the per-query histogram is back to zero
+        assert not back(ws, np.uint32).reshape(n_q, -1)[:, :4096].any()
     return got
 
 
