@@ -170,8 +170,9 @@ int rivoli_index_score(const float* q, const float* w, const unsigned short* kca
 /* The paged, batched form: query qi (q [n_queries][nh][hd], w [n_queries][nh]) scores its
  * first nts[qi] tokens (nt when nts is null) through block_table[qi] over the paged key
  * cache kpool[n_pages*page_tokens][hd] bf16, into scores[qi*stride + t]. Tokens whose page id
- * is outside [0, n_pages) are not written. Same guards, plus 1002 for stride < nt and 1004
- * for page_tokens % 32 (a 32-token block must sit inside one page). */
+ * is outside [0, n_pages) are not written. Same guards, plus 1002 for stride < nt, for
+ * nt > max_blocks_per_seq * page_tokens (a scored token without a block-table entry) or for
+ * n_queries > 65535, and 1004 for page_tokens % 32 (a 32-token block must sit inside one page). */
 int rivoli_index_score_paged(const float* q, const float* w, const unsigned short* kpool,
                              const int* block_table, const int* nts, const unsigned int* heads,
                              int n_queries, int max_blocks_per_seq, int stride, int nt, int nh,

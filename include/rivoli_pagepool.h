@@ -12,7 +12,8 @@
  * the kernels in rivoli_kvcache.h consume. Not thread-safe: one decode thread owns a pool,
  * as one thread issues all launches in the reference (crates/backend/src/gpustream.rs:83-91).
  * Return convention: >= 0 success / value, negative = refusal:
- *   -1001 invalid argument or unknown sequence, -1005 pool exhausted (nothing was changed).
+ *   -1001 invalid argument or unknown sequence, -1005 pool exhausted, -1006 out of host memory
+ *   (nothing was changed in either case; no C++ exception leaves an entry point).
  */
 #ifndef RIVOLI_PAGEPOOL_H
 #define RIVOLI_PAGEPOOL_H

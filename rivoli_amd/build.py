@@ -27,16 +27,33 @@ def offload_arch() -> str:
 
 
 def build_kernels(verbose: bool = False) -> str:
-    cmd = [hipcc(), f"--offload-arch={offload_arch()}", "-O3", "-std=c++17", "-fPIC", "-shared",
-           # packed-f32 instructions stay off: plain f32 math only
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           "-I", os.path.join(os.path.dirname(CSRC), "..", "include"),
-           "-o", LIB_PATH] + [os.path.join(CSRC, k) for k in KERNELS]
-    res = subprocess.run(cmd, capture_output=True, text=True)
+    """Every source to an object of its own (in parallel, under build/), then one link."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    objdir = os.path.join(CSRC, "build")
+    os.makedirs(objdir, exist_ok=True)
+    common = [hipcc(), f"--offload-arch={offload_arch()}", "-O3", "-std=c++17", "-fPIC",
+              # packed-f32 instructions stay off: plain f32 math only
+              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+              "-I", os.path.join(os.path.dirname(CSRC), "..", "include")]
+
+    def compile_one(k: str) -> str:
+        obj = os.path.join(objdir, k.replace(".hip", ".o"))
+        res = subprocess.run(common + ["-c", os.path.join(CSRC, k), "-o", obj], capture_output=True, text=True)
+        if verbose or res.returncode != 0:
+            sys.stderr.write(res.stdout + res.stderr)
+        if res.returncode != 0:
+            raise RuntimeError("hipcc failed compiling " + k)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+        objs = list(pool.map(compile_one, KERNELS))
+    res = subprocess.run([hipcc(), f"--offload-arch={offload_arch()}", "-shared", "-fPIC", "-o", LIB_PATH] + objs,
+                         capture_output=True, text=True)
     if verbose or res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed building " + LIB_PATH)
+        raise RuntimeError("hipcc failed linking " + LIB_PATH)
     return LIB_PATH
 
 

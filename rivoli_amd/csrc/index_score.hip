@@ -263,6 +263,8 @@ static int index_score_launch(const float* q, const float* w, const unsigned sho
     if (block_table && (max_blocks_per_seq <= 0 || page_tokens <= 0 || n_pages <= 0)) return 1001;
     if (nact > kScoreMaxHeads || hd > kScoreMaxHd || stride < nt || n_queries > 65535) return 1002;
     if ((hd % 16) != 0 || (block_table && (page_tokens % 32) != 0)) return 1004;
+    // every scored token needs an entry in its query's block-table row
+    if (block_table && (long long)nt > (long long)max_blocks_per_seq * page_tokens) return 1002;
     // the histogram is only wanted where the selection of this shape runs split over the chip
     if (topk_workspace && !aligned16(topk_workspace)) return 1004;
     uint32_t* ws = topk_runs_split(n_queries, nt) ? (uint32_t*)topk_workspace : nullptr;

@@ -235,7 +235,9 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
             w.n_here = 0, w.tile_off = 0, w.tile_scale_off = 0;
             if (pos0 >= r_end) return;
             const int blk = pos0 >> a.page_shift, off = pos0 & (a.page_tokens - 1);
-            const int page = __builtin_amdgcn_readfirstlane(table_at(blk));
+            // a position the block table has no entry for is skipped and counted, like a page
+            // id outside the pool: the table row of the next sequence is never read
+            const int page = blk < a.max_blocks ? __builtin_amdgcn_readfirstlane(table_at(blk)) : -1;
             const int n = min(kTile, r_end - pos0);
             if ((unsigned)page < (unsigned)a.n_pages) {
                 w.n_here = n;

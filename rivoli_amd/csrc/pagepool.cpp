@@ -2,7 +2,14 @@
 // follows (crates/core/src/arena.rs:132-149) are in include/rivoli_pagepool.h.
 #include "rivoli_pagepool.h"
 
+#include <cstddef>
+#include <new>
 #include <vector>
+
+// No C++ exception may cross the C boundary: an allocation failure inside an entry point is
+// reported as kOutOfHostMemory, and every entry point reserves what it will need BEFORE it changes
+// the pool, so a failed call leaves the pool exactly as it found it.
+static constexpr int kOutOfHostMemory = -1006;
 
 struct rivoli_pagepool {
     int n_pages = 0;
@@ -37,9 +44,16 @@ struct rivoli_pagepool {
 extern "C" rivoli_pagepool* rivoli_pagepool_create(int n_pages, int page_tokens) {
     if (n_pages <= 0 || page_tokens <= 0) return nullptr;
     if ((long long)n_pages * page_tokens > 0x7fffffffLL) return nullptr;  // slots must fit int
-    auto* p = new rivoli_pagepool();
+    auto* p = new (std::nothrow) rivoli_pagepool();
+    if (!p) return nullptr;
     p->n_pages = n_pages;
     p->page_tokens = page_tokens;
+    try {
+        p->free_list.reserve((std::size_t)n_pages);  // freeing pages can then never allocate
+    } catch (...) {
+        delete p;
+        return nullptr;
+    }
     return p;
 }
 
@@ -53,7 +67,13 @@ extern "C" int rivoli_pagepool_seq_create(rivoli_pagepool* pool) {
         pool->free_ids.pop_back();
     } else {
         id = (int)pool->seqs.size();
-        pool->seqs.emplace_back();
+        try {
+            // room for this id on the list of freed ids too, so seq_free cannot fail
+            pool->free_ids.reserve(pool->seqs.size() + 1);
+            pool->seqs.emplace_back();
+        } catch (...) {
+            return kOutOfHostMemory;
+        }
     }
     pool->seqs[id].live = true;
     pool->seqs[id].len = 0;
@@ -85,6 +105,11 @@ extern "C" int rivoli_pagepool_seq_extend(rivoli_pagepool* pool, int seq, int n_
     const long long blocks_needed = (new_len + pt - 1) / pt;
     const long long extra = blocks_needed - (long long)s->pages.size();
     if (extra > pool->available()) return -1005;
+    try {
+        s->pages.reserve((std::size_t)blocks_needed);  // all or nothing: the pushes below cannot throw
+    } catch (...) {
+        return kOutOfHostMemory;
+    }
     for (long long i = 0; i < extra; ++i) s->pages.push_back(pool->take_page());
     pool->owned += (int)extra;
     if (slots_out) {

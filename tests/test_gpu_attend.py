@@ -183,6 +183,20 @@ def test_bad_pages_are_left_out_and_counted(oracle):
     assert back(bad, np.uint32)[0] == 64
 
 
+def test_lengths_past_the_block_table_are_left_out_and_counted(oracle):
+    """A length that claims more rows than the block table can address (4 blocks = 256 rows
+    here): the rows past the table are skipped and counted, the neighbouring sequence's table
+    row is never used in their place, and nothing past the table is read."""
+    c = paged_case(oracle, [200, 200], H=64, seed=610)
+    assert c["table"].shape[1] == 4
+    want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], c["lens"], None, None,
+                                   KVL, ROPE, PT, c["scale"])
+    bad = dzeros(4)
+    got = run_paged(dict(c, lens=np.array([300, 300], np.int32)), 300, bad=bad)
+    check(got, want, 2, "rows past the table")
+    assert back(bad, np.uint32)[0] == 2 * (300 - 256)
+
+
 def test_guards():
     b = dzeros(4096)
     ok = dict(n_seqs=1, H=64, max_rows=64, mb=1, kvl=512, rope=64, pt=64, n_pages=1)

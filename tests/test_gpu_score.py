@@ -70,6 +70,10 @@ def test_index_score_guards():
         with pytest.raises(hip.LaunchError) as e:
             hip.launch_index_score(b, b, b, None, *args, 1.0, 1.0, b)
         assert e.value.code == code, args
+    # paged: every scored token needs a block-table entry (here 2 blocks x 64 tokens < nt = 129)
+    with pytest.raises(hip.LaunchError) as e:
+        hip.launch_index_score_paged(b, b, b, b, None, None, 1, 2, 129, 129, 8, 8, 16, 64, 4, 1.0, 1.0, b)
+    assert e.value.code == 1002
 
 
 def test_paged_index_append_and_score(oracle):
