@@ -155,6 +155,26 @@ int rivoli_dsa_select_gather_paged(const float* scores, int n_queries, int strid
                                    int max_blocks_per_seq, int width, int page_tokens, int n_pages,
                                    unsigned int* bad_rows, void* stream);
 
+/* rivoli_dsa_select_gather_paged for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no
+ * counterpart in the reference. Same arguments without `workspace` and `hist_ready`, same
+ * results bit for bit: the selection's workspace is a 4.5 MiB array inside the library's own
+ * device image (one copy per GPU, held until the process ends), and the call makes no
+ * hipMalloc / hipFree and calls no allocating routine. Shapes that run split must fit it:
+ * n_queries * rivoli_index_topk_workspace_bytes(1, nt) <= 4 718 592 bytes (16 queries of 65536
+ * scores do), else 1002; shorter queries (nt <= 16384) need no workspace and are not limited.
+ * Every call on a GPU shares that GPU's array, so calls that overlap on one GPU (two streams,
+ * two threads) race; calls that follow each other on one stream are fine, whatever their shapes
+ * (the call clears what must start at zero with a fill kernel, not a memset). The first call on
+ * a device looks the array's address up (hipGetSymbolAddress): make it outside a graph capture.
+ * Other guards as rivoli_dsa_select_gather_paged. */
+int rivoli_dsa_select_gather_paged_noalloc(const float* scores, int n_queries, int stride,
+                                           const int* nts, int nt, int k, unsigned int* rows,
+                                           const unsigned char* pool, const int* block_table,
+                                           unsigned short* out, int max_blocks_per_seq, int width,
+                                           int page_tokens, int n_pages, unsigned int* bad_rows,
+                                           void* stream);
+
 /* Replaces crates/backend/kernels/indexer.hip:278-295 (launch_index_score,
  * crates/backend/src/hip_attn.rs:464-476): scores[t] = sum over the active heads h of
  * w[h]*wscale*max((q_h . k_t)*dscale, 0) for t < nt, over the LINEAR bf16 key cache

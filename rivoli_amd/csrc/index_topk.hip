@@ -38,6 +38,7 @@
 //     shape (1)'s radix passes over the whole query in every workgroup — slower, same answer.
 //     The histogram is left zeroed for the next call.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
+#include <mutex>
 #include <type_traits>
 
 #include "gather_common.hpp"
@@ -1466,6 +1467,56 @@ static int sel_fill_launch(const SelShape& s, int win, int ratio, int start_pos,
     return launch_status();
 }
 
+// ---------------------------------------------------------------------------------------------
+// The selection workspace for callers that cannot allocate: one array per GPU, inside the
+// library's own image, held until the process ends. Sized for 16 queries of 65536 scores.
+// ---------------------------------------------------------------------------------------------
+constexpr size_t kStaticWsWords = 1179648;  // 4.5 MiB
+constexpr int kStaticWsMaxDevices = 64;
+static __device__ __align__(256) uint32_t scratch[kStaticWsWords];
+static std::mutex g_scratch_mutex;
+static uint32_t* g_scratch_ptr[kStaticWsMaxDevices];  // per device: where ITS copy of the array is
+
+// The current device's copy of `scratch` (looked up once per device); 0, a guard code, or
+// -(int)hipError_t.
+static int static_workspace(uint32_t** out) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return -(int)e;
+    if (device < 0 || device >= kStaticWsMaxDevices) return 1002;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return -(int)e;
+        if (!p) return -(int)hipErrorInvalidSymbol;
+        g_scratch_ptr[device] = (uint32_t*)p;
+    }
+    *out = g_scratch_ptr[device];
+    return 0;
+}
+
+// The histogram of every query back to zero (a fill kernel, so that the call can sit in a
+// captured graph): the array keeps what the last call left, and a call of another shape left
+// its lists where this one's histograms are.
+__global__ __launch_bounds__(kSplitThreads) void topk_ws_clear_kernel(uint32_t* __restrict__ ws,
+                                                                      size_t ws_stride) {
+    reinterpret_cast<u32x4*>(ws + (size_t)blockIdx.x * ws_stride)[threadIdx.x] = u32x4{0u, 0u, 0u, 0u};
+}
+
+// What both forms of the select-and-gather call refuse before anything is launched.
+static int dsa_guard(const float* scores, int n_queries, int stride, int nt, int k,
+                     const unsigned int* rows, const unsigned char* pool, const int* block_table,
+                     const unsigned short* out, int max_blocks_per_seq, int width, int page_tokens,
+                     int n_pages) {
+    if (!scores || !rows || !pool || !block_table || !out) return 1001;
+    if (n_queries <= 0 || nt <= 0 || k <= 0) return 1001;
+    if (max_blocks_per_seq <= 0 || width <= 0 || page_tokens <= 0 || n_pages <= 0) return 1001;
+    if (stride < nt || n_queries > 65535) return 1002;
+    if (!gather_shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
+    return 0;
+}
+
 }  // namespace rk
 
 extern "C" int rivoli_sel_shape(int win, int ratio, int index_topk, int seqlen, int start_pos,
@@ -1540,10 +1591,9 @@ extern "C" int rivoli_dsa_select_gather_paged(const float* scores, int n_queries
                                               int width, int page_tokens, int n_pages,
                                               unsigned int* bad_rows, void* stream) {
     using namespace rk;
-    if (!pool || !block_table || !out) return 1001;
-    if (max_blocks_per_seq <= 0 || width <= 0 || page_tokens <= 0 || n_pages <= 0) return 1001;
-    if (n_queries > 65535) return 1002;
-    if (!gather_shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
+    const int refused = dsa_guard(scores, n_queries, stride, nt, k, rows, pool, block_table, out,
+                                  max_blocks_per_seq, width, page_tokens, n_pages);
+    if (refused) return refused;
     if (workspace && !aligned16(workspace)) return 1004;
     const GatherArgs ga = {pool, block_table, out, max_blocks_per_seq, width, page_tokens, n_pages,
                            bad_rows};
@@ -1560,4 +1610,32 @@ extern "C" int rivoli_dsa_select_gather_paged(const float* scores, int n_queries
     return gather_rows_launch(pool, block_table, rows, nts, out, n_queries, k,
                                         k < nt ? k : nt, max_blocks_per_seq, width, page_tokens,
                                         n_pages, bad_rows, stream);
+}
+
+extern "C" int rivoli_dsa_select_gather_paged_noalloc(const float* scores, int n_queries,
+                                                      int stride, const int* nts, int nt, int k,
+                                                      unsigned int* rows, const unsigned char* pool,
+                                                      const int* block_table, unsigned short* out,
+                                                      int max_blocks_per_seq, int width,
+                                                      int page_tokens, int n_pages,
+                                                      unsigned int* bad_rows, void* stream) {
+    using namespace rk;
+    const int refused = dsa_guard(scores, n_queries, stride, nt, k, rows, pool, block_table, out,
+                                  max_blocks_per_seq, width, page_tokens, n_pages);
+    if (refused) return refused;
+    uint32_t* ws = nullptr;
+    if (topk_runs_split(n_queries, nt)) {
+        const size_t ws_stride = topk_ws_words(topk_segments(nt));
+        if ((size_t)n_queries * ws_stride > kStaticWsWords) return 1002;
+        const int code = static_workspace(&ws);
+        if (code) return code;
+        (void)hipGetLastError();
+        hipLaunchKernelGGL(topk_ws_clear_kernel, dim3((unsigned)n_queries), dim3(kSplitThreads), 0,
+                           (hipStream_t)stream, ws, ws_stride);
+        const int launched = launch_status();
+        if (launched) return launched;
+    }
+    return rivoli_dsa_select_gather_paged(scores, n_queries, stride, nts, nt, k, rows, ws, 0, pool,
+                                          block_table, out, max_blocks_per_seq, width, page_tokens,
+                                          n_pages, bad_rows, stream);
 }

@@ -47,6 +47,8 @@ _SIGNATURES = {
     "rivoli_index_score_paged_hist": [_VP] * 6 + [_I] * 9 + [_F, _F, _VP, _VP, _VP],
     "rivoli_dsa_select_gather_paged": [_VP, _I, _I, _VP, _I, _I, _VP, _VP, _I, _VP, _VP, _VP,
                                        _I, _I, _I, _I, _VP, _VP],
+    "rivoli_dsa_select_gather_paged_noalloc": [_VP, _I, _I, _VP, _I, _I, _VP, _VP, _VP, _VP,
+                                               _I, _I, _I, _I, _VP, _VP],
     "rivoli_index_append_paged": [_VP, _VP, _VP, _I, _I, _I, _I, _VP, _VP],
     "rivoli_hash_rows": [_VP, _I, _I, _ULL, _VP, _VP],
     "rivoli_device_sync": [],
@@ -246,6 +248,16 @@ def launch_dsa_select_gather_paged(scores, n_queries, stride, nts, nt, k, rows, 
         _p(scores), n_queries, stride, _p(nts), nt, k, _p(rows), _p(workspace), 1 if hist_ready else 0,
         _p(pool), _p(block_table), _p(out), max_blocks_per_seq, width, page_tokens, n_pages,
         _p(bad_rows), _s(stream)), "dsa_select_gather_paged")
+
+
+def launch_dsa_select_gather_paged_noalloc(scores, n_queries, stride, nts, nt, k, rows, pool, block_table,
+                                           out, max_blocks_per_seq, width, page_tokens, n_pages,
+                                           bad_rows=None, stream=NULL_STREAM) -> None:
+    """launch_dsa_select_gather_paged over the library's own workspace: allocates nothing."""
+    ensure_hip_status(lib().rivoli_dsa_select_gather_paged_noalloc(
+        _p(scores), n_queries, stride, _p(nts), nt, k, _p(rows), _p(pool), _p(block_table), _p(out),
+        max_blocks_per_seq, width, page_tokens, n_pages, _p(bad_rows), _s(stream)),
+        "dsa_select_gather_paged_noalloc")
 
 
 # ---- attention: the reference's single-token launcher over its linear slabs ----------------
