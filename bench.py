@@ -40,10 +40,10 @@ def parse():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=32768)
-    ap.add_argument("--workload", choices=["decode", "prefill", "dsa", "dsa_scored", "dsa_attend", "attend", "v4",
+    ap.add_argument("--workload", choices=["all", "decode", "prefill", "dsa", "dsa_scored", "dsa_attend", "attend", "v4",
                                            "v4_attend"],
-                    default="decode",
-                    help="decode = configuration 3 (the headline line); prefill = configuration 2 "
+                    default="all",
+                    help="all (default) = the headline line with every other configuration attached under `configs`; decode = configuration 3 (the headline line) alone; prefill = configuration 2 "
                          "bulk append; dsa = configuration 4 top-k + sparse gather on synthetic "
                          "scores; dsa_scored = the same with the scores computed on the device; "
                          "dsa_attend = configuration 4 with the sparse gather replaced by MLA decode "
@@ -64,6 +64,12 @@ def parse():
     ap.add_argument("--ragged", action="store_true",
                     help="decode / attend: per-sequence context drawn uniformly from [1024, ctx] "
                          "(configuration 3 as written) instead of every sequence at ctx (its metric point)")
+    ap.add_argument("--table-blocks", type=int, default=0,
+                    help="decode: columns of the block tables (default: what ctx needs); more = tables sized "
+                         "for a context limit above ctx, their extra columns unused")
+    ap.add_argument("--gather-form", choices=["packed", "grid"], default="packed",
+                    help="decode: rivoli_kv_gather_paged_packed (the caller passes the batch's token count) "
+                         "or rivoli_kv_gather_paged")
     ap.add_argument("--tokens", type=int, default=8192, help="prefill: new tokens per step")
     ap.add_argument("--topk", type=int, default=2048)
     ap.add_argument("--unfused", action="store_true",
@@ -103,16 +109,86 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    if a.workload == "prefill":
+    if a.workload != "all":
+        res = run_workload(a.workload, a, torch, hip)
+        print(json.dumps(res), flush=True)
+        return
+    # the default run: the headline (configuration 3 at its metric point) and, in the same
+    # line, the other configurations, each with its own oracle check
+    res = bench_decode(a, torch, hip)
+    short = min(a.cpu_seconds, 2.0)
+    others = (("cfg3_ragged", "decode", dict(ragged=True, cpu_seconds=short)),
+              ("cfg4_dsa", "dsa", dict(cpu_seconds=short)),
+              ("cfg4_dsa_scored", "dsa_scored", {}),
+              ("cfg2_prefill_8192", "prefill", dict(tokens=8192, cpu_seconds=short)),
+              ("cfg2_prefill_1048576", "prefill", dict(tokens=1048576, cpu_seconds=short)))
+    res["configs"] = {}
+    for name, workload, over in others:
+        torch.cuda.empty_cache()
+        sub = run_workload(workload, argparse.Namespace(**{**vars(a), **over}), torch, hip)
+        res["configs"][name] = brief(sub)
+    print(json.dumps(res), flush=True)
+
+
+def run_workload(workload, a, torch, hip):
+    if workload == "decode":
+        return bench_decode(a, torch, hip)
+    if workload == "prefill":
         return bench_prefill(a, torch, hip)
-    if a.workload in ("dsa", "dsa_scored", "dsa_attend"):
-        return bench_dsa(a, torch, hip, scored=a.workload == "dsa_scored", attend=a.workload == "dsa_attend")
-    if a.workload == "attend":
+    if workload in ("dsa", "dsa_scored", "dsa_attend"):
+        return bench_dsa(a, torch, hip, scored=workload == "dsa_scored", attend=workload == "dsa_attend")
+    if workload == "attend":
         return bench_attend(a, torch, hip)
-    if a.workload == "v4":
+    if workload == "v4":
         return bench_v4(a, torch, hip)
-    if a.workload == "v4_attend":
+    if workload == "v4_attend":
         return bench_v4_attend(a, torch, hip)
+    raise SystemExit(f"unknown workload {workload}")
+
+
+def brief(res):
+    """What a secondary configuration contributes to the default run's line."""
+    keep = ("metric", "value", "unit", "ms_per_step", "layer_us", "hbm_peak_frac", "tokens_per_s", "rows_per_s",
+            "kernels_ms", "roofline", "index_score", "config")
+    out = {k: res[k] for k in keep if k in res}
+    if "cpu_baseline" in res:
+        out["checked"] = res["cpu_baseline"]["sample"]
+        out["cpu_baseline"] = {k: res["cpu_baseline"][k] for k in ("value", "unit", "cores", "nproc", "kind")
+                               if k in res["cpu_baseline"]}
+    return out
+
+
+def host_threads():
+    """(threads the CPU baseline uses, processors this process may run on, processors the box has)."""
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return max(1, min(16, usable)), usable, os.cpu_count() or 1
+
+
+_TRAFFIC = None
+
+
+def measured_traffic(key):
+    """HBM bytes per launch of a workload's dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
+    WRITE_SIZE runs of that workload scaled by a plain copy of known size. Counters cannot be
+    read from inside the process, so the figures are kept in profiles/traffic.json by shape;
+    a shape that was not measured reports null."""
+    global _TRAFFIC
+    if _TRAFFIC is None:
+        try:
+            with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+                _TRAFFIC = json.load(f)
+        except (OSError, ValueError):
+            _TRAFFIC = {}
+    entry = _TRAFFIC.get(key)
+    return entry["bytes"] if isinstance(entry, dict) else None
+
+
+def bench_decode(a, torch, hip):
+    """Benchmark configuration 3: per layer, append one token per sequence, then gather and
+    dequantize every sequence's context."""
     L, B, ctx = a.layers, a.batch, a.ctx
     blocks = -(-ctx // PT)
     n_pages = B * blocks
@@ -127,6 +203,9 @@ def main():
     tables_np = perm.reshape(B, blocks)
     pos = np.arange(ctx)
     slots_np = np.concatenate([tables_np[s][pos // PT] * PT + pos % PT for s in range(B)]).astype(np.int32)
+    cols = max(blocks, a.table_blocks)
+    if cols > blocks:
+        tables_np = np.concatenate([tables_np, np.full((B, cols - blocks), -1, np.int32)], axis=1)
     tables = torch.from_numpy(tables_np.copy()).cuda()
     slots_all = torch.from_numpy(slots_np).cuda()
     seq_lens_np = context_lengths(a, rng)
@@ -157,8 +236,12 @@ def main():
             if events is not None:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)
-            hip.launch_kv_gather_paged(pools[layer], tables, seq_lens, cu, out, B, blocks, W, PT,
-                                       n_pages, None, sh)
+            if a.gather_form == "packed":
+                hip.launch_kv_gather_paged_packed(pools[layer], tables, seq_lens, cu, out, B, cols, n_att, W,
+                                                  PT, n_pages, None, sh)
+            else:
+                hip.launch_kv_gather_paged(pools[layer], tables, seq_lens, cu, out, B, cols, W, PT, n_pages,
+                                           None, sh)
             if events is not None:
                 e1.record(stream)
                 events.append((e0, e1))
@@ -195,23 +278,20 @@ def main():
                    "layers": L, "batch": B, "ctx": ctx, "page_tokens": PT, "width": W,
                    "stored": "fp8 e4m3 + 1 f32 scale/token", "out": "bf16",
                    "contexts": "uniform in [1024, ctx]" if a.ragged else "all at ctx",
-                   "tokens_per_layer": n_att},
+                   "tokens_per_layer": n_att, "table_blocks": cols, "gather_form": a.gather_form},
         "decode_step_kv_ms": round(ms_per_step, 4),
         "tokens_per_s": round(L * n_att / (ms_per_step * 1e-3), 1),
         "hbm_peak_frac": round(value * 1e9 / HBM_PEAK, 4),
         "roofline": {"bound": "hbm", "kernel": "kv_gather_paged_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": round(achieved * 1e9 / HBM_PEAK, 4),
                      "avg_launch_ms": round(gather_ms, 5), "bytes_per_launch": gather_bytes_layer,
-                     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-                     # this workload, scaled by a known 1 GiB copy (profiles/); it cannot be
-                     # read live, so it is only reported for the shape it was measured on
-                     "traffic": 1821500000 if (B, ctx) == (32, 32768) and not a.ragged else None},
+                     "traffic": measured_traffic(f"decode:b{B}:ctx{ctx}:{'ragged' if a.ragged else 'uniform'}")},
     }
 
     if not a.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(pools[0], tables_np, seq_lens_np, out, a.cpu_seconds,
-                                              hip, tables, seq_lens, cu, B, blocks, n_pages)
-    print(json.dumps(result), flush=True)
+                                              hip, tables, seq_lens, cu, B, cols, n_pages)
+    return result
 
 
 def timed(torch, stream, steps, warmup, step):
@@ -289,13 +369,12 @@ def bench_prefill(a, torch, hip):
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                         "frac": round(nbytes / (per["append"] * 1e-3) / HBM_PEAK, 5),
                         "avg_launch_ms": round(per["append"], 5), "bytes_per_launch": nbytes,
-                        # rocprofv3 FETCH_SIZE + WRITE_SIZE of this kernel at 1 048 576 tokens, scaled
-                        # by a known 1 GiB copy (profiles/); not readable from inside the process
-                        "traffic": 1833300000 if n == 1048576 else None}}
+                        "traffic": measured_traffic(f"prefill:tokens{n}")}}
     if not a.no_cpu_baseline:
         from oracle.kvoracle import oracle as get_oracle
 
-        ora, cores = get_oracle(), max(1, min(16, os.cpu_count() or 1))
+        ora = get_oracle()
+        cores, usable, nproc = host_threads()
         rows_h = rows.view(torch.int16).cpu().numpy().view(np.uint16)
         slots_h, pool_h = slots.cpu().numpy(), np.zeros(n_pages * page_bytes, np.uint8)
         reps, spent = 0, 0.0
@@ -307,10 +386,10 @@ def bench_prefill(a, torch, hip):
         if not np.array_equal(pool.cpu().numpy(), pool_h):
             raise SystemExit("bench: GPU append differs from the CPU oracle")
         res["cpu_baseline"] = {"value": round(nbytes / (spent / reps) / 1e9, 3), "unit": "GB/s",
-                               "cores": cores, "kind": "port",
+                               "cores": cores, "nproc": nproc, "usable": usable, "kind": "port",
                                "sample": f"the same {n}-token append x{reps} reps, {cores} host "
                                          "threads; GPU pool bytes checked equal"}
-    print(json.dumps(res), flush=True)
+    return res
 
 
 def ordered_bf16(ora, x):
@@ -672,7 +751,8 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
     if not a.no_cpu_baseline and not scored and not attend:
         from oracle.kvoracle import oracle as get_oracle
 
-        ora, cores = get_oracle(), max(1, min(16, os.cpu_count() or 1))
+        ora = get_oracle()
+        cores, usable, nproc = host_threads()
         sc_h, pool_h = scores[0].cpu().numpy(), pools[0].cpu().numpy()
         reps, spent = 0, 0.0
         while spent < a.cpu_seconds and reps < 50:
@@ -693,10 +773,10 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
         if not np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16).reshape(B, k, W), want_rows):
             raise SystemExit("bench: GPU sparse gather differs from the CPU oracle")
         res["cpu_baseline"] = {"value": round(layer_bytes / (spent / reps) / 1e9, 3), "unit": "GB/s",
-                               "cores": cores, "kind": "port",
+                               "cores": cores, "nproc": nproc, "usable": usable, "kind": "port",
                                "sample": f"one layer (top-k on {cores} host threads, sparse gather "
                                          f"single-threaded) x{reps} reps; GPU indices and rows checked equal"}
-    print(json.dumps(res), flush=True)
+    return res
 
 
 def bench_attend(a, torch, hip):
@@ -771,12 +851,13 @@ def bench_attend(a, torch, hip):
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                         "frac": round(attend_bytes / (per["attend"] * 1e-3) / HBM_PEAK, 4),
                         "avg_launch_ms": round(per["attend"], 5), "bytes_per_launch": attend_bytes,
-                        "traffic": 679990000 if (B, ctx, H) == (32, 32768, 64) and not a.ragged else None,
+                        "traffic": measured_traffic(f"attend:b{B}:ctx{ctx}:h{H}:{'ragged' if a.ragged else 'uniform'}"),
                         "tflops": round(flops / (per["attend"] * 1e-3) / 1e12, 1)}}
     if not a.no_cpu_baseline:
         from oracle.kvoracle import oracle as get_oracle
 
-        ora, cores = get_oracle(), max(1, min(16, os.cpu_count() or 1))
+        ora = get_oracle()
+        cores, usable, nproc = host_threads()
         # bounded sample: the first `cores` sequences cut to 2048 tokens, all heads, layer 0
         ns, cut = min(B, cores), min(ctx, 2048)
         lens_cut = np.zeros(B, np.int32)
@@ -796,11 +877,11 @@ def bench_attend(a, torch, hip):
             raise SystemExit(f"bench: GPU attention differs from the CPU oracle: err={err:.3e} max={mx:.3e}")
         sample_bytes = ns * cut * REC + ns * H * (W + KVL) * 4
         res["cpu_baseline"] = {"value": round(sample_bytes / spent / 1e9, 4), "unit": "GB/s", "cores": cores,
-                               "kind": "port",
+                               "nproc": nproc, "usable": usable, "kind": "port",
                                "sample": f"attention of {ns} sequences x {cut} tokens x {H} heads (layer 0, same "
                                          f"pool) on {cores} host threads; GPU output within {err / mx:.1e} of it",
                                "tokens_per_s": round(ns * cut / spent, 1)}
-    print(json.dumps(res), flush=True)
+    return res
 
 
 def cpu_baseline(pool0, tables_np, seq_lens_np, out, budget_s, hip, tables, seq_lens, cu, B, blocks,
@@ -812,7 +893,7 @@ def cpu_baseline(pool0, tables_np, seq_lens_np, out, budget_s, hip, tables, seq_
     from oracle.kvoracle import oracle as get_oracle
 
     ora = get_oracle()
-    cores = max(1, min(16, os.cpu_count() or 1))
+    cores, usable, nproc = host_threads()
     pool_host = pool0.cpu().numpy()
     n_tok = int(seq_lens_np.sum())
     out_host = np.empty((n_tok, W), np.uint16)
@@ -838,8 +919,8 @@ def cpu_baseline(pool0, tables_np, seq_lens_np, out, budget_s, hip, tables, seq_
                                out_host))
     if not same:
         raise SystemExit("bench: GPU gather differs from the CPU oracle at full size")
-    return {"value": round(bytes_layer / per_layer_s / 1e9, 3), "unit": "GB/s", "cores": cores,
-            "kind": "port",
+    return {"value": round(bytes_layer / per_layer_s / 1e9, 3), "unit": "GB/s", "cores": cores, "nproc": nproc,
+            "usable": usable, "kind": "port",
             "sample": f"gather+dequantize of one layer ({n_tok} tokens, same pool and block "
                       f"tables) x{reps} reps, {cores} host threads; GPU output checked equal",
             "tokens_per_s": round(n_tok / per_layer_s, 1),

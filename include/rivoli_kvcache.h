@@ -110,6 +110,20 @@ int rivoli_kv_gather_paged(const unsigned char* pool, const int* block_table,
                            int n_seqs, int max_blocks_per_seq, int width, int page_tokens,
                            int n_pages, unsigned int* bad_pages, void* stream);
 
+/* rivoli_kv_gather_paged for a caller that knows how many rows the batch holds (it sized
+ * `out` by that number): total_tokens >= the sum of seq_lens. Same results. When the batch
+ * fills less than a quarter of what its block tables could address (tables sized for a context
+ * limit far above the sequences' lengths), the launch is sized by total_tokens instead of by
+ * n_seqs * max_blocks_per_seq pages and each workgroup finds its sequence from the device-side
+ * lengths; otherwise this is rivoli_kv_gather_paged. Rows may be left out if total_tokens
+ * understates the sum. Guards as above, plus 1001 for total_tokens < 0 and 1002 when
+ * total_tokens / 4 does not fit a launch. */
+int rivoli_kv_gather_paged_packed(const unsigned char* pool, const int* block_table,
+                                  const int* seq_lens, const int* cu_seqlens, unsigned short* out,
+                                  int n_seqs, int max_blocks_per_seq, long long total_tokens,
+                                  int width, int page_tokens, int n_pages, unsigned int* bad_pages,
+                                  void* stream);
+
 /* Sparse row gather + dequantize (the `rows` argument of rivoli_mla_attend,
  * crates/backend/kernels/attn.hip:125,175): for query q < n_queries and j < n_rows[q]
  * (k when n_rows is null): out[(q*k + j)*width ..] = dequantized token rows[q*k + j] of

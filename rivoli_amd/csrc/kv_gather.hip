@@ -30,19 +30,16 @@ constexpr int kRowsPerGroup = 32;  // sparse gather: rows resolved per workgroup
 // on a compact, nearly sequential frontier of the output and run ~7% faster than one
 // workgroup per page.
 template <int W, int PT, int THREADS, int ROWS>
-__global__ __launch_bounds__(THREADS) void kv_gather_paged_kernel(
-    const uint8_t* __restrict__ pool, const int* __restrict__ block_table,
-    const int* __restrict__ seq_lens, const int* __restrict__ cu_seqlens,
-    uint16_t* __restrict__ out, int max_blocks_per_seq, int width_rt, int page_tokens_rt,
-    int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_pages) {
+__device__ __forceinline__ void gather_unit(const uint8_t* __restrict__ pool,
+                                            const int* __restrict__ block_table,
+                                            const int* __restrict__ cu_seqlens,
+                                            uint16_t* __restrict__ out, int s, int blk, int part,
+                                            int len, int max_blocks_per_seq, int width_rt,
+                                            int page_tokens_rt, int n_pages, size_t page_bytes,
+                                            unsigned int* __restrict__ bad_pages) {
     const int width = W ? W : width_rt;
     const int pt = PT ? PT : page_tokens_rt;
-    const int parts = pt / ROWS;
-    const int s = blockIdx.y;
-    const int blk = (int)blockIdx.x / parts;
-    const int part = (int)blockIdx.x - blk * parts;
     const int t0 = blk * pt + part * ROWS;
-    const int len = seq_lens[s];
     if (t0 >= len) return;
     const int valid = min(ROWS, len - t0);
     const int page = block_table[(size_t)s * max_blocks_per_seq + blk];
@@ -76,6 +73,91 @@ __global__ __launch_bounds__(THREADS) void kv_gather_paged_kernel(
             if (c < n_chunks) __builtin_nontemporal_store(dequant8_bf16(raw[u], scl[u]), dst + c);
         }
     }
+}
+
+// The grid spans what the block tables could hold: blockIdx.y = sequence, blockIdx.x = its
+// (page, part). Right when every sequence is about as long as the longest; with uneven lengths
+// most workgroups only find out that they have nothing to do.
+template <int W, int PT, int THREADS, int ROWS>
+__global__ __launch_bounds__(THREADS) void kv_gather_paged_kernel(
+    const uint8_t* __restrict__ pool, const int* __restrict__ block_table,
+    const int* __restrict__ seq_lens, const int* __restrict__ cu_seqlens,
+    uint16_t* __restrict__ out, int max_blocks_per_seq, int width_rt, int page_tokens_rt,
+    int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_pages) {
+    const int parts = (PT ? PT : page_tokens_rt) / ROWS;
+    const int s = blockIdx.y;
+    const int blk = (int)blockIdx.x / parts;
+    const int part = (int)blockIdx.x - blk * parts;
+    gather_unit<W, PT, THREADS, ROWS>(pool, block_table, cu_seqlens, out, s, blk, part, seq_lens[s],
+                                      max_blocks_per_seq, width_rt, page_tokens_rt, n_pages,
+                                      page_bytes, bad_pages);
+}
+
+// The same units on a flat grid sized by the batch's real token count: workgroup u finds the
+// sequence its unit belongs to from the device-side lengths; sequence s owns ceil(len_s / ROWS)
+// consecutive units. Up to kScalarScanSeqs sequences the lengths are walked with uniform
+// (scalar) loads, 16 at a time: those go through the scalar cache, apart from the vector memory
+// pipeline that the streaming traffic keeps full, and the table lookup that follows stays a
+// scalar load too. Longer batches scan 64 lengths per round across the lanes. No LDS, no barrier; at most n_seqs workgroups of the launch (the rounding
+// of each sequence's last unit) find nothing to do.
+constexpr int kScalarScanSeqs = 128;
+template <int W, int PT, int THREADS, int ROWS>
+__global__ __launch_bounds__(THREADS) void kv_gather_flat_kernel(
+    const uint8_t* __restrict__ pool, const int* __restrict__ block_table,
+    const int* __restrict__ seq_lens, const int* __restrict__ cu_seqlens,
+    uint16_t* __restrict__ out, int n_seqs, int max_blocks_per_seq, int width_rt,
+    int page_tokens_rt, int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_pages) {
+    const int pt = PT ? PT : page_tokens_rt;
+    const int parts = pt / ROWS;
+    const uint32_t u = blockIdx.x;
+    const int cap = max_blocks_per_seq * pt;  // rows a block-table row can address
+    uint32_t first = 0;                       // units of the sequences before s
+    int s = -1, my_len = 0;
+    if (n_seqs <= kScalarScanSeqs) {
+        for (int base = 0; base < n_seqs && s < 0; base += 16) {
+            int l[16];
+            if (base + 16 <= n_seqs) {  // one wide scalar load
+#pragma unroll
+                for (int j = 0; j < 16; ++j) l[j] = seq_lens[base + j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) l[j] = base + j < n_seqs ? seq_lens[base + j] : 0;
+            }
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int len = min(max(l[j], 0), cap);
+                const uint32_t units = (uint32_t)(len + ROWS - 1) / ROWS;
+                if (s < 0) {
+                    if (u < first + units) s = base + j, my_len = len;
+                    else first += units;
+                }
+            }
+        }
+    } else {
+        const int lane = threadIdx.x & (kWave - 1);
+        for (int s0 = 0; s0 < n_seqs; s0 += kWave) {
+            int len = 0;
+            if (s0 + lane < n_seqs) len = min(max(seq_lens[s0 + lane], 0), cap);
+            const uint32_t units = (uint32_t)(len + ROWS - 1) / ROWS;
+            const uint32_t incl = first + wave_inclusive_sum(units);
+            const int passed = __popcll(__ballot(incl <= u));  // sequences ending at or before u
+            if (passed < kWave) {
+                if (s0 + passed < n_seqs) {
+                    if (passed) first = (uint32_t)__builtin_amdgcn_readlane((int)incl, passed - 1);
+                    s = s0 + passed;
+                    my_len = __builtin_amdgcn_readlane(len, passed);
+                }
+                break;
+            }
+            first = wave_total(incl);
+        }
+    }
+    if (s < 0) return;  // past the last sequence's last unit
+    const int unit = (int)(u - first);
+    const int blk = unit / parts;
+    gather_unit<W, PT, THREADS, ROWS>(pool, block_table, cu_seqlens, out, s, blk, unit - blk * parts,
+                                      my_len, max_blocks_per_seq, width_rt, page_tokens_rt, n_pages,
+                                      page_bytes, bad_pages);
 }
 
 template <int W, int PT, int UNROLL>
@@ -123,11 +205,12 @@ __global__ void e4m3_dequant_bf16_kernel(const uint8_t* __restrict__ codes, floa
 
 }  // namespace rk
 
-extern "C" int rivoli_kv_gather_paged(const unsigned char* pool, const int* block_table,
-                                      const int* seq_lens, const int* cu_seqlens,
-                                      unsigned short* out, int n_seqs, int max_blocks_per_seq,
-                                      int width, int page_tokens, int n_pages,
-                                      unsigned int* bad_pages, void* stream) {
+// total_tokens < 0: not known, the grid spans what the block tables could hold.
+static int gather_paged_launch(const unsigned char* pool, const int* block_table,
+                               const int* seq_lens, const int* cu_seqlens, unsigned short* out,
+                               int n_seqs, int max_blocks_per_seq, long long total_tokens,
+                               int width, int page_tokens, int n_pages, unsigned int* bad_pages,
+                               void* stream) {
     using namespace rk;
     if (!pool || !block_table || !seq_lens || !cu_seqlens || !out) return 1001;
     if (n_seqs <= 0 || max_blocks_per_seq <= 0 || width <= 0 || page_tokens <= 0 || n_pages <= 0)
@@ -135,27 +218,61 @@ extern "C" int rivoli_kv_gather_paged(const unsigned char* pool, const int* bloc
     if (n_seqs > 65535) return 1002;
     if (!gather_shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
     const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
+    const long long capacity = (long long)n_seqs * max_blocks_per_seq * page_tokens;
+    // The flat grid pays for finding each workgroup's sequence (measured on MI355X at 32
+    // sequences of 1 K - 32 K rows, 578 K rows in tables that hold 1 M: 199 us against 177 us for
+    // the grid form, whose 29 K idle workgroups cost 10 us) and saves the idle workgroups, so it
+    // is taken when the block tables are mostly empty — tables sized for a context limit far
+    // above what the sequences hold.
+    const bool flat = total_tokens >= 0 && total_tokens < capacity / 4;
     (void)hipGetLastError();
-    if (width == 576 && page_tokens == 64) {
-        constexpr int kRows = 16, kThreads = 768;
-        dim3 grid((unsigned)max_blocks_per_seq * (64 / kRows), (unsigned)n_seqs);
-        hipLaunchKernelGGL((kv_gather_paged_kernel<576, 64, kThreads, kRows>), grid, dim3(kThreads),
-                           0, (hipStream_t)stream, pool, block_table, seq_lens, cu_seqlens, out,
-                           max_blocks_per_seq, width, page_tokens, n_pages, page_bytes, bad_pages);
-    } else if (page_tokens % 16 == 0) {
-        dim3 grid((unsigned)max_blocks_per_seq * (unsigned)(page_tokens / 16), (unsigned)n_seqs);
-        hipLaunchKernelGGL((kv_gather_paged_kernel<0, 0, kGatherThreads, 16>), grid,
-                           dim3(kGatherThreads), 0, (hipStream_t)stream, pool, block_table,
-                           seq_lens, cu_seqlens, out, max_blocks_per_seq, width, page_tokens,
-                           n_pages, page_bytes, bad_pages);
-    } else {
-        dim3 grid((unsigned)max_blocks_per_seq * (unsigned)(page_tokens / 4), (unsigned)n_seqs);
-        hipLaunchKernelGGL((kv_gather_paged_kernel<0, 0, kGatherThreads, 4>), grid,
-                           dim3(kGatherThreads), 0, (hipStream_t)stream, pool, block_table,
-                           seq_lens, cu_seqlens, out, max_blocks_per_seq, width, page_tokens,
-                           n_pages, page_bytes, bad_pages);
-    }
+#define RK_GATHER(WV, PTV, THREADS, FLAT_THREADS, ROWS)                                            \
+    do {                                                                                           \
+        const unsigned parts = (unsigned)(page_tokens / (ROWS));                                   \
+        if (flat) {                                                                                \
+            const long long units = (total_tokens + (ROWS) - 1) / (ROWS) + n_seqs;                 \
+            if (units > 0x7fffffffLL) return 1002;                                                 \
+            hipLaunchKernelGGL((kv_gather_flat_kernel<WV, PTV, FLAT_THREADS, ROWS>),               \
+                               dim3((unsigned)units), dim3(FLAT_THREADS), 0, (hipStream_t)stream, pool, \
+                               block_table, seq_lens, cu_seqlens, out, n_seqs, max_blocks_per_seq, \
+                               width, page_tokens, n_pages, page_bytes, bad_pages);                \
+        } else {                                                                                   \
+            hipLaunchKernelGGL((kv_gather_paged_kernel<WV, PTV, THREADS, ROWS>),                   \
+                               dim3((unsigned)max_blocks_per_seq * parts, (unsigned)n_seqs),       \
+                               dim3(THREADS), 0, (hipStream_t)stream, pool, block_table, seq_lens, \
+                               cu_seqlens, out, max_blocks_per_seq, width, page_tokens, n_pages,   \
+                               page_bytes, bad_pages);                                             \
+        }                                                                                          \
+    } while (0)
+    if (width == 576 && page_tokens == 64)
+        RK_GATHER(576, 64, 768, 384, 16);
+    else if (page_tokens % 16 == 0)
+        RK_GATHER(0, 0, kGatherThreads, kGatherThreads, 16);
+    else
+        RK_GATHER(0, 0, kGatherThreads, kGatherThreads, 4);
+#undef RK_GATHER
     return launch_status();
+}
+
+extern "C" int rivoli_kv_gather_paged(const unsigned char* pool, const int* block_table,
+                                      const int* seq_lens, const int* cu_seqlens,
+                                      unsigned short* out, int n_seqs, int max_blocks_per_seq,
+                                      int width, int page_tokens, int n_pages,
+                                      unsigned int* bad_pages, void* stream) {
+    return gather_paged_launch(pool, block_table, seq_lens, cu_seqlens, out, n_seqs,
+                               max_blocks_per_seq, -1, width, page_tokens, n_pages, bad_pages, stream);
+}
+
+extern "C" int rivoli_kv_gather_paged_packed(const unsigned char* pool, const int* block_table,
+                                             const int* seq_lens, const int* cu_seqlens,
+                                             unsigned short* out, int n_seqs,
+                                             int max_blocks_per_seq, long long total_tokens,
+                                             int width, int page_tokens, int n_pages,
+                                             unsigned int* bad_pages, void* stream) {
+    if (total_tokens < 0) return 1001;
+    return gather_paged_launch(pool, block_table, seq_lens, cu_seqlens, out, n_seqs,
+                               max_blocks_per_seq, total_tokens, width, page_tokens, n_pages,
+                               bad_pages, stream);
 }
 
 // Query q gathers its first min(n_rows[q], nr_cap) listed rows (nr_cap when n_rows is null);

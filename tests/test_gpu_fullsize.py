@@ -60,6 +60,12 @@ def test_config3_one_layer_ragged_batch32(oracle):
     n_words = int(cu[-1]) * W // 2
     assert device_fold(out, n_words) == oracle.xor_fold(want)      # one u64 for 600+ MB
     assert np.array_equal(back(out, np.uint16).reshape(-1, W), want)
+    # the launch sized by the batch's token count: the same bytes
+    out2 = dzeros(int(cu[-1]) * W * 2)
+    hip.launch_kv_gather_paged_packed(pool, dev(tables), dev(lens), dev(cu), out2, B, max_blocks,
+                                      int(cu[-1]), W, PT, n_pages)
+    assert device_fold(out2, n_words) == oracle.xor_fold(want)
+    assert np.array_equal(back(out2, np.uint16).reshape(-1, W), want)
 
 
 def test_config4_one_layer_topk_then_sparse_gather(oracle):

@@ -26,15 +26,37 @@ def build_pool(oracle, seq_lens, n_pages, seed, width=W, pt=PT, outlier_frac=0.0
 
 
 def gpu_gather(pool, tables, seq_lens, width=W, pt=PT, n_pages=None, fill=0x5A):
+    """The gather through both entry points — the grid over what the block tables could hold and
+    the one sized by the batch's token count (exact, and overstated) — which must agree byte
+    for byte, fill included."""
     seq_lens = np.asarray(seq_lens, np.int32)
     cu = np.zeros(seq_lens.size + 1, np.int32)
     np.cumsum(seq_lens, out=cu[1:])
-    out = dzeros(max(int(cu[-1]), 1) * width * 2, fill)
-    bad = dzeros(4)
     n_pages = n_pages or pool.size // (pt * (width + 4))
-    hip.launch_kv_gather_paged(dev(pool), dev(tables), dev(seq_lens), dev(cu), out, seq_lens.size,
-                               tables.shape[1], width, pt, n_pages, bad)
-    return back(out, np.uint16).reshape(-1, width), int(back(bad, np.uint32)[0])
+    pool_d, tables_d, lens_d, cu_d = dev(pool), dev(tables), dev(seq_lens), dev(cu)
+    total = int(np.minimum(np.maximum(seq_lens, 0), tables.shape[1] * pt).sum())
+    # the same tables with four times as many (unused) columns: a batch that fills less than a
+    # quarter of its tables takes the launch sized by the token count
+    wide = np.full((tables.shape[0], 4 * tables.shape[1] + 1), -1, np.int32)
+    wide[:, : tables.shape[1]] = tables
+    wide_d = dev(wide)
+    results = []
+    for form in ("grid", "packed", "packed-wide", "packed-wide+slack"):
+        out = dzeros(max(int(cu[-1]), 1) * width * 2, fill)
+        bad = dzeros(4)
+        if form == "grid":
+            hip.launch_kv_gather_paged(pool_d, tables_d, lens_d, cu_d, out, seq_lens.size,
+                                       tables.shape[1], width, pt, n_pages, bad)
+        else:
+            t_d, t = (wide_d, wide) if "wide" in form else (tables_d, tables)
+            hip.launch_kv_gather_paged_packed(pool_d, t_d, lens_d, cu_d, out, seq_lens.size, t.shape[1],
+                                              total + (37 if form.endswith("slack") else 0),
+                                              width, pt, n_pages, bad)
+        results.append((back(out, np.uint16).reshape(-1, width), int(back(bad, np.uint32)[0])))
+    for got, bad in results[1:]:
+        assert bad == results[0][1]
+        assert np.array_equal(got, results[0][0])
+    return results[0]
 
 
 def test_config1_gather_full_context(oracle):
@@ -68,6 +90,18 @@ def test_zero_length_sequences_and_untouched_tail(oracle):
     hip.launch_kv_gather_paged(dev(pool), dev(tables), dev(sl), dev(cu), out, 4, tables.shape[1],
                                W, PT, 16)
     assert np.all(back(out)[cu_total * W * 2:] == 0x5A)
+
+
+def test_many_uneven_sequences(oracle):
+    """More sequences than a wave has lanes, lengths from 0 to a few pages, block tables mostly
+    empty: the token-count-sized launch scans the lengths in several rounds."""
+    rng = np.random.default_rng(150)
+    seq_lens = [int(x) for x in rng.integers(0, 300, size=150)]
+    seq_lens[0], seq_lens[63], seq_lens[64], seq_lens[149] = 0, 299, 1, 17
+    pool, tables = build_pool(oracle, [max(n, 1) for n in seq_lens], 150 * 5 + 7, seed=150)
+    want = oracle.kv_gather_paged(pool, tables, seq_lens, W, PT)
+    got, bad = gpu_gather(pool, tables, seq_lens)
+    assert bad == 0 and np.array_equal(got, want)
 
 
 def test_gather_is_invariant_under_page_permutation(oracle):
