@@ -732,7 +732,7 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
                         "frac": round(dom_bytes / (per[rows_kernel] * 1e-3) / HBM_PEAK, 5),
                         "avg_launch_ms": round(per[rows_kernel], 5),
                         "bytes_per_launch": dom_bytes,
-                        "traffic": None}}
+                        "traffic": measured_traffic(f"dsa:b{B}:ctx{nt}:k{k}") if fused and not scored else None}}
     if not fused:
         res["topk"] = {"achieved": round(topk_bytes / (per["topk"] * 1e-3) / 1e9, 2), "unit": "GB/s",
                        "avg_launch_ms": round(per["topk"], 5), "bytes_per_launch": topk_bytes}
