@@ -195,8 +195,10 @@ int rivoli_dsa_select_gather_paged_noalloc(const float* scores, int n_queries, i
  * kcache[nt][hd]. q is [nh][hd] f32, w [nh] f32; heads (nullable) lists the nact active
  * heads, null = heads 0..nact-1. Results agree with the reference's within 1e-5 of the
  * largest score (its own test bar), not bit for bit: the dots run on the matrix cores.
- * Guards: 1001 as the reference (non-positive dims, nact > nh); 1002 nact > 64 or hd > 128
- * (the reference allows up to 1024 heads); 1004 hd % 16. Null stream. */
+ * Guards: the reference's own — 1001 non-positive dims or nact > nh; 1002 more than 1024 active
+ * heads, or (hd + the next power of two >= max(nact, 32)) * 4 > 65536. Up to 64 active heads
+ * with hd <= 128, hd % 16 == 0 and 16-byte-aligned q and kcache run on the matrix cores; every
+ * other accepted shape takes a plain f32 kernel (same bar). Null stream. */
 int rivoli_index_score(const float* q, const float* w, const unsigned short* kcache,
                        const unsigned int* heads, int nt, int nh, int nact, int hd, float wscale,
                        float dscale, float* scores);
@@ -206,7 +208,7 @@ int rivoli_index_score(const float* q, const float* w, const unsigned short* kca
  * cache kpool[n_pages*page_tokens][hd] bf16, into scores[qi*stride + t]. Tokens whose page id
  * is outside [0, n_pages) are not written. Same guards, plus 1002 for stride < nt, for
  * nt > max_blocks_per_seq * page_tokens (a scored token without a block-table entry) or for
- * n_queries > 65535, and 1004 for page_tokens % 32 (a 32-token block must sit inside one page). */
+ * n_queries > 65535. A page size that is not a multiple of 32 takes the plain f32 kernel. */
 int rivoli_index_score_paged(const float* q, const float* w, const unsigned short* kpool,
                              const int* block_table, const int* nts, const unsigned int* heads,
                              int n_queries, int max_blocks_per_seq, int stride, int nt, int nh,

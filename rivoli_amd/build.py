@@ -13,7 +13,7 @@ import sys
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(CSRC, "librivoli_kvcache.so")
 HOST_LIB_PATH = os.path.join(CSRC, "librivoli_pagepool.so")
-KERNELS = ["kv_append.hip", "kv_gather.hip", "index_topk.hip", "index_score.hip", "mla_attend.hip", "mla_attend_linear.hip",
+KERNELS = ["kv_append.hip", "kv_gather.hip", "index_topk.hip", "index_score.hip", "mla_attend.hip",
            "act_quant.hip", "kv_compress.hip", "kv_ring.hip", "gather_attn.hip", "hash_rows.hip"]
 HOST_SOURCES = ["pagepool.cpp"]
 

@@ -228,6 +228,80 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
     }
 }
 
+// Shapes outside the matrix-core kernel's limits (more than 64 active heads, a head dimension
+// above 128 or not a multiple of 16): plain f32 arithmetic, any shape the reference's launcher
+// accepts (crates/backend/kernels/indexer.hip:283-289). A wave owns a token: its key row sits
+// in registers (lane L holds dims L, L + 64, ...), every active head is one coalesced pass over
+// the query row (from LDS when the active heads fit 64 KiB, else from memory), a butterfly sum
+// and the ReLU-weighted accumulate. A workgroup of four waves walks 64 tokens.
+constexpr int kPlainTokensPerGroup = 64;
+constexpr int kPlainMaxRegs = 8;  // key dims held per lane before the row is re-read per head
+__global__ __launch_bounds__(kScoreThreads) void index_score_plain_kernel(
+    const float* __restrict__ q, const float* __restrict__ w,
+    const uint16_t* __restrict__ kpool, const int* __restrict__ block_table,
+    const int* __restrict__ nts, const unsigned int* __restrict__ heads, int max_blocks_per_seq,
+    int stride, int nt_all, int nh, int nact, int hd, int page_tokens, int n_pages, float wscale,
+    float dscale, float* __restrict__ scores, uint32_t* __restrict__ topk_ws, size_t ws_stride,
+    int q_in_lds) {
+    extern __shared__ float s_q[];  // [nact][hd] when q_in_lds
+    const int qi = blockIdx.y;
+    const int nt = nts ? min(nts[qi], nt_all) : nt_all;
+    const int t0 = (int)blockIdx.x * kPlainTokensPerGroup;
+    if (t0 >= nt) return;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    auto head_of = [&](int a) -> int {
+        const int h = heads ? (int)heads[a] : a;
+        return (unsigned)h < (unsigned)nh ? h : -1;  // a head id outside [0, nh) contributes nothing
+    };
+    if (q_in_lds) {
+        for (int i = tid; i < nact * hd; i += kScoreThreads) {
+            const int a = i / hd, h = head_of(a);
+            s_q[i] = h >= 0 ? q[((size_t)qi * nh + h) * hd + (i - a * hd)] : 0.0f;
+        }
+        __syncthreads();
+    }
+    const bool in_regs = hd <= kPlainMaxRegs * kWave;
+    for (int t = t0 + wave; t < min(t0 + kPlainTokensPerGroup, nt); t += kScoreWaves) {
+        size_t slot = (size_t)t;
+        if (block_table) {
+            const int page = block_table[(size_t)qi * max_blocks_per_seq + t / page_tokens];
+            if ((unsigned)page >= (unsigned)n_pages) continue;  // not readable: not written
+            slot = (size_t)page * page_tokens + (size_t)(t % page_tokens);
+        }
+        const uint16_t* krow = kpool + slot * hd;
+        float kreg[kPlainMaxRegs];
+#pragma unroll
+        for (int j = 0; j < kPlainMaxRegs; ++j) {
+            const int d = lane + j * kWave;
+            kreg[j] = (in_regs && d < hd) ? bf16_lo_to_f32((uint32_t)krow[d]) : 0.0f;
+        }
+        float total = 0.0f;
+        for (int a = 0; a < nact; ++a) {
+            const int h = head_of(a);
+            if (h < 0) continue;
+            const float* qrow = q_in_lds ? s_q + (size_t)a * hd : q + ((size_t)qi * nh + h) * hd;
+            float dot = 0.0f;
+            if (in_regs) {
+#pragma unroll
+                for (int j = 0; j < kPlainMaxRegs; ++j) {
+                    const int d = lane + j * kWave;
+                    if (d < hd) dot += qrow[d] * kreg[j];
+                }
+            } else {
+                for (int d = lane; d < hd; d += kWave) dot += qrow[d] * bf16_lo_to_f32((uint32_t)krow[d]);
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, kWave);
+            total += w[(size_t)qi * nh + h] * wscale * fmaxf(dot * dscale, 0.0f);
+        }
+        if (lane == 0) {
+            scores[(size_t)qi * stride + t] = total;
+            if (topk_ws) atomicAdd(&topk_ws[(size_t)qi * ws_stride + (topk_key(total) >> kLowBits)], 1u);
+        }
+    }
+}
+
 // kpool[slot*hd + i] = bf16(k[t*hd + i]); 8 elements per thread.
 __global__ __launch_bounds__(256) void index_append_paged_kernel(
     const float* __restrict__ k, const int* __restrict__ slot_mapping,
@@ -261,8 +335,14 @@ static int index_score_launch(const float* q, const float* w, const unsigned sho
     if (!q || !w || !kpool || !scores) return 1001;
     if (n_queries <= 0 || nt <= 0 || nh <= 0 || nact <= 0 || nact > nh || hd <= 0) return 1001;
     if (block_table && (max_blocks_per_seq <= 0 || page_tokens <= 0 || n_pages <= 0)) return 1001;
-    if (nact > kScoreMaxHeads || hd > kScoreMaxHd || stride < nt || n_queries > 65535) return 1002;
-    if ((hd % 16) != 0 || (block_table && (page_tokens % 32) != 0)) return 1004;
+    if (stride < nt || n_queries > 65535) return 1002;
+    {   // what the reference's launcher refuses (crates/backend/kernels/indexer.hip:283-289)
+        int bd = 32;
+        while (bd < nact) bd <<= 1;
+        if (bd > 1024 || ((size_t)hd + bd) * sizeof(float) > 65536) return 1002;
+    }
+    const bool plain = nact > kScoreMaxHeads || hd > kScoreMaxHd || (hd % 16) != 0 ||
+                       (block_table && (page_tokens % 32) != 0) || !aligned16(q) || !aligned16(kpool);
     // every scored token needs an entry in its query's block-table row
     if (block_table && (long long)nt > (long long)max_blocks_per_seq * page_tokens) return 1002;
     // the histogram is only wanted where the selection of this shape runs split over the chip
@@ -272,6 +352,17 @@ static int index_score_launch(const float* q, const float* w, const unsigned sho
     dim3 grid((unsigned)((nt + kScoreTokensPerGroup - 1) / kScoreTokensPerGroup),
               (unsigned)n_queries);
     (void)hipGetLastError();
+    if (plain) {
+        const size_t q_bytes = (size_t)nact * hd * sizeof(float);
+        const int q_in_lds = q_bytes <= 65536;
+        hipLaunchKernelGGL(index_score_plain_kernel,
+                           dim3((unsigned)((nt + kPlainTokensPerGroup - 1) / kPlainTokensPerGroup),
+                                (unsigned)n_queries),
+                           dim3(kScoreThreads), q_in_lds ? q_bytes : 0, stream, q, w, kpool, block_table,
+                           nts, heads, max_blocks_per_seq, stride, nt, nh, nact, hd, page_tokens, n_pages,
+                           wscale, dscale, scores, ws, ws_stride, q_in_lds);
+        return launch_status();
+    }
 #define RK_SCORE(RBV, HDV)                                                                      \
     hipLaunchKernelGGL((index_score_kernel<RBV, HDV>), grid, dim3(kScoreThreads), 0, stream, q, w, \
                        kpool, block_table, nts, heads, max_blocks_per_seq, stride, nt, nh, nact,  \

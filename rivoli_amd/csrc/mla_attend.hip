@@ -47,6 +47,8 @@
 // ascending order; the plan is a pure function of the call's shape and of the lengths, so
 // equal calls give bit-equal results.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
+#include <type_traits>
+
 #include "attend_common.hpp"
 
 namespace rk {
@@ -63,7 +65,9 @@ constexpr int kKrBytes = kTile * kKrRowBytes;
 constexpr int kBufs = 3;                   // LDS tiles in rotation: tile t is staged while t-2 is consumed
 constexpr int kXchBytes = 2 * kAttWaves * kWave * 8 * 4;  // partial scores, 8 f32 per lane, two parities
 constexpr int kTableLds = 1024;            // block-table entries staged per workgroup
-constexpr int kAttSmemBytes = kBufs * kKrBytes + 2 * kBufs * kTile * 4 + kXchBytes + kTableLds * 4;
+constexpr int kBlockScaleBytes = kBufs * kTile * 16;  // linear slabs: four block scales per token
+constexpr int kAttSmemBytes =
+    kBufs * kKrBytes + 2 * kBufs * kTile * 4 + kXchBytes + kTableLds * 4 + kBlockScaleBytes;
 static_assert(kAttSmemBytes + (1024 + 8 + 8) * 4 <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
 
 // Work plan. `n_splits` is a pure function of the call's shape; with more than one split the
@@ -122,6 +126,13 @@ struct AttendArgs {
     const int* n_rows;            // sparse: rows per sequence (null = k)
     int k;
     int H, max_blocks, page_tokens, n_pages;
+    int kvl, rope, row_w;         // widths of a cache row: latent, rope, and their sum (512 / 64 / 576 on the fast path)
+    // MODE == kLinear, the reference's slabs: e4m3 latent codes [t][kvl] with one f32 scale per
+    // 128 of them [t][n_blocks], and the roped key as bf16 [t][rope]
+    const uint8_t* lc8;
+    const float* lscale;
+    const uint16_t* rc;
+    int n_blocks;
     int page_shift;               // log2(page_tokens) when that is a power of two, else -1
     size_t page_bytes;
     float qscale;                 // softmax scale * log2(e)
@@ -136,17 +147,26 @@ struct AttendArgs {
 enum : int {
     kDense = 0,      // token = row position, any page size: one table lookup per token
     kSparse = 1,     // token = rows[position]: one list entry and one table lookup per token
-    kDensePaged = 2  // token = row position and page_tokens is a power of two >= the tile: a
+    kDensePaged = 2, // token = row position and page_tokens is a power of two >= the tile: a
                      // tile lies inside ONE page, so a tile costs one (scalar) table lookup
+    kLinear = 3      // the reference's linear slabs (one sequence): token = rows ? rows[position]
+                     // : position, addressed by the token index, block scales, bf16 rope
 };
+// ANY: the row widths are runtime values (kvl a multiple of 128 up to 512, rope up to 64): the
+// tile keeps its 512 + 64 layout and the dims a cache does not have are staged as zeros, so a
+// narrower cache costs the matrix cores the same as the full one. The fast path (ANY = false)
+// is the shipped 512 + 64 row.
 
 // One part of a workgroup's work: rows [r_begin, r_end) of sequence `seq`, heads 64*hb ..+63.
 // `whole`: the part is the whole sequence, so the normalised result goes straight to clat;
 // otherwise the unnormalised accumulators and (m, l) go to the partial record pa / pml.
-template <int QSPLIT, int PSPLIT, int MODE>
+template <int QSPLIT, int PSPLIT, int MODE, bool ANY>
 __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb, int r_begin,
                                                       int r_end, bool whole, float* pa, float* pml) {
     constexpr bool SPARSE = MODE == kSparse;
+    constexpr bool LINEAR = MODE == kLinear;
+    static_assert(!LINEAR || (ANY && QSPLIT == 2 && PSPLIT == 2), "the linear slabs run in the parity mode");
+    const int kvl = ANY ? a.kvl : kKvl, ropew = ANY ? a.rope : kRopeW, row_w = ANY ? a.row_w : kRowW;
     // operand fragments requested together ahead of the MFMAs that consume them: as many
     // as the register budget of two waves per SIMD (256) leaves room for
     constexpr int kFragBlock = QSPLIT == 2 ? 3 : 9;   // score side, K-steps (2 fragments each)
@@ -162,6 +182,7 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
     const lds_ptr<float> sbias = sc + kBufs * kTile;                       // [kBufs][32]
     const lds_ptr<f32x4> xch = (lds_ptr<f32x4>)(sbias + kBufs * kTile);    // [2 parities][8 waves][64 lanes][2]
     const lds_ptr<int> tbl = (lds_ptr<int>)(xch + 2 * kAttWaves * kWave * 2);
+    const lds_ptr<f32x4> sc4 = (lds_ptr<f32x4>)(tbl + kTableLds);  // [kBufs][32], linear slabs only
 
 
     const int tid = threadIdx.x;
@@ -174,10 +195,10 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
     const int n_tiles = (r_end - r_begin + kTile - 1) / kTile;
 
     // ---- block-table slice into LDS -----------------------------------------------------
-    const int* const table_g = a.block_table + (size_t)seq * a.max_blocks;
-    const int tbl_first = SPARSE ? 0 : r_begin / a.page_tokens;
+    const int* const table_g = LINEAR ? nullptr : a.block_table + (size_t)seq * a.max_blocks;
+    const int tbl_first = (SPARSE || LINEAR) ? 0 : r_begin / a.page_tokens;
     const int tbl_last = SPARSE ? a.max_blocks - 1 : min(a.max_blocks - 1, (r_end - 1) / a.page_tokens);
-    const int tbl_count = min(kTableLds, tbl_last - tbl_first + 1);
+    const int tbl_count = LINEAR ? 0 : min(kTableLds, tbl_last - tbl_first + 1);
     for (int i = tid; i < tbl_count; i += kAttThreads) tbl[i] = table_g[tbl_first + i];
 
     // ---- this wave's half of its 16 query heads as the B operand, for the whole kernel ---
@@ -185,15 +206,24 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
     {
         const int head = hb * 64 + 16 * hw + n16;
         const bool live = head < a.H;
-        const float* qa = a.qabs + ((size_t)seq * a.H + (live ? head : 0)) * kKvl + 8 * g;
-        const float* qr = a.qrope + ((size_t)seq * a.H + (live ? head : 0)) * kRopeW + 8 * g;
+        const size_t qrow = (size_t)seq * a.H + (live ? head : 0);
+        const float* qa = a.qabs + qrow * kvl + 8 * g;
+        const float* qr = a.qrope + qrow * ropew + 8 * g;
 #pragma unroll
         for (int j = 0; j < kKStepsHalf; ++j) {
             const int ks = half * kKStepsHalf + j;  // uniform: 0..8 or 9..17 (16, 17 are the rope)
-            const float4* src = reinterpret_cast<const float4*>(ks < 16 ? qa + 32 * ks : qr + 32 * (ks - 16));
-            float4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
-            if (live) v0 = src[0], v1 = src[1];
-            const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+            float v[8];
+            if constexpr (!ANY) {
+                const float4* src = reinterpret_cast<const float4*>(ks < 16 ? qa + 32 * ks : qr + 32 * (ks - 16));
+                float4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
+                if (live) v0 = src[0], v1 = src[1];
+                v[0] = v0.x, v[1] = v0.y, v[2] = v0.z, v[3] = v0.w, v[4] = v1.x, v[5] = v1.y, v[6] = v1.z, v[7] = v1.w;
+            } else {  // a dim this cache does not have multiplies a staged zero: its q is zero too
+                const float* src = ks < 16 ? qa + 32 * ks : qr + 32 * (ks - 16);
+                const int left = (ks < 16 ? kvl - 32 * ks : ropew - 32 * (ks - 16)) - 8 * g;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = (live && i < left) ? src[i] : 0.0f;
+            }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const float x = v[i] * a.qscale;
@@ -222,11 +252,12 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
         unsigned long long tile_off, tile_scale_off;  // uniform, kDensePaged
         int n_here;                                    // uniform, kDensePaged: valid rows in the tile
     };
-    const unsigned int* const rows_g = SPARSE ? a.rows + (size_t)seq * a.k : nullptr;
+    const unsigned int* const rows_g = SPARSE ? a.rows + (size_t)seq * a.k : (LINEAR ? a.rows : nullptr);
     auto row_token = [&](int tile) -> unsigned int {  // sparse: the row list entry, else the position
         if (MODE == kDensePaged) return 0;
         const int pos = r_begin + tile * kTile + tile_pos_of(wave, lane & 3);
         if (lane >= 4 || pos >= r_end) return 0xffffffffu;
+        if (LINEAR) return rows_g ? rows_g[pos] : (unsigned)pos;
         return SPARSE ? rows_g[pos] : (unsigned)pos;
     };
     auto resolve = [&](int tile, unsigned int tok, Where& w) {
@@ -241,9 +272,9 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
             const int n = min(kTile, r_end - pos0);
             if ((unsigned)page < (unsigned)a.n_pages) {
                 w.n_here = n;
-                w.tile_off = (unsigned long long)page * a.page_bytes + (unsigned long long)off * kRowW;
+                w.tile_off = (unsigned long long)page * a.page_bytes + (unsigned long long)off * row_w;
                 w.tile_scale_off = (unsigned long long)page * a.page_bytes +
-                                   (unsigned long long)a.page_tokens * kRowW + (unsigned long long)off * 4;
+                                   (unsigned long long)a.page_tokens * row_w + (unsigned long long)off * 4;
             } else if (a.bad_rows && hb == 0 && tid == 0) {
                 atomicAdd(a.bad_rows, (unsigned)n);
             }
@@ -251,40 +282,56 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
         }
         w.code_off = kNone, w.scale_off = 0;
         if (tok == 0xffffffffu) return;
+        if (LINEAR) {  // addressed by the token index itself
+            w.code_off = tok;
+            return;
+        }
         unsigned int blk, off;
         if (a.page_shift >= 0) blk = tok >> a.page_shift, off = tok & (unsigned)(a.page_tokens - 1);
         else blk = tok / (unsigned)a.page_tokens, off = tok - blk * (unsigned)a.page_tokens;
         const int page = blk < (unsigned)a.max_blocks ? table_at((int)blk) : -1;
         if ((unsigned)page < (unsigned)a.n_pages) {
             const unsigned long long pbase = (unsigned long long)page * a.page_bytes;
-            w.code_off = pbase + (unsigned long long)off * kRowW;
-            w.scale_off = pbase + (unsigned long long)a.page_tokens * kRowW + (unsigned long long)off * 4;
+            w.code_off = pbase + (unsigned long long)off * row_w;
+            w.scale_off = pbase + (unsigned long long)a.page_tokens * row_w + (unsigned long long)off * 4;
         } else if (a.bad_rows && hb == 0) {
             atomicAdd(a.bad_rows, 1u);
         }
     };
 
     u32x2 raw[4];
-    uint32_t raw_rope;
+    uint32_t raw_rope;          // four rope codes; linear slabs: raw_rope / raw_rope_hi hold four bf16
+    uint32_t raw_rope_hi = 0;
     float raw_scale, raw_bias;  // lanes 0..3
+    f32x4 raw_scale4 = {0, 0, 0, 0};  // linear slabs, lanes 0..3: the token's block scales
     const int my_pos0 = tile_pos_of(wave, 0);  // the wave's 4 tokens are consecutive tile positions
+    // ANY: a lane whose chunk lies past the row's latent (rope) width loads the row's first
+    // chunk instead and discards it: no branch sits between the loads of a tile
+    const bool lat_ok = !ANY || 8 * lane < kvl;
+    const bool rope_ok = !ANY || 4 * (lane & 15) < ropew;
+    const int lat_at = lat_ok ? 8 * lane : 0, rope_at = kvl + (rope_ok ? 4 * (lane & 15) : 0);
     auto issue_loads = [&](const Where& w) {
         if (MODE == kDensePaged) {
-            const uint8_t* const base = a.pool + w.tile_off + (size_t)my_pos0 * kRowW;
+            const uint8_t* const base = a.pool + w.tile_off + (size_t)my_pos0 * row_w;
             if (my_pos0 + 3 < w.n_here) {  // the common case: all four rows are there
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    raw[i] = *reinterpret_cast<const u32x2*>(base + i * kRowW + 8 * lane);
-                raw_rope = *reinterpret_cast<const uint32_t*>(base + (lane >> 4) * kRowW + kKvl + 4 * (lane & 15));
+                    raw[i] = *reinterpret_cast<const u32x2*>(base + i * row_w + lat_at);
+                raw_rope = *reinterpret_cast<const uint32_t*>(base + (lane >> 4) * row_w + rope_at);
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     raw[i] = u32x2{0, 0};
-                    if (my_pos0 + i < w.n_here) raw[i] = *reinterpret_cast<const u32x2*>(base + i * kRowW + 8 * lane);
+                    if (my_pos0 + i < w.n_here) raw[i] = *reinterpret_cast<const u32x2*>(base + i * row_w + lat_at);
                 }
                 raw_rope = 0;
                 if (my_pos0 + (lane >> 4) < w.n_here)
-                    raw_rope = *reinterpret_cast<const uint32_t*>(base + (lane >> 4) * kRowW + kKvl + 4 * (lane & 15));
+                    raw_rope = *reinterpret_cast<const uint32_t*>(base + (lane >> 4) * row_w + rope_at);
+            }
+            if (ANY) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) raw[i] = lat_ok ? raw[i] : u32x2{0, 0};
+                raw_rope = rope_ok ? raw_rope : 0u;
             }
             raw_scale = 0.0f, raw_bias = -INFINITY;
             if (lane < 4 && my_pos0 + lane < w.n_here) {
@@ -294,16 +341,45 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
             return;
         }
         const uint32_t lo = (uint32_t)w.code_off, hi = (uint32_t)(w.code_off >> 32);
+        if constexpr (LINEAR) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t blo = __builtin_amdgcn_readlane(lo, i), bhi = __builtin_amdgcn_readlane(hi, i);
+                const unsigned long long t = ((unsigned long long)bhi << 32) | blo;
+                raw[i] = u32x2{0, 0};
+                if (t != kNone && lat_ok) raw[i] = *reinterpret_cast<const u32x2*>(a.lc8 + t * kvl + 8 * lane);
+            }
+            // the roped key is bf16 already: four values per lane, read one by one (any width, any alignment)
+            const unsigned long long tr = __shfl(w.code_off, lane >> 4, kWave);
+            uint32_t r4[4] = {0, 0, 0, 0};
+            if (tr != kNone) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int d = 4 * (lane & 15) + e;
+                    if (d < ropew) r4[e] = a.rc[tr * ropew + d];
+                }
+            }
+            raw_rope = r4[0] | (r4[1] << 16), raw_rope_hi = r4[2] | (r4[3] << 16);
+            raw_scale = 0.0f, raw_bias = -INFINITY, raw_scale4 = f32x4{0, 0, 0, 0};
+            if (lane < 4 && w.code_off != kNone) {
+                const float* sp = a.lscale + w.code_off * a.n_blocks;
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    if (128 * b < kvl) raw_scale4[b] = sp[b];
+                raw_scale = 1.0f, raw_bias = 0.0f;
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t blo = __builtin_amdgcn_readlane(lo, i), bhi = __builtin_amdgcn_readlane(hi, i);
             const unsigned long long b = ((unsigned long long)bhi << 32) | blo;
             raw[i] = u32x2{0, 0};
-            if (b != kNone) raw[i] = *reinterpret_cast<const u32x2*>(a.pool + b + 8 * lane);
+            if (b != kNone && lat_ok) raw[i] = *reinterpret_cast<const u32x2*>(a.pool + b + 8 * lane);
         }
         const unsigned long long br = __shfl(w.code_off, lane >> 4, kWave);
         raw_rope = 0;
-        if (br != kNone) raw_rope = *reinterpret_cast<const uint32_t*>(a.pool + br + kKvl + 4 * (lane & 15));
+        if (br != kNone && rope_ok) raw_rope = *reinterpret_cast<const uint32_t*>(a.pool + br + kvl + 4 * (lane & 15));
         raw_scale = 0.0f, raw_bias = -INFINITY;
         if (lane < 4 && w.code_off != kNone) {
             raw_scale = *reinterpret_cast<const float*>(a.pool + w.scale_off);
@@ -320,9 +396,11 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
             *(lds_ptr<u32x4>)(krb + (my_pos0 + i) * kKrRowBytes + 16 * lane) = u32x4{r[0], r[1], r[2], r[3]};
         }
         uint32_t rr0, rr1;
-        e4m3x4_to_bf16(raw_rope, rr0, rr1);
+        if constexpr (LINEAR) rr0 = raw_rope, rr1 = raw_rope_hi;
+        else e4m3x4_to_bf16(raw_rope, rr0, rr1);
         *(lds_ptr<u32x2>)(krb + (my_pos0 + (lane >> 4)) * kKrRowBytes + kKvl * 2 + 8 * (lane & 15)) =
             u32x2{rr0, rr1};
+        if (LINEAR && lane < 4) sc4[buf * kTile + 4 * wave + lane] = raw_scale4;
         if (lane < 4) {
             // a scale that is not a positive number cannot come from the append: such a
             // token is left out like one that is not there
@@ -368,11 +446,47 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
         const lds_ptr<bf16x8> a0p = (lds_ptr<bf16x8>)(krb + n16 * kKrRowBytes + 16 * g);
         const lds_ptr<bf16x8> a1p = (lds_ptr<bf16x8>)(krb + (16 + n16) * kKrRowBytes + 16 * g);
         f32x4 s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0};
+        if constexpr (LINEAR) {
+            // One scale per token AND per 128 latent dims: each block's dots are folded into the
+            // running score with that block's scales before the next block starts; the roped
+            // dims (K-steps 16, 17) carry no scale. Which K-steps close a block depends on the
+            // half of the dims this wave owns, so the loop is written once per half.
+            f32x4 t0 = {0, 0, 0, 0}, t1 = {0, 0, 0, 0};
+            auto run = [&](auto half_c) {
+                constexpr int HF = decltype(half_c)::value;
+#pragma unroll
+                for (int j = 0; j < kKStepsHalf; ++j) {
+                    const bf16x8 f0 = a0p[j * 4], f1 = a1p[j * 4];
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, qh[j], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1, qh[j], s1, 0, 0, 0);
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, ql[j], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1, ql[j], s1, 0, 0, 0);
+                    const int ks = HF * kKStepsHalf + j;
+                    const int blk = ks < 16 ? ks / 4 : 4;
+                    const int blk_next = j + 1 == kKStepsHalf ? -1 : (ks + 1 < 16 ? (ks + 1) / 4 : 4);
+                    if (blk_next != blk) {
+                        if (blk < 4) {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) {
+                                t0[i] += s0[i] * sc4[buf * kTile + 8 * g + i][blk];
+                                t1[i] += s1[i] * sc4[buf * kTile + 8 * g + 4 + i][blk];
+                            }
+                        } else {
+                            t0 += s0, t1 += s1;
+                        }
+                        s0 = f32x4{0, 0, 0, 0}, s1 = f32x4{0, 0, 0, 0};
+                    }
+                }
+            };
+            if (half == 0) run(std::integral_constant<int, 0>{});
+            else run(std::integral_constant<int, 1>{});
+            s0 = t0, s1 = t1;
+        }
         // The operand fragments of a block of K-steps are all requested before the first MFMA
         // of the block; left alone the compiler keeps two reads in flight and every pair of
         // MFMAs then waits out a full LDS round trip.
 #pragma unroll
-        for (int j0 = 0; j0 < kKStepsHalf; j0 += kFragBlock) {
+        for (int j0 = 0; j0 < (LINEAR ? 0 : kKStepsHalf); j0 += kFragBlock) {
             bf16x8 fa0[kFragBlock], fa1[kFragBlock];
 #pragma unroll
             for (int i = 0; i < kFragBlock; ++i) fa0[i] = a0p[(j0 + i) * 4], fa1[i] = a1p[(j0 + i) * 4];
@@ -454,10 +568,19 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
         // magnitude, and vanishes when one token holds the whole softmax. Carried as
         // hi + lo the weights are good to 2^-17 and the denominator sums p_t itself.
         bf16x8 p, p_lo;
+        bf16x8 p2, p2_lo;  // linear slabs: the weights under the scales of the wave's second column block
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const float e = __builtin_amdgcn_exp2f(v[i] - mu);  // not there -> 0
-            const float x = e * scl[i];
+            float x = e * scl[i];
+            if constexpr (LINEAR) {  // columns 256*half .. +127 and +128 .. +255 are blocks 2*half, 2*half + 1
+                const f32x4 s4 = sc4[buf * kTile + 8 * g + i];
+                x = e * (half ? s4[2] : s4[0]);
+                const float x2 = e * (half ? s4[3] : s4[1]);
+                const __bf16 w2 = (__bf16)x2;
+                p2[i] = w2;
+                p2_lo[i] = (__bf16)(x2 - (float)w2);
+            }
             const __bf16 w = (__bf16)x;
             p[i] = w;
             if (PSPLIT == 2) {
@@ -478,9 +601,10 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
             }
 #pragma unroll
             for (int i = 0; i < kValueAhead; ++i) {
-                o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p, fb[i], o[n0 + i], 0, 0, 0);
+                const bool second = LINEAR && n0 + i >= kColTilesHalf / 2;  // known when unrolled
+                o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(second ? p2 : p, fb[i], o[n0 + i], 0, 0, 0);
                 if (PSPLIT == 2)
-                    o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_lo, fb[i], o[n0 + i], 0, 0, 0);
+                    o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(second ? p2_lo : p_lo, fb[i], o[n0 + i], 0, 0, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -523,15 +647,16 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
             const int head = head0 + 4 * g + i;
             const float inv = l_h[i] > 0.0f ? 1.0f / l_h[i] : 0.0f;
             if (head < a.H) {
-                float* const dst = a.clat + ((size_t)seq * a.H + head) * kKvl;
+                float* const dst = a.clat + ((size_t)seq * a.H + head) * kvl;
 #pragma unroll
-                for (int nt = 0; nt < kColTilesHalf; ++nt) dst[col0 + 16 * nt] = o[nt][i] * inv;
+                for (int nt = 0; nt < kColTilesHalf; ++nt)
+                    if (!ANY || col0 + 16 * nt < kvl) dst[col0 + 16 * nt] = o[nt][i] * inv;
             }
         }
     }
 }
 
-template <int QSPLIT, int PSPLIT, int MODE>
+template <int QSPLIT, int PSPLIT, int MODE, bool ANY>
 __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const AttendArgs a) {
     __shared__ int pre[kDealMaxSeqs + 8];  // tiles before each sequence, when dealing
     __shared__ int wave_total[kAttWaves];
@@ -542,6 +667,7 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     auto attended = [&](int s) -> int {
+        if (MODE == kLinear) return a.k;
         if (SPARSE) return a.n_rows ? max(min(a.n_rows[s], a.k), 0) : a.k;
         return max(min(a.seq_lens[s], a.k), 0);
     };
@@ -606,14 +732,15 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         r_end = attended(seq);
         if (r_end <= 0) {
             // a sequence with nothing to attend gets zeros, like the reference's `l > 0 ? 1/l : 0`
-            for (int i = tid; i < 64 * kKvl; i += kAttThreads) {
-                const int h = hb * 64 + i / kKvl;
-                if (h < a.H) a.clat[((size_t)seq * a.H + h) * kKvl + (i % kKvl)] = 0.0f;
+            const int kvl = ANY ? a.kvl : kKvl;
+            for (int i = tid; i < 64 * kvl; i += kAttThreads) {
+                const int h = hb * 64 + i / kvl;
+                if (h < a.H) a.clat[((size_t)seq * a.H + h) * kvl + (i % kvl)] = 0.0f;
             }
             return;
         }
     }
-    attend_part<QSPLIT, PSPLIT, MODE>(a, seq, hb, r_begin, r_end, whole, pa, pml);
+    attend_part<QSPLIT, PSPLIT, MODE, ANY>(a, seq, hb, r_begin, r_end, whole, pa, pml);
     if (a.n_items == 0) break;
   }  // parts of this workgroup
 }
@@ -624,14 +751,14 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
 // whole was written by it directly; one with nothing to attend gets zeros.
 __global__ __launch_bounds__(128) void mla_attend_combine_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, const int* __restrict__ seq_lens,
-    const int* __restrict__ n_rows, int sparse, int k, int n_seqs, int n_items, int H,
+    const int* __restrict__ n_rows, int sparse, int k, int n_seqs, int n_items, int H, int kvl,
     float* __restrict__ clat) {
     __shared__ long long s_sum[3][2];  // per wave: tiles before seq, tiles of seq .. end
     const int head = blockIdx.x, seq = blockIdx.y;
     // tiles before this sequence, of this sequence, and in all
     long long before = 0, mine = 0, total = 0;
     for (int s = threadIdx.x; s < n_seqs; s += 128) {
-        int n = sparse ? (n_rows ? min(n_rows[s], k) : k) : min(seq_lens[s], k);
+        int n = (sparse || !seq_lens) ? (n_rows ? min(n_rows[s], k) : k) : min(seq_lens[s], k);
         n = max(n, 0);
         const long long t = (n + kTile - 1) / kTile;
         total += t;
@@ -650,7 +777,8 @@ __global__ __launch_bounds__(128) void mla_attend_combine_kernel(
     }
     __syncthreads();
     before = s_sum[0][0] + s_sum[0][1], mine = s_sum[1][0] + s_sum[1][1], total = s_sum[2][0] + s_sum[2][1];
-    float4* const dst = reinterpret_cast<float4*>(clat + ((size_t)seq * H + head) * kKvl) + threadIdx.x;
+    if (4 * (int)threadIdx.x >= kvl) return;  // the records are 512 wide whatever the cache's width
+    float4* const dst = reinterpret_cast<float4*>(clat + ((size_t)seq * H + head) * kvl) + threadIdx.x;
     if (mine == 0) {
         *dst = float4{0, 0, 0, 0};
         return;
@@ -678,7 +806,35 @@ __global__ __launch_bounds__(128) void mla_attend_combine_kernel(
     *dst = float4{sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv};
 }
 
+// What both launchers share once the arguments are in place: the attention kernel of the right
+// mode, then the merge of the partial records when the plan has any.
+template <int MODE>
+static int attend_launch(const AttendArgs& a, const AttendPlan& plan, int n_seqs, int max_rows, bool any,
+                         int precise, const int* seq_lens, const int* n_rows, bool listed, hipStream_t st) {
+    const dim3 grid(plan.n_items ? (unsigned)plan.n_items : 1u, plan.n_items ? 1u : (unsigned)n_seqs,
+                    (unsigned)((a.H + 63) / 64));
+    (void)hipGetLastError();
+    // A cache of other widths than 512 + 64 always runs in the parity mode.
+    if (any || MODE == kLinear)
+        hipLaunchKernelGGL((mla_attend_paged_kernel<2, 2, MODE, true>), grid, dim3(kAttThreads), 0, st, a);
+    else if constexpr (MODE != kLinear) {
+        if (precise >= 2)
+            hipLaunchKernelGGL((mla_attend_paged_kernel<2, 2, MODE, false>), grid, dim3(kAttThreads), 0, st, a);
+        else if (precise == 1)
+            hipLaunchKernelGGL((mla_attend_paged_kernel<2, 1, MODE, false>), grid, dim3(kAttThreads), 0, st, a);
+        else
+            hipLaunchKernelGGL((mla_attend_paged_kernel<1, 1, MODE, false>), grid, dim3(kAttThreads), 0, st, a);
+    }
+    const int rc = launch_status();
+    if (rc != 0 || plan.n_splits <= 1) return rc;
+    hipLaunchKernelGGL(mla_attend_combine_kernel, dim3((unsigned)a.H, (unsigned)n_seqs), dim3(128), 0, st,
+                       a.part_acc, a.part_ml, seq_lens, n_rows, listed ? 1 : 0, max_rows, n_seqs, plan.n_items,
+                       a.H, a.kvl, a.clat);
+    return launch_status();
+}
+
 }  // namespace rk
+
 
 extern "C" size_t rivoli_mla_attend_paged_scratch_floats(int n_seqs, int H, int max_rows) {
     if (n_seqs <= 0 || H <= 0 || max_rows <= 0) return 0;
@@ -700,43 +856,123 @@ extern "C" int rivoli_mla_attend_paged(const float* qabs, const float* qrope,
         page_tokens <= 0 || n_pages <= 0)
         return 1001;
     if (n_seqs > 65535 || H > 64 * 65535) return 1002;
-    if (kvl != kKvl || rope != kRopeW) return 1004;  // the page row is 512 latent + 64 rope codes
+    // the latent width as the reference's launcher has it (crates/backend/kernels/attn.hip:
+    // 284-293: a multiple of 128 up to 512); the rope codes fill at most two 32-wide steps
+    if (kvl > kKvl || (kvl % 128) != 0 || rope > kRopeW || (rope % 8) != 0) return 1004;
     if (!aligned16(qabs) || !aligned16(qrope) || !aligned16(pool) || !aligned16(clat) || !aligned16(partial))
         return 1004;
     const AttendPlan plan = attend_plan(n_seqs, H, max_rows);
     if (plan.n_splits > 1 && !partial) return 1001;
-    AttendArgs a;
+    AttendArgs a = {};
     a.qabs = qabs, a.qrope = qrope, a.pool = pool, a.block_table = block_table;
     a.seq_lens = seq_lens, a.rows = rows, a.n_rows = n_rows, a.k = max_rows;
     a.H = H, a.max_blocks = max_blocks_per_seq, a.page_tokens = page_tokens, a.n_pages = n_pages;
+    a.kvl = kvl, a.rope = rope, a.row_w = kvl + rope;
     a.page_shift = (page_tokens & (page_tokens - 1)) == 0 ? __builtin_ctz((unsigned)page_tokens) : -1;
-    a.page_bytes = (size_t)page_tokens * kRowW + (size_t)page_tokens * 4;
+    a.page_bytes = (size_t)page_tokens * a.row_w + (size_t)page_tokens * 4;
     a.qscale = scale * kLog2e;
     a.n_seqs = n_seqs, a.n_items = plan.n_items;
     a.clat = clat, a.bad_rows = bad_rows;
     a.part_acc = plan.n_items ? partial : nullptr;
     a.part_ml = plan.n_items ? partial + (size_t)plan.n_records * H * kKvl : nullptr;
-    const dim3 grid(plan.n_items ? (unsigned)plan.n_items : 1u, plan.n_items ? 1u : (unsigned)n_seqs,
-                    (unsigned)((H + 63) / 64));
-    (void)hipGetLastError();
+    const bool any = kvl != kKvl || rope != kRopeW;
     hipStream_t st = (hipStream_t)stream;
-#define RK_ATTEND_LAUNCH(Q, P, M) \
-    hipLaunchKernelGGL((mla_attend_paged_kernel<Q, P, M>), grid, dim3(kAttThreads), 0, st, a)
-#define RK_ATTEND_MODES(M)                          \
-    do {                                            \
-        if (precise >= 2) RK_ATTEND_LAUNCH(2, 2, M); \
-        else if (precise == 1) RK_ATTEND_LAUNCH(2, 1, M); \
-        else RK_ATTEND_LAUNCH(1, 1, M);             \
-    } while (0)
-    if (rows) RK_ATTEND_MODES(kSparse);
-    else if (a.page_shift >= 0 && page_tokens >= kTile) RK_ATTEND_MODES(kDensePaged);
-    else RK_ATTEND_MODES(kDense);
-#undef RK_ATTEND_MODES
-#undef RK_ATTEND_LAUNCH
-    int rc = launch_status();
-    if (rc != 0 || plan.n_splits <= 1) return rc;
-    hipLaunchKernelGGL(mla_attend_combine_kernel, dim3((unsigned)H, (unsigned)n_seqs), dim3(128), 0, st,
-                       a.part_acc, a.part_ml, seq_lens, n_rows, rows ? 1 : 0, max_rows, n_seqs, plan.n_items, H,
-                       clat);
-    return launch_status();
+    if (rows) return attend_launch<kSparse>(a, plan, n_seqs, max_rows, any, precise, seq_lens, n_rows, true, st);
+    if (a.page_shift >= 0 && page_tokens >= kTile)
+        return attend_launch<kDensePaged>(a, plan, n_seqs, max_rows, any, precise, seq_lens, n_rows, false, st);
+    return attend_launch<kDense>(a, plan, n_seqs, max_rows, any, precise, seq_lens, n_rows, false, st);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The reference's single-token launcher over its linear slabs, signature and guards kept
+// (crates/backend/kernels/attn.hip:95-103,279-308): latent e4m3 codes with one f32 scale per
+// 128 values, the roped key as bf16, token = rows ? rows[j] : j for j < nr. The same kernel as
+// above with a third address mode: the caller's scratch (sized by the reference's rule,
+// 16 * H * (kvl + 2) floats) holds as many 512-wide partial records as fit it.
+// ---------------------------------------------------------------------------------------------
+namespace rk {
+constexpr int kRefMaxSplits = 16;  // what rivoli_mla_attend_scratch_floats prices (attn.hip:66,98-103)
+
+// Shapes the tile kernel does not take (a roped key wider than 64, slabs that are not 8-byte
+// aligned): a wave per head walks the rows one at a time, lanes over the dims, online softmax.
+__global__ __launch_bounds__(256) void mla_attend_rowwise_kernel(
+    const float* __restrict__ qabs, const float* __restrict__ qrope, const uint8_t* __restrict__ lc8,
+    const float* __restrict__ lscale, const uint16_t* __restrict__ rc, const unsigned int* __restrict__ rows,
+    int H, int nr, int kvl, int rope, int n_blocks, float qscale, float* __restrict__ clat) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int head = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (head >= H) return;
+    const float* qa = qabs + (size_t)head * kvl;
+    const float* qr = qrope + (size_t)head * rope;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // columns lane, lane + 64, ... (kvl <= 512)
+    float m = -INFINITY, l = 0.0f;
+    for (int j = 0; j < nr; ++j) {
+        const size_t t = rows ? rows[j] : (unsigned)j;
+        float lat[8], dot = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const int i = lane + c * kWave;
+            lat[c] = 0.0f;
+            if (i < kvl)
+                lat[c] = __builtin_amdgcn_cvt_pk_f32_fp8((uint32_t)lc8[t * kvl + i], false)[0] * lscale[t * n_blocks + i / 128];
+            if (i < kvl) dot += qa[i] * lat[c];
+        }
+        for (int i = lane; i < rope; i += kWave) dot += qr[i] * bf16_lo_to_f32((uint32_t)rc[t * rope + i]);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, kWave);
+        const float sv = dot * qscale;  // log2 units
+        const float m_new = fmaxf(m, sv);
+        const float corr = exp2f(m - m_new), pw = exp2f(sv - m_new);
+        l = l * corr + pw;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc[c] = acc[c] * corr + pw * lat[c];
+        m = m_new;
+    }
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int i = lane + c * kWave;
+        if (i < kvl) clat[(size_t)head * kvl + i] = acc[c] * inv;
+    }
+}
+}  // namespace rk
+
+extern "C" size_t rivoli_mla_attend_scratch_floats(int H, int kvl) {
+    if (H <= 0 || kvl <= 0) return 0;
+    return (size_t)rk::kRefMaxSplits * (size_t)H * ((size_t)kvl + 2);
+}
+
+extern "C" int rivoli_mla_attend(const float* qabs, const float* qrope, const unsigned char* Lc8,
+                                 const float* Lscale, const unsigned short* Rc,
+                                 const unsigned int* rows, int H, int nr, int kvl, int rope,
+                                 int n_blocks, float scale, float* clat, float* partial) {
+    using namespace rk;
+    if (H <= 0 || nr <= 0 || kvl <= 0 || rope <= 0 || n_blocks <= 0) return 1001;
+    if (((size_t)kvl + rope) * 16 * sizeof(float) > 65536) return 1002;  // the reference's LDS bound
+    if (kvl > kKvl || kvl % 128) return 1004;
+    if (!qabs || !qrope || !Lc8 || !Lscale || !Rc || !clat) return 1001;
+    (void)hipGetLastError();
+    if (rope > kRopeW || (reinterpret_cast<uintptr_t>(Lc8) & 7u) != 0 || H > 64 * 65535) {
+        hipLaunchKernelGGL(mla_attend_rowwise_kernel, dim3((unsigned)((H + 3) / 4)), dim3(256), 0, nullptr, qabs,
+                           qrope, Lc8, Lscale, Rc, rows, H, nr, kvl, rope, n_blocks, scale * kLog2e, clat);
+        return launch_status();
+    }
+    // split plan: as the batched launcher's for one sequence, capped by what the scratch holds
+    AttendPlan plan = attend_plan(1, H, nr);
+    const int fit = (int)((size_t)kRefMaxSplits * ((size_t)kvl + 2) / (kKvl + 2)) - 1;  // records - 1
+    if (plan.n_splits > fit) plan.n_splits = fit;
+    if (!partial || plan.n_splits < 2) plan.n_splits = 1;
+    plan.n_items = plan.n_splits > 1 ? plan.n_splits : 0;
+    plan.n_records = plan.n_items ? plan.n_items + 1 : 0;
+    AttendArgs a = {};
+    a.qabs = qabs, a.qrope = qrope, a.rows = rows, a.k = nr, a.H = H;
+    a.lc8 = Lc8, a.lscale = Lscale, a.rc = Rc, a.n_blocks = n_blocks;
+    a.kvl = kvl, a.rope = rope, a.row_w = kvl + rope;
+    a.max_blocks = 1, a.page_tokens = 1, a.n_pages = 1, a.page_shift = 0, a.page_bytes = 0;
+    a.qscale = scale * kLog2e;
+    a.n_seqs = 1, a.n_items = plan.n_items;
+    a.clat = clat;
+    a.part_acc = plan.n_items ? partial : nullptr;
+    a.part_ml = plan.n_items ? partial + (size_t)plan.n_records * H * kKvl : nullptr;
+    return attend_launch<kLinear>(a, plan, 1, nr, true, 2, nullptr, nullptr, rows != nullptr, nullptr);
 }

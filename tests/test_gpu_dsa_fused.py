@@ -122,11 +122,12 @@ def test_select_gather_guards(oracle):
         assert e.value.code == code, kw
 
 
-def test_score_kernel_fills_the_selection_histogram(oracle):
+@pytest.mark.parametrize("nh", [32, 72])
+def test_score_kernel_fills_the_selection_histogram(oracle, nh):
     """index_score_paged_hist -> select (hist_ready) gives the rows that the plain score kernel
     followed by the full selection gives on the same device scores, and the oracle's rows for
-    those scores."""
-    hd, pt, nh, nt, k, n_q = 128, 64, 32, 20000, 700, 3
+    those scores. 72 heads are past the matrix-core kernel: the f32 kernel fills the histogram."""
+    hd, pt, nt, k, n_q = 128, 64, 20000, 700, 3
     rng = np.random.default_rng(31)
     blocks = -(-nt // pt)
     n_pages = n_q * blocks

@@ -51,7 +51,13 @@ def test_index_score_head_weights_land_on_the_right_heads(oracle):
 
 
 @pytest.mark.parametrize("nt,nh,nact,hd", [(1, 8, 8, 16), (31, 32, 32, 64), (33, 32, 17, 128),
-                                           (513, 64, 64, 128), (2000, 40, 33, 96), (512, 4, 4, 32)])
+                                           (513, 64, 64, 128), (2000, 40, 33, 96), (512, 4, 4, 32),
+                                           # beyond the matrix-core kernel: more than 64 active heads,
+                                           # wider heads, a width that is not a multiple of 16, and
+                                           # the reference's own upper limits (1024 heads; 64 KiB of LDS)
+                                           (300, 128, 128, 128), (200, 8, 8, 256), (100, 8, 5, 24),
+                                           (70, 100, 65, 40), (9, 1024, 1024, 16), (5, 4, 4, 16000),
+                                           (130, 200, 200, 128)])
 def test_index_score_shapes(oracle, nt, nh, nact, hd):
     rng = np.random.default_rng(nt)
     q = rng.standard_normal((nh, hd), dtype=np.float32)
@@ -66,7 +72,7 @@ def test_index_score_shapes(oracle, nt, nh, nact, hd):
 def test_index_score_guards():
     b = dzeros(1 << 16)
     for args, code in (((0, 8, 8, 16), 1001), ((4, 8, 9, 16), 1001), ((4, 0, 0, 16), 1001),
-                       ((4, 128, 65, 16), 1002), ((4, 8, 8, 256), 1002), ((4, 8, 8, 24), 1004)):
+                       ((4, 2048, 1025, 16), 1002), ((4, 8, 8, 16384), 1002)):     # the reference's own limits
         with pytest.raises(hip.LaunchError) as e:
             hip.launch_index_score(b, b, b, None, *args, 1.0, 1.0, b)
         assert e.value.code == code, args
@@ -76,13 +82,15 @@ def test_index_score_guards():
     assert e.value.code == 1002
 
 
-def test_paged_index_append_and_score(oracle):
+@pytest.mark.parametrize("pt,n_pages,blocks,nh", [(64, 40, 12, 32), (16, 160, 48, 32), (64, 40, 12, 96)])
+def test_paged_index_append_and_score(oracle, pt, n_pages, blocks, nh):
     """Keys appended through a slot mapping into a fragmented pool, then scored through the
-    block tables for three queries of different lengths."""
-    hd, pt, n_pages, nh = 128, 64, 40, 32
+    block tables for three queries of different lengths (pages of 16 tokens and 96 heads take
+    the plain kernel)."""
+    hd = 128
     rng = np.random.default_rng(8)
     nts = np.array([760, 64, 300], np.int32)
-    tables = rng.permutation(n_pages)[:36].reshape(3, 12).astype(np.int32)
+    tables = rng.permutation(n_pages)[:3 * blocks].reshape(3, blocks).astype(np.int32)
     q = rng.standard_normal((3, nh, hd), dtype=np.float32)
     w = rng.standard_normal((3, nh), dtype=np.float32)
     want_pool = np.full((n_pages * pt, hd), 0x1234, np.uint16)
@@ -101,7 +109,7 @@ def test_paged_index_append_and_score(oracle):
     assert np.array_equal(back(kpool, np.uint16).reshape(-1, hd), want_pool)   # bit-exact keys
     stride = 768
     out = dzeros(3 * stride * 4, 0x7F)
-    hip.launch_index_score_paged(dev(q), dev(w), kpool, dev(tables), dev(nts), None, 3, 12, stride,
+    hip.launch_index_score_paged(dev(q), dev(w), kpool, dev(tables), dev(nts), None, 3, blocks, stride,
                                  stride, nh, nh, hd, pt, n_pages, 0.75, 0.125, out)
     got = back(out, np.float32).reshape(3, stride)
     want = oracle.index_score_paged(q, w, want_pool, tables, nts, None, stride, hd, pt, 0.75, 0.125,
