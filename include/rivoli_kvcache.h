@@ -402,7 +402,7 @@ typedef struct rivoli_comp_finish {
  * the derived values), 1004 (ents > 128), 1010 (overlap and ratio disagree); 1001 null buffer;
  * 1005 s <= 0; 1008 slot0 out of range. */
 int rivoli_kv_compress_deposit(const float* kv, const float* score, const float* ape,
-                               float* kv_state, float* score_state, const rivoli_comp_geom* p,
+                               float* kv_state, float* score_state, const rivoli_comp_geom* pp,
                                int s, int slot0, void* stream);
 
 /* Replaces kvcompress.hip:439-456. For block b < nblk: per feature, softmax over the window's
@@ -412,15 +412,15 @@ int rivoli_kv_compress_deposit(const float* kv, const float* score, const float*
  * bf16 store, rotation of adjacent pairs of the last rd dims at position b * ratio, bf16 store;
  * out[b][d] holds bf16 values in f32. Codes as above, plus 1002 d > 8192, 1006 nblk <= 0. */
 int rivoli_kv_compress_prefill(const float* kv, const float* score, const float* ape,
-                               const rivoli_comp_finish* f, const rivoli_comp_geom* p, int nblk,
+                               const rivoli_comp_finish* ff, const rivoli_comp_geom* pp, int nblk,
                                void* stream);
 
-/* Replaces kvcompress.hip:458-478. Pools the completed window out of the state into f->out[d]
+/* Replaces kvcompress.hip:458-478. Pools the completed window out of the state into ff->out[d]
  * (rotated at the block's first position, (start_pos / ratio) * ratio), then slides the window
  * on overlapping layers. One workgroup. Codes as above, plus 1007 start_pos <= 0 and 1009 when
  * start_pos + 1 is not a multiple of ratio. */
-int rivoli_kv_compress_decode(float* kv_state, float* score_state, const rivoli_comp_finish* f,
-                              const rivoli_comp_geom* p, int start_pos, void* stream);
+int rivoli_kv_compress_decode(float* kv_state, float* score_state, const rivoli_comp_finish* ff,
+                              const rivoli_comp_geom* pp, int start_pos, void* stream);
 
 /* Element codecs as launchers (what formats.hpp:42-57,99-106 and fwd.hip:20-45 are to the
  * reference's kernels), for census tests of the device codecs on arbitrary inputs:

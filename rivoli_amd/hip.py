@@ -76,6 +76,16 @@ _SIGNATURES = {
 }
 
 
+# the sizing functions: pure host arithmetic, size_t results
+_SIZE_SIGNATURES = {
+    "rivoli_kv_page_bytes": [_I, _I],
+    "rivoli_index_topk_workspace_bytes": [_I, _I],
+    "rivoli_mla_attend_paged_scratch_floats": [_I, _I, _I],
+    "rivoli_mla_attend_scratch_floats": [_I, _I],
+    "rivoli_gather_attn_scratch_floats": [_I, _I, _I, _I],
+}
+
+
 def lib() -> C.CDLL:
     """The loaded HIP library. Raises if it was never built — there is no other path."""
     global _LIB
@@ -97,15 +107,9 @@ def lib() -> C.CDLL:
         for name, args in _SIGNATURES.items():
             fn = getattr(handle, name)
             fn.restype, fn.argtypes = C.c_int, args
-        for name in ("rivoli_kv_page_bytes", "rivoli_index_topk_workspace_bytes"):
+        for name, args in _SIZE_SIGNATURES.items():
             fn = getattr(handle, name)
-            fn.restype, fn.argtypes = C.c_size_t, [_I, _I]
-        fn = handle.rivoli_mla_attend_paged_scratch_floats
-        fn.restype, fn.argtypes = C.c_size_t, [_I, _I, _I]
-        fn = handle.rivoli_mla_attend_scratch_floats
-        fn.restype, fn.argtypes = C.c_size_t, [_I, _I]
-        fn = handle.rivoli_gather_attn_scratch_floats
-        fn.restype, fn.argtypes = C.c_size_t, [_I, _I, _I, _I]
+            fn.restype, fn.argtypes = C.c_size_t, args
         _LIB = handle
     return _LIB
 
