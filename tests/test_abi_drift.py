@@ -134,6 +134,13 @@ def test_ctypes_table_matches_the_header():
         assert sym in head, f"{sym}: in rivoli_amd/hip.py, not in the header"
 
 
+def test_cpp_mirror_has_a_launcher_for_every_status_returning_entry_point():
+    text = open(os.path.join(ROOT, "include", "rivoli_launchers.hpp")).read()
+    wrapped = set(re.findall(r"RIVOLI_LAUNCHER\(\s*\w+\s*,\s*(rivoli_\w+)", text)) | set(re.findall(r"(rivoli_\w+)\(", text))
+    for sym in header_prototypes():
+        assert sym in wrapped, f"{sym}: no launcher in include/rivoli_launchers.hpp"
+
+
 @pytest.mark.skipif(not os.path.isdir(REFERENCE_KERNELS), reason="the reference tree is not mounted")
 def test_reference_signatures_are_kept_argument_for_argument():
     """Every entry point the header shares with the reference's kernels/*.hip has the reference's
