@@ -24,8 +24,9 @@
 // up with 8 slots of ONE head, which is the A layout of the value MFMA, so P never leaves
 // registers; the value operand is the same LDS tile through the transposing load
 // (ds_read_b64_tr_b16). Online softmax in base 2 with a lazily moved reference maximum; three
-// LDS tiles rotate so one barrier per tile suffices. Other widths take a plain kernel: one
-// workgroup per (query, head), a wave per logit, threads over output dims.
+// LDS tiles rotate so one barrier per tile suffices. Other widths (and rows that must not be
+// rounded to bf16) take an f32 kernel: a wave per (query, head), lanes over the dims, one
+// online-softmax pass over the list.
 // Launch-only; see include/rivoli_kvcache.h for the contract.
 #include "attend_common.hpp"
 
@@ -416,77 +417,62 @@ __global__ __launch_bounds__(128) void gather_attn_combine_kernel(
                   (float)(__bf16)(sum.w / l_g)};
 }
 
-// Any width: one workgroup of 4 waves per (query, head). Logits: a wave per slot, lanes over
-// dims; then the two-pass softmax of the reference over the logits in LDS; values: threads
-// over output dims, slots ascending.
-constexpr int kGaPlainThreads = 256;
-constexpr int kGaPlainAcc = 4;  // output dims per thread: d <= 1024
+// Any width, and rows kept exactly as they are (no rounding to bf16): a wave per (query, head),
+// the four heads of a workgroup walking the same query's list together so that a listed row
+// comes out of the first-level cache for three of them. A lane owns dims lane, lane + 64, ...:
+// the query and the running output sit in its registers, a slot is one coalesced pass over the
+// row (kept for the value side), a butterfly sum, and an online-softmax update. One pass over
+// the list, no LDS, no barrier; a masked slot (index outside [0, n_kv)) is never dereferenced.
+constexpr int kGaRowThreads = 256;
+constexpr int kGaRowDims = 16;  // dims per lane: d <= 1024
 
-__global__ __launch_bounds__(kGaPlainThreads) void gather_attn_plain_kernel(
+__global__ __launch_bounds__(kGaRowThreads) void gather_attn_rowwise_kernel(
     const float* __restrict__ q, const float* __restrict__ kv, const float* __restrict__ sink,
     const int* __restrict__ idxs, int h, int d, int topk, int n_kv, float scale,
     float* __restrict__ o) {
-    extern __shared__ float ga_lds[];
-    float* qs = ga_lds;      // [d]
-    float* lg = ga_lds + d;  // [topk] logits, then weights
-    __shared__ float red[kGaPlainThreads / kWave];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int head = blockIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int head = (int)blockIdx.x * (kGaRowThreads / kWave) + (threadIdx.x >> 6);
+    if (head >= h) return;
     const size_t t = blockIdx.y;
     const float* qrow = q + (t * h + head) * d;
-    const int* ix = idxs + t * topk;
-    for (int i = tid; i < d; i += kGaPlainThreads) qs[i] = qrow[i];
-    __syncthreads();
-
-    float mx = -INFINITY;
-    for (int j = wave; j < topk; j += kGaPlainThreads / kWave) {
-        const int p = ix[j];
-        float l = -INFINITY;
-        if ((unsigned)p < (unsigned)n_kv) {
-            const float* kr = kv + (size_t)p * d;
-            float acc = 0.0f;
-            for (int i = lane; i < d; i += kWave) acc += qs[i] * kr[i];
-            for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
-            l = acc * scale;
-        }
-        if (lane == 0) lg[j] = l;
-        mx = fmaxf(mx, l);
-    }
-    if (lane == 0) red[wave] = mx;
-    __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    __syncthreads();
-
-    float ps = 0.0f;
-    for (int j = tid; j < topk; j += kGaPlainThreads) {
-        const float l = lg[j];
-        const float e = l == -INFINITY ? 0.0f : expf(l - mx);
-        lg[j] = e;
-        ps += e;
-    }
-    for (int off = 32; off > 0; off >>= 1) ps += __shfl_xor(ps, off, kWave);
-    if (lane == 0) red[wave] = ps;
-    __syncthreads();
-    const float denom = isfinite(mx) ? (red[0] + red[1]) + (red[2] + red[3]) + expf(sink[head] - mx) : NAN;
-
-    float acc[kGaPlainAcc];
+    const int* list = idxs + t * topk;
+    const int steps = (d + kWave - 1) / kWave;  // wave-uniform
+    float qv[kGaRowDims], acc[kGaRowDims];
 #pragma unroll
-    for (int c = 0; c < kGaPlainAcc; ++c) acc[c] = 0.0f;
+    for (int c = 0; c < kGaRowDims; ++c) {
+        const int i = lane + c * kWave;
+        qv[c] = (c < steps && i < d) ? qrow[i] * (scale * kLog2e) : 0.0f;  // scores in log2 units
+        acc[c] = 0.0f;
+    }
+    float top = -INFINITY, denom = 0.0f;
     for (int j = 0; j < topk; ++j) {
-        const float e = lg[j];
-        if (e == 0.0f) continue;  // masked, or a weight that underflowed: adds nothing either way
-        const float* kr = kv + (size_t)ix[j] * d;
+        const int row = list[j];
+        if ((unsigned)row >= (unsigned)n_kv) continue;  // masked (wave-uniform)
+        const float* src = kv + (size_t)row * d;
+        float val[kGaRowDims], dot = 0.0f;
 #pragma unroll
-        for (int c = 0; c < kGaPlainAcc; ++c) {
-            const int i = tid + c * kGaPlainThreads;
-            if (i < d) acc[c] += e * kr[i];
+        for (int c = 0; c < kGaRowDims; ++c) {
+            const int i = lane + c * kWave;
+            val[c] = (c < steps && i < d) ? src[i] : 0.0f;
+            dot += qv[c] * val[c];
         }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, kWave);
+        const float top_new = fmaxf(top, dot);
+        const float keep = exp2f(top - top_new), w = exp2f(dot - top_new);  // 2^-inf = 0 on the first slot
+        denom = denom * keep + w;
+#pragma unroll
+        for (int c = 0; c < kGaRowDims; ++c) acc[c] = acc[c] * keep + w * val[c];
+        top = top_new;
     }
+    // the sink joins the denominator only; a query whose every slot is masked has no maximum
+    // to measure the sink against and comes out NaN, as in the reference (attn.hip:415-420)
+    const float total = top == -INFINITY ? NAN : denom + exp2f(sink[head] * kLog2e - top);
     float* orow = o + (t * h + head) * d;
 #pragma unroll
-    for (int c = 0; c < kGaPlainAcc; ++c) {
-        const int i = tid + c * kGaPlainThreads;
-        if (i < d) orow[i] = (float)(__bf16)(acc[c] / denom);
+    for (int c = 0; c < kGaRowDims; ++c) {
+        const int i = lane + c * kWave;
+        if (c < steps && i < d) orow[i] = (float)(__bf16)(acc[c] / total);
     }
 }
 
@@ -517,12 +503,12 @@ static int gather_attn_launch(const float* q, const float* kv, const float* sink
                            a.part_acc, a.part_ml, sink, a.n_splits, h, o);
         return launch_status();
     }
-    // the plain kernel keeps the reference launcher's limits (attn.hip:450-458)
-    if (d > kGaPlainThreads * kGaPlainAcc || m > 65535) return 1002;
-    const size_t lds = ((size_t)d + (size_t)topk) * sizeof(float);
-    if (lds + sizeof(float) * (kGaPlainThreads + 2) > 65536) return 1006;
-    hipLaunchKernelGGL(gather_attn_plain_kernel, dim3((unsigned)h, (unsigned)m), dim3(kGaPlainThreads),
-                       (unsigned)lds, stream, q, kv, sink, idxs, h, d, topk, n_kv, scale, o);
+    // the reference launcher's limits, kept (attn.hip:450-458): d within 1024, its LDS budget
+    if (d > kGaRowDims * kWave || m > 65535) return 1002;
+    if (((size_t)d + (size_t)topk + 256 + 2) * sizeof(float) > 65536) return 1006;
+    hipLaunchKernelGGL(gather_attn_rowwise_kernel,
+                       dim3((unsigned)((h + kGaRowThreads / kWave - 1) / (kGaRowThreads / kWave)), (unsigned)m),
+                       dim3(kGaRowThreads), 0, stream, q, kv, sink, idxs, h, d, topk, n_kv, scale, o);
     return launch_status();
 }
 

@@ -254,34 +254,36 @@ __global__ __launch_bounds__(SLOTS ? 256 : 1024) void kv_compress_decode_kernel(
     }
 }
 
-// kvcompress.hip:227-262, both phases: a prefill of s tokens starts at slot 0, a decode step
-// deposits its one row at slot0 = start_pos % ratio.
-__global__ void kv_compress_deposit_kernel(const float* __restrict__ kv,
-                                           const float* __restrict__ score,
-                                           const float* __restrict__ ape,
-                                           float* __restrict__ kv_state,
-                                           float* __restrict__ score_state, CompGeom p, int s,
-                                           int slot0) {
-    const int remainder = s % p.ratio, cutoff = s - remainder;
-    const bool overlap = p.coff == 2;
-    const int state_off = overlap ? p.ratio : 0;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (overlap && cutoff >= p.ratio) {
-        const size_t n = (size_t)p.ratio * p.cd, src0 = (size_t)(cutoff - p.ratio) * p.cd;
-        for (size_t i = tid; i < n; i += stride) {
-            kv_state[i] = kv[src0 + i];
-            score_state[i] = score[src0 + i] + ape[i];
-        }
+// The state update every call makes before it pools (crates/backend/kernels/kvcompress.hip:
+// 215-262; model.py:335-336): up to two runs of whole rows move from the call's kv / score
+// rows into the state, the scores picking up the position embedding of their slot.
+//   carry: on an overlapping layer, the last COMPLETE block of the call -> state rows
+//          [0, ratio), embedding rows [0, ratio)            (prefill only: a call of >= ratio rows)
+//   tail:  the rows after the last complete block -> state rows [state_off + slot0, ..),
+//          embedding rows [slot0, ..)                       (a decode step is one tail row)
+// Both runs are contiguous on both sides, so the launch is one flat range of VEC-float pieces,
+// carry first, exactly as many threads as pieces, one 16-byte load per source and store per
+// destination when VEC == 4.
+struct DepositRun {
+    size_t src, dst, emb, n;  // element offsets into kv/score, the state, ape; length
+};
+template <int VEC>
+__global__ __launch_bounds__(256) void kv_compress_deposit_kernel(
+    const float* __restrict__ kv, const float* __restrict__ score, const float* __restrict__ ape,
+    float* __restrict__ kv_state, float* __restrict__ score_state, DepositRun carry, DepositRun tail) {
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
+    size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+    DepositRun r = carry;
+    if (i >= carry.n) {
+        i -= carry.n;
+        r = tail;
+        if (i >= tail.n) return;
     }
-    if (remainder > 0) {
-        const size_t n = (size_t)remainder * p.cd, src0 = (size_t)cutoff * p.cd;
-        const size_t dst0 = (size_t)(state_off + slot0) * p.cd, ape0 = (size_t)slot0 * p.cd;
-        for (size_t i = tid; i < n; i += stride) {
-            kv_state[dst0 + i] = kv[src0 + i];
-            score_state[dst0 + i] = score[src0 + i] + ape[ape0 + i];
-        }
-    }
+    const vec_t k = *reinterpret_cast<const vec_t*>(kv + r.src + i);
+    const vec_t sc = *reinterpret_cast<const vec_t*>(score + r.src + i);
+    const vec_t e = *reinterpret_cast<const vec_t*>(ape + r.emb + i);
+    *reinterpret_cast<vec_t*>(kv_state + r.dst + i) = k;
+    *reinterpret_cast<vec_t*>(score_state + r.dst + i) = sc + e;
 }
 
 // kvcompress.hip:386-405.
@@ -343,10 +345,24 @@ extern "C" int rivoli_kv_compress_deposit(const float* kv, const float* score, c
     if (s <= 0) return 1005;
     if (slot0 < 0 || slot0 + s % p.ratio > p.ratio) return 1008;
     (void)hipGetLastError();
-    const int rem = s % p.ratio;
-    const size_t n = (size_t)(p.ratio > rem ? p.ratio : rem) * p.cd;
-    hipLaunchKernelGGL(rk::kv_compress_deposit_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256),
-                       0, (hipStream_t)stream, kv, score, ape, kv_state, score_state, p, s, slot0);
+    const int rem = s % p.ratio, cutoff = s - rem;
+    const size_t cd = (size_t)p.cd;
+    rk::DepositRun carry = {0, 0, 0, 0}, tail = {0, 0, 0, 0};
+    if (p.coff == 2 && cutoff >= p.ratio) carry = {(size_t)(cutoff - p.ratio) * cd, 0, 0, (size_t)p.ratio * cd};
+    if (rem > 0)
+        tail = {(size_t)cutoff * cd, (size_t)((p.coff == 2 ? p.ratio : 0) + slot0) * cd, (size_t)slot0 * cd,
+                (size_t)rem * cd};
+    if (carry.n + tail.n == 0) return 0;  // whole blocks on a layer without overlap: nothing to keep
+    const bool vec = (p.cd % 4) == 0 && rk::aligned16(kv) && rk::aligned16(score) && rk::aligned16(ape) &&
+                     rk::aligned16(kv_state) && rk::aligned16(score_state);
+    const size_t pieces = (carry.n + tail.n) / (vec ? 4 : 1);
+    const dim3 grid((unsigned)((pieces + 255) / 256));
+    if (vec)
+        hipLaunchKernelGGL(rk::kv_compress_deposit_kernel<4>, grid, dim3(256), 0, (hipStream_t)stream, kv, score,
+                           ape, kv_state, score_state, carry, tail);
+    else
+        hipLaunchKernelGGL(rk::kv_compress_deposit_kernel<1>, grid, dim3(256), 0, (hipStream_t)stream, kv, score,
+                           ape, kv_state, score_state, carry, tail);
     return rk::launch_status();
 }
 
