@@ -258,8 +258,17 @@ int rivoli_index_append_paged(const float* k, const int* slot_mapping, unsigned 
  * asserts.rs), though not bit for bit; 1 carries only q that way (weights rounded to bf16
  * once: errors up to ~1e-3 of the SPREAD of the attended rows); 0 rounds q to bf16 once as
  * well (a score is off by ~2^-10 |q||k|: ordinary bf16 flash-attention numerics).
+ * 3 and 4 (512 + 64 rows only) run both contractions on the 8-bit matrix instructions, the
+ * cache codes going into them untouched and q / the weights as sums of e4m3 terms under
+ * power-of-two block scales: 3 = two terms each (the accuracy class of 0), 4 = three terms for
+ * q and two for the weights (the class of 1; inside the reference's bar on the test caches).
+ * Correct and tested, but slower than 0 - 2 today (register allocation, not the instruction
+ * rate, bounds them): kept as the measured starting point of that design.
+ * Other row widths (kvl a multiple of 128 up to 512, rope a multiple of 8 up to 64) always run
+ * as 2.
  * Guards: 1001 null / non-positive, or a null `partial` when scratch is needed; 1002
- * n_seqs > 65535; 1004 unless kvl == 512 and rope == 64 (the 576-code page row). */
+ * n_seqs > 65535; 1004 for a latent width that is not a multiple of 128 or above 512, a rope
+ * width that is not a multiple of 8 or above 64, or a buffer that is not 16-byte aligned. */
 size_t rivoli_mla_attend_paged_scratch_floats(int n_seqs, int H, int max_rows);
 int rivoli_mla_attend_paged(const float* qabs, const float* qrope, const unsigned char* pool,
                             const int* block_table, const int* seq_lens,

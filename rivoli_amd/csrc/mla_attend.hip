@@ -656,10 +656,18 @@ __device__ __forceinline__ void attend_part(const AttendArgs& a, int seq, int hb
     }
 }
 
-template <int QSPLIT, int PSPLIT, int MODE, bool ANY>
-__global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const AttendArgs a) {
+}  // namespace rk
+#include "mla_attend_f8.hpp"
+namespace rk {
+
+// F8: the contractions run on the 8-bit matrix instructions with QSPLIT / PSPLIT e4m3 terms for
+// q / the softmax weights (mla_attend_f8.hpp); else on the bf16 ones.
+template <int QSPLIT, int PSPLIT, int MODE, bool ANY, bool F8 = false>
+__global__ __launch_bounds__(F8 ? kF8Threads : kAttThreads) void mla_attend_paged_kernel(const AttendArgs a) {
+    constexpr int THREADS = F8 ? kF8Threads : kAttThreads;
+    constexpr int PER = kDealMaxSeqs / THREADS;  // sequences per thread in the prefix below
     __shared__ int pre[kDealMaxSeqs + 8];  // tiles before each sequence, when dealing
-    __shared__ int wave_total[kAttWaves];
+    __shared__ int wave_total[THREADS / kWave];
     constexpr bool SPARSE = MODE == kSparse;
     const int hb = blockIdx.z;
     const int tid = threadIdx.x;
@@ -678,11 +686,14 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
     long long t_lo = 0, t_hi = 0;
     int seq = blockIdx.y;
     if (a.n_items > 0) {
-        // inclusive prefix of tiles per sequence, two sequences per thread
-        const int s0 = 2 * tid, s1 = 2 * tid + 1;
-        const int c0 = s0 < a.n_seqs ? (attended(s0) + kTile - 1) / kTile : 0;
-        const int c1 = s1 < a.n_seqs ? (attended(s1) + kTile - 1) / kTile : 0;
-        int run = c0 + c1;
+        // inclusive prefix of tiles per sequence, PER consecutive sequences per thread
+        int c[PER], run = 0;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int s = PER * tid + j;
+            c[j] = s < a.n_seqs ? (attended(s) + kTile - 1) / kTile : 0;
+            run += c[j];
+        }
 #pragma unroll
         for (int off = 1; off < kWave; off <<= 1) {
             const int up = __shfl_up(run, off, kWave);
@@ -692,10 +703,14 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         __syncthreads();
         int before = 0;
         for (int w = 0; w < wave; ++w) before += wave_total[w];
-        run += before;  // tiles of sequences 0 .. s1
+        run += before;  // tiles of sequence 0 .. the thread's last one
         if (tid == 0) pre[0] = 0;
-        if (s0 < a.n_seqs) pre[s0 + 1] = run - c1;
-        if (s1 < a.n_seqs) pre[s1 + 1] = run;
+#pragma unroll
+        for (int j = PER - 1; j >= 0; --j) {
+            const int s = PER * tid + j;
+            if (s < a.n_seqs) pre[s + 1] = run;
+            run -= c[j];
+        }
         __syncthreads();
         const long long total = pre[a.n_seqs];
         t_lo = deal_lo(blockIdx.x, a.n_items, total);
@@ -733,14 +748,15 @@ __global__ __launch_bounds__(kAttThreads) void mla_attend_paged_kernel(const Att
         if (r_end <= 0) {
             // a sequence with nothing to attend gets zeros, like the reference's `l > 0 ? 1/l : 0`
             const int kvl = ANY ? a.kvl : kKvl;
-            for (int i = tid; i < 64 * kvl; i += kAttThreads) {
+            for (int i = tid; i < 64 * kvl; i += THREADS) {
                 const int h = hb * 64 + i / kvl;
                 if (h < a.H) a.clat[((size_t)seq * a.H + h) * kvl + (i % kvl)] = 0.0f;
             }
             return;
         }
     }
-    attend_part<QSPLIT, PSPLIT, MODE, ANY>(a, seq, hb, r_begin, r_end, whole, pa, pml);
+    if constexpr (F8) attend_part_f8<QSPLIT, PSPLIT, MODE == kSparse>(a, seq, hb, r_begin, r_end, whole, pa, pml);
+    else attend_part<QSPLIT, PSPLIT, MODE, ANY>(a, seq, hb, r_begin, r_end, whole, pa, pml);
     if (a.n_items == 0) break;
   }  // parts of this workgroup
 }
@@ -818,7 +834,13 @@ static int attend_launch(const AttendArgs& a, const AttendPlan& plan, int n_seqs
     if (any || MODE == kLinear)
         hipLaunchKernelGGL((mla_attend_paged_kernel<2, 2, MODE, true>), grid, dim3(kAttThreads), 0, st, a);
     else if constexpr (MODE != kLinear) {
-        if (precise >= 2)
+        if (precise == 3)
+            hipLaunchKernelGGL((mla_attend_paged_kernel<2, 2, MODE == kSparse ? kSparse : kDense, false, true>), grid,
+                               dim3(kF8Threads), 0, st, a);
+        else if (precise == 4)
+            hipLaunchKernelGGL((mla_attend_paged_kernel<3, 2, MODE == kSparse ? kSparse : kDense, false, true>), grid,
+                               dim3(kF8Threads), 0, st, a);
+        else if (precise >= 2)
             hipLaunchKernelGGL((mla_attend_paged_kernel<2, 2, MODE, false>), grid, dim3(kAttThreads), 0, st, a);
         else if (precise == 1)
             hipLaunchKernelGGL((mla_attend_paged_kernel<2, 1, MODE, false>), grid, dim3(kAttThreads), 0, st, a);

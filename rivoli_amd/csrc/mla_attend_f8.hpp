@@ -1,0 +1,404 @@
+// MLA decode attention over the paged fp8 cache on gfx950's 8-bit matrix instructions
+// (v_mfma_scale_f32_16x16x128_f8f6f4), included by mla_attend.hip.
+//
+// The cache rows ARE e4m3 codes, so they go from memory into LDS and from LDS into the matrix
+// cores untouched: no conversion, half the LDS bytes of the bf16 kernel, a quarter of its matrix
+// instructions. What is not e4m3 is carried as a short sum of e4m3 terms under power-of-two
+// block scales (the instruction's own E8M0 scale operands):
+//   q      = sum_t 2^(e - 4(t-1)) * q_t,  e from the largest |q| of the (head, 128-dim step)
+//   p * s  = sum_t 2^(e - 4(t-1)) * p_t,  e from the largest weight of the (head, 128-token tile)
+// Each term adds four significant bits (term t quantizes what terms 1..t-1 left over), so TQ / TP
+// terms give q / the softmax weights 4 TQ / 4 TP bits: two terms are bf16-class, four the parity
+// mode's. The scale operands are uniform over a row's four lanes, which makes the instruction's
+// own assignment of scale lanes to K blocks immaterial.
+//
+// Mapping: as the bf16 kernel, a 512-thread workgroup owns 64 heads and a run of rows, waves w
+// and w + 4 share heads 16 (w & 3) .. +15; wave half h takes K-steps {0, 1, rope} or {2, 3} of the
+// scores (a K-step is 128 dims; the rope's 64 fill half a step) and output columns 256 h .. +255.
+// Tiles are 128 tokens — the K of the value contraction — held ONCE in LDS as raw code rows; the
+// XX scores S^T[token][head] (A = the rows, 32 contiguous bytes per
+// lane, B = the q terms resident in registers), exchange of the two halves' partial scores
+// through LDS, barrier, online softmax in base 2 with a lazily moved maximum, weights to e4m3
+// terms in registers — a lane's 32 weights are exactly its A operand of the value contraction —
+// values O[head][col] += P . V with V read from the same tile through the transposing byte load
+// (ds_read_b64_tr_b8) in the token order the weights have, barrier.
+#pragma once
+
+namespace rk {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kF8Threads = 256;              // four waves, one per SIMD, each with the full register file
+constexpr int kF8Waves = kF8Threads / kWave;
+constexpr int kF8Tile = 128;                 // tokens per tile
+constexpr int kF8RowBytes = 592;             // 576 codes + 16 of padding
+constexpr int kF8TileBytes = kF8Tile * kF8RowBytes;
+constexpr int kF8ZeroBytes = 64;
+constexpr int kF8Steps = 5;                  // K-steps of the scores: four of 128 latent dims, one for the rope
+constexpr int kF8ColTiles = kKvl / 16;       // 32 output column tiles per wave
+constexpr int kF8RowGranules = kF8RowBytes / 16;  // 37: 36 of codes, one of padding
+constexpr int kF8SmemBytes = 2 * kF8TileBytes + kF8ZeroBytes + 2 * 2 * kF8Tile * 4 + kF8Tile * 8 + kTableLds * 4;
+static_assert(kF8SmemBytes + (1024 + 8 + 8) * 4 <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
+constexpr int kScaleOne = 0x7f7f7f7f;        // E8M0 1.0 in every byte
+
+// 2^e as a float, e in [-126, 127].
+__device__ __forceinline__ float pow2i(int e) { return __uint_as_float((uint32_t)(e + 127) << 23); }
+// The block exponent for a largest magnitude `amax`: values / 2^e land below 256 (e4m3 holds 448).
+__device__ __forceinline__ int block_exp(float amax) {
+    const int e = (int)((__float_as_uint(amax) >> 23) & 0xffu) - 127 - 7;
+    return amax > 0.0f ? max(min(e, 100), -100) : 0;  // (a tile of vanishing weights keeps a scale whose finer terms still exist)
+}
+// x[0..3] (already divided by the block scale) -> four e4m3 codes, and x -= their values.
+__device__ __forceinline__ uint32_t e4m3x4_and_residual(float (&x)[4]) {
+    int w = 0;
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], w, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(x[2], x[3], w, true);
+    const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+    x[0] -= lo[0], x[1] -= lo[1], x[2] -= hi[0], x[3] -= hi[1];
+    return (uint32_t)w;
+}
+
+template <int TQ, int TP, bool SPARSE>
+__device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int hb, int r_begin, int r_end,
+                                               bool whole, float* pa, float* pml) {
+    __shared__ __attribute__((aligned(16))) uint8_t smem8[kF8SmemBytes];
+    const lds_ptr<uint8_t> tiles = (lds_ptr<uint8_t>)smem8;               // [2][128] rows of codes
+    const lds_ptr<uint8_t> zeros = tiles + 2 * kF8TileBytes;
+    const lds_ptr<float> sc = (lds_ptr<float>)(zeros + kF8ZeroBytes);     // [2][128] token scales (0 = not there)
+    const lds_ptr<float> sbias = sc + 2 * kF8Tile;                         // [2][128] 0 or -inf
+    const lds_ptr<unsigned long long> rowbase = (lds_ptr<unsigned long long>)(sbias + 2 * kF8Tile);  // [128] where a row's codes are
+    const lds_ptr<int> tbl = (lds_ptr<int>)(rowbase + kF8Tile);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // = which 16 heads of the block
+    const int g = lane >> 4, n16 = lane & 15;
+    const int n_tiles = (r_end - r_begin + kF8Tile - 1) / kF8Tile;
+
+    // ---- block-table slice, zero area -------------------------------------------------------
+    const int* const table_g = a.block_table + (size_t)seq * a.max_blocks;
+    const int tbl_first = SPARSE ? 0 : r_begin / a.page_tokens;
+    const int tbl_last = SPARSE ? a.max_blocks - 1 : min(a.max_blocks - 1, (r_end - 1) / a.page_tokens);
+    const int tbl_count = min(kTableLds, tbl_last - tbl_first + 1);
+    for (int i = tid; i < tbl_count; i += kF8Threads) tbl[i] = table_g[tbl_first + i];
+    if (tid < kF8ZeroBytes / 4) ((lds_ptr<int>)zeros)[tid] = 0;
+
+    // ---- this wave's 16 query heads as e4m3 terms, for the whole kernel ----------------------
+    // step s < 4: latent dims 128 s .. +127; step 4: the rope (its 64 dims in lane groups 0 and 1)
+    i32x8 qt[TQ][kF8Steps];
+    int qscale_lo[TQ], qscale_hi[TQ];  // E8M0 scales: bytes 0..3 = steps 0..3, byte 0 of _hi = step 4
+    {
+        const int head = hb * 64 + 16 * wave + n16;
+        const bool live = head < a.H;
+        const size_t qrow = (size_t)seq * a.H + (live ? head : 0);
+#pragma unroll
+        for (int t = 0; t < TQ; ++t) qscale_lo[t] = qscale_hi[t] = kScaleOne;
+#pragma unroll
+        for (int s = 0; s < kF8Steps; ++s) {
+            float x[32];
+            const bool there = live && (s < 4 || g < 2);
+            const float* src = s == 4 ? a.qrope + qrow * kRopeW + 32 * g : a.qabs + qrow * kKvl + 128 * s + 32 * g;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                float4 v = {0, 0, 0, 0};
+                if (there) v = reinterpret_cast<const float4*>(src)[c];
+                x[4 * c] = v.x * a.qscale, x[4 * c + 1] = v.y * a.qscale, x[4 * c + 2] = v.z * a.qscale,
+                x[4 * c + 3] = v.w * a.qscale;
+            }
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(x[i]));
+            amax = rows_max(amax);  // over the head's four lanes: one scale per (head, step)
+            const int e = block_exp(amax);
+            const float inv = pow2i(-e);
+#pragma unroll
+            for (int i = 0; i < 32; ++i) x[i] *= inv;
+#pragma unroll
+            for (int t = 0; t < TQ; ++t) {
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    float y[4] = {x[4 * c], x[4 * c + 1], x[4 * c + 2], x[4 * c + 3]};
+                    qt[t][s][c] = (int)e4m3x4_and_residual(y);
+                    // what is left over, at the next term's scale (16 times finer)
+                    x[4 * c] = y[0] * 16.0f, x[4 * c + 1] = y[1] * 16.0f, x[4 * c + 2] = y[2] * 16.0f,
+                    x[4 * c + 3] = y[3] * 16.0f;
+                }
+                const int byte = max(e - 4 * t + 127, 1);
+                if (s < 4) qscale_lo[t] = (qscale_lo[t] & ~(0xff << (8 * s))) | (byte << (8 * s));
+                else qscale_hi[t] = (qscale_hi[t] & ~0xff) | byte;
+            }
+        }
+    }
+    __syncthreads();  // table slice and zero area visible
+
+    auto table_at = [&](int blk) -> int {
+        const int rel = blk - tbl_first;
+        return (rel >= 0 && rel < tbl_count) ? tbl[rel] : table_g[blk];
+    };
+
+    // ---- where the wave's 32 tokens of a tile are: lanes 0..31 resolve one each --------------
+    constexpr unsigned long long kNone = ~0ull;
+    const unsigned int* const rows_g = SPARSE ? a.rows + (size_t)seq * a.k : nullptr;
+    auto resolve = [&](int t, unsigned long long& code_off, unsigned long long& scale_off) {
+        code_off = kNone, scale_off = 0;
+        const int pos = r_begin + t * kF8Tile + 32 * wave + lane;
+        if (lane >= 32 || t >= n_tiles || pos >= r_end) return;
+        const unsigned int tok = SPARSE ? rows_g[pos] : (unsigned)pos;
+        unsigned int blk, off;
+        if (a.page_shift >= 0) blk = tok >> a.page_shift, off = tok & (unsigned)(a.page_tokens - 1);
+        else blk = tok / (unsigned)a.page_tokens, off = tok - blk * (unsigned)a.page_tokens;
+        const int page = blk < (unsigned)a.max_blocks ? table_at((int)blk) : -1;
+        if ((unsigned)page < (unsigned)a.n_pages) {
+            const unsigned long long pbase = (unsigned long long)page * a.page_bytes;
+            code_off = pbase + (unsigned long long)off * kRowW;
+            scale_off = pbase + (unsigned long long)a.page_tokens * kRowW + (unsigned long long)off * 4;
+        } else if (a.bad_rows && hb == 0) {
+            atomicAdd(a.bad_rows, 1u);
+        }
+    };
+    // A tile goes from memory straight into LDS (global_load_lds, 16 bytes per lane, a wave's 64
+    // lanes filling 1 KiB of consecutive LDS): no registers hold it on the way. The wave's 32 rows
+    // of 37 granules (36 of codes + the padding one) are that consecutive range, so lane L of
+    // request I fills granule 64 I + L = row (64 I + L) / 37, granule (64 I + L) % 37 of the
+    // row, from wherever that row's page is. A row that is not there is zero-filled by hand: its
+    // codes must be finite, they meet a zero weight and a -inf bias, never a NaN.
+    float next_scale = 0.0f;  // lanes 0..31: the scale of the row this lane resolved
+    auto request_tile = [&](int t, int buf) {
+        unsigned long long code_off, scale_off;
+        resolve(t, code_off, scale_off);
+        if (lane < 32) rowbase[32 * wave + lane] = code_off;
+        next_scale = 0.0f;
+        if (code_off != kNone) next_scale = *reinterpret_cast<const float*>(a.pool + scale_off);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+        const lds_ptr<uint8_t> dst0 = tiles + buf * kF8TileBytes + (32 * wave) * kF8RowBytes;
+        // (the per-request row and granule depend only on the lane: recomputed here each time
+        // rather than kept live across the whole tile loop, where they would cost ~60 registers)
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+#pragma unroll
+        for (int i = 0; i < (32 * kF8RowGranules + kWave - 1) / kWave; ++i) {
+            const int gi = kWave * i + ln;
+            const int row = gi / kF8RowGranules, c = gi - row * kF8RowGranules;
+            if (row < 32 && c < kRowW / 16) {
+                const unsigned long long base = rowbase[32 * wave + row];
+                if (base != kNone) {
+                    __builtin_amdgcn_global_load_lds(
+                        (const __attribute__((address_space(1))) void*)(a.pool + base + 16 * c),
+                        (__attribute__((address_space(3))) void*)(dst0 + 1024 * i), 16, 0, 0);
+                } else {
+                    *(lds_ptr<u32x4>)(dst0 + 16 * gi) = u32x4{0, 0, 0, 0};
+                }
+            }
+        }
+    };
+    auto publish_scales = [&](int buf) {  // the scales of the tile request_tile last asked for
+        if (lane < 32) {
+            const bool ok = next_scale > 0.0f;  // a token that is not there has scale 0
+            sc[buf * kF8Tile + 32 * wave + lane] = ok ? next_scale : 0.0f;
+            sbias[buf * kF8Tile + 32 * wave + lane] = ok ? 0.0f : -INFINITY;
+        }
+    };
+
+    // ---- per-lane LDS addresses ---------------------------------------------------------------
+    // scores: row 16 mb + n16, this lane's 32 bytes of K-step s; the rope step's upper half
+    // (lane groups 2 and 3) reads zeros
+    const int a_row = n16 * kF8RowBytes + 32 * g;
+    const bool rope_zero = g >= 2;
+    // values: transposing load r (of 4) hands this lane bytes 8 r .. 8 r + 7 of its operand = the
+    // tokens 16 (2 r + e / 4) + 4 g + e % 4, e = 0..7, of column 16 nt + n16; source lane pair e
+    // addresses token e's row, its two lanes the two 8-byte halves of the 16 columns.
+    int v_off[4];
+    {
+        const int e = n16 >> 1;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            v_off[r] = (16 * (2 * r + (e >> 2)) + 4 * g + (e & 3)) * kF8RowBytes + 8 * (n16 & 1);
+    }
+
+    f32x4 o[kF8ColTiles];
+#pragma unroll
+    for (int nt = 0; nt < kF8ColTiles; ++nt) o[nt] = f32x4{0, 0, 0, 0};
+    float m_ref = -INFINITY, l_sum = 0.0f;
+
+    // prologue: tile 0 into LDS
+    request_tile(0, 0);
+    publish_scales(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    for (int t = 0; t < n_tiles; ++t) {
+        const int buf = t & 1;
+        const lds_ptr<uint8_t> tile = tiles + buf * kF8TileBytes;
+        const lds_ptr<float> sc_t = sc + buf * kF8Tile, sbias_t = sbias + buf * kF8Tile;
+        // tile t + 1 starts on its way into the other buffer (which held tile t - 1: every wave
+        // left it before the barrier that ended the previous iteration)
+        if (t + 1 < n_tiles) request_tile(t + 1, buf ^ 1);
+
+        // ---- scores: S^T[token][head] over the five K-steps ---------------------------------
+        f32x4 acc[8];
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) acc[mb] = f32x4{0, 0, 0, 0};
+        // Operand fragments are requested four row blocks at a time, ahead of the matrix
+        // instructions that consume them; the scheduling fences keep the compiler from hoisting
+        // every step's reads to the top (and spilling them).
+#pragma unroll
+        for (int s = 0; s < kF8Steps; ++s) {
+#pragma unroll
+            for (int m0 = 0; m0 < 8; m0 += 4) {
+                i32x8 af[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const lds_ptr<uint8_t> src =
+                        (s == 4 && rope_zero) ? zeros : tile + (m0 + j) * 16 * kF8RowBytes + a_row + 128 * s;
+                    const u32x4 lo4 = *(lds_ptr<u32x4>)(src), hi4 = *(lds_ptr<u32x4>)(src + 16);
+                    af[j] = i32x8{(int)lo4.x, (int)lo4.y, (int)lo4.z, (int)lo4.w, (int)hi4.x, (int)hi4.y, (int)hi4.z, (int)hi4.w};
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int tq = 0; tq < TQ; ++tq)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int mb = m0 + j;
+                        if (s == 0)
+                            acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[j], qt[tq][0], acc[mb], 0, 0, 0, kScaleOne, 0, qscale_lo[tq]);
+                        else if (s == 1)
+                            acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[j], qt[tq][1], acc[mb], 0, 0, 0, kScaleOne, 1, qscale_lo[tq]);
+                        else if (s == 2)
+                            acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[j], qt[tq][2], acc[mb], 0, 0, 0, kScaleOne, 2, qscale_lo[tq]);
+                        else if (s == 3)
+                            acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[j], qt[tq][3], acc[mb], 0, 0, 0, kScaleOne, 3, qscale_lo[tq]);
+                        else
+                            acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[j], qt[tq][4], acc[mb], 0, 0, 0, kScaleOne, 0, qscale_hi[tq]);
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+
+        // ---- online softmax over the lane's 32 tokens of head n16: tokens 16 mb + 4 g + i ----
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) {
+            const f32x4 s4 = *(lds_ptr<f32x4>)(sc_t + 16 * mb + 4 * g);
+            const f32x4 b4 = *(lds_ptr<f32x4>)(sbias_t + 16 * mb + 4 * g);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[mb][i] = __builtin_fmaf(acc[mb][i], s4[i], b4[i]);  // -inf where the token is not there
+                tmax = fmaxf(tmax, acc[mb][i]);
+            }
+        }
+        tmax = rows_max(tmax);
+        const bool grow = tmax > m_ref + kLazyRescale;  // false while everything is masked
+        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+            const float corr = grow ? __builtin_amdgcn_exp2f(m_ref - tmax) : 1.0f;
+            if (grow) m_ref = tmax;
+            l_sum *= corr;
+            float c[4];  // the lane's accumulators are heads 4g+i; corr lives in lanes n16 == head
+#pragma unroll
+            for (int i = 0; i < 4; ++i) c[i] = __shfl(corr, 4 * g + i, kWave);
+#pragma unroll
+            for (int nt = 0; nt < kF8ColTiles; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[nt][i] *= c[i];
+        }
+        const float mu = m_ref == -INFINITY ? 0.0f : m_ref;
+        // weights w_t = 2^(v_t - mu) * s_t, as TP e4m3 terms under one scale per (head, tile)
+        float wmax = 0.0f;
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) {
+            const f32x4 s4 = *(lds_ptr<f32x4>)(sc_t + 16 * mb + 4 * g);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[mb][i] = __builtin_amdgcn_exp2f(acc[mb][i] - mu) * s4[i];  // not there -> 0
+                wmax = fmaxf(wmax, acc[mb][i]);
+            }
+        }
+        wmax = rows_max(wmax);
+        const int pe = block_exp(wmax);
+        const float pinv = pow2i(-pe);
+        // what one unit of the last residual is worth: 2^pe / 16^(TP - 1)
+        const float last_unit = pow2i(pe - 4 * (TP - 1));
+        i32x8 pt[TP];
+        int pscale[TP];
+#pragma unroll
+        for (int tp = 0; tp < TP; ++tp) pscale[tp] = (int)((uint32_t)max(pe - 4 * tp + 127, 1) * 0x01010101u);
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) {
+            const f32x4 s4 = *(lds_ptr<f32x4>)(sc_t + 16 * mb + 4 * g);
+            float y[4] = {acc[mb][0] * pinv, acc[mb][1] * pinv, acc[mb][2] * pinv, acc[mb][3] * pinv};
+#pragma unroll
+            for (int tp = 0; tp < TP; ++tp) {
+                pt[tp][mb] = (int)e4m3x4_and_residual(y);
+                if (tp + 1 < TP) y[0] *= 16.0f, y[1] *= 16.0f, y[2] *= 16.0f, y[3] *= 16.0f;
+            }
+            // The denominator sums the weights the numerator really holds (w_t less the last
+            // residual), over the token scale: the result is an exactly normalised average under
+            // weights perturbed by 2^-4TP each.
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float held = acc[mb][i] - y[i] * last_unit;
+                l_sum += s4[i] > 0.0f ? held * __builtin_amdgcn_rcpf(s4[i]) : 0.0f;
+            }
+        }
+
+        // ---- values: O[head][col] += P . V over all 512 columns -------------------------------
+#pragma unroll
+        for (int n0 = 0; n0 < kF8ColTiles; n0 += 4) {
+            i32x8 vf[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const i32x2 two =
+                        __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr<i32x2>)(tile + v_off[r] + 16 * (n0 + j)));
+                    vf[j][2 * r] = two[0], vf[j][2 * r + 1] = two[1];
+                }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int tp = 0; tp < TP; ++tp)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    o[n0 + j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pt[tp], vf[j], o[n0 + j], 0, 0, 0, pscale[tp], 0, kScaleOne);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        if (t + 1 < n_tiles) publish_scales(buf ^ 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's part of tile t + 1 has landed
+        __syncthreads();  // tile t + 1 is in LDS; every wave is done with tile t
+    }
+
+    // ---- epilogue ---------------------------------------------------------------------------
+    l_sum = rows_sum(l_sum);
+    float l_h[4];  // the lane's accumulators are heads 4g+i; their (m, l) live in lanes with n16 == 4g+i
+#pragma unroll
+    for (int i = 0; i < 4; ++i) l_h[i] = __shfl(l_sum, 4 * g + i, kWave);
+    const int head0 = hb * 64 + 16 * wave;
+    if (!whole) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int head = head0 + 4 * g + i;
+            if (head < a.H) {
+#pragma unroll
+                for (int nt = 0; nt < kF8ColTiles; ++nt) pa[(size_t)head * kKvl + n16 + 16 * nt] = o[nt][i];
+            }
+        }
+        if (g == 0 && head0 + n16 < a.H) {
+            pml[(head0 + n16) * 2] = m_ref;
+            pml[(head0 + n16) * 2 + 1] = l_sum;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int head = head0 + 4 * g + i;
+            const float inv = l_h[i] > 0.0f ? 1.0f / l_h[i] : 0.0f;
+            if (head < a.H) {
+                float* const dst = a.clat + ((size_t)seq * a.H + head) * kKvl;
+#pragma unroll
+                for (int nt = 0; nt < kF8ColTiles; ++nt) dst[n16 + 16 * nt] = o[nt][i] * inv;
+            }
+        }
+    }
+}
+
+}  // namespace rk
