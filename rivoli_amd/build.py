@@ -15,6 +15,10 @@ LIB_PATH = os.path.join(CSRC, "librivoli_kvcache.so")
 HOST_LIB_PATH = os.path.join(CSRC, "librivoli_pagepool.so")
 KERNELS = ["kv_append.hip", "kv_gather.hip", "index_topk.hip", "index_score.hip", "mla_attend.hip",
            "act_quant.hip", "kv_compress.hip", "kv_ring.hip", "gather_attn.hip", "hash_rows.hip"]
+# Matrix-instruction results in ordinary registers: the 8-bit attention kernel keeps its 128
+# accumulators there and its q terms in the accumulation registers (mla_attend_f8.hpp); the bf16
+# kernels of the same file time the same either way.
+EXTRA_FLAGS = {"mla_attend.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 HOST_SOURCES = ["pagepool.cpp"]
 
 
@@ -39,7 +43,8 @@ def build_kernels(verbose: bool = False) -> str:
 
     def compile_one(k: str) -> str:
         obj = os.path.join(objdir, k.replace(".hip", ".o"))
-        res = subprocess.run(common + ["-c", os.path.join(CSRC, k), "-o", obj], capture_output=True, text=True)
+        res = subprocess.run(common + EXTRA_FLAGS.get(k, []) + ["-c", os.path.join(CSRC, k), "-o", obj],
+                             capture_output=True, text=True)
         if verbose or res.returncode != 0:
             sys.stderr.write(res.stdout + res.stderr)
         if res.returncode != 0:

@@ -1,27 +1,36 @@
 // MLA decode attention over the paged fp8 cache on gfx950's 8-bit matrix instructions
 // (v_mfma_scale_f32_16x16x128_f8f6f4), included by mla_attend.hip.
 //
-// The cache rows ARE e4m3 codes, so they go from memory into LDS and from LDS into the matrix
-// cores untouched: no conversion, half the LDS bytes of the bf16 kernel, a quarter of its matrix
-// instructions. What is not e4m3 is carried as a short sum of e4m3 terms under power-of-two
-// block scales (the instruction's own E8M0 scale operands):
-//   q      = sum_t 2^(e - 4(t-1)) * q_t,  e from the largest |q| of the (head, 128-dim step)
-//   p * s  = sum_t 2^(e - 4(t-1)) * p_t,  e from the largest weight of the (head, 128-token tile)
-// Each term adds four significant bits (term t quantizes what terms 1..t-1 left over), so TQ / TP
-// terms give q / the softmax weights 4 TQ / 4 TP bits: two terms are bf16-class, four the parity
-// mode's. The scale operands are uniform over a row's four lanes, which makes the instruction's
-// own assignment of scale lanes to K blocks immaterial.
+// The cache rows ARE e4m3 codes, so they go from memory into LDS (global_load_lds: no registers
+// on the way) and from LDS into the matrix cores untouched: no conversion, half the LDS bytes of
+// the bf16 kernel, a quarter of its matrix instructions. What is not e4m3 is carried as a short
+// sum of e4m3 terms under power-of-two block scales (the instruction's own E8M0 scale operands):
+//   q      = sum_t 2^(e - 4t) * q_t,  e from the largest |q| of the (head, 128-dim step)
+//   p * s  = sum_t 2^(e - 4t) * p_t,  e from the largest weight of the (head, tile)
+// Each term adds four significant bits (term t quantizes what the terms before it left over): two
+// terms are bf16-class; three of q and two of the weights stay inside the reference's bar.
 //
-// Mapping: as the bf16 kernel, a 512-thread workgroup owns 64 heads and a run of rows, waves w
-// and w + 4 share heads 16 (w & 3) .. +15; wave half h takes K-steps {0, 1, rope} or {2, 3} of the
-// scores (a K-step is 128 dims; the rope's 64 fill half a step) and output columns 256 h .. +255.
-// Tiles are 128 tokens — the K of the value contraction — held ONCE in LDS as raw code rows; the
-// XX scores S^T[token][head] (A = the rows, 32 contiguous bytes per
-// lane, B = the q terms resident in registers), exchange of the two halves' partial scores
-// through LDS, barrier, online softmax in base 2 with a lazily moved maximum, weights to e4m3
-// terms in registers — a lane's 32 weights are exactly its A operand of the value contraction —
-// values O[head][col] += P . V with V read from the same tile through the transposing byte load
-// (ds_read_b64_tr_b8) in the token order the weights have, barrier.
+// Mapping: a 256-thread workgroup — one wave per SIMD, each with the whole register file — owns
+// 64 heads and a run of rows; wave w owns heads 16 w .. +15 and all 512 output columns (128
+// accumulators). Two q terms live in the accumulation half of the register file, which the
+// matrix instructions read directly (a third, when there is one, in LDS). Tiles are 64 tokens,
+// two buffers of raw code rows in LDS. Per tile a wave
+//   requests the next tile into the other buffer;
+//   scores: S^T[token][head] = rows x q, 4 row blocks x 5 K-steps (128 dims; the rope's 64 fill
+//     half a step) x TQ terms, A = 32 contiguous bytes of a row per lane;
+//   online softmax in base 2 with a lazily moved reference, the weights to two e4m3 terms in
+//     registers: a lane's 16 weights per term are exactly its share of the next operand;
+//   values: O[head][col] += P V. The contraction's K is 128 = the tile's 64 tokens once per
+//     term: bytes 0..15 of a lane's weight operand hold the first term of its 16 tokens, bytes
+//     16..31 the second (the instruction takes K block b's scale from lane 16 b + row, so lane
+//     groups 2 and 3 carry the finer scale), and the value operand — the same tile, read through
+//     the transposing byte load (ds_read_b64_tr_b8) — repeats its 16 bytes;
+//   waits for its part of the next tile and meets the other waves at the one barrier of the step.
+// Operand fragments are requested one unit ahead of the matrix instructions that use them.
+// The file must be compiled with -mllvm -amdgpu-mfma-vgpr-form (the build does): the kernel's
+// register budget assumes the output tiles in ordinary registers and the q terms in the
+// accumulation registers, and without the switch the compiler moves all 128 accumulators
+// between the two halves every tile.
 #pragma once
 
 namespace rk {
@@ -31,15 +40,23 @@ typedef int i32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kF8Threads = 256;              // four waves, one per SIMD, each with the full register file
 constexpr int kF8Waves = kF8Threads / kWave;
-constexpr int kF8Tile = 128;                 // tokens per tile
+constexpr int kF8Tile = 64;                  // tokens per tile
+constexpr int kF8Bufs = 2;
 constexpr int kF8RowBytes = 592;             // 576 codes + 16 of padding
 constexpr int kF8TileBytes = kF8Tile * kF8RowBytes;
 constexpr int kF8ZeroBytes = 64;
 constexpr int kF8Steps = 5;                  // K-steps of the scores: four of 128 latent dims, one for the rope
+constexpr int kF8RowBlocks = kF8Tile / 16;   // 4 score row blocks per tile
 constexpr int kF8ColTiles = kKvl / 16;       // 32 output column tiles per wave
 constexpr int kF8RowGranules = kF8RowBytes / 16;  // 37: 36 of codes, one of padding
-constexpr int kF8SmemBytes = 2 * kF8TileBytes + kF8ZeroBytes + 2 * 2 * kF8Tile * 4 + kF8Tile * 8 + kTableLds * 4;
-static_assert(kF8SmemBytes + (1024 + 8 + 8) * 4 <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
+constexpr int kF8WaveRows = kF8Tile / kF8Waves;    // rows of a tile one wave brings in
+constexpr int kF8Requests = (kF8WaveRows * kF8RowGranules + kWave - 1) / kWave;
+template <int TQ>
+constexpr int f8_q_bytes() { return TQ > 2 ? (TQ - 2) * 64 * kF8RowBytes : 16; }  // q terms past the second: the block's 64 heads, rows padded like the tiles'
+constexpr int kF8SmemBytes =
+    kF8Bufs * kF8TileBytes + kF8ZeroBytes + 2 * kF8Bufs * kF8Tile * 4 + kF8Tile * 8 + kTableLds * 4;
+static_assert(kF8SmemBytes + f8_q_bytes<3>() + (1024 + 8 + 8) * 4 <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
+constexpr int kWaitLds0 = 0xC07F;           // s_waitcnt lgkmcnt(0), the other counters left alone
 constexpr int kScaleOne = 0x7f7f7f7f;        // E8M0 1.0 in every byte
 
 // 2^e as a float, e in [-126, 127].
@@ -59,16 +76,25 @@ __device__ __forceinline__ uint32_t e4m3x4_and_residual(float (&x)[4]) {
     return (uint32_t)w;
 }
 
+// Sixteen bytes per lane from memory straight into LDS: lane L's land at dst + 16 L (dst is
+// wave-uniform). Issued as text: through the builtin the compiler makes every later LDS read wait
+// for the transfer, whichever buffer it reads. The caller waits (vmcnt) before the data is used.
+__device__ __forceinline__ void dma16(const uint8_t* src, lds_ptr<uint8_t> dst) {
+    const uint32_t base = (uint32_t)(uintptr_t)dst;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+}
+
 template <int TQ, int TP, bool SPARSE>
 __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int hb, int r_begin, int r_end,
                                                bool whole, float* pa, float* pml) {
-    __shared__ __attribute__((aligned(16))) uint8_t smem8[kF8SmemBytes];
-    const lds_ptr<uint8_t> tiles = (lds_ptr<uint8_t>)smem8;               // [2][128] rows of codes
-    const lds_ptr<uint8_t> zeros = tiles + 2 * kF8TileBytes;
-    const lds_ptr<float> sc = (lds_ptr<float>)(zeros + kF8ZeroBytes);     // [2][128] token scales (0 = not there)
-    const lds_ptr<float> sbias = sc + 2 * kF8Tile;                         // [2][128] 0 or -inf
-    const lds_ptr<unsigned long long> rowbase = (lds_ptr<unsigned long long>)(sbias + 2 * kF8Tile);  // [128] where a row's codes are
+    __shared__ __attribute__((aligned(16))) uint8_t smem8[kF8SmemBytes + f8_q_bytes<TQ>()];
+    const lds_ptr<uint8_t> tiles = (lds_ptr<uint8_t>)smem8;               // [2][64] rows of codes
+    const lds_ptr<uint8_t> zeros = tiles + kF8Bufs * kF8TileBytes;
+    const lds_ptr<float> sc = (lds_ptr<float>)(zeros + kF8ZeroBytes);     // [2][64] token scales (0 = not there)
+    const lds_ptr<float> sbias = sc + kF8Bufs * kF8Tile;                     // [2][64] 0 or -inf
+    const lds_ptr<unsigned long long> rowbase = (lds_ptr<unsigned long long>)(sbias + kF8Bufs * kF8Tile);  // [64] where a row's codes are
     const lds_ptr<int> tbl = (lds_ptr<int>)(rowbase + kF8Tile);
+    const lds_ptr<uint8_t> qlds = (lds_ptr<uint8_t>)(tbl + kTableLds);  // [TQ - 2][64 heads] rows of q codes
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -86,7 +112,8 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
 
     // ---- this wave's 16 query heads as e4m3 terms, for the whole kernel ----------------------
     // step s < 4: latent dims 128 s .. +127; step 4: the rope (its 64 dims in lane groups 0 and 1)
-    i32x8 qt[TQ][kF8Steps];
+    constexpr int TQR = TQ > 2 ? 2 : TQ;  // terms in (accumulation) registers; a third one lives in LDS
+    i32x8 qt[TQR ? TQR : 1][kF8Steps];
     int qscale_lo[TQ], qscale_hi[TQ];  // E8M0 scales: bytes 0..3 = steps 0..3, byte 0 of _hi = step 4
     {
         const int head = hb * 64 + 16 * wave + n16;
@@ -119,7 +146,12 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
 #pragma unroll
                 for (int c = 0; c < 8; ++c) {
                     float y[4] = {x[4 * c], x[4 * c + 1], x[4 * c + 2], x[4 * c + 3]};
-                    qt[t][s][c] = (int)e4m3x4_and_residual(y);
+                    const uint32_t w4 = e4m3x4_and_residual(y);
+                    int qa;
+                    asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(qa) : "v"(w4));
+                    if (t < TQR) qt[t < TQR ? t : 0][s][c] = qa;
+                    else if (s < 4 || g < 2)
+                        *(lds_ptr<uint32_t>)(qlds + ((t - TQR) * 64 + 16 * wave + n16) * kF8RowBytes + 128 * s + 32 * g + 4 * c) = w4;
                     // what is left over, at the next term's scale (16 times finer)
                     x[4 * c] = y[0] * 16.0f, x[4 * c + 1] = y[1] * 16.0f, x[4 * c + 2] = y[2] * 16.0f,
                     x[4 * c + 3] = y[3] * 16.0f;
@@ -137,13 +169,13 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         return (rel >= 0 && rel < tbl_count) ? tbl[rel] : table_g[blk];
     };
 
-    // ---- where the wave's 32 tokens of a tile are: lanes 0..31 resolve one each --------------
+    // ---- where the wave's 16 rows of a tile are: lanes 0..15 resolve one each ------------------
     constexpr unsigned long long kNone = ~0ull;
     const unsigned int* const rows_g = SPARSE ? a.rows + (size_t)seq * a.k : nullptr;
     auto resolve = [&](int t, unsigned long long& code_off, unsigned long long& scale_off) {
         code_off = kNone, scale_off = 0;
-        const int pos = r_begin + t * kF8Tile + 32 * wave + lane;
-        if (lane >= 32 || t >= n_tiles || pos >= r_end) return;
+        const int pos = r_begin + t * kF8Tile + kF8WaveRows * wave + lane;
+        if (lane >= kF8WaveRows || t >= n_tiles || pos >= r_end) return;
         const unsigned int tok = SPARSE ? rows_g[pos] : (unsigned)pos;
         unsigned int blk, off;
         if (a.page_shift >= 0) blk = tok >> a.page_shift, off = tok & (unsigned)(a.page_tokens - 1);
@@ -157,47 +189,74 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             atomicAdd(a.bad_rows, 1u);
         }
     };
-    // A tile goes from memory straight into LDS (global_load_lds, 16 bytes per lane, a wave's 64
-    // lanes filling 1 KiB of consecutive LDS): no registers hold it on the way. The wave's 32 rows
-    // of 37 granules (36 of codes + the padding one) are that consecutive range, so lane L of
-    // request I fills granule 64 I + L = row (64 I + L) / 37, granule (64 I + L) % 37 of the
-    // row, from wherever that row's page is. A row that is not there is zero-filled by hand: its
-    // codes must be finite, they meet a zero weight and a -inf bias, never a NaN.
-    float next_scale = 0.0f;  // lanes 0..31: the scale of the row this lane resolved
-    auto request_tile = [&](int t, int buf) {
+    // A tile goes from memory straight into LDS (16 bytes per lane, a wave's 64 lanes filling
+    // 1 KiB of consecutive LDS). The wave's 16 rows of 37 granules (36 of codes + the padding one)
+    // are that consecutive range, so lane L of request I fills granule 64 I + L = row
+    // (64 I + L) / 37, granule (64 I + L) % 37 of the row, from wherever that row's page is. A row
+    // that is not there is zero-filled by hand: its codes must be finite, they meet a zero weight
+    // and a -inf bias, never a NaN.
+    float next_scale = 0.0f;  // lanes 0..15: the scale of the row this lane resolved
+    // Dense fast path: the wave's 16 rows of a tile are 16 consecutive rows of one page (tiles
+    // start on multiples of 32 tokens and the page holds a multiple of 16), so granule 64 i +
+    // lane comes from byte goff[i] past the first of them: no lookups, one request per 1 KiB.
+    int goff[kF8Requests];
+#pragma unroll
+    for (int i = 0; i < kF8Requests; ++i) {
+        const int gi = min(kWave * i + lane, kF8WaveRows * kF8RowGranules - 1);
+        const int row = gi / kF8RowGranules, c = min(gi - row * kF8RowGranules, kRowW / 16 - 1);
+        goff[i] = row * kRowW + 16 * c;  // (the padding granule repeats the one before it)
+    }
+    const bool pages_hold_runs = !SPARSE && a.page_shift >= 4;
+    auto request_tile = [&](int t, lds_ptr<uint8_t> dst_tile) {
+        const lds_ptr<uint8_t> dst_w = dst_tile + (kF8WaveRows * wave) * kF8RowBytes;
+        if (pages_hold_runs) {
+            const int pos0 = r_begin + t * kF8Tile + kF8WaveRows * wave;
+            if (pos0 + kF8WaveRows <= r_end) {
+                const int blk = pos0 >> a.page_shift, off = pos0 & (a.page_tokens - 1);
+                const int page = blk < a.max_blocks ? __builtin_amdgcn_readfirstlane(table_at(blk)) : -1;
+                if ((unsigned)page < (unsigned)a.n_pages) {
+                    const uint8_t* const pg = a.pool + (size_t)page * a.page_bytes;
+                    const uint8_t* const src = pg + (size_t)off * kRowW;
+                    next_scale = 0.0f;
+                    if (lane < kF8WaveRows)
+                        next_scale = reinterpret_cast<const float*>(pg + (size_t)a.page_tokens * kRowW)[off + lane];
+#pragma unroll
+                    for (int i = 0; i < kF8Requests; ++i)
+                        if (kWave * (i + 1) <= kF8WaveRows * kF8RowGranules || lane < kF8WaveRows * kF8RowGranules - kWave * i)
+                            dma16(src + goff[i], dst_w + 1024 * i);
+                    return;
+                }
+            }
+        }
         unsigned long long code_off, scale_off;
         resolve(t, code_off, scale_off);
-        if (lane < 32) rowbase[32 * wave + lane] = code_off;
+        if (lane < kF8WaveRows) rowbase[kF8WaveRows * wave + lane] = code_off;
         next_scale = 0.0f;
         if (code_off != kNone) next_scale = *reinterpret_cast<const float*>(a.pool + scale_off);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-        const lds_ptr<uint8_t> dst0 = tiles + buf * kF8TileBytes + (32 * wave) * kF8RowBytes;
-        // (the per-request row and granule depend only on the lane: recomputed here each time
-        // rather than kept live across the whole tile loop, where they would cost ~60 registers)
-        int ln = lane;
-        asm volatile("" : "+v"(ln));
+        const lds_ptr<uint8_t> dst0 = dst_w;
 #pragma unroll
-        for (int i = 0; i < (32 * kF8RowGranules + kWave - 1) / kWave; ++i) {
+        for (int i = 0; i < kF8Requests; ++i) {
+            int ln = lane;
+            asm volatile("" : "+v"(ln));  // (kept out of the registers that live across the tile loop)
             const int gi = kWave * i + ln;
             const int row = gi / kF8RowGranules, c = gi - row * kF8RowGranules;
-            if (row < 32 && c < kRowW / 16) {
-                const unsigned long long base = rowbase[32 * wave + row];
+            if (row < kF8WaveRows && c < kRowW / 16) {
+                const unsigned long long base = rowbase[kF8WaveRows * wave + row];
                 if (base != kNone) {
-                    __builtin_amdgcn_global_load_lds(
-                        (const __attribute__((address_space(1))) void*)(a.pool + base + 16 * c),
-                        (__attribute__((address_space(3))) void*)(dst0 + 1024 * i), 16, 0, 0);
+                    dma16(a.pool + base + 16 * c, dst0 + 1024 * i);
                 } else {
-                    *(lds_ptr<u32x4>)(dst0 + 16 * gi) = u32x4{0, 0, 0, 0};
+                    *(lds_ptr<u32x4>)(dst0 + 16 * (kWave * i + lane)) = u32x4{0, 0, 0, 0};
                 }
             }
         }
     };
     auto publish_scales = [&](int buf) {  // the scales of the tile request_tile last asked for
-        if (lane < 32) {
+        if (lane < kF8WaveRows) {
             const bool ok = next_scale > 0.0f;  // a token that is not there has scale 0
-            sc[buf * kF8Tile + 32 * wave + lane] = ok ? next_scale : 0.0f;
-            sbias[buf * kF8Tile + 32 * wave + lane] = ok ? 0.0f : -INFINITY;
+            sc[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? next_scale : 0.0f;
+            sbias[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? 0.0f : -INFINITY;
         }
     };
 
@@ -206,14 +265,15 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     // (lane groups 2 and 3) reads zeros
     const int a_row = n16 * kF8RowBytes + 32 * g;
     const bool rope_zero = g >= 2;
+    const int q_row = (16 * wave + n16) * kF8RowBytes + 32 * g;
     // values: transposing load r (of 4) hands this lane bytes 8 r .. 8 r + 7 of its operand = the
     // tokens 16 (2 r + e / 4) + 4 g + e % 4, e = 0..7, of column 16 nt + n16; source lane pair e
     // addresses token e's row, its two lanes the two 8-byte halves of the 16 columns.
-    int v_off[4];
+    int v_off[2];
     {
         const int e = n16 >> 1;
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+        for (int r = 0; r < 2; ++r)
             v_off[r] = (16 * (2 * r + (e >> 2)) + 4 * g + (e & 3)) * kF8RowBytes + 8 * (n16 & 1);
     }
 
@@ -223,68 +283,81 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     float m_ref = -INFINITY, l_sum = 0.0f;
 
     // prologue: tile 0 into LDS
-    request_tile(0, 0);
+    request_tile(0, tiles);
     publish_scales(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     for (int t = 0; t < n_tiles; ++t) {
         const int buf = t & 1;
-        const lds_ptr<uint8_t> tile = tiles + buf * kF8TileBytes;
+        const lds_ptr<uint8_t> tile = tiles + buf * kF8TileBytes, next = tiles + (buf ^ 1) * kF8TileBytes;
         const lds_ptr<float> sc_t = sc + buf * kF8Tile, sbias_t = sbias + buf * kF8Tile;
         // tile t + 1 starts on its way into the other buffer (which held tile t - 1: every wave
         // left it before the barrier that ended the previous iteration)
-        if (t + 1 < n_tiles) request_tile(t + 1, buf ^ 1);
+        if (t + 1 < n_tiles) request_tile(t + 1, next);
 
         // ---- scores: S^T[token][head] over the five K-steps ---------------------------------
-        f32x4 acc[8];
+        // A K-step's four operand fragments are requested while the matrix instructions of the
+        // step before run; the scheduling fences keep that order.
+        f32x4 acc[kF8RowBlocks];
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb) acc[mb] = f32x4{0, 0, 0, 0};
-        // Operand fragments are requested four row blocks at a time, ahead of the matrix
-        // instructions that consume them; the scheduling fences keep the compiler from hoisting
-        // every step's reads to the top (and spilling them).
+        for (int mb = 0; mb < kF8RowBlocks; ++mb) acc[mb] = f32x4{0, 0, 0, 0};
+        i32x8 af[2][2], qf[2][TQ > TQR ? TQ - TQR : 1];
+        auto read32 = [&](lds_ptr<uint8_t> src) -> i32x8 {
+            const u32x4 lo4 = *(lds_ptr<u32x4>)(src), hi4 = *(lds_ptr<u32x4>)(src + 16);
+            return i32x8{(int)lo4.x, (int)lo4.y, (int)lo4.z, (int)lo4.w, (int)hi4.x, (int)hi4.y, (int)hi4.z, (int)hi4.w};
+        };
+        // unit u: K-step u / 2, row blocks 2 (u & 1) + {0, 1}; a step's q fragments come with its first unit
+        auto load_unit = [&](int u) {
+            const int s = u >> 1;
+            const bool z = s == 4 && rope_zero;
 #pragma unroll
-        for (int s = 0; s < kF8Steps; ++s) {
+            for (int j = 0; j < 2; ++j)
+                af[u & 1][j] = read32(z ? zeros : tile + (2 * (u & 1) + j) * 16 * kF8RowBytes + a_row + 128 * s);
+            if ((u & 1) == 0) {
 #pragma unroll
-            for (int m0 = 0; m0 < 8; m0 += 4) {
-                i32x8 af[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const lds_ptr<uint8_t> src =
-                        (s == 4 && rope_zero) ? zeros : tile + (m0 + j) * 16 * kF8RowBytes + a_row + 128 * s;
-                    const u32x4 lo4 = *(lds_ptr<u32x4>)(src), hi4 = *(lds_ptr<u32x4>)(src + 16);
-                    af[j] = i32x8{(int)lo4.x, (int)lo4.y, (int)lo4.z, (int)lo4.w, (int)hi4.x, (int)hi4.y, (int)hi4.z, (int)hi4.w};
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int tq = 0; tq < TQ; ++tq)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const int mb = m0 + j;
-                        if (s == 0)
-                            acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[j], qt[tq][0], acc[mb], 0, 0, 0, kScaleOne, 0, qscale_lo[tq]);
-                        else if (s == 1)
-                            acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[j], qt[tq][1], acc[mb], 0, 0, 0, kScaleOne, 1, qscale_lo[tq]);
-                        else if (s == 2)
-                            acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[j], qt[tq][2], acc[mb], 0, 0, 0, kScaleOne, 2, qscale_lo[tq]);
-                        else if (s == 3)
-                            acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[j], qt[tq][3], acc[mb], 0, 0, 0, kScaleOne, 3, qscale_lo[tq]);
-                        else
-                            acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[j], qt[tq][4], acc[mb], 0, 0, 0, kScaleOne, 0, qscale_hi[tq]);
-                    }
-                __builtin_amdgcn_sched_barrier(0);
+                for (int tq = 0; tq < TQ - TQR; ++tq)
+                    qf[s & 1][tq] = read32(z ? zeros : qlds + tq * 64 * kF8RowBytes + q_row + 128 * s);
             }
+        };
+        load_unit(0);
+#pragma unroll
+        for (int u = 0; u < 2 * kF8Steps; ++u) {
+            __builtin_amdgcn_s_waitcnt(kWaitLds0);  // this unit's fragments are in
+            __builtin_amdgcn_sched_barrier(0);
+            if (u + 1 < 2 * kF8Steps) load_unit(u + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            const int s = u >> 1;
+#pragma unroll
+            for (int tq = 0; tq < TQ; ++tq)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const i32x8 fa = af[u & 1][j], fq = tq < TQR ? qt[tq < TQR ? tq : 0][s] : qf[s & 1][tq < TQR ? 0 : tq - TQR];
+                    const int mb = 2 * (u & 1) + j;
+                    if (s == 0)
+                        acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa, fq, acc[mb], 0, 0, 0, kScaleOne, 0, qscale_lo[tq]);
+                    else if (s == 1)
+                        acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa, fq, acc[mb], 0, 0, 0, kScaleOne, 1, qscale_lo[tq]);
+                    else if (s == 2)
+                        acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa, fq, acc[mb], 0, 0, 0, kScaleOne, 2, qscale_lo[tq]);
+                    else if (s == 3)
+                        acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa, fq, acc[mb], 0, 0, 0, kScaleOne, 3, qscale_lo[tq]);
+                    else
+                        acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa, fq, acc[mb], 0, 0, 0, kScaleOne, 0, qscale_hi[tq]);
+                }
+            __builtin_amdgcn_sched_barrier(0);
         }
 
-        // ---- online softmax over the lane's 32 tokens of head n16: tokens 16 mb + 4 g + i ----
+        // ---- online softmax over the lane's 16 tokens of head n16: tokens 16 mb + 4 g + i ----
         float tmax = -INFINITY;
+        f32x4 s4[kF8RowBlocks];
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb) {
-            const f32x4 s4 = *(lds_ptr<f32x4>)(sc_t + 16 * mb + 4 * g);
+        for (int mb = 0; mb < kF8RowBlocks; ++mb) {
+            s4[mb] = *(lds_ptr<f32x4>)(sc_t + 16 * mb + 4 * g);
             const f32x4 b4 = *(lds_ptr<f32x4>)(sbias_t + 16 * mb + 4 * g);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                acc[mb][i] = __builtin_fmaf(acc[mb][i], s4[i], b4[i]);  // -inf where the token is not there
+                acc[mb][i] = __builtin_fmaf(acc[mb][i], s4[mb][i], b4[i]);  // -inf where the token is not there
                 tmax = fmaxf(tmax, acc[mb][i]);
             }
         }
@@ -306,60 +379,58 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         // weights w_t = 2^(v_t - mu) * s_t, as TP e4m3 terms under one scale per (head, tile)
         float wmax = 0.0f;
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb) {
-            const f32x4 s4 = *(lds_ptr<f32x4>)(sc_t + 16 * mb + 4 * g);
+        for (int mb = 0; mb < kF8RowBlocks; ++mb)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                acc[mb][i] = __builtin_amdgcn_exp2f(acc[mb][i] - mu) * s4[i];  // not there -> 0
+                acc[mb][i] = __builtin_amdgcn_exp2f(acc[mb][i] - mu) * s4[mb][i];  // not there -> 0
                 wmax = fmaxf(wmax, acc[mb][i]);
             }
-        }
         wmax = rows_max(wmax);
         const int pe = block_exp(wmax);
-        const float pinv = pow2i(-pe);
-        // what one unit of the last residual is worth: 2^pe / 16^(TP - 1)
-        const float last_unit = pow2i(pe - 4 * (TP - 1));
-        i32x8 pt[TP];
-        int pscale[TP];
+        const float pinv = pow2i(-pe), unit = pow2i(pe - 4);  // what one unit of the second term is worth
+        i32x8 pt;  // bytes 0..15: the first term of the lane's 16 tokens, 16..31: the second
+        // (the instruction takes K block b's scale from lane 16 b + row: blocks 0, 1 are the
+        // first term of lane groups 0,1 / 2,3, blocks 2, 3 the second term, 16 times finer)
+        const int pscale = (int)((uint32_t)max(pe - 4 * (g >> 1) + 127, 1) * 0x01010101u);
 #pragma unroll
-        for (int tp = 0; tp < TP; ++tp) pscale[tp] = (int)((uint32_t)max(pe - 4 * tp + 127, 1) * 0x01010101u);
-#pragma unroll
-        for (int mb = 0; mb < 8; ++mb) {
-            const f32x4 s4 = *(lds_ptr<f32x4>)(sc_t + 16 * mb + 4 * g);
+        for (int mb = 0; mb < kF8RowBlocks; ++mb) {
             float y[4] = {acc[mb][0] * pinv, acc[mb][1] * pinv, acc[mb][2] * pinv, acc[mb][3] * pinv};
+            pt[mb] = (int)e4m3x4_and_residual(y);
 #pragma unroll
-            for (int tp = 0; tp < TP; ++tp) {
-                pt[tp][mb] = (int)e4m3x4_and_residual(y);
-                if (tp + 1 < TP) y[0] *= 16.0f, y[1] *= 16.0f, y[2] *= 16.0f, y[3] *= 16.0f;
-            }
+            for (int i = 0; i < 4; ++i) y[i] *= 16.0f;
+            pt[4 + mb] = (int)e4m3x4_and_residual(y);
             // The denominator sums the weights the numerator really holds (w_t less the last
             // residual), over the token scale: the result is an exactly normalised average under
-            // weights perturbed by 2^-4TP each.
+            // weights perturbed by 2^-8 each.
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float held = acc[mb][i] - y[i] * last_unit;
-                l_sum += s4[i] > 0.0f ? held * __builtin_amdgcn_rcpf(s4[i]) : 0.0f;
+                const float held = acc[mb][i] - y[i] * unit;
+                l_sum += s4[mb][i] > 0.0f ? held * __builtin_amdgcn_rcpf(s4[mb][i]) : 0.0f;
             }
         }
 
         // ---- values: O[head][col] += P . V over all 512 columns -------------------------------
+        static_assert(TP == 2, "two terms fill the value contraction's K exactly");
+        constexpr int CU = 4;  // column tiles per unit
+        i32x8 vf[2][CU];
+        auto load_cols = [&](int n0, i32x8 (&f)[CU]) {
 #pragma unroll
-        for (int n0 = 0; n0 < kF8ColTiles; n0 += 4) {
-            i32x8 vf[4];
+            for (int j = 0; j < CU; ++j) {
+                const i32x2 r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr<i32x2>)(tile + v_off[0] + 16 * (n0 + j)));
+                const i32x2 r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr<i32x2>)(tile + v_off[1] + 16 * (n0 + j)));
+                f[j] = i32x8{r0[0], r0[1], r1[0], r1[1], r0[0], r0[1], r1[0], r1[1]};
+            }
+        };
+        load_cols(0, vf[0]);
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const i32x2 two =
-                        __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr<i32x2>)(tile + v_off[r] + 16 * (n0 + j)));
-                    vf[j][2 * r] = two[0], vf[j][2 * r + 1] = two[1];
-                }
+        for (int n0 = 0; n0 < kF8ColTiles; n0 += CU) {
+            __builtin_amdgcn_s_waitcnt(kWaitLds0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (n0 + CU < kF8ColTiles) load_cols(n0 + CU, vf[((n0 / CU) + 1) & 1]);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int tp = 0; tp < TP; ++tp)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    o[n0 + j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pt[tp], vf[j], o[n0 + j], 0, 0, 0, pscale[tp], 0, kScaleOne);
+            for (int j = 0; j < CU; ++j)
+                o[n0 + j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pt, vf[(n0 / CU) & 1][j], o[n0 + j], 0, 0, 0, pscale, 0, kScaleOne);
             __builtin_amdgcn_sched_barrier(0);
         }
 
