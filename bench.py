@@ -60,7 +60,9 @@ def parse():
     ap.add_argument("--heads", type=int, default=64, help="attend: query heads")
     ap.add_argument("--precise", type=int, default=2, choices=[0, 1, 2, 3, 4],
                     help="attend: 2 = q and softmax weights as bf16 hi+lo (parity mode), "
-                         "1 = q only, 0 = plain bf16")
+                         "1 = q only, 0 = plain bf16; on the 8-bit matrix instructions: 4 = q as three "
+                         "e4m3 terms and the weights as two (inside the reference's bar), 3 = two and two "
+                         "(bf16-class)")
     ap.add_argument("--ragged", action="store_true",
                     help="decode / attend: per-sequence context drawn uniformly from [1024, ctx] "
                          "(configuration 3 as written) instead of every sequence at ctx (its metric point)")
@@ -121,7 +123,11 @@ def main():
               ("cfg4_dsa", "dsa", dict(cpu_seconds=short)),
               ("cfg4_dsa_scored", "dsa_scored", {}),
               ("cfg2_prefill_8192", "prefill", dict(tokens=8192, cpu_seconds=short)),
-              ("cfg2_prefill_1048576", "prefill", dict(tokens=1048576, cpu_seconds=short)))
+              ("cfg2_prefill_1048576", "prefill", dict(tokens=1048576, cpu_seconds=short)),
+              # the cache's consumer at configuration 3's shape: inside the reference's own bar on
+              # the 8-bit matrix instructions, and the tighter bf16 hi + lo mode
+              ("attend_decode", "attend", dict(precise=4)),
+              ("attend_decode_bf16x2", "attend", dict(precise=2)))
     res["configs"] = {}
     for name, workload, over in others:
         torch.cuda.empty_cache()
@@ -872,7 +878,7 @@ def bench_attend(a, torch, hip):
         torch.cuda.synchronize()
         got = clat.cpu().numpy()[:ns]
         err, mx = float(np.abs(got - want).max()), float(np.abs(want).max())
-        bar = {2: 1e-4, 1: 2e-3, 0: 3e-2, 3: 3e-2, 4: 2e-3}[a.precise] * mx
+        bar = {2: 1e-4, 1: 2e-3, 0: 3e-2, 3: 3e-2, 4: 1e-3}[a.precise] * mx
         if not err <= bar:
             raise SystemExit(f"bench: GPU attention differs from the CPU oracle: err={err:.3e} max={mx:.3e}")
         sample_bytes = ns * cut * REC + ns * H * (W + KVL) * 4
