@@ -81,7 +81,11 @@ __device__ __forceinline__ uint32_t e4m3x4_and_residual(float (&x)[4]) {
 // for the transfer, whichever buffer it reads. The caller waits (vmcnt) before the data is used.
 __device__ __forceinline__ void dma16(const uint8_t* src, lds_ptr<uint8_t> dst) {
     const uint32_t base = (uint32_t)(uintptr_t)dst;
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+    uint32_t keep;  // m0 is the instruction's LDS base; the compiler's own value of it is put back
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(keep)
+                 : "v"(src), "s"(base)
+                 : "memory");
 }
 
 template <int TQ, int TP, bool SPARSE>
