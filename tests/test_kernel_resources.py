@@ -1,0 +1,41 @@
+"""The 8-bit attention kernels' register budget is part of their design: one wave per SIMD with
+the whole register file, 128 accumulators in ordinary registers, two q terms in the accumulation
+registers (rivoli_amd/csrc/mla_attend_f8.hpp). A compiler or source change that makes them spill
+still gives right answers, only several times slower, so the build's own resource report is held
+to "no scratch memory" here. Compiles one file; needs hipcc, no GPU."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+from rivoli_amd import build
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.skipif(shutil.which(build.hipcc()) is None, reason="hipcc not found")
+def test_eight_bit_attention_kernels_do_not_spill(tmp_path):
+    src = os.path.join(build.CSRC, "mla_attend.hip")
+    cmd = [build.hipcc(), f"--offload-arch={build.offload_arch()}", "-O3", "-std=c++17", "-fPIC",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I", os.path.join(ROOT, "include")] + build.EXTRA_FLAGS.get("mla_attend.hip", []) + \
+          ["-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", str(tmp_path / "m.o")]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    # remarks come in blocks: "Function Name: <mangled>" followed by that kernel's figures
+    blocks = re.split(r"remark: Function Name: ", res.stderr)[1:]
+    seen = 0
+    for b in blocks:
+        name = b.split()[0]
+        if "mla_attend_paged_kernel" not in name or not name.endswith("Lb1EEEvNS_10AttendArgsE"):
+            continue  # the last template argument (true) marks the 8-bit kernels
+        seen += 1
+        scratch = int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b).group(1))
+        occupancy = int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", b).group(1))
+        lds = int(re.search(r"LDS Size \[bytes/block\]: (\d+)", b).group(1))
+        assert scratch == 0, f"{name} spills {scratch} bytes per lane"
+        assert occupancy == 1, name
+        assert lds <= 160 * 1024, name
+    assert seen == 4, f"expected the dense and row-list kernels of both 8-bit modes, saw {seen}"
