@@ -241,7 +241,9 @@ launchers! {
     /// `launch_attend` for a whole decode batch over the paged fp8 cache, dense (`rows`
     /// null, `seq_lens` given) or over DSA row lists (`rows[s*max_rows + j]`, `j <
     /// n_rows[s]`). `partial`: [`attend_paged_scratch_floats`] floats, or null when that is 0.
-    /// `precise`: 2 = q and softmax weights as bf16 hi + lo (parity), 1 = q only, 0 = bf16.
+    /// `precise`: 2 = q and softmax weights as bf16 hi + lo (parity), 1 = q only, 0 = bf16;
+    /// 4 / 3 = both contractions on the 8-bit matrix instructions (q as three / two e4m3 terms):
+    /// the fastest modes, 4 inside the reference's bar for this kernel.
     launch_attend_paged -> rivoli_mla_attend_paged, "mla_attend_paged" (
         qabs: *const f32,
         qrope: *const f32,
