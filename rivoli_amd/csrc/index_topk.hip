@@ -1106,14 +1106,43 @@ __device__ __forceinline__ void select_bisect(const float* __restrict__ s, int n
     const int rem = nt - seg0;
     const int limit = (rem < per_wave ? rem : per_wave) - lane;  // element j exists iff j*64 < limit
 
+    // Every load of the row is in flight before the first is used: an element past the row's
+    // end reads the row's last score instead (and becomes key 0), because a load under a
+    // per-lane condition is a branch with a wait of its own — 32 memory round trips in a row.
+    // The wave-uniform choice among 8, 16, 24 or 32 loads keeps short rows from paying for
+    // long ones; each arm is straight-line code.
     uint32_t key[ITEMS];
     {
-        const float* sp = s + seg0 + lane;
+        float v[ITEMS];
+        const uint32_t first = (uint32_t)(seg0 + lane), last = (uint32_t)(nt - 1);
+        auto fetch = [&](auto n_tag) {
+            constexpr int N = decltype(n_tag)::value;
 #pragma unroll
-        for (int j = 0; j < ITEMS; ++j)
-            key[j] = j * kWave < limit ? KEY::of(sp[j * kWave]) : 0u;
+            for (int j = 0; j < ITEMS; ++j)
+                v[j] = j < N ? s[min(first + (uint32_t)(j * kWave), last)] : 0.0f;
+        };
+        if (ITEMS <= 8 || steps > 24)
+            fetch(std::integral_constant<int, ITEMS>{});
+        else if (steps > 16)
+            fetch(std::integral_constant<int, 24>{});
+        else if (steps > 8)
+            fetch(std::integral_constant<int, 16>{});
+        else
+            fetch(std::integral_constant<int, 8>{});
+        // ---- the top kSelBits of the k-th largest key, by one LDS histogram -------------------
+        // (sign, exponent and the first mantissa bit of a score): one atomic per key instead
+        // of a bisection step per bit. The atomic sits with the key's conversion so that the
+        // per-element "exists" masks do not stay live (32 of them overflow the scalar file).
+        __syncthreads();  // the histogram is clear (the loads above are in flight meanwhile)
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            key[j] = 0u;
+            if (j * kWave < limit) {
+                key[j] = KEY::of(v[j]);
+                atomicAdd(&lds[kSelMisc + (key[j] >> kSelLow)], 1u);
+            }
+        }
     }
-    __syncthreads();  // the histogram is clear
     // keys >= cand over the whole row, cand >= 1 (so the zero keys of absent elements never
     // count). `turn` alternates the LDS slots so that one barrier per call is enough.
     auto count_ge = [&](uint32_t cand, int turn) -> uint32_t {
@@ -1139,19 +1168,9 @@ __device__ __forceinline__ void select_bisect(const float* __restrict__ s, int n
         return c;
     };
 
-    // ---- the top kSelBits of the k-th largest key, by one LDS histogram -----------------------
-    // (sign, exponent and the first mantissa bit of a score): one atomic per key instead of a
-    // bisection step per bit. s_hist was cleared and a barrier passed before this point.
     uint32_t* s_hist = lds + kSelMisc;
     uint32_t* s_cand = s_hist;  // the list reuses the histogram once the pivot bin is known
     uint32_t* s_pv = lds + 4 * WAVES;  // [0] pivot bin, [1] keys in higher bins, [2] keys in it, [3] list fill
-#pragma unroll
-    for (int j0 = 0; j0 < ITEMS; j0 += 8) {
-        if (j0 >= steps) break;
-#pragma unroll
-        for (int j = j0; j < j0 + 8 && j < ITEMS; ++j)
-            if (j * kWave < limit) atomicAdd(&s_hist[key[j] >> kSelLow], 1u);
-    }
     __syncthreads();
     if (wave == 0) {
         // a lane owns 16 consecutive bins; suffix sums over the lanes find the lane where the
@@ -1188,9 +1207,13 @@ __device__ __forceinline__ void select_bisect(const float* __restrict__ s, int n
 
     // T: select key > T, and the first `need` (in index order) of key == T
     uint32_t T = 0, need = 0;
+    // Absent elements hold key 0, which no test below can tell from a live key 0 — and none has
+    // to: they sit past every live element in index order, and kq < nt leaves at least one live
+    // key unselected, so ties at the threshold are used up before an absent element's turn. Only
+    // the list must not meet them (the histogram did not count them), hence pbin != 0 there.
     if (need_in_bin == in_bin) {
         T = (pbin << kSelLow) - 1u;  // the whole bin is selected (pbin == 0 would need every key: kq < nt)
-    } else if (in_bin <= (uint32_t)kSelCand) {
+    } else if (pbin != 0u && in_bin <= (uint32_t)kSelCand) {
         // ---- the other bits among the bin's members only: they are listed (any order) in LDS
         // and one wave bisects them from registers
         uint32_t fill = 0;  // where this wave's members start in the list
@@ -1201,7 +1224,7 @@ __device__ __forceinline__ void select_bisect(const float* __restrict__ s, int n
                 if (j0 >= steps) break;
 #pragma unroll
                 for (int j = j0; j < j0 + 8 && j < ITEMS; ++j)
-                    mine += (uint32_t)__popcll(__ballot(j * kWave < limit && (key[j] >> kSelLow) == pbin));
+                    mine += (uint32_t)__popcll(__ballot((key[j] >> kSelLow) == pbin));
             }
             uint32_t* s_cnt = lds;  // the count_ge slots are idle here
             if (lane == 0) s_cnt[wave] = mine;
@@ -1213,7 +1236,7 @@ __device__ __forceinline__ void select_bisect(const float* __restrict__ s, int n
             if (j0 >= steps) break;
 #pragma unroll
             for (int j = j0; j < j0 + 8 && j < ITEMS; ++j) {
-                const bool is = j * kWave < limit && (key[j] >> kSelLow) == pbin;
+                const bool is = (key[j] >> kSelLow) == pbin;
                 const unsigned long long m = __ballot(is);
                 if (is) s_cand[fill + lanes_below(m)] = key[j];
                 fill += (uint32_t)__popcll(m);
@@ -1281,18 +1304,26 @@ __device__ __forceinline__ void select_bisect(const float* __restrict__ s, int n
         }
     }
 
-    uint32_t cnt_gt = 0, cnt_eq = 0;
-    if constexpr (WAVES > 1) {
-#pragma unroll
-        for (int j = 0; j < ITEMS; ++j) {
-            const bool live = j * kWave < limit;
-            cnt_gt += live && key[j] > T ? 1u : 0u;
-            cnt_eq += live && key[j] == T ? 1u : 0u;
-        }
-    }
+    // ---- emission in index order. A wave's share of the selection comes from ballots (scalar
+    // popcounts), and its compares are kept apart from the emission's by passing T through an
+    // empty asm: shared, their 64 masks would have to stay live across the exchange.
+    T = __builtin_amdgcn_readfirstlane(T);  // the same in every lane: say so to the compiler
+    need = __builtin_amdgcn_readfirstlane(need);
+    const bool ties = need != 0u;  // distinct keys end the bisection on an exact count: need == 0
     uint32_t run_gt = 0, run_eq = 0;
     if constexpr (WAVES > 1) {
-        const uint32_t gt_total = wave_sum(cnt_gt), eq_total = wave_sum(cnt_eq);
+        uint32_t Tc = T;
+        asm volatile("" : "+s"(Tc));
+        uint32_t gt_total = 0, eq_total = 0;
+#pragma unroll
+        for (int j0 = 0; j0 < ITEMS; j0 += 8) {
+            if (j0 >= steps) break;
+#pragma unroll
+            for (int j = j0; j < j0 + 8 && j < ITEMS; ++j) {
+                gt_total += (uint32_t)__popcll(__ballot(key[j] > Tc));
+                if (ties) eq_total += (uint32_t)__popcll(__ballot(key[j] == Tc));
+            }
+        }
         uint32_t* s_gt = lds + 2 * WAVES;
         uint32_t* s_eq = s_gt + WAVES;
         if (lane == 0) {
@@ -1305,28 +1336,37 @@ __device__ __forceinline__ void select_bisect(const float* __restrict__ s, int n
             run_eq += s_eq[w];
         }
     }
+    // slot < kq holds by construction; the compare keeps a wrong threshold from ever turning
+    // into a write outside the caller's buffer
+    if (!ties) {
+#pragma unroll
+        for (int j0 = 0; j0 < ITEMS; j0 += 8) {
+            if (j0 >= steps) break;
+#pragma unroll
+            for (int j = j0; j < j0 + 8 && j < ITEMS; ++j) {
+                const bool g = key[j] > T;
+                const unsigned long long mg = __ballot(g);
+                const uint32_t slot = run_gt + lanes_below(mg);
+                if (g && slot < kq) out[slot] = (uint32_t)(seg0 + j * kWave + lane) + add;
+                run_gt += (uint32_t)__popcll(mg);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j0 = 0; j0 < ITEMS; j0 += 8) {
         if (j0 >= steps) break;
 #pragma unroll
         for (int j = j0; j < j0 + 8 && j < ITEMS; ++j) {
-            const bool live = j * kWave < limit;
-            const bool g = live && key[j] > T;
-            const bool e = live && key[j] == T;
+            const bool g = key[j] > T;
+            const bool e = key[j] == T;
             const unsigned long long mg = __ballot(g), me = __ballot(e);
             const uint32_t G = run_gt + lanes_below(mg);
-            // slot < kq holds by construction; the compare keeps a wrong threshold from ever
-            // turning into a write outside the caller's buffer
-            if (me == 0ull) {  // no key equal to the threshold in this step: the usual case
-                const uint32_t slot = G + (run_eq < need ? run_eq : need);
-                if (g && slot < kq) out[slot] = (uint32_t)(seg0 + j * kWave + lane) + add;
-            } else {
-                const uint32_t E = run_eq + lanes_below(me);
-                const uint32_t slot = G + (E < need ? E : need);
-                if ((g || (e && E < need)) && slot < kq)
-                    out[slot] = (uint32_t)(seg0 + j * kWave + lane) + add;
-                run_eq += (uint32_t)__popcll(me);
-            }
+            const uint32_t E = run_eq + lanes_below(me);
+            const uint32_t slot = G + (E < need ? E : need);
+            if ((g || (e && E < need)) && slot < kq)
+                out[slot] = (uint32_t)(seg0 + j * kWave + lane) + add;
+            run_eq += (uint32_t)__popcll(me);
             run_gt += (uint32_t)__popcll(mg);
         }
     }
