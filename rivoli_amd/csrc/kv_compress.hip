@@ -74,33 +74,36 @@ __device__ __forceinline__ Entry state_entry(const float* kv_state, const float*
 }
 
 // Softmax over the entries of VEC features starting at e, then the weighted sum
-// (kvcompress.hip:117-150), from registers.
+// (kvcompress.hip:117-150), from registers. Every load of the window is issued before the
+// first is used: a masked entry (and a missing embedding) reads `safe` instead — any address
+// that holds a feature row — and is dropped afterwards. A load under a condition, even a
+// workgroup-uniform one, compiles to a branch that waits for its own data: one memory round
+// trip per entry, one after the other.
 template <int VEC, int SLOTS, class GetEntry>
-__device__ __forceinline__ void pool_registers(GetEntry&& entry, int ents, int e, float (&out)[VEC]) {
+__device__ __forceinline__ void pool_registers(GetEntry&& entry, const float* safe, int ents, int e,
+                                               float (&out)[VEC]) {
     static_assert(SLOTS <= kCompRegEnts, "register windows are short");
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
     float v[SLOTS][VEC], k[SLOTS][VEC];
     bool live[SLOTS];
+    {
+        vec_t s_raw[SLOTS], k_raw[SLOTS], a_raw[SLOTS];
+        bool emb[SLOTS];
 #pragma unroll
-    for (int j = 0; j < SLOTS; ++j) {
-        live[j] = false;
-        if (j < ents) {
-            const Entry en = entry(j);
+        for (int j = 0; j < SLOTS; ++j) {
+            const Entry en = j < ents ? entry(j) : Entry{nullptr, nullptr, nullptr};
             live[j] = en.sc != nullptr;
-            if (live[j]) {
-                if constexpr (VEC == 4) {
-                    const f32x4 s4 = *reinterpret_cast<const f32x4*>(en.sc + e);
-                    const f32x4 k4 = *reinterpret_cast<const f32x4*>(en.kv + e);
-                    f32x4 a4 = {0, 0, 0, 0};
-                    if (en.ape) a4 = *reinterpret_cast<const f32x4*>(en.ape + e);
+            emb[j] = live[j] && en.ape != nullptr;
+            s_raw[j] = *reinterpret_cast<const vec_t*>((live[j] ? en.sc : safe) + e);
+            k_raw[j] = *reinterpret_cast<const vec_t*>((live[j] ? en.kv : safe) + e);
+            a_raw[j] = *reinterpret_cast<const vec_t*>((emb[j] ? en.ape : safe) + e);
+        }
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        v[j][i] = en.ape ? s4[i] + a4[i] : s4[i] + 0.0f;
-                        k[j][i] = k4[i];
-                    }
-                } else {
-                    v[j][0] = en.sc[e] + (en.ape ? en.ape[e] : 0.0f);
-                    k[j][0] = en.kv[e];
-                }
+        for (int j = 0; j < SLOTS; ++j) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                v[j][i] = s_raw[j][i] + (emb[j] ? a_raw[j][i] : 0.0f);
+                k[j][i] = k_raw[j][i];
             }
         }
     }
@@ -109,7 +112,7 @@ __device__ __forceinline__ void pool_registers(GetEntry&& entry, int ents, int e
         float mx = -INFINITY;
 #pragma unroll
         for (int j = 0; j < SLOTS; ++j)
-            if (j < ents && live[j]) mx = fmaxf(mx, v[j][i]);
+            if (live[j]) mx = fmaxf(mx, v[j][i]);
         if (!isfinite(mx)) {  // every entry masked: a zero row, as the CPU statement has it
             out[i] = 0.0f;
             continue;
@@ -117,7 +120,7 @@ __device__ __forceinline__ void pool_registers(GetEntry&& entry, int ents, int e
         float ex[SLOTS], sum = 0.0f;
 #pragma unroll
         for (int j = 0; j < SLOTS; ++j) {
-            if (j < ents && live[j]) {
+            if (live[j]) {
                 ex[j] = expf(v[j][i] - mx);
                 sum += ex[j];
             }
@@ -125,7 +128,7 @@ __device__ __forceinline__ void pool_registers(GetEntry&& entry, int ents, int e
         float acc = 0.0f;
 #pragma unroll
         for (int j = 0; j < SLOTS; ++j)
-            if (j < ents && live[j]) acc += k[j][i] * (ex[j] / sum);
+            if (live[j]) acc += k[j][i] * (ex[j] / sum);
         out[i] = acc;
     }
 }
@@ -173,15 +176,26 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 // VEC == 4 requires d % 4 == 0 and 16-byte-aligned rows.
 // SLOTS: 8 or 16 = the window is held in that many register slots; 0 = streamed.
 template <int VEC, int SLOTS, class GetEntry>
-__device__ __forceinline__ void compress_row(GetEntry&& entry, const CompFinish& f, float* out_row,
+__device__ __forceinline__ void compress_row(GetEntry&& entry, const float* safe, const CompFinish& f, float* out_row,
                                              int pos, const CompGeom& p, float* row, float* red) {
     const int tid = threadIdx.x, nthr = blockDim.x;
+    // what the finishing steps read (this lane's first norm weights and rotation pair) is
+    // requested now, with the window, instead of one round trip after each barrier
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
+    const float* t = f.freqs + (size_t)pos * p.rd;
+    vec_t norm0 = 0.0f;
+    float cos0 = 0.0f, sin0 = 0.0f;
+    if (tid * VEC < p.d) norm0 = *reinterpret_cast<const vec_t*>(f.norm + tid * VEC);
+    if (tid < p.rd / 2) {
+        cos0 = t[2 * tid];
+        sin0 = t[2 * tid + 1];
+    }
     float ss = 0.0f;
     for (int e = tid * VEC; e < p.d; e += nthr * VEC) {
         float pooled[VEC];
         static_assert(VEC == 1 || VEC == 4, "one feature or four");
         if constexpr (SLOTS > 0) {
-            pool_registers<VEC, SLOTS>(entry, p.ents, e, pooled);
+            pool_registers<VEC, SLOTS>(entry, safe, p.ents, e, pooled);
         } else {
 #pragma unroll
             for (int i = 0; i < VEC; ++i) pooled[i] = pool_streamed(entry, p.ents, e + i);
@@ -197,13 +211,15 @@ __device__ __forceinline__ void compress_row(GetEntry&& entry, const CompFinish&
     const float rs = 1.0f / sqrtf(block_sum(ss, red) / (float)p.d + p.eps);
     for (int e = tid * VEC; e < p.d; e += nthr * VEC) {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) row[e + i] = rbf16(f.norm[e + i] * (row[e + i] * rs));
+        for (int i = 0; i < VEC; ++i) {
+            const float nw = e == tid * VEC ? norm0[i] : f.norm[e + i];
+            row[e + i] = rbf16(nw * (row[e + i] * rs));
+        }
     }
     __syncthreads();
-    const float* t = f.freqs + (size_t)pos * p.rd;
     float* seg = row + (p.d - p.rd);
     for (int i = tid; i < p.rd / 2; i += nthr) {
-        const float c = t[2 * i], s = t[2 * i + 1];
+        const float c = i == tid ? cos0 : t[2 * i], s = i == tid ? sin0 : t[2 * i + 1];
         const float a = seg[2 * i], b = seg[2 * i + 1];
         seg[2 * i] = rbf16(a * c - b * s);
         seg[2 * i + 1] = rbf16(a * s + b * c);
@@ -230,7 +246,7 @@ __global__ __launch_bounds__(SLOTS ? 256 : 1024) void kv_compress_prefill_kernel
     float* red = lds + p.d;
     const int b = blockIdx.x;
     auto entry = [&](int j) { return prefill_entry(kv, score, ape, p, b, j); };
-    compress_row<VEC, SLOTS>(entry, f, f.out + (size_t)b * p.d, b * p.ratio, p, row, red);
+    compress_row<VEC, SLOTS>(entry, score, f, f.out + (size_t)b * p.d, b * p.ratio, p, row, red);
 }
 
 // One workgroup: its barriers order the pooling's reads against the window slide.
@@ -242,7 +258,7 @@ __global__ __launch_bounds__(SLOTS ? 256 : 1024) void kv_compress_decode_kernel(
     float* red = lds + p.d;
     auto entry = [&](int j) { return state_entry(kv_state, score_state, p, j); };
     // the block's first absolute position, not its index (kvcompress.hip:360-371)
-    compress_row<VEC, SLOTS>(entry, f, f.out, (start_pos / p.ratio) * p.ratio, p, row, red);
+    compress_row<VEC, SLOTS>(entry, score_state, f, f.out, (start_pos / p.ratio) * p.ratio, p, row, red);
     __syncthreads();
     if (p.coff == 2) {
         // this block's normal half becomes the next block's overlap half
