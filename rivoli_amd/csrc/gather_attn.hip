@@ -99,25 +99,31 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
 
     // ---- a tile's slots: lanes 0..3 hold the wave's 4 list entries ------------------------
     const int my_pos0 = tile_pos_of(wave, 0);  // the wave's 4 slots are consecutive tile positions
-    auto list_entry = [&](int tile) -> int {
-        const int pos = (tile0 + tile) * kGaTile + my_pos0 + (lane & 3);
-        if (lane >= 4 || pos >= a.topk) return -1;
-        const int p = ix[pos];
-        return (unsigned)p < (unsigned)a.n_kv ? p : -1;
+    // The fetch is unconditional (a position past the list reads the list's last entry) and
+    // apart from the test of what it returns: a load under a per-lane condition compiles to a
+    // branch that waits for its own data, and that wait (vmcnt(0)) would also drain the rows
+    // requested for the tiles ahead — one exposed memory round trip per tile.
+    auto list_fetch = [&](int tile) -> int {
+        const long long pos = (long long)(tile0 + tile) * kGaTile + my_pos0 + (lane & 3);
+        return ix[pos < a.topk ? pos : a.topk - 1];
+    };
+    auto list_entry = [&](int tile, int p) -> int {
+        const long long pos = (long long)(tile0 + tile) * kGaTile + my_pos0 + (lane & 3);
+        return (tile < n_tiles && lane < 4 && pos < a.topk && (unsigned)p < (unsigned)a.n_kv) ? p : -1;
     };
     struct RawTile {
         float4 row[4][2];
         float bias;  // lanes 0..3: 0, or -inf for a masked slot
+        int live;    // bit i: row i was listed (a masked slot fetches row 0 and is staged as zeros)
     };
     auto issue_loads = [&](RawTile& r, int entry) {
+        r.live = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int p = __builtin_amdgcn_readlane(entry, i);
-            r.row[i][0] = float4{0, 0, 0, 0}, r.row[i][1] = float4{0, 0, 0, 0};
-            if (p >= 0) {
-                const float4* src = reinterpret_cast<const float4*>(a.kv + (size_t)p * kGaD) + 2 * lane;
-                r.row[i][0] = src[0], r.row[i][1] = src[1];
-            }
+            r.live |= (p >= 0 ? 1 : 0) << i;
+            const float4* src = reinterpret_cast<const float4*>(a.kv + (size_t)(p >= 0 ? p : 0) * kGaD) + 2 * lane;
+            r.row[i][0] = src[0], r.row[i][1] = src[1];
         }
         r.bias = entry >= 0 ? 0.0f : -INFINITY;
     };
@@ -130,8 +136,9 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
         const lds_ptr<uint8_t> krb = kr + buf * kGaTileBytes;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const u32x4 v = {pack2(r.row[i][0].x, r.row[i][0].y), pack2(r.row[i][0].z, r.row[i][0].w),
-                             pack2(r.row[i][1].x, r.row[i][1].y), pack2(r.row[i][1].z, r.row[i][1].w)};
+            u32x4 v = {pack2(r.row[i][0].x, r.row[i][0].y), pack2(r.row[i][0].z, r.row[i][0].w),
+                       pack2(r.row[i][1].x, r.row[i][1].y), pack2(r.row[i][1].z, r.row[i][1].w)};
+            if (!((r.live >> i) & 1)) v = u32x4{0u, 0u, 0u, 0u};
             *(lds_ptr<u32x4>)(krb + (my_pos0 + i) * kGaRowBytes + 16 * lane) = v;
         }
         if (lane < 4) sbias[buf * kGaTile + 4 * wave + lane] = r.bias;
@@ -142,13 +149,11 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
     // entries of tiles 0..3, the query (oldest request, so its wait leaves the rows in
     // flight), the rows of tiles 0 and 1. Then: query -> B-operand fragments, tiles 0 and 1
     // staged, tile 2 requested.
-    const int e0 = list_entry(0);
-    const int e1 = n_tiles > 1 ? list_entry(1) : -1;
-    const int e2 = n_tiles > 2 ? list_entry(2) : -1;
-    int entry_next = n_tiles > 3 ? list_entry(3) : -1;
+    const int f0 = list_fetch(0), f1 = list_fetch(1), f2 = list_fetch(2), f3 = list_fetch(3);
     // this wave's half of its 16 query heads as the B operand, for the whole kernel
     bf16x8 qh[kGaKStepsHalf], ql[QSPLIT == 2 ? kGaKStepsHalf : 1];
     RawTile raw;
+    raw.live = 0;
     {
         const int head = hb * 64 + 16 * hw + n16;
         const bool live = head < a.h;
@@ -157,9 +162,9 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
 #pragma unroll
         for (int j = 0; j < kGaKStepsHalf; ++j) {
             const float4* src = reinterpret_cast<const float4*>(qa + 32 * j);
-            qv[j][0] = float4{0, 0, 0, 0}, qv[j][1] = float4{0, 0, 0, 0};
-            if (live) qv[j][0] = src[0], qv[j][1] = src[1];
+            qv[j][0] = src[0], qv[j][1] = src[1];  // a head past h reads head 0 and is zeroed below
         }
+        const int e0 = list_entry(0, f0), e1 = list_entry(1, f1);
         RawTile second;
         issue_loads(raw, e0);
         if (n_tiles > 1) issue_loads(second, e1);
@@ -169,7 +174,7 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
                                 qv[j][1].x, qv[j][1].y, qv[j][1].z, qv[j][1].w};
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float x = v[i];  // unscaled: a bf16-valued q stays exact in its hi part
+                const float x = live ? v[i] : 0.0f;  // unscaled: a bf16-valued q stays exact in its hi part
                 const __bf16 hi = (__bf16)x;
                 qh[j][i] = hi;
                 if (QSPLIT == 2) ql[j][i] = (__bf16)(x - (float)hi);
@@ -178,7 +183,8 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
         stage(raw, 0);
         if (n_tiles > 1) stage(second, 1);
     }
-    if (n_tiles > 2) issue_loads(raw, e2);
+    if (n_tiles > 2) issue_loads(raw, list_entry(2, f2));
+    int entry_next = list_entry(3, f3);
     __syncthreads();
 
     f32x4 o[kGaColTilesHalf];
@@ -229,7 +235,7 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
         x[0] = s0, x[1] = s1;
     }
     for (int tile = 0; tile < n_tiles; ++tile) {
-        const int entry_ahead = tile + 4 < n_tiles ? list_entry(tile + 4) : -1;
+        const int fetch_ahead = list_fetch(tile + 4);  // looked at when this iteration ends
         const lds_ptr<f32x4> xch_peer = xch + (((tile & 1) * kGaWaves + (wave ^ 4)) * kWave + lane) * 2;
         const lds_ptr<f32x4> xch_next = xch + ((((tile + 1) & 1) * kGaWaves + wave) * kWave + lane) * 2;
         const int buf_next = buf == 2 ? 0 : buf + 1;
@@ -335,8 +341,13 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
         }
         // ---- stage tile + 2, request tile + 3 ---------------------------------------------
         if (tile + 2 < n_tiles) stage(raw, buf == 0 ? 2 : buf - 1);
-        if (tile + 3 < n_tiles) issue_loads(raw, entry_next);
-        entry_next = entry_ahead;
+        // the list entry fetched at the top is looked at BEFORE the rows are requested: past
+        // the conditional request the compiler no longer knows how many loads are in flight
+        // and would wait for all of them
+        const int entry_now = entry_next;
+        entry_next = list_entry(tile + 4, fetch_ahead);
+        asm volatile("" : "+v"(entry_next));  // here, not wherever the scheduler would sink it
+        if (tile + 3 < n_tiles) issue_loads(raw, entry_now);
         buf = buf_next;
     }
 
