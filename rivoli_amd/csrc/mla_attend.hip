@@ -687,11 +687,22 @@ __global__ __launch_bounds__(F8 ? kF8Threads : kAttThreads) void mla_attend_page
     int seq = blockIdx.y;
     if (a.n_items > 0) {
         // inclusive prefix of tiles per sequence, PER consecutive sequences per thread
+        // (the lengths are read unconditionally, a sequence past the last re-reading the last
+        // one: under `s < n_seqs` each read would be a branch with a wait of its own)
         int c[PER], run = 0;
+        const int* const lens = MODE == kLinear ? nullptr : (SPARSE ? a.n_rows : a.seq_lens);
+        if (lens) {
+#pragma unroll
+            for (int j = 0; j < PER; ++j) c[j] = lens[min(PER * tid + j, a.n_seqs - 1)];
+#pragma unroll
+            for (int j = 0; j < PER; ++j) c[j] = max(min(c[j], a.k), 0);
+        } else {
+#pragma unroll
+            for (int j = 0; j < PER; ++j) c[j] = a.k;
+        }
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
-            const int s = PER * tid + j;
-            c[j] = s < a.n_seqs ? (attended(s) + kTile - 1) / kTile : 0;
+            c[j] = PER * tid + j < a.n_seqs ? (c[j] + kTile - 1) / kTile : 0;
             run += c[j];
         }
 #pragma unroll

@@ -125,17 +125,27 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         const size_t qrow = (size_t)seq * a.H + (live ? head : 0);
 #pragma unroll
         for (int t = 0; t < TQ; ++t) qscale_lo[t] = qscale_hi[t] = kScaleOne;
+        // every load of q is requested before the first is used, from addresses that always
+        // exist (a head past H reads head 0, lane groups 2 and 3 re-read the rope's halves) and
+        // dropped afterwards: a load under a condition is a branch with a wait of its own
+        float4 raw[kF8Steps][8];
+#pragma unroll
+        for (int s = 0; s < kF8Steps; ++s) {
+            const float* src =
+                s == 4 ? a.qrope + qrow * kRopeW + 32 * (g & 1) : a.qabs + qrow * kKvl + 128 * s + 32 * g;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) raw[s][c] = reinterpret_cast<const float4*>(src)[c];
+        }
 #pragma unroll
         for (int s = 0; s < kF8Steps; ++s) {
             float x[32];
             const bool there = live && (s < 4 || g < 2);
-            const float* src = s == 4 ? a.qrope + qrow * kRopeW + 32 * g : a.qabs + qrow * kKvl + 128 * s + 32 * g;
+            const float keep = there ? a.qscale : 0.0f;
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
-                float4 v = {0, 0, 0, 0};
-                if (there) v = reinterpret_cast<const float4*>(src)[c];
-                x[4 * c] = v.x * a.qscale, x[4 * c + 1] = v.y * a.qscale, x[4 * c + 2] = v.z * a.qscale,
-                x[4 * c + 3] = v.w * a.qscale;
+                const float4 v = raw[s][c];
+                x[4 * c] = there ? v.x * keep : 0.0f, x[4 * c + 1] = there ? v.y * keep : 0.0f;
+                x[4 * c + 2] = there ? v.z * keep : 0.0f, x[4 * c + 3] = there ? v.w * keep : 0.0f;
             }
             float amax = 0.0f;
 #pragma unroll
