@@ -95,12 +95,12 @@ __global__ __launch_bounds__(THREADS) void kv_gather_paged_kernel(
 
 // The same units on a flat grid sized by the batch's real token count: workgroup u finds the
 // sequence its unit belongs to from the device-side lengths; sequence s owns ceil(len_s / ROWS)
-// consecutive units. Up to kScalarScanSeqs sequences the lengths are walked with uniform
-// (scalar) loads, 16 at a time: those go through the scalar cache, apart from the vector memory
-// pipeline that the streaming traffic keeps full, and the table lookup that follows stays a
-// scalar load too. Longer batches scan 64 lengths per round across the lanes. No LDS, no barrier; at most n_seqs workgroups of the launch (the rounding
-// of each sequence's last unit) find nothing to do.
-constexpr int kScalarScanSeqs = 128;
+// consecutive units. The lengths are scanned 64 per round across the lanes of every wave (one
+// coalesced load, a DPP prefix sum, a ballot); walking them with uniform loads and scalar
+// compares instead costs ~500 scalar instructions per 16 sequences per wave, which saturates
+// the compute unit's one scalar pipe (measured: 0.63 against 0.66 of peak at 32 sequences,
+// 0.37 against 0.63 at 128). No LDS, no barrier; at most n_seqs workgroups of the launch (the
+// rounding of each sequence's last unit) find nothing to do.
 template <int W, int PT, int THREADS, int ROWS>
 __global__ __launch_bounds__(THREADS) void kv_gather_flat_kernel(
     const uint8_t* __restrict__ pool, const int* __restrict__ block_table,
@@ -113,31 +113,11 @@ __global__ __launch_bounds__(THREADS) void kv_gather_flat_kernel(
     const int cap = max_blocks_per_seq * pt;  // rows a block-table row can address
     uint32_t first = 0;                       // units of the sequences before s
     int s = -1, my_len = 0;
-    if (n_seqs <= kScalarScanSeqs) {
-        for (int base = 0; base < n_seqs && s < 0; base += 16) {
-            int l[16];
-            if (base + 16 <= n_seqs) {  // one wide scalar load
-#pragma unroll
-                for (int j = 0; j < 16; ++j) l[j] = seq_lens[base + j];
-            } else {
-#pragma unroll
-                for (int j = 0; j < 16; ++j) l[j] = base + j < n_seqs ? seq_lens[base + j] : 0;
-            }
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const int len = min(max(l[j], 0), cap);
-                const uint32_t units = (uint32_t)(len + ROWS - 1) / ROWS;
-                if (s < 0) {
-                    if (u < first + units) s = base + j, my_len = len;
-                    else first += units;
-                }
-            }
-        }
-    } else {
+    {
         const int lane = threadIdx.x & (kWave - 1);
         for (int s0 = 0; s0 < n_seqs; s0 += kWave) {
-            int len = 0;
-            if (s0 + lane < n_seqs) len = min(max(seq_lens[s0 + lane], 0), cap);
+            int len = seq_lens[min(s0 + lane, n_seqs - 1)];
+            len = s0 + lane < n_seqs ? min(max(len, 0), cap) : 0;
             const uint32_t units = (uint32_t)(len + ROWS - 1) / ROWS;
             const uint32_t incl = first + wave_inclusive_sum(units);
             const int passed = __popcll(__ballot(incl <= u));  // sequences ending at or before u
@@ -219,12 +199,11 @@ static int gather_paged_launch(const unsigned char* pool, const int* block_table
     if (!gather_shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
     const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
     const long long capacity = (long long)n_seqs * max_blocks_per_seq * page_tokens;
-    // The flat grid pays for finding each workgroup's sequence (measured on MI355X at 32
-    // sequences of 1 K - 32 K rows, 578 K rows in tables that hold 1 M: 199 us against 177 us for
-    // the grid form, whose 29 K idle workgroups cost 10 us) and saves the idle workgroups, so it
-    // is taken when the block tables are mostly empty — tables sized for a context limit far
-    // above what the sequences hold.
-    const bool flat = total_tokens >= 0 && total_tokens < capacity / 4;
+    // The flat grid pays for finding each workgroup's sequence (a constant 0.665 of the HBM peak
+    // at 32 ragged sequences whatever the tables' size) and saves the idle workgroups of the
+    // grid form, which reaches 0.70 with tables half full, 0.66 a third full and 0.62 a quarter
+    // full: flat when the batch fills less than a third of what its block tables could hold.
+    const bool flat = total_tokens >= 0 && total_tokens < capacity / 3;
     (void)hipGetLastError();
 #define RK_GATHER(WV, PTV, THREADS, FLAT_THREADS, ROWS)                                            \
     do {                                                                                           \
