@@ -1,8 +1,14 @@
-"""The 8-bit attention kernels' register budget is part of their design: one wave per SIMD with
+"""Register budgets that are part of a kernel's design, held to the build's own resource report.
+
+The 8-bit attention kernels' register budget is part of their design: one wave per SIMD with
 the whole register file, 128 accumulators in ordinary registers, two q terms in the accumulation
 registers (rivoli_amd/csrc/mla_attend_f8.hpp). A compiler or source change that makes them spill
 still gives right answers, only several times slower, so the build's own resource report is held
-to "no scratch memory" here. Compiles one file; needs hipcc, no GPU."""
+to "no scratch memory" here. The scored block selection keeps a row's keys in registers and its
+phases must not share per-element lane masks: 32 of them do not fit the scalar registers, and
+when they spilled (to lanes of a vector register, a write and a read each) a quarter of the
+kernel's vector instructions were spill traffic. Compiles one file per test; needs hipcc, no
+GPU."""
 import os
 import re
 import shutil
@@ -39,3 +45,29 @@ def test_eight_bit_attention_kernels_do_not_spill(tmp_path):
         assert occupancy == 1, name
         assert lds <= 160 * 1024, name
     assert seen == 4, f"expected the dense and row-list kernels of both 8-bit modes, saw {seen}"
+
+
+def _resource_blocks(src_name):
+    src = os.path.join(build.CSRC, src_name)
+    cmd = [build.hipcc(), f"--offload-arch={build.offload_arch()}", "-O3", "-std=c++17", "-fPIC",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I", os.path.join(ROOT, "include")] + build.EXTRA_FLAGS.get(src_name, []) + \
+          ["-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", os.devnull]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    return re.split(r"remark: Function Name: ", res.stderr)[1:]
+
+
+@pytest.mark.skipif(shutil.which(build.hipcc()) is None, reason="hipcc not found")
+def test_block_selection_keeps_its_masks_out_of_memory():
+    seen = 0
+    for b in _resource_blocks("index_topk.hip"):
+        name = b.split()[0]
+        if "block_select_bisect_kernel" not in name:
+            continue
+        seen += 1
+        assert int(re.search(r"SGPRs Spill: (\d+)", b).group(1)) == 0, name
+        assert int(re.search(r"VGPRs Spill: (\d+)", b).group(1)) == 0, name
+        assert int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b).group(1)) == 0, name
+        assert int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", b).group(1)) == 8, name
+    assert seen == 6, f"expected the six widths of the register form, saw {seen}"
