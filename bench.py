@@ -127,7 +127,10 @@ def main():
               # the cache's consumer at configuration 3's shape: inside the reference's own bar on
               # the 8-bit matrix instructions, and the tighter bf16 hi + lo mode
               ("attend_decode", "attend", dict(precise=4)),
-              ("attend_decode_bf16x2", "attend", dict(precise=2)))
+              ("attend_decode_bf16x2", "attend", dict(precise=2)),
+              # the second cache format's own operators, at prefill
+              ("v4_prefill_32768", "v4", dict(tokens=32768)),
+              ("v4_attend_prefill_8192", "v4_attend", dict(tokens=8192, precise=2)))
     res["configs"] = {}
     for name, workload, over in others:
         torch.cuda.empty_cache()
@@ -155,7 +158,7 @@ def run_workload(workload, a, torch, hip):
 def brief(res):
     """What a secondary configuration contributes to the default run's line."""
     keep = ("metric", "value", "unit", "ms_per_step", "layer_us", "hbm_peak_frac", "tokens_per_s", "rows_per_s",
-            "kernels_ms", "roofline", "index_score", "config")
+            "kernels_ms", "kernels", "roofline", "index_score", "decode_one_query_us", "queries_per_s", "config")
     out = {k: res[k] for k in keep if k in res}
     if "cpu_baseline" in res:
         out["checked"] = res["cpu_baseline"]["sample"]
@@ -519,7 +522,7 @@ def bench_v4(a, torch, hip):
                                "sample": f"the first {nr} rows of the same inputs through the oracle's "
                                          "compressor pooling, act_quant and scored_rows, one host thread; "
                                          "GPU results checked (pooling within 2 bf16 codes, the others equal)"}
-    print(json.dumps(res), flush=True)
+    return res
 
 
 def bench_v4_attend(a, torch, hip):
@@ -622,7 +625,7 @@ def bench_v4_attend(a, torch, hip):
                                "sample": f"the last {nq} queries of the same inputs through the oracle's "
                                          f"sparse_attn, one host thread; GPU output within {err:.2g} of the "
                                          "largest element (bar 1/128)"}
-    print(json.dumps(res), flush=True)
+    return res
 
 
 def bench_dsa(a, torch, hip, scored=False, attend=False):
