@@ -291,7 +291,12 @@ def bench_decode(a, torch, hip):
         "decode_step_kv_ms": round(ms_per_step, 4),
         "tokens_per_s": round(L * n_att / (ms_per_step * 1e-3), 1),
         "hbm_peak_frac": round(value * 1e9 / HBM_PEAK, 4),
-        "roofline": {"bound": "hbm", "kernel": "kv_gather_paged_kernel", "achieved": round(achieved, 1),
+        # rivoli_kv_gather_paged_packed takes the launch sized by the token count when the batch fills
+        # less than 0.7 of what its block tables could hold (kv_gather.hip: gather_paged_launch)
+        "roofline": {"bound": "hbm",
+                     "kernel": ("kv_gather_flat_kernel" if a.gather_form == "packed" and n_att * 10 < B * cols * PT * 7
+                                else "kv_gather_paged_kernel"),
+                     "achieved": round(achieved, 1),
                      "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": round(achieved * 1e9 / HBM_PEAK, 4),
                      "avg_launch_ms": round(gather_ms, 5), "bytes_per_launch": gather_bytes_layer,
                      "traffic": measured_traffic(f"decode:b{B}:ctx{ctx}:{'ragged' if a.ragged else 'uniform'}")},

@@ -112,8 +112,8 @@ int rivoli_kv_gather_paged(const unsigned char* pool, const int* block_table,
 
 /* rivoli_kv_gather_paged for a caller that knows how many rows the batch holds (it sized
  * `out` by that number): total_tokens >= the sum of seq_lens. Same results. When the batch
- * fills less than a third of what its block tables could address (tables sized for a context
- * limit far above the sequences' lengths), the launch is sized by total_tokens instead of by
+ * fills less than 0.7 of what its block tables could address (ragged batches, or tables sized
+ * for a context limit above the sequences' lengths), the launch is sized by total_tokens instead of by
  * n_seqs * max_blocks_per_seq pages and each workgroup finds its sequence from the device-side
  * lengths; otherwise this is rivoli_kv_gather_paged. Rows may be left out if total_tokens
  * understates the sum. Guards as above, plus 1001 for total_tokens < 0 and 1002 when

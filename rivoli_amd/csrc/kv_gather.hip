@@ -107,6 +107,7 @@ __global__ __launch_bounds__(THREADS) void kv_gather_flat_kernel(
     const int* __restrict__ seq_lens, const int* __restrict__ cu_seqlens,
     uint16_t* __restrict__ out, int n_seqs, int max_blocks_per_seq, int width_rt,
     int page_tokens_rt, int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_pages) {
+    static_assert(THREADS % kWave == 0, "the scan below runs in every wave and needs all 64 lanes of each");
     const int pt = PT ? PT : page_tokens_rt;
     const int parts = pt / ROWS;
     const uint32_t u = blockIdx.x;
@@ -199,11 +200,12 @@ static int gather_paged_launch(const unsigned char* pool, const int* block_table
     if (!gather_shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
     const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
     const long long capacity = (long long)n_seqs * max_blocks_per_seq * page_tokens;
-    // The flat grid pays for finding each workgroup's sequence (a constant 0.665 of the HBM peak
-    // at 32 ragged sequences whatever the tables' size) and saves the idle workgroups of the
-    // grid form, which reaches 0.70 with tables half full, 0.66 a third full and 0.62 a quarter
-    // full: flat when the batch fills less than a third of what its block tables could hold.
-    const bool flat = total_tokens >= 0 && total_tokens < capacity / 3;
+    // The flat grid pays for finding each workgroup's sequence and saves the idle workgroups of
+    // the grid form. Measured at 32 ragged sequences (1 K - 32 K rows): flat 0.72 of the HBM peak
+    // whatever the tables' size, grid 0.70 with tables half full, 0.66 a third full, 0.62 a
+    // quarter full; with every sequence at the tables' full length grid 0.75, flat 0.72. So:
+    // flat when the batch fills less than 0.7 of what its block tables could hold.
+    const bool flat = total_tokens >= 0 && total_tokens * 10 < capacity * 7;
     (void)hipGetLastError();
 #define RK_GATHER(WV, PTV, THREADS, FLAT_THREADS, ROWS)                                            \
     do {                                                                                           \
@@ -224,7 +226,7 @@ static int gather_paged_launch(const unsigned char* pool, const int* block_table
         }                                                                                          \
     } while (0)
     if (width == 576 && page_tokens == 64)
-        RK_GATHER(576, 64, 768, 384, 16);
+        RK_GATHER(576, 64, 768, 576, 16);  // flat: 576 threads = two 8-byte chunks each
     else if (page_tokens % 16 == 0)
         RK_GATHER(0, 0, kGatherThreads, kGatherThreads, 16);
     else

@@ -35,8 +35,8 @@ def gpu_gather(pool, tables, seq_lens, width=W, pt=PT, n_pages=None, fill=0x5A):
     n_pages = n_pages or pool.size // (pt * (width + 4))
     pool_d, tables_d, lens_d, cu_d = dev(pool), dev(tables), dev(seq_lens), dev(cu)
     total = int(np.minimum(np.maximum(seq_lens, 0), tables.shape[1] * pt).sum())
-    # the same tables with four times as many (unused) columns: a batch that fills less than a
-    # third of its tables takes the launch sized by the token count
+    # the same tables with four times as many (unused) columns: a batch that fills less than
+    # 0.7 of its tables takes the launch sized by the token count
     wide = np.full((tables.shape[0], 4 * tables.shape[1] + 1), -1, np.int32)
     wide[:, : tables.shape[1]] = tables
     wide_d = dev(wide)
