@@ -813,20 +813,39 @@ __global__ __launch_bounds__(128) void mla_attend_combine_kernel(
     const int first = deal_item_of(before, n_items, total);
     const int last = deal_item_of(before + mine - 1, n_items, total);
     if (first == last) return;  // one work item had the whole sequence and wrote it
+    // Records are fetched eight at a time, every load of a batch issued before the first use
+    // (a record past the last re-reads the last and is left out): one round trip per batch
+    // instead of one per record. The sums run in ascending record order as before.
+    constexpr int kBatch = 8;
     float m_g = -INFINITY;
-    for (int it = first; it <= last; ++it)
-        m_g = fmaxf(m_g, part_ml[((size_t)(it + seq) * H + head) * 2]);
+    for (int b0 = first; b0 <= last; b0 += kBatch) {
+        float m_r[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u)
+            m_r[u] = part_ml[((size_t)(min(b0 + u, last) + seq) * H + head) * 2];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) m_g = fmaxf(m_g, m_r[u]);
+    }
     float4 sum = {0, 0, 0, 0};
     float l_g = 0.0f;
     if (m_g != -INFINITY) {
-        for (int it = first; it <= last; ++it) {
-            const size_t rec = (size_t)it + seq;
-            const float m_r = part_ml[(rec * H + head) * 2];
-            if (m_r == -INFINITY) continue;
-            const float w = exp2f(m_r - m_g);
-            l_g += part_ml[(rec * H + head) * 2 + 1] * w;
-            const float4 v = reinterpret_cast<const float4*>(part_acc + (rec * H + head) * kKvl)[threadIdx.x];
-            sum.x += v.x * w, sum.y += v.y * w, sum.z += v.z * w, sum.w += v.w * w;
+        for (int b0 = first; b0 <= last; b0 += kBatch) {
+            float m_r[kBatch], l_r[kBatch];
+            float4 v[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const size_t rec = (size_t)min(b0 + u, last) + seq;
+                m_r[u] = part_ml[(rec * H + head) * 2];
+                l_r[u] = part_ml[(rec * H + head) * 2 + 1];
+                v[u] = reinterpret_cast<const float4*>(part_acc + (rec * H + head) * kKvl)[threadIdx.x];
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                if (b0 + u > last || m_r[u] == -INFINITY) continue;
+                const float w = exp2f(m_r[u] - m_g);
+                l_g += l_r[u] * w;
+                sum.x += v[u].x * w, sum.y += v[u].y * w, sum.z += v[u].z * w, sum.w += v[u].w * w;
+            }
         }
     }
     const float inv = l_g > 0.0f ? 1.0f / l_g : 0.0f;
