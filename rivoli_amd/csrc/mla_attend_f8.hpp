@@ -54,7 +54,7 @@ constexpr int kF8Requests = (kF8WaveRows * kF8RowGranules + kWave - 1) / kWave;
 template <int TQ>
 constexpr int f8_q_bytes() { return TQ > 2 ? (TQ - 2) * 64 * kF8RowBytes : 16; }  // q terms past the second: the block's 64 heads, rows padded like the tiles'
 constexpr int kF8SmemBytes =
-    kF8Bufs * kF8TileBytes + kF8ZeroBytes + 2 * kF8Bufs * kF8Tile * 4 + kF8Tile * 8 + kTableLds * 4;
+    kF8Bufs * kF8TileBytes + kF8ZeroBytes + 3 * kF8Bufs * kF8Tile * 4 + kF8Tile * 8 + kTableLds * 4;
 static_assert(kF8SmemBytes + f8_q_bytes<3>() + (1024 + 8 + 8) * 4 <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
 constexpr int kWaitLds0 = 0xC07F;           // s_waitcnt lgkmcnt(0), the other counters left alone
 constexpr int kScaleOne = 0x7f7f7f7f;        // E8M0 1.0 in every byte
@@ -96,7 +96,8 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     const lds_ptr<uint8_t> zeros = tiles + kF8Bufs * kF8TileBytes;
     const lds_ptr<float> sc = (lds_ptr<float>)(zeros + kF8ZeroBytes);     // [2][64] token scales (0 = not there)
     const lds_ptr<float> sbias = sc + kF8Bufs * kF8Tile;                     // [2][64] 0 or -inf
-    const lds_ptr<unsigned long long> rowbase = (lds_ptr<unsigned long long>)(sbias + kF8Bufs * kF8Tile);  // [64] where a row's codes are
+    const lds_ptr<float> rsc = sbias + kF8Bufs * kF8Tile;                    // [2][64] 1 / scale (0 = not there)
+    const lds_ptr<unsigned long long> rowbase = (lds_ptr<unsigned long long>)(rsc + kF8Bufs * kF8Tile);  // [64] where a row's codes are
     const lds_ptr<int> tbl = (lds_ptr<int>)(rowbase + kF8Tile);
     const lds_ptr<uint8_t> qlds = (lds_ptr<uint8_t>)(tbl + kTableLds);  // [TQ - 2][64 heads] rows of q codes
 
@@ -271,6 +272,9 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             const bool ok = next_scale > 0.0f;  // a token that is not there has scale 0
             sc[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? next_scale : 0.0f;
             sbias[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? 0.0f : -INFINITY;
+            // the denominator divides every held weight by its token's scale: the reciprocal is
+            // taken once per token here, not once per (token, head) in the softmax
+            rsc[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? __builtin_amdgcn_rcpf(next_scale) : 0.0f;
         }
     };
 
@@ -305,7 +309,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     for (int t = 0; t < n_tiles; ++t) {
         const int buf = t & 1;
         const lds_ptr<uint8_t> tile = tiles + buf * kF8TileBytes, next = tiles + (buf ^ 1) * kF8TileBytes;
-        const lds_ptr<float> sc_t = sc + buf * kF8Tile, sbias_t = sbias + buf * kF8Tile;
+        const lds_ptr<float> sc_t = sc + buf * kF8Tile, sbias_t = sbias + buf * kF8Tile, rsc_t = rsc + buf * kF8Tile;
         // tile t + 1 starts on its way into the other buffer (which held tile t - 1: every wave
         // left it before the barrier that ended the previous iteration)
         if (t + 1 < n_tiles) request_tile(t + 1, next);
@@ -364,10 +368,11 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
 
         // ---- online softmax over the lane's 16 tokens of head n16: tokens 16 mb + 4 g + i ----
         float tmax = -INFINITY;
-        f32x4 s4[kF8RowBlocks];
+        f32x4 s4[kF8RowBlocks], r4[kF8RowBlocks];
 #pragma unroll
         for (int mb = 0; mb < kF8RowBlocks; ++mb) {
             s4[mb] = *(lds_ptr<f32x4>)(sc_t + 16 * mb + 4 * g);
+            r4[mb] = *(lds_ptr<f32x4>)(rsc_t + 16 * mb + 4 * g);
             const f32x4 b4 = *(lds_ptr<f32x4>)(sbias_t + 16 * mb + 4 * g);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -418,8 +423,8 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             // weights perturbed by 2^-8 each.
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float held = acc[mb][i] - y[i] * unit;
-                l_sum += s4[mb][i] > 0.0f ? held * __builtin_amdgcn_rcpf(s4[mb][i]) : 0.0f;
+                const float held = acc[mb][i] - y[i] * unit;  // 0 for a token that is not there
+                l_sum += held * r4[mb][i];
             }
         }
 
