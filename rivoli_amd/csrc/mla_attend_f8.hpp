@@ -95,7 +95,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     const lds_ptr<uint8_t> tiles = (lds_ptr<uint8_t>)smem8;               // [2][64] rows of codes
     const lds_ptr<uint8_t> zeros = tiles + kF8Bufs * kF8TileBytes;
     const lds_ptr<float> sc = (lds_ptr<float>)(zeros + kF8ZeroBytes);     // [2][64] token scales (0 = not there)
-    const lds_ptr<float> sbias = sc + kF8Bufs * kF8Tile;                     // [2][64] 0 or -inf
+    const lds_ptr<float> sbias = sc + kF8Bufs * kF8Tile;                     // [2][64] log2 scale, or -inf
     const lds_ptr<float> rsc = sbias + kF8Bufs * kF8Tile;                    // [2][64] 1 / scale (0 = not there)
     const lds_ptr<unsigned long long> rowbase = (lds_ptr<unsigned long long>)(rsc + kF8Bufs * kF8Tile);  // [64] where a row's codes are
     const lds_ptr<int> tbl = (lds_ptr<int>)(rowbase + kF8Tile);
@@ -271,7 +271,9 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         if (lane < kF8WaveRows) {
             const bool ok = next_scale > 0.0f;  // a token that is not there has scale 0
             sc[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? next_scale : 0.0f;
-            sbias[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? 0.0f : -INFINITY;
+            // the bias added to a token's scores: log2 of its scale (its weights then carry the
+            // scale the value contraction needs), -inf for a token that is not there
+            sbias[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? __builtin_amdgcn_logf(next_scale) : -INFINITY;
             // the denominator divides every held weight by its token's scale: the reciprocal is
             // taken once per token here, not once per (token, head) in the softmax
             rsc[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? __builtin_amdgcn_rcpf(next_scale) : 0.0f;
@@ -395,25 +397,23 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
                 for (int i = 0; i < 4; ++i) o[nt][i] *= c[i];
         }
         const float mu = m_ref == -INFINITY ? 0.0f : m_ref;
-        // weights w_t = 2^(v_t - mu) * s_t, as TP e4m3 terms under one scale per (head, tile)
-        float wmax = 0.0f;
-#pragma unroll
-        for (int mb = 0; mb < kF8RowBlocks; ++mb)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                acc[mb][i] = __builtin_amdgcn_exp2f(acc[mb][i] - mu) * s4[mb][i];  // not there -> 0
-                wmax = fmaxf(wmax, acc[mb][i]);
-            }
-        wmax = rows_max(wmax);
-        const int pe = block_exp(wmax);
-        const float pinv = pow2i(-pe), unit = pow2i(pe - 4);  // what one unit of the second term is worth
+        // weights w_t = 2^(v_t - mu) * s_t = 2^(v'_t - mu) with v' = v + log2 s_t (the published
+        // bias carries log2 s_t, so the token scale costs nothing here), as TP e4m3 terms under
+        // one scale 2^pe per (head, tile). The largest weight of the head's 64 tokens is
+        // 2^(tmax - mu), exp2 being monotonic: no second maximum is taken. The terms are cut from
+        // y = w / 2^pe, computed as one exponential.
+        const int pe = block_exp(__builtin_amdgcn_exp2f(tmax - mu));
+        const float shift = mu + (float)pe, unit = pow2i(pe);
         i32x8 pt;  // bytes 0..15: the first term of the lane's 16 tokens, 16..31: the second
         // (the instruction takes K block b's scale from lane 16 b + row: blocks 0, 1 are the
         // first term of lane groups 0,1 / 2,3, blocks 2, 3 the second term, 16 times finer)
         const int pscale = (int)((uint32_t)max(pe - 4 * (g >> 1) + 127, 1) * 0x01010101u);
+        float l_tile = 0.0f;  // in units of 2^pe
 #pragma unroll
         for (int mb = 0; mb < kF8RowBlocks; ++mb) {
-            float y[4] = {acc[mb][0] * pinv, acc[mb][1] * pinv, acc[mb][2] * pinv, acc[mb][3] * pinv};
+            float y[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) y[i] = acc[mb][i] = __builtin_amdgcn_exp2f(acc[mb][i] - shift);  // not there -> 0
             pt[mb] = (int)e4m3x4_and_residual(y);
 #pragma unroll
             for (int i = 0; i < 4; ++i) y[i] *= 16.0f;
@@ -423,10 +423,11 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             // weights perturbed by 2^-8 each.
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float held = acc[mb][i] - y[i] * unit;  // 0 for a token that is not there
-                l_sum += held * r4[mb][i];
+                const float held = __builtin_fmaf(y[i], -0.0625f, acc[mb][i]);  // 0 for a token that is not there
+                l_tile = __builtin_fmaf(held, r4[mb][i], l_tile);
             }
         }
+        l_sum = __builtin_fmaf(l_tile, unit, l_sum);
 
         // ---- values: O[head][col] += P . V over all 512 columns -------------------------------
         static_assert(TP == 2, "two terms fill the value contraction's K exactly");
