@@ -323,6 +323,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
 #pragma unroll
         for (int mb = 0; mb < kF8RowBlocks; ++mb) acc[mb] = f32x4{0, 0, 0, 0};
         i32x8 af[2][2], qf[2][TQ > TQR ? TQ - TQR : 1];
+        f32x4 s4[kF8RowBlocks], r4[kF8RowBlocks], b4[kF8RowBlocks];  // token scales, their reciprocals, biases
         auto read32 = [&](lds_ptr<uint8_t> src) -> i32x8 {
             const u32x4 lo4 = *(lds_ptr<u32x4>)(src), hi4 = *(lds_ptr<u32x4>)(src + 16);
             return i32x8{(int)lo4.x, (int)lo4.y, (int)lo4.z, (int)lo4.w, (int)hi4.x, (int)hi4.y, (int)hi4.z, (int)hi4.w};
@@ -345,7 +346,17 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         for (int u = 0; u < 2 * kF8Steps; ++u) {
             __builtin_amdgcn_s_waitcnt(kWaitLds0);  // this unit's fragments are in
             __builtin_amdgcn_sched_barrier(0);
-            if (u + 1 < 2 * kF8Steps) load_unit(u + 1);
+            if (u + 1 < 2 * kF8Steps) {
+                load_unit(u + 1);
+            } else {
+                // under the last unit's matrix instructions: what the softmax reads first
+#pragma unroll
+                for (int mb = 0; mb < kF8RowBlocks; ++mb) {
+                    s4[mb] = *(lds_ptr<f32x4>)(sc_t + 16 * mb + 4 * g);
+                    r4[mb] = *(lds_ptr<f32x4>)(rsc_t + 16 * mb + 4 * g);
+                    b4[mb] = *(lds_ptr<f32x4>)(sbias_t + 16 * mb + 4 * g);
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
             const int s = u >> 1;
 #pragma unroll
@@ -370,15 +381,11 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
 
         // ---- online softmax over the lane's 16 tokens of head n16: tokens 16 mb + 4 g + i ----
         float tmax = -INFINITY;
-        f32x4 s4[kF8RowBlocks], r4[kF8RowBlocks];
 #pragma unroll
         for (int mb = 0; mb < kF8RowBlocks; ++mb) {
-            s4[mb] = *(lds_ptr<f32x4>)(sc_t + 16 * mb + 4 * g);
-            r4[mb] = *(lds_ptr<f32x4>)(rsc_t + 16 * mb + 4 * g);
-            const f32x4 b4 = *(lds_ptr<f32x4>)(sbias_t + 16 * mb + 4 * g);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                acc[mb][i] = __builtin_fmaf(acc[mb][i], s4[mb][i], b4[i]);  // -inf where the token is not there
+                acc[mb][i] = __builtin_fmaf(acc[mb][i], s4[mb][i], b4[mb][i]);  // -inf where the token is not there
                 tmax = fmaxf(tmax, acc[mb][i]);
             }
         }
