@@ -312,9 +312,6 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         const int buf = t & 1;
         const lds_ptr<uint8_t> tile = tiles + buf * kF8TileBytes, next = tiles + (buf ^ 1) * kF8TileBytes;
         const lds_ptr<float> sc_t = sc + buf * kF8Tile, sbias_t = sbias + buf * kF8Tile, rsc_t = rsc + buf * kF8Tile;
-        // tile t + 1 starts on its way into the other buffer (which held tile t - 1: every wave
-        // left it before the barrier that ended the previous iteration)
-        if (t + 1 < n_tiles) request_tile(t + 1, next);
 
         // ---- scores: S^T[token][head] over the five K-steps ---------------------------------
         // A K-step's four operand fragments are requested while the matrix instructions of the
@@ -342,6 +339,11 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             }
         };
         load_unit(0);
+        __builtin_amdgcn_sched_barrier(0);
+        // tile t + 1 starts on its way into the other buffer (which held tile t - 1: every wave
+        // left it before the barrier that ended the previous iteration); the address arithmetic of
+        // its requests runs while the first fragments above come out of LDS
+        if (t + 1 < n_tiles) request_tile(t + 1, next);
 #pragma unroll
         for (int u = 0; u < 2 * kF8Steps; ++u) {
             __builtin_amdgcn_s_waitcnt(kWaitLds0);  // this unit's fragments are in
@@ -378,6 +380,22 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
                 }
             __builtin_amdgcn_sched_barrier(0);
         }
+
+        // the value contraction's first operands are requested now: they do not depend on the
+        // softmax, whose arithmetic then hides their way out of LDS
+        static_assert(TP == 2, "two terms fill the value contraction's K exactly");
+        constexpr int CU = 4;  // column tiles per unit
+        i32x8 vf[2][CU];
+        auto load_cols = [&](int n0, i32x8 (&f)[CU]) {
+#pragma unroll
+            for (int j = 0; j < CU; ++j) {
+                const i32x2 r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr<i32x2>)(tile + v_off[0] + 16 * (n0 + j)));
+                const i32x2 r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr<i32x2>)(tile + v_off[1] + 16 * (n0 + j)));
+                f[j] = i32x8{r0[0], r0[1], r1[0], r1[1], r0[0], r0[1], r1[0], r1[1]};
+            }
+        };
+        load_cols(0, vf[0]);
+        __builtin_amdgcn_sched_barrier(0);
 
         // ---- online softmax over the lane's 16 tokens of head n16: tokens 16 mb + 4 g + i ----
         float tmax = -INFINITY;
@@ -436,19 +454,8 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         }
         l_sum = __builtin_fmaf(l_tile, unit, l_sum);
 
-        // ---- values: O[head][col] += P . V over all 512 columns -------------------------------
-        static_assert(TP == 2, "two terms fill the value contraction's K exactly");
-        constexpr int CU = 4;  // column tiles per unit
-        i32x8 vf[2][CU];
-        auto load_cols = [&](int n0, i32x8 (&f)[CU]) {
-#pragma unroll
-            for (int j = 0; j < CU; ++j) {
-                const i32x2 r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr<i32x2>)(tile + v_off[0] + 16 * (n0 + j)));
-                const i32x2 r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr<i32x2>)(tile + v_off[1] + 16 * (n0 + j)));
-                f[j] = i32x8{r0[0], r0[1], r1[0], r1[1], r0[0], r0[1], r1[0], r1[1]};
-            }
-        };
-        load_cols(0, vf[0]);
+        // ---- values: O[head][col] += P . V over all 512 columns (the first unit's operands were
+        // requested before the softmax) --------------------------------------------------------
 #pragma unroll
         for (int n0 = 0; n0 < kF8ColTiles; n0 += CU) {
             __builtin_amdgcn_s_waitcnt(kWaitLds0);
