@@ -384,7 +384,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         // the value contraction's first operands are requested now: they do not depend on the
         // softmax, whose arithmetic then hides their way out of LDS
         static_assert(TP == 2, "two terms fill the value contraction's K exactly");
-        constexpr int CU = 4;  // column tiles per unit
+        constexpr int CU = 8;  // column tiles per unit
         i32x8 vf[2][CU];
         auto load_cols = [&](int n0, i32x8 (&f)[CU]) {
 #pragma unroll
