@@ -262,7 +262,7 @@ int rivoli_index_append_paged(const float* k, const int* slot_mapping, unsigned 
  * cache codes going into them untouched and q / the weights as sums of e4m3 terms under
  * power-of-two block scales: 3 = two terms each (the accuracy class of 0), 4 = three terms for
  * q and two for the weights (the class of 1; inside the reference's bar on the test caches).
- * They are the fastest modes: about a quarter less time per launch than 0 / 2.
+ * They are the fastest modes: about 30 % less time per launch than 0 / 2.
  * Other row widths (kvl a multiple of 128 up to 512, rope a multiple of 8 up to 64) always run
  * as 2.
  * Guards: 1001 null / non-positive, or a null `partial` when scratch is needed; 1002
