@@ -116,10 +116,19 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     if (tid < kF8ZeroBytes / 4) ((lds_ptr<int>)zeros)[tid] = 0;
 
     // ---- this wave's 16 query heads as e4m3 terms, for the whole kernel ----------------------
-    // step s < 4: latent dims 128 s .. +127; step 4: the rope (its 64 dims in lane groups 0 and 1)
+    // step s < 4: latent dims 128 s .. +127. Step 4, the rope, has 64 dims for a K of 128: its
+    // operand holds the rope's FIRST TWO TERMS side by side, term 0 in lane groups 0 and 1, term 1
+    // in lane groups 2 and 3 (qt[0][4]; the key rows' rope bytes are read by both pairs of lane
+    // groups), so one matrix instruction does what two half-empty ones would. An element of
+    // lane group g, byte b belongs to K block (g >> 1) + 2 (b / 16) and block k takes its scale
+    // from lane group k: term 0 sits in blocks 0 and 2, term 1 in blocks 1 and 3, hence a scale
+    // register that alternates between the two terms' scales by lane group (qscale_rope). A
+    // third term keeps the half-empty form (zeros in lane groups 2 and 3).
     constexpr int TQR = TQ > 2 ? 2 : TQ;  // terms in (accumulation) registers; a third one lives in LDS
-    i32x8 qt[TQR ? TQR : 1][kF8Steps];
+    static_assert(TQR == 2, "the rope step pairs the first two terms");
+    i32x8 qt[TQR][kF8Steps];  // qt[1][4] is not used
     int qscale_lo[TQ], qscale_hi[TQ];  // E8M0 scales: bytes 0..3 = steps 0..3, byte 0 of _hi = step 4
+    int qscale_rope = kScaleOne;
     {
         const int head = hb * 64 + 16 * wave + n16;
         const bool live = head < a.H;
@@ -140,7 +149,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
 #pragma unroll
         for (int s = 0; s < kF8Steps; ++s) {
             float x[32];
-            const bool there = live && (s < 4 || g < 2);
+            const bool there = live;  // (the rope step: lane groups 2, 3 hold what 0, 1 hold)
             const float keep = there ? a.qscale : 0.0f;
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
@@ -156,16 +165,20 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             const float inv = pow2i(-e);
 #pragma unroll
             for (int i = 0; i < 32; ++i) x[i] *= inv;
+            uint32_t first_term[8];  // the rope step: term 0's codes, until term 1's join them
 #pragma unroll
             for (int t = 0; t < TQ; ++t) {
 #pragma unroll
                 for (int c = 0; c < 8; ++c) {
                     float y[4] = {x[4 * c], x[4 * c + 1], x[4 * c + 2], x[4 * c + 3]};
-                    const uint32_t w4 = e4m3x4_and_residual(y);
-                    int qa;
-                    asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(qa) : "v"(w4));
-                    if (t < TQR) qt[t < TQR ? t : 0][s][c] = qa;
-                    else if (s < 4 || g < 2)
+                    uint32_t w4 = e4m3x4_and_residual(y);
+                    if (s == 4 && t == 0) first_term[c] = w4;
+                    if (s == 4 && t == 1) w4 = g < 2 ? first_term[c] : w4;
+                    if (t < TQR && !(s == 4 && t == 0)) {
+                        int qa;
+                        asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(qa) : "v"(w4));
+                        qt[s == 4 ? 0 : t][s][c] = qa;
+                    } else if (t >= TQR && (s < 4 || g < 2))
                         *(lds_ptr<uint32_t>)(qlds + ((t - TQR) * 64 + 16 * wave + n16) * kF8RowBytes + 128 * s + 32 * g + 4 * c) = w4;
                     // what is left over, at the next term's scale (16 times finer)
                     x[4 * c] = y[0] * 16.0f, x[4 * c + 1] = y[1] * 16.0f, x[4 * c + 2] = y[2] * 16.0f,
@@ -174,6 +187,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
                 const int byte = max(e - 4 * t + 127, 1);
                 if (s < 4) qscale_lo[t] = (qscale_lo[t] & ~(0xff << (8 * s))) | (byte << (8 * s));
                 else qscale_hi[t] = (qscale_hi[t] & ~0xff) | byte;
+                if (s == 4 && t < 2 && (g & 1) == t) qscale_rope = (qscale_rope & ~0xff) | byte;
             }
         }
     }
@@ -284,7 +298,8 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     // scores: row 16 mb + n16, this lane's 32 bytes of K-step s; the rope step's upper half
     // (lane groups 2 and 3) reads zeros
     const int a_row = n16 * kF8RowBytes + 32 * g;
-    const bool rope_zero = g >= 2;
+    const int a_rope = n16 * kF8RowBytes + kKvl + 32 * (g & 1);  // both pairs of lane groups read the rope
+    const bool rope_zero = g >= 2;  // a third q term's rope fragment
     const int q_row = (16 * wave + n16) * kF8RowBytes + 32 * g;
     // values: transposing load r (of 4) hands this lane bytes 8 r .. 8 r + 7 of its operand = the
     // tokens 16 (2 r + e / 4) + 4 g + e % 4, e = 0..7, of column 16 nt + n16; source lane pair e
@@ -331,7 +346,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             const bool z = s == 4 && rope_zero;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                af[u & 1][j] = read32(z ? zeros : tile + (2 * (u & 1) + j) * 16 * kF8RowBytes + a_row + 128 * s);
+                af[u & 1][j] = read32(tile + (2 * (u & 1) + j) * 16 * kF8RowBytes + (s == 4 ? a_rope : a_row + 128 * s));
             if ((u & 1) == 0) {
 #pragma unroll
                 for (int tq = 0; tq < TQ - TQR; ++tq)
@@ -365,6 +380,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             for (int tq = 0; tq < TQ; ++tq)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
+                    if (s == 4 && tq == 1) continue;  // the rope's second term rode with the first
                     const i32x8 fa = af[u & 1][j], fq = tq < TQR ? qt[tq < TQR ? tq : 0][s] : qf[s & 1][tq < TQR ? 0 : tq - TQR];
                     const int mb = 2 * (u & 1) + j;
                     if (s == 0)
@@ -376,7 +392,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
                     else if (s == 3)
                         acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa, fq, acc[mb], 0, 0, 0, kScaleOne, 3, qscale_lo[tq]);
                     else
-                        acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa, fq, acc[mb], 0, 0, 0, kScaleOne, 0, qscale_hi[tq]);
+                        acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa, fq, acc[mb], 0, 0, 0, kScaleOne, 0, tq == 0 ? qscale_rope : qscale_hi[tq]);
                 }
             __builtin_amdgcn_sched_barrier(0);
         }
