@@ -40,29 +40,39 @@ __device__ __forceinline__ float rbf16(float x) {
     return __uint_as_float((uint32_t)f32_to_bf16(x) << 16);
 }
 
-// Where entry j of a window lives: null score = masked.
+// Where entry j of a window lives. The two facts are flags, not null pointers: a pointer
+// that was computed must be compared with null again, entry by entry, in scalar code.
 struct Entry {
     const float* kv;
     const float* sc;
-    const float* ape;  // null: already in the score
+    const float* ape;
+    bool live;  // false: masked, the pointers mean nothing
+    bool emb;   // false: the embedding is already in the score
 };
+__device__ __forceinline__ Entry masked_entry() { return Entry{nullptr, nullptr, nullptr, false, false}; }
 
-// Prefill's overlap_transform as an index map (kvcompress.hip:264-309).
-__device__ __forceinline__ Entry prefill_entry(const float* kv, const float* score,
+// Prefill's overlap_transform as an index map (kvcompress.hip:264-309). kv_own / sc_own point
+// at the first row of block b: the one 64-bit product of the address is taken once per
+// workgroup and an entry adds a small signed element offset. OVERLAP (two halves per row,
+// ratio 4, eight entries: the guard admits no other overlapping geometry) is a compile-time
+// fact so that which row and half entry j reads is one too. Decided per entry at run time, the
+// scalar arithmetic in front of a row's first load was ~600 instructions and spilled scalar
+// registers; it is ~200 now. The launch took the same time either way.
+template <bool OVERLAP>
+__device__ __forceinline__ Entry prefill_entry(const float* kv_own, const float* sc_own,
                                                const float* ape, const CompGeom& p, int b, int j) {
-    int sblk = b, src_j = j, half = 0;
-    if (p.coff == 2) {
-        if (j >= p.ratio) {
-            src_j = j - p.ratio;
-            half = p.d;
-        } else if (b > 0) {
-            sblk = b - 1;
-        } else {
-            return Entry{nullptr, nullptr, nullptr};
+    if constexpr (OVERLAP) {
+        constexpr int kRatio = 4;
+        if (j >= kRatio) {  // this block's rows, their second half
+            const int rel = (j - kRatio) * p.cd + p.d;
+            return Entry{kv_own + rel, sc_own + rel, ape + rel, true, true};
         }
+        const int rel = (j - kRatio) * p.cd;  // the block before, first half: block 0 has none
+        return Entry{kv_own + rel, sc_own + rel, ape + j * p.cd, b != 0, b != 0};
+    } else {
+        const int rel = j * p.cd;
+        return Entry{kv_own + rel, sc_own + rel, ape + rel, true, true};
     }
-    const size_t src = (size_t)(sblk * p.ratio + src_j) * p.cd + half;
-    return Entry{kv + src, score + src, ape + (size_t)src_j * p.cd + half};
 }
 // Decode reads the state: low slots their overlap half, high slots their normal half
 // (kvcompress.hip:340-349).
@@ -70,7 +80,7 @@ __device__ __forceinline__ Entry state_entry(const float* kv_state, const float*
                                              const CompGeom& p, int j) {
     const int half = (p.coff == 2 && j >= p.ratio) ? p.d : 0;
     const size_t src = (size_t)j * p.cd + half;
-    return Entry{kv_state + src, score_state + src, nullptr};
+    return Entry{kv_state + src, score_state + src, nullptr, true, false};
 }
 
 // Softmax over the entries of VEC features starting at e, then the weighted sum
@@ -91,9 +101,9 @@ __device__ __forceinline__ void pool_registers(GetEntry&& entry, const float* sa
         bool emb[SLOTS];
 #pragma unroll
         for (int j = 0; j < SLOTS; ++j) {
-            const Entry en = j < ents ? entry(j) : Entry{nullptr, nullptr, nullptr};
-            live[j] = en.sc != nullptr;
-            emb[j] = live[j] && en.ape != nullptr;
+            const Entry en = j < ents ? entry(j) : masked_entry();
+            live[j] = en.live;
+            emb[j] = en.live && en.emb;
             s_raw[j] = *reinterpret_cast<const vec_t*>((live[j] ? en.sc : safe) + e);
             k_raw[j] = *reinterpret_cast<const vec_t*>((live[j] ? en.kv : safe) + e);
             a_raw[j] = *reinterpret_cast<const vec_t*>((emb[j] ? en.ape : safe) + e);
@@ -139,21 +149,21 @@ __device__ __forceinline__ float pool_streamed(GetEntry&& entry, int ents, int e
     float mx = -INFINITY;
     for (int j = 0; j < ents; ++j) {
         const Entry en = entry(j);
-        if (!en.sc) continue;
-        mx = fmaxf(mx, en.sc[e] + (en.ape ? en.ape[e] : 0.0f));
+        if (!en.live) continue;
+        mx = fmaxf(mx, en.sc[e] + (en.emb ? en.ape[e] : 0.0f));
     }
     if (!isfinite(mx)) return 0.0f;
     float sum = 0.0f;
     for (int j = 0; j < ents; ++j) {
         const Entry en = entry(j);
-        if (!en.sc) continue;
-        sum += expf(en.sc[e] + (en.ape ? en.ape[e] : 0.0f) - mx);
+        if (!en.live) continue;
+        sum += expf(en.sc[e] + (en.emb ? en.ape[e] : 0.0f) - mx);
     }
     float acc = 0.0f;
     for (int j = 0; j < ents; ++j) {
         const Entry en = entry(j);
-        if (!en.sc) continue;
-        acc += en.kv[e] * (expf(en.sc[e] + (en.ape ? en.ape[e] : 0.0f) - mx) / sum);
+        if (!en.live) continue;
+        acc += en.kv[e] * (expf(en.sc[e] + (en.emb ? en.ape[e] : 0.0f) - mx) / sum);
     }
     return acc;
 }
@@ -177,7 +187,7 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 // SLOTS: 8 or 16 = the window is held in that many register slots; 0 = streamed.
 template <int VEC, int SLOTS, class GetEntry>
 __device__ __forceinline__ void compress_row(GetEntry&& entry, const float* safe, const CompFinish& f, float* out_row,
-                                             int pos, const CompGeom& p, float* row, float* red) {
+                                             int pos, int ents, const CompGeom& p, float* row, float* red) {
     const int tid = threadIdx.x, nthr = blockDim.x;
     // what the finishing steps read (this lane's first norm weights and rotation pair) is
     // requested now, with the window, instead of one round trip after each barrier
@@ -195,10 +205,10 @@ __device__ __forceinline__ void compress_row(GetEntry&& entry, const float* safe
         float pooled[VEC];
         static_assert(VEC == 1 || VEC == 4, "one feature or four");
         if constexpr (SLOTS > 0) {
-            pool_registers<VEC, SLOTS>(entry, safe, p.ents, e, pooled);
+            pool_registers<VEC, SLOTS>(entry, safe, ents, e, pooled);
         } else {
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) pooled[i] = pool_streamed(entry, p.ents, e + i);
+            for (int i = 0; i < VEC; ++i) pooled[i] = pool_streamed(entry, ents, e + i);
         }
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
@@ -236,7 +246,7 @@ __device__ __forceinline__ void compress_row(GetEntry&& entry, const float* safe
 }
 
 // A window held in registers wants a small workgroup; wide windows stream and want many lanes.
-template <int VEC, int SLOTS>
+template <int VEC, int SLOTS, bool OVERLAP>
 __global__ __launch_bounds__(SLOTS ? 256 : 1024) void kv_compress_prefill_kernel(const float* __restrict__ kv,
                                            const float* __restrict__ score,
                                            const float* __restrict__ ape, CompFinish f,
@@ -245,9 +255,20 @@ __global__ __launch_bounds__(SLOTS ? 256 : 1024) void kv_compress_prefill_kernel
     float* row = lds;
     float* red = lds + p.d;
     const int b = blockIdx.x;
-    auto entry = [&](int j) { return prefill_entry(kv, score, ape, p, b, j); };
-    compress_row<VEC, SLOTS>(entry, score, f, f.out + (size_t)b * p.d, b * p.ratio, p, row, red);
+    const size_t own = (size_t)b * p.ratio * p.cd;
+    const float* const kv_own = kv + own;
+    const float* const sc_own = score + own;
+    auto entry = [&](int j) { return prefill_entry<OVERLAP>(kv_own, sc_own, ape, p, b, j); };
+    compress_row<VEC, SLOTS>(entry, score, f, f.out + (size_t)b * p.d, b * p.ratio,
+                             OVERLAP ? 8 : p.ents, p, row, red);
 }
+
+// Names the kernel by its window shape alone, as the dispatch below does.
+template <bool OVERLAP>
+struct PrefillKernel {
+    template <int VEC, int SLOTS>
+    static constexpr auto fn = &kv_compress_prefill_kernel<VEC, SLOTS, OVERLAP>;
+};
 
 // One workgroup: its barriers order the pooling's reads against the window slide.
 template <int VEC, int SLOTS>
@@ -258,7 +279,7 @@ __global__ __launch_bounds__(SLOTS ? 256 : 1024) void kv_compress_decode_kernel(
     float* red = lds + p.d;
     auto entry = [&](int j) { return state_entry(kv_state, score_state, p, j); };
     // the block's first absolute position, not its index (kvcompress.hip:360-371)
-    compress_row<VEC, SLOTS>(entry, score_state, f, f.out, (start_pos / p.ratio) * p.ratio, p, row, red);
+    compress_row<VEC, SLOTS>(entry, score_state, f, f.out, (start_pos / p.ratio) * p.ratio, p.ents, p, row, red);
     __syncthreads();
     if (p.coff == 2) {
         // this block's normal half becomes the next block's overlap half
@@ -396,8 +417,12 @@ extern "C" int rivoli_kv_compress_prefill(const float* kv, const float* score, c
                          rk::aligned16(ff->out);
     const rk::RowLaunch r = rk::row_launch(p, aligned);
     (void)hipGetLastError();
-    RK_COMPRESS_DISPATCH(rk::kv_compress_prefill_kernel, dim3((unsigned)nblk), r, p.ents,
-                         (hipStream_t)stream, kv, score, ape, *ff, p);
+    if (p.coff == 2)
+        RK_COMPRESS_DISPATCH(rk::PrefillKernel<true>::fn, dim3((unsigned)nblk), r, p.ents,
+                             (hipStream_t)stream, kv, score, ape, *ff, p);
+    else
+        RK_COMPRESS_DISPATCH(rk::PrefillKernel<false>::fn, dim3((unsigned)nblk), r, p.ents,
+                             (hipStream_t)stream, kv, score, ape, *ff, p);
     return rk::launch_status();
 }
 
