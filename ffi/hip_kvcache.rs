@@ -486,3 +486,5 @@ pub fn sel_shape(win: usize, ratio: usize, index_topk: usize, seqlen: usize, sta
 //   rivoli_kv_compress_deposit           launch_kv_compress_deposit, hip_attn.rs:547-605
 //   rivoli_kv_compress_prefill           launch_kv_compress_prefill, hip_attn.rs:547-605
 //   rivoli_kv_compress_decode            launch_kv_compress_decode, hip_attn.rs:547-605
+//   rivoli_act_quant_f4_rotated          launch_act_quant_f4_rotated, hip_linalg.rs:620
+//   rivoli_index_score_blocks            launch_index_score_blocks, hip.rs:497-520

@@ -291,6 +291,31 @@ int rivoli_mla_attend_paged(const float* qabs, const float* qrope, const unsigne
 int rivoli_act_quant_f8_prefix(const float* src, float* dst, int rows, int row_stride, int n,
                                int block, void* stream);
 
+/* Replaces crates/backend/kernels/blockindex.hip:241-262 (launch_act_quant_f4_rotated,
+ * crates/backend/src/hip_linalg.rs:620; callers crates/engine/src/v4/blocksel.rs:218 on the
+ * indexer's q rows and v4/kvcompress.rs:388 as the indexer compressor's finish): every row of
+ * x [rows][d], in place, becomes bf16(fp4(bf16(H x / sqrt(d)))) — H the natural-order
+ * (Sylvester) Hadamard matrix, the butterflies in the reference's stage order; fp4 = blocks of
+ * 32 with amax floored at 6 * 2^-126, scale 2^ceil(log2(amax / 6)), e2m1 nearest with ties to
+ * the even mantissa (actquant.hpp:45-105, formats.hpp:285-293). Bit-identical to the
+ * reference's kernel. Guards as the reference's: 1001 non-positive sizes (also a null
+ * pointer), 1002 d > 256, 1003 d not a power of two, 1004 d not a multiple of 32 (also x not
+ * 16-byte aligned). */
+int rivoli_act_quant_f4_rotated(float* x, int rows, int d, void* stream);
+
+/* Replaces crates/backend/kernels/blockindex.hip:264-281 (launch_index_score_blocks,
+ * crates/backend/src/hip.rs:497-520; caller v4/blocksel.rs:248): score[t][c] =
+ * bf16(sum_h bf16(relu(bf16(q[t][h] . kv[c])) * w[t][h])) for q [s][heads][hd], kv
+ * [n_comp][hd], w [s][heads], score [s][n_comp] — what rivoli_index_select_blocks ranks. The
+ * dot is a sequential f32 fold of separately rounded products and the head sum a sequential
+ * f32 fold rounded once, exactly as the reference's kernel, so the result is bit-identical
+ * to it. hd = 128 (the shipped width) with a 16-byte-aligned kv takes the register-resident
+ * kernel; any other width a slower one. Guards as the reference's: 1001 non-positive s, heads
+ * or hd (also null pointers); 1005 n_comp <= 0 (no block has completed: the caller must not
+ * rank an unwritten buffer). */
+int rivoli_index_score_blocks(const float* q, const float* kv, const float* w, float* score,
+                              int s, int n_comp, int heads, int hd, void* stream);
+
 /* The scored block selection that crates/engine/src/v4/select.rs:153-188 (scored_rows) performs
  * on the host after a device-to-host copy of the scores, as one launch on the device. scores is
  * [rows][n_comp] f32 (what launch_index_score_blocks wrote; illegal slots need not be masked).

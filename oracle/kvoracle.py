@@ -93,6 +93,40 @@ class _V4Mixin:
             _ptr(freqs, C.c_float), _ptr(out, C.c_float), C.byref(geom), nblk))
         return code, out[:max(nblk, 0)]
 
+    def e2m1_encode(self, x) -> int:
+        return int(self.lib.ro_e2m1_encode(float(np.float32(x))))
+
+    def e2m1_decode(self, code: int) -> np.float32:
+        return np.float32(self.lib.ro_e2m1_decode(int(code)))
+
+    def hadamard_rotate(self, row) -> np.ndarray:
+        out = _c(row, np.float32).copy()
+        self.lib.ro_hadamard_rotate(_ptr(out, C.c_float), out.size)
+        return out
+
+    def fp4_act_quant(self, row, block: int = 32) -> np.ndarray:
+        out = _c(row, np.float32).copy()
+        self.lib.ro_fp4_act_quant_inplace(_ptr(out, C.c_float), out.size, block)
+        return out
+
+    def act_quant_f4_rotated(self, x):
+        """x: [rows, d] f32. Returns (code, spread rows); the input is not modified."""
+        out = _c(x, np.float32).copy()
+        rows, d = out.shape
+        code = int(self.lib.ro_act_quant_f4_rotated(_ptr(out, C.c_float), rows, d))
+        return code, out
+
+    def index_score_blocks(self, q, kv, w):
+        """q: [s, heads, hd]; kv: [n_comp, hd]; w: [s, heads]. Returns (code, score[s, n_comp])."""
+        q, kv, w = _c(q, np.float32), _c(kv, np.float32), _c(w, np.float32)
+        s, heads, hd = q.shape
+        n_comp = kv.shape[0]
+        score = np.zeros((s, max(n_comp, 1)), np.float32)
+        code = int(self.lib.ro_index_score_blocks(_ptr(q, C.c_float), _ptr(kv, C.c_float),
+                                                  _ptr(w, C.c_float), _ptr(score, C.c_float), s, n_comp,
+                                                  heads, hd))
+        return code, score[:, :n_comp]
+
     def kv_compress_decode(self, kv_state, score_state, norm, freqs, geom: CompGeom, start_pos: int):
         """Returns (code, out[d]); the states are updated in place (the window slides)."""
         norm, freqs = _c(norm, np.float32), _c(freqs, np.float32)
@@ -231,6 +265,12 @@ class Oracle(_V4Mixin):
             "ro_kv_compress_deposit": (C.c_int, [f32p] * 5 + [C.POINTER(CompGeom), C.c_int, C.c_int]),
             "ro_kv_compress_prefill": (C.c_int, [f32p] * 6 + [C.POINTER(CompGeom), C.c_int]),
             "ro_kv_compress_decode": (C.c_int, [f32p] * 5 + [C.POINTER(CompGeom), C.c_int]),
+            "ro_e2m1_encode": (C.c_uint8, [C.c_float]),
+            "ro_e2m1_decode": (C.c_float, [C.c_uint8]),
+            "ro_hadamard_rotate": (None, [f32p, C.c_int]),
+            "ro_fp4_act_quant_inplace": (None, [f32p, C.c_int, C.c_int]),
+            "ro_act_quant_f4_rotated": (C.c_int, [f32p, C.c_int, C.c_int]),
+            "ro_index_score_blocks": (C.c_int, [f32p] * 4 + [C.c_int] * 4),
         }
         for name, (res, args) in sig.items():
             fn = getattr(lib, name)

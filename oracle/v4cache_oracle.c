@@ -443,3 +443,102 @@ int ro_kv_compress_decode(float* kv_state, float* score_state, const float* norm
     }
     return 0;
 }
+
+/* ------------------------------------------------------------------------------------------
+ * The indexer's spread (Hadamard + simulated fp4) and its block scorer
+ * ---------------------------------------------------------------------------------------- */
+
+/* formats.hpp:285-293 / numerics.rs e2m1_encode: the code is the number of midpoints passed;
+ * a tie goes up at an odd-indexed midpoint (to the even mantissa). NaN passes none. */
+uint8_t ro_e2m1_encode(float x) {
+    static const float mid[7] = {0.25f, 0.75f, 1.25f, 1.75f, 2.5f, 3.5f, 5.0f};
+    const float a = fabsf(x);
+    unsigned code = 0;
+    for (int i = 0; i < 7; ++i) code += (a > mid[i] || (a == mid[i] && (i & 1))) ? 1u : 0u;
+    return (uint8_t)((signbit(x) ? 8u : 0u) | code);
+}
+
+float ro_e2m1_decode(uint8_t c) {
+    static const float mag[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+    const float m = mag[c & 7u];
+    return (c & 8u) ? -m : m;
+}
+
+/* numerics.rs:324-353: Sylvester (natural-order) butterflies, h = 1, 2, 4, ..., then one
+ * multiply by 1 / sqrt(n) with a correctly rounded square root and a true divide. */
+void ro_hadamard_rotate(float* row, int n) {
+    for (int h = 1; h < n; h *= 2)
+        for (int i = 0; i < n; i += 2 * h)
+            for (int j = i; j < i + h; ++j) {
+                const float a = row[j], b = row[j + h];
+                row[j] = a + b;
+                row[j + h] = a - b;
+            }
+    const float scale = 1.0f / sqrtf((float)n);
+    for (int i = 0; i < n; ++i) row[i] *= scale;
+}
+
+/* numerics.rs:245-298 with the fp4 constants (actquant.hpp:45-51): block amax floored at
+ * 6 * 2^-126, scale rounded up to a power of two, clamp by comparisons, e2m1 round trip. */
+void ro_fp4_act_quant_inplace(float* row, int n, int block) {
+    const float fp4_max = 6.0f;
+    const float floor_amax = fp4_max * float_of(1u << 23);
+    for (int b0 = 0; b0 < n; b0 += block) {
+        const int len = n - b0 < block ? n - b0 : block;
+        float amax = 0.0f;
+        for (int i = 0; i < len; ++i) amax = fmaxf(amax, fabsf(row[b0 + i]));
+        amax = fmaxf(amax, floor_amax);
+        const float s = ro_fast_round_scale(amax, 1.0f / fp4_max);
+        for (int i = 0; i < len; ++i) {
+            float q = row[b0 + i] / s;
+            q = q < -fp4_max ? -fp4_max : (q > fp4_max ? fp4_max : q);
+            row[b0 + i] = ro_e2m1_decode(ro_e2m1_encode(q)) * s;
+        }
+    }
+}
+
+/* blockindex.hip:99-136 behind the launcher's guards (:241-262): rotate, store as bf16,
+ * quantize in blocks of 32, store as bf16 — the order of kernel_v4_indexer.rs:149-156. */
+int ro_act_quant_f4_rotated(float* x, int rows, int d) {
+    if (rows <= 0 || d <= 0) return 1001;
+    if (d > 256) return 1002;
+    if (d & (d - 1)) return 1003;
+    if (d % 32) return 1004;
+    for (int r = 0; r < rows; ++r) {
+        float* row = x + (size_t)r * d;
+        ro_hadamard_rotate(row, d);
+        for (int i = 0; i < d; ++i) row[i] = round_bf16(row[i]);
+        ro_fp4_act_quant_inplace(row, d, 32);
+        for (int i = 0; i < d; ++i) row[i] = round_bf16(row[i]);
+    }
+    return 0;
+}
+
+/* blockindex.hip:209-235 (and kernel_v4_indexer.rs:437-462, the same fold on the host) behind
+ * the launcher's guards (:264-281). q: [s][heads][hd]; kv: [n_comp][hd]; w: [s][heads];
+ * score: [s][n_comp]. Products and sums are separate roundings (this file is built with
+ * -ffp-contract=off); the head sum is carried in f32 and rounded to bf16 once. */
+int ro_index_score_blocks(const float* q, const float* kv, const float* w, float* score, int s,
+                          int n_comp, int heads, int hd) {
+    if (s <= 0 || heads <= 0 || hd <= 0) return 1001;
+    if (n_comp <= 0) return 1005;
+    for (int t = 0; t < s; ++t)
+        for (int c = 0; c < n_comp; ++c) {
+            const float* kvr = kv + (size_t)c * hd;
+            float acc = 0.0f;
+            for (int hh = 0; hh < heads; ++hh) {
+                const float* qh = q + ((size_t)t * heads + hh) * hd;
+                float dot = 0.0f;
+                for (int i = 0; i < hd; ++i) {
+                    const float prod = qh[i] * kvr[i];
+                    dot = dot + prod;
+                }
+                dot = round_bf16(dot);
+                dot = dot > 0.0f ? dot : 0.0f;  /* the sign of a zero cannot reach the output */
+                const float term = dot * w[(size_t)t * heads + hh];
+                acc = acc + round_bf16(term);
+            }
+            score[(size_t)t * n_comp + c] = round_bf16(acc);
+        }
+    return 0;
+}

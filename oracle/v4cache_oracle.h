@@ -31,6 +31,24 @@
  *                         with the same per-feature fold). The reference's expectation for
  *                         these kernels is computed at test time from seeded weights
  *                         (crates/engine/tests/kernel_v4_compress.rs); it stores no vectors.
+ *   ro_e2m1_encode / ro_e2m1_decode  (tests/test_oracle_v4_blockindex.py, as all of this group)
+ *                         the seven midpoints as crates/oracles/tests/v4_oracle_codecs.rs:163-180
+ *                         writes them, nearest magnitude by enumeration, saturation at +-1e9,
+ *                         every code its own nearest (ibid. :181-207)
+ *   ro_hadamard_rotate    equality with scipy's Sylvester matrix on integer inputs (exact in
+ *                         f32, so a different basis order fails); involution and norm
+ *                         (v4_oracle_codecs.rs:387-420)
+ *   ro_fp4_act_quant_inplace  scale = smallest power of two >= amax / 6 from frexp; every output
+ *                         the nearest of the eight magnitudes times that scale; the floor
+ *   ro_act_quant_f4_rotated  the four steps in the order of
+ *                         crates/engine/tests/kernel_v4_indexer.rs:149-156 from the parts above
+ *                         (the store between rotation and quantization shown to matter);
+ *                         power-of-two equivariance over 60 binades (ibid. :246-277); guards
+ *                         (:287-320); on the GPU also the reference's own kernel
+ *   ro_index_score_blocks the reference's known answer 1.125 (kernel_v4_indexer.rs:689-726);
+ *                         closed forms that isolate each bf16 store, the relu and signed
+ *                         weights; inputs on which a reordered or fused dot changes the
+ *                         bits; guards; on the GPU also the reference's own kernel
  *   ro_v4_scored_rows     the three reference KATs (crates/engine/src/v4/select.rs:645-747:
  *                         below the cap the row is offset+0..limit-1 then -1; three-way tie
  *                         keeps the lower indices; a prefill row cannot take a block that
@@ -156,6 +174,25 @@ int ro_kv_compress_prefill(const float* kv, const float* score, const float* ape
  * then slide the window when overlapping. Code 1000 / guard / 1007 / 1009 / 0. */
 int ro_kv_compress_decode(float* kv_state, float* score_state, const float* norm,
                           const float* freqs, float* out, const ro_comp_geom* p, int start_pos);
+
+/* ---- the indexer's spread and block scorer (crates/backend/kernels/blockindex.hip) ---- */
+
+/* formats.hpp:285-293 and its decode table {0, .5, 1, 1.5, 2, 3, 4, 6}; bit 3 is the sign. */
+uint8_t ro_e2m1_encode(float x);
+float ro_e2m1_decode(uint8_t code);
+
+/* crates/oracles/src/v4oracle/numerics.rs:324-353, n a power of two, in place. */
+void ro_hadamard_rotate(float* row, int n);
+
+/* numerics.rs:245-298 with actquant.hpp:45-51's constants, in place over n values. */
+void ro_fp4_act_quant_inplace(float* row, int n, int block);
+
+/* blockindex.hip:99-136 + :241-262, x: [rows][d] in place. Code 1001-1004 or 0. */
+int ro_act_quant_f4_rotated(float* x, int rows, int d);
+
+/* blockindex.hip:209-235 + :264-281. Code 1001, 1005 or 0. */
+int ro_index_score_blocks(const float* q, const float* kv, const float* w, float* score, int s,
+                          int n_comp, int heads, int hd);
 
 #ifdef __cplusplus
 }

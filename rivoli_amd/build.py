@@ -14,7 +14,8 @@ CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(CSRC, "librivoli_kvcache.so")
 HOST_LIB_PATH = os.path.join(CSRC, "librivoli_pagepool.so")
 KERNELS = ["kv_append.hip", "kv_gather.hip", "index_topk.hip", "index_score.hip", "mla_attend.hip",
-           "act_quant.hip", "kv_compress.hip", "kv_ring.hip", "gather_attn.hip", "hash_rows.hip"]
+           "act_quant.hip", "kv_compress.hip", "kv_ring.hip", "gather_attn.hip", "hash_rows.hip",
+           "block_index.hip"]
 # Matrix-instruction results in ordinary registers: the 8-bit attention kernel keeps its 128
 # accumulators there and its q terms in the accumulation registers (mla_attend_f8.hpp); the bf16
 # kernels of the same file time the same either way.

@@ -1,0 +1,226 @@
+// The second cache format's block indexer: the Hadamard + simulated-fp4 spread of its q rows
+// and of its compressor's pooled rows, and the block scorer that ranks compressed blocks for a
+// query (crates/backend/kernels/blockindex.hip:99-136 and :209-235, launchers :241-281; CPU
+// statements crates/oracles/src/v4oracle/numerics.rs:245-353 and
+// crates/engine/tests/kernel_v4_indexer.rs:437-462). Both are bit-exact by construction: every
+// value is produced by the reference's tree of f32 operations; what differs is who computes
+// which value and where the operands wait.
+//
+// Spread. The reference gives a row to a 128-thread workgroup and walks LDS log2(d) times with
+// a barrier per stage, then hands each fp4 block of 32 to one thread. Here a lane holds four
+// consecutive values of a row (one 16-byte load and store, a wave moves 1 KiB per instruction),
+// d / 4 neighbouring lanes hold a row, and a wave holds 64 / (d / 4) rows. The butterflies of
+// stages 1 and 2 pair values of one lane; stage h >= 4 pairs lane L with lane L ^ (h / 4): the
+// lane whose bit is clear holds the pair's first value and computes a + b, the other computes
+// a - b from the same two numbers. A block of 32 is eight lanes; its amax is a maximum (exact
+// in any order) over three lane exchanges. No LDS, no barrier; 8 bytes of traffic per value.
+//
+// Scorer. score[t][c] = bf16(sum_h bf16(relu(bf16(q[t][h] . kv[c])) * w[t][h])), the dot a
+// sequential f32 fold of separately rounded products and the head sum a sequential f32 fold
+// (blockindex.hip:138-207 argues each). That order rules out the matrix cores and any split of
+// a dot over lanes; what is free is where the operands come from. A lane owns block c and
+// keeps its 128-value row in registers for the whole launch; a wave's 64 lanes share the query,
+// so q[t][h][i] and w[t][h] are wave-uniform and come through scalar loads straight into the
+// multiply's scalar operand. Per (t, h) a wave issues 128 multiplies and 128 adds for 64
+// scores and reads 512 bytes through the scalar cache: bound by vector issue, two
+// instructions per multiply-add because the reference's rounding is two roundings.
+// Widths other than 128 re-read the block's row through the vector cache instead.
+#include "codec.hpp"
+
+#include <cmath>
+
+#include "rivoli_kvcache.h"
+
+#pragma clang fp contract(off)
+
+namespace rk {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr float kFp4Max = 6.0f;
+constexpr float kFp4MaxInv = 1.0f / kFp4Max;
+constexpr float kFp4AmaxFloor = kFp4Max * 1.17549435082228750797e-38f;  // 6 * 2^-126 (actquant.hpp:51)
+constexpr int kSpreadMaxD = 256;   // blockindex.hip:40-42
+constexpr int kSpreadThreads = 256;
+constexpr int kSpreadInFlight = 4;  // row groups per wave, all requested before the first is used
+
+__device__ __forceinline__ float round_bf16(float x) {
+    return __uint_as_float((uint32_t)f32_to_bf16(x) << 16);
+}
+
+// formats.hpp:285-293 followed by its decode: the magnitude is the last of the eight whose
+// midpoint was passed; a tie passes an odd-indexed midpoint only. The sign is q's sign bit.
+__device__ __forceinline__ float e2m1_round_trip(float q) {
+    const float mid[7] = {0.25f, 0.75f, 1.25f, 1.75f, 2.5f, 3.5f, 5.0f};
+    const float mag[7] = {0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+    const float a = fabsf(q);
+    float v = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 7; ++i)
+        if (a > mid[i] || (a == mid[i] && (i & 1))) v = mag[i];
+    return __builtin_signbit(q) ? -v : v;
+}
+
+// LPR: lanes per row (d / 4). scale = 1 / sqrt(d), taken on the host (a correctly rounded
+// square root and a true divide, blockindex.hip:107-113).
+template <int LPR>
+__global__ __launch_bounds__(kSpreadThreads) void f4_rotated_kernel(float* __restrict__ x,
+                                                                     long long rows, float scale) {
+    constexpr int kRowsPerWave = kWave / LPR;
+    constexpr int d = LPR * 4;
+    const int lane = threadIdx.x & (kWave - 1);
+    const long long wave = (long long)blockIdx.x * (kSpreadThreads / kWave) + (threadIdx.x >> 6);
+    const long long row0 = wave * (kRowsPerWave * kSpreadInFlight) + lane / LPR;
+    const int col = (lane % LPR) * 4;
+
+    f32x4 v[kSpreadInFlight];
+#pragma unroll
+    for (int u = 0; u < kSpreadInFlight; ++u) {
+        const long long r = row0 + (long long)u * kRowsPerWave;
+        // unconditional: a row past the end re-reads the last row and is not stored
+        v[u] = *reinterpret_cast<const f32x4*>(x + (r < rows ? r : rows - 1) * d + col);
+    }
+#pragma unroll
+    for (int u = 0; u < kSpreadInFlight; ++u) {
+        float e[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+        // stages h = 1, 2: inside the lane
+        {
+            const float a0 = e[0] + e[1], a1 = e[0] - e[1], a2 = e[2] + e[3], a3 = e[2] - e[3];
+            e[0] = a0 + a2, e[2] = a0 - a2, e[1] = a1 + a3, e[3] = a1 - a3;
+        }
+        // stages h = 4 .. d / 2: lane L with lane L ^ (h / 4)
+#pragma unroll
+        for (int m = 1; m < LPR; m <<= 1) {
+            const bool upper = (lane & m) != 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float other = __shfl_xor(e[i], m, kWave);
+                e[i] = upper ? other - e[i] : e[i] + other;
+            }
+        }
+        // the bf16 store between rotation and quantization (blockindex.hip:91-96)
+        float amax = kFp4AmaxFloor;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            e[i] = round_bf16(e[i] * scale);
+            amax = fmaxf(amax, fabsf(e[i]));
+        }
+        // a block of 32 is 8 lanes; d = 32 is the whole row
+#pragma unroll
+        for (int m = 1; m < 8; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m, kWave));
+        // actquant.hpp:65-75: the smallest power of two >= amax / 6, by exponent surgery
+        const uint32_t b = __float_as_uint(amax * kFp4MaxInv);
+        const int ex = (int)((b >> 23) & 0xffu) - 127 + ((b & 0x7fffffu) ? 1 : 0);
+        const float s = __uint_as_float((uint32_t)(ex + 127) << 23);
+        f32x4 out;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float q = e[i] / s;  // s is a power of two: exact unless the quotient leaves the range
+            q = q < -kFp4Max ? -kFp4Max : (q > kFp4Max ? kFp4Max : q);  // a NaN stays a NaN
+            out[i] = round_bf16(e2m1_round_trip(q) * s);
+        }
+        const long long r = row0 + (long long)u * kRowsPerWave;
+        if (r < rows) *reinterpret_cast<f32x4*>(x + r * d + col) = out;
+    }
+}
+
+// ---- the block scorer -------------------------------------------------------------------------
+constexpr int kScoreThreads = 256;           // four waves, 64 blocks each
+constexpr int kScoreQueriesPerGroup = 16;    // queries a workgroup walks with its rows held
+
+// One (query, block) score from a row held in registers (HD > 0) or re-read (HD == 0).
+template <int HD>
+__global__ __launch_bounds__(kScoreThreads) void index_score_blocks_kernel(
+    const float* __restrict__ q, const float* __restrict__ kv, const float* __restrict__ w,
+    float* __restrict__ score, int s, int n_comp, int heads, int hd_rt, int t_per_group) {
+    const int hd = HD ? HD : hd_rt;
+    const long long c = (long long)blockIdx.x * kScoreThreads + threadIdx.x;
+    const float* const kvr = kv + (size_t)(c < n_comp ? c : n_comp - 1) * hd;
+    float row[HD ? HD : 1];
+    if constexpr (HD > 0) {
+#pragma unroll
+        for (int i = 0; i < HD; i += 4) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(kvr + i);
+            row[i] = v.x, row[i + 1] = v.y, row[i + 2] = v.z, row[i + 3] = v.w;
+        }
+    }
+    const int t0 = blockIdx.y * t_per_group;
+    const int t1 = min(s, t0 + t_per_group);
+    for (int t = t0; t < t1; ++t) {
+        float acc = 0.0f;
+        for (int hh = 0; hh < heads; ++hh) {
+            const float* const qh = q + ((size_t)t * heads + hh) * hd;  // wave-uniform
+            float dot = 0.0f;
+            if constexpr (HD > 0) {
+#pragma unroll
+                for (int i = 0; i < HD; ++i) {
+                    const float prod = qh[i] * row[i];
+                    dot = dot + prod;
+                }
+            } else {
+                for (int i = 0; i < hd; ++i) {
+                    const float prod = qh[i] * kvr[i];
+                    dot = dot + prod;
+                }
+            }
+            // bf16 first, then the relu (blockindex.hip:224-228); the sign of a zero cannot
+            // reach the output
+            dot = round_bf16(dot);
+            dot = dot > 0.0f ? dot : 0.0f;
+            const float term = dot * w[(size_t)t * heads + hh];
+            acc = acc + round_bf16(term);
+        }
+        if (c < n_comp) score[(size_t)t * n_comp + c] = round_bf16(acc);
+    }
+}
+
+}  // namespace rk
+
+extern "C" int rivoli_act_quant_f4_rotated(float* x, int rows, int d, void* stream) {
+    if (rows <= 0 || d <= 0) return 1001;
+    if (d > rk::kSpreadMaxD) return 1002;
+    if (d & (d - 1)) return 1003;
+    if (d % 32) return 1004;
+    if (!x) return 1001;
+    if (!rk::aligned16(x)) return 1004;  // rows are moved 16 bytes at a time
+    (void)hipGetLastError();
+    const float scale = 1.0f / std::sqrt((float)d);
+    const int lpr = d / 4;
+    const long long rows_per_group = (long long)(rk::kWave / lpr) * rk::kSpreadInFlight *
+                                     (rk::kSpreadThreads / rk::kWave);
+    const dim3 grid((unsigned)((rows + rows_per_group - 1) / rows_per_group)), block(rk::kSpreadThreads);
+    hipStream_t st = (hipStream_t)stream;
+    switch (lpr) {
+        case 8: hipLaunchKernelGGL(rk::f4_rotated_kernel<8>, grid, block, 0, st, x, (long long)rows, scale); break;
+        case 16: hipLaunchKernelGGL(rk::f4_rotated_kernel<16>, grid, block, 0, st, x, (long long)rows, scale); break;
+        case 32: hipLaunchKernelGGL(rk::f4_rotated_kernel<32>, grid, block, 0, st, x, (long long)rows, scale); break;
+        default: hipLaunchKernelGGL(rk::f4_rotated_kernel<64>, grid, block, 0, st, x, (long long)rows, scale); break;
+    }
+    return rk::launch_status();
+}
+
+extern "C" int rivoli_index_score_blocks(const float* q, const float* kv, const float* w,
+                                         float* score, int s, int n_comp, int heads, int hd,
+                                         void* stream) {
+    if (s <= 0 || heads <= 0 || hd <= 0) return 1001;
+    // refused, not an empty success: the reference produces no score tensor at all before the
+    // first block completes (blockindex.hip:268-273)
+    if (n_comp <= 0) return 1005;
+    if (!q || !kv || !w || !score) return 1001;
+    (void)hipGetLastError();
+    // enough workgroups to fill the part while a workgroup keeps its rows for several queries
+    const unsigned c_groups = (unsigned)(((long long)n_comp + rk::kScoreThreads - 1) / rk::kScoreThreads);
+    int t_per_group = rk::kScoreQueriesPerGroup;
+    while (t_per_group > 1 && (long long)c_groups * ((s + t_per_group - 1) / t_per_group) < 2048) t_per_group >>= 1;
+    while ((s + t_per_group - 1) / t_per_group > 65535) t_per_group <<= 1;  // the grid's second extent
+    const unsigned t_groups = (unsigned)((s + t_per_group - 1) / t_per_group);
+    const dim3 grid(c_groups, t_groups), block(rk::kScoreThreads);
+    hipStream_t st = (hipStream_t)stream;
+    if (hd == 128 && rk::aligned16(kv))
+        hipLaunchKernelGGL(rk::index_score_blocks_kernel<128>, grid, block, 0, st, q, kv, w, score, s,
+                           n_comp, heads, hd, t_per_group);
+    else
+        hipLaunchKernelGGL(rk::index_score_blocks_kernel<0>, grid, block, 0, st, q, kv, w, score, s,
+                           n_comp, heads, hd, t_per_group);
+    return rk::launch_status();
+}

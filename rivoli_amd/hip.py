@@ -59,6 +59,8 @@ _SIGNATURES = {
     "rivoli_mla_attend": [_VP] * 6 + [_I] * 5 + [_F, _VP, _VP],
     "rivoli_mla_attend_paged": [_VP] * 7 + [_I] * 8 + [_F, _I, _VP, _VP, _VP, _VP],
     "rivoli_act_quant_f8_prefix": [_VP, _VP] + [_I] * 4 + [_VP],
+    "rivoli_act_quant_f4_rotated": [_VP, _I, _I, _VP],
+    "rivoli_index_score_blocks": [_VP] * 4 + [_I] * 4 + [_VP],
     "rivoli_index_select_blocks": [_VP] + [_I] * 6 + [_VP, _VP],
     "rivoli_sel_shape": [_I] * 5 + [_VP, _VP],
     "rivoli_sel_gather": [_I] * 5 + [_VP, _VP],
@@ -311,6 +313,18 @@ def launch_act_quant_f8_prefix(src, dst, rows, row_stride, n, block, stream=NULL
     [0, n) of every row in blocks of `block`; src may be dst."""
     ensure_hip_status(lib().rivoli_act_quant_f8_prefix(_p(src), _p(dst), rows, row_stride, n, block,
                                                        _s(stream)), "act_quant_f8_prefix")
+
+
+def launch_act_quant_f4_rotated(x, rows, d, stream=NULL_STREAM) -> None:
+    """crates/backend/src/hip_linalg.rs:620 launch_act_quant_f4_rotated: the Hadamard + fp4
+    spread of every row of x [rows][d], in place."""
+    ensure_hip_status(lib().rivoli_act_quant_f4_rotated(_p(x), rows, d, _s(stream)), "act_quant_f4_rotated")
+
+
+def launch_index_score_blocks(q, kv, w, score, s, n_comp, heads, hd, stream=NULL_STREAM) -> None:
+    """crates/backend/src/hip.rs:497-520 launch_index_score_blocks: block scores [s][n_comp]."""
+    ensure_hip_status(lib().rivoli_index_score_blocks(_p(q), _p(kv), _p(w), _p(score), s, n_comp, heads, hd,
+                                                      _s(stream)), "index_score_blocks")
 
 
 def launch_index_select_blocks(scores, rows, n_comp, ratio, index_topk, prefill, offset, out,

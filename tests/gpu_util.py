@@ -65,6 +65,11 @@ def ref_kernels():
             h.rivoli_kv_compress_prefill.argtypes = [vp] * 5 + [i, vp]
             h.rivoli_kv_compress_decode.restype = i
             h.rivoli_kv_compress_decode.argtypes = [vp] * 4 + [i, vp]
+        if hasattr(h, "rivoli_index_score_blocks"):
+            h.rivoli_act_quant_f4_rotated.restype = i
+            h.rivoli_act_quant_f4_rotated.argtypes = [vp, i, i, vp]
+            h.rivoli_index_score_blocks.restype = i
+            h.rivoli_index_score_blocks.argtypes = [vp] * 4 + [i] * 4 + [vp]
         h.rivoli_hash_rows.restype = i
         h.rivoli_hash_rows.argtypes = [vp, i, i, C.c_ulonglong, vp, vp]
         _REF = h

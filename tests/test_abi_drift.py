@@ -22,7 +22,7 @@ REFERENCE_ROWS = {
     "rivoli_append_kv", "rivoli_index_append", "rivoli_index_topk", "rivoli_index_score", "rivoli_hash_rows",
     "rivoli_mla_attend", "rivoli_mla_attend_scratch_floats", "rivoli_device_sync", "rivoli_act_quant_f8_prefix",
     "rivoli_gather_attn_shared_kv", "rivoli_kv_compress_deposit", "rivoli_kv_compress_prefill",
-    "rivoli_kv_compress_decode",
+    "rivoli_kv_compress_decode", "rivoli_act_quant_f4_rotated", "rivoli_index_score_blocks",
 }
 
 C_ELEM = {"float": "f32", "unsigned char": "u8", "unsigned short": "u16", "int": "i32", "unsigned int": "u32",
