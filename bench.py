@@ -41,7 +41,7 @@ def parse():
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=32768)
     ap.add_argument("--workload", choices=["all", "decode", "prefill", "dsa", "dsa_scored", "dsa_attend", "attend", "v4",
-                                           "v4_attend"],
+                                           "v4_attend", "v4_index"],
                     default="all",
                     help="all (default) = the headline line with every other configuration attached under `configs`; decode = configuration 3 (the headline line) alone; prefill = configuration 2 "
                          "bulk append; dsa = configuration 4 top-k + sparse gather on synthetic "
@@ -55,7 +55,10 @@ def parse():
                          "query row (ratio 4, cap --index-topk); "
                          "v4_attend = the second cache format's consumer at prefill: ring write, the "
                          "[window | scored blocks] selection rectangle, and the index-list attention "
-                         "of `tokens` queries x --heads heads over it")
+                         "of `tokens` queries x --heads heads over it; "
+                         "v4_index = the second cache format's block indexer at prefill: the Hadamard + "
+                         "fp4 spread of `tokens` x --heads query rows of 128 and the block scores of "
+                         "every query against the tokens / 4 compressed blocks")
     ap.add_argument("--index-topk", type=int, default=512, help="v4: blocks kept per query row")
     ap.add_argument("--heads", type=int, default=64, help="attend: query heads")
     ap.add_argument("--precise", type=int, default=2, choices=[0, 1, 2, 3, 4],
@@ -130,7 +133,8 @@ def main():
               ("attend_decode_bf16x2", "attend", dict(precise=2)),
               # the second cache format's own operators, at prefill
               ("v4_prefill_32768", "v4", dict(tokens=32768)),
-              ("v4_attend_prefill_8192", "v4_attend", dict(tokens=8192, precise=2)))
+              ("v4_attend_prefill_8192", "v4_attend", dict(tokens=8192, precise=2)),
+              ("v4_index_prefill_4096", "v4_index", dict(tokens=4096)))
     res["configs"] = {}
     for name, workload, over in others:
         torch.cuda.empty_cache()
@@ -152,6 +156,8 @@ def run_workload(workload, a, torch, hip):
         return bench_v4(a, torch, hip)
     if workload == "v4_attend":
         return bench_v4_attend(a, torch, hip)
+    if workload == "v4_index":
+        return bench_v4_index(a, torch, hip)
     raise SystemExit(f"unknown workload {workload}")
 
 
@@ -527,6 +533,84 @@ def bench_v4(a, torch, hip):
                                "sample": f"the first {nr} rows of the same inputs through the oracle's "
                                          "compressor pooling, act_quant and scored_rows, one host thread; "
                                          "GPU results checked (pooling within 2 bf16 codes, the others equal)"}
+    return res
+
+
+def bench_v4_index(a, torch, hip):
+    """The second cache format's block indexer at prefill (crates/engine/src/v4/blocksel.rs:218-248):
+    `tokens` queries x `heads` index heads of 128 are spread in place (Hadamard + simulated fp4),
+    then every query is scored against the tokens / 4 compressed blocks (spread rows as well)."""
+    s, heads, hd, ratio = a.tokens, a.heads, 128, 4
+    n_comp = max(s // ratio, 1)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0x5EED0007)
+    q_raw = torch.randn(s * heads, hd, generator=g, device="cuda", dtype=torch.float32).bfloat16().float()
+    kv = torch.randn(n_comp, hd, generator=g, device="cuda", dtype=torch.float32).bfloat16().float()
+    w = (torch.randn(s, heads, generator=g, device="cuda", dtype=torch.float32) * hd ** -0.5).bfloat16().float()
+    hip.launch_act_quant_f4_rotated(kv, n_comp, hd)     # the indexer compressor's finish
+    q = q_raw.clone()
+    score = torch.empty(s, n_comp, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.Stream()
+    sh = stream.cuda_stream
+
+    def step(events):
+        bracket(torch, stream, events, "spread", lambda: hip.launch_act_quant_f4_rotated(q, s * heads, hd, sh))
+        bracket(torch, stream, events, "score",
+                lambda: hip.launch_index_score_blocks(q, kv, w, score, s, n_comp, heads, hd, sh))
+
+    ms, per = timed(torch, stream, a.steps, a.warmup, step)
+    spread_bytes = s * heads * hd * 8                                   # f32 in, f32 out
+    score_flops = 2 * s * n_comp * heads * hd                           # one multiply and one add per term
+    score_bytes = s * heads * hd * 4 + n_comp * hd * 4 + s * n_comp * 4
+    # the timed steps spread the same buffer again and again; the check runs one step on a fresh copy
+    q.copy_(q_raw)
+    torch.cuda.synchronize()
+    step(None)
+    stream.synchronize()
+    res = {"metric": "v4_block_index_scores_per_s", "value": round(s * n_comp / (ms * 1e-3), 1), "unit": "scores/s",
+           "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "second cache format, prefill: Hadamard + fp4 spread of the index queries, block "
+                                  "scores of every query against every compressed block (sequential f32 folds, "
+                                  "bit-identical to the reference's kernel)",
+                      "tokens": s, "heads": heads, "head_dim": hd, "ratio": ratio, "n_comp": n_comp},
+           "tokens_per_s": round(s / (ms * 1e-3), 1),
+           "kernels": {"f4_rotated_kernel": {"avg_launch_ms": round(per["spread"], 5), "bytes_per_launch": spread_bytes,
+                                             "GBps": round(spread_bytes / (per["spread"] * 1e-3) / 1e9, 1)},
+                       "index_score_blocks_kernel": {"avg_launch_ms": round(per["score"], 5),
+                                                     "flops_per_launch": score_flops, "bytes_per_launch": score_bytes,
+                                                     "TFLOPps": round(score_flops / (per["score"] * 1e-3) / 1e12, 2)}},
+           # the scorer is bound by vector issue, not by memory or the matrix cores: the published
+           # fp32 vector peak counts a fused multiply-add on packed pairs as four operations per lane
+           # and cycle; the reference's two roundings per term allow one
+           "roofline": {"bound": "fp32", "kernel": "index_score_blocks_kernel",
+                        "achieved": round(score_flops / (per["score"] * 1e-3) / 1e12, 2), "peak": 157.3,
+                        "unit": "TFLOP/s", "frac": round(score_flops / (per["score"] * 1e-3) / 157.3e12, 4),
+                        "unfused_unpacked_peak": 39.3,
+                        "frac_of_unfused_unpacked_peak": round(score_flops / (per["score"] * 1e-3) / 39.3e12, 4),
+                        "avg_launch_ms": round(per["score"], 5), "traffic": None}}
+    if not a.no_cpu_baseline:
+        from oracle.kvoracle import oracle as get_oracle
+
+        ora = get_oracle()
+        rows = sorted({0, 1, s // 2, s - 1} | set(range(min(s, 12))))
+        q_h = q_raw.view(s, heads, hd)[rows].cpu().numpy()
+        kv_h, w_h = kv.cpu().numpy(), w[rows].cpu().numpy()
+        t0 = time.perf_counter()
+        code_q, want_q = ora.act_quant_f4_rotated(q_h.reshape(-1, hd))
+        code_s, want_s = ora.index_score_blocks(want_q.reshape(len(rows), heads, hd), kv_h, w_h)
+        spent = time.perf_counter() - t0
+        got_q = q.view(s, heads, hd)[rows].cpu().numpy().reshape(-1, hd)
+        got_s = score[rows].cpu().numpy()
+        if code_q != 0 or not np.array_equal(got_q.view(np.uint32), want_q.view(np.uint32)):
+            raise SystemExit("bench: GPU spread differs from the CPU oracle")
+        if code_s != 0 or not np.array_equal(got_s.view(np.uint32), want_s.view(np.uint32)):
+            raise SystemExit("bench: GPU block scores differ from the CPU oracle")
+        res["cpu_baseline"] = {"value": round(len(rows) * n_comp / spent, 1), "unit": "scores/s", "cores": 1,
+                               "kind": "port",
+                               "sample": f"{len(rows)} query rows of the same inputs through the oracle's spread and "
+                                         "block scorer, one host thread; GPU results bit-equal"}
+        res["cpu_baseline"]["nproc"] = host_threads()[2]
     return res
 
 

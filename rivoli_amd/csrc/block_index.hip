@@ -128,22 +128,101 @@ __global__ __launch_bounds__(kSpreadThreads) void f4_rotated_kernel(float* __res
 constexpr int kScoreThreads = 256;           // four waves, 64 blocks each
 constexpr int kScoreQueriesPerGroup = 16;    // queries a workgroup walks with its rows held
 
-// One (query, block) score from a row held in registers (HD > 0) or re-read (HD == 0).
-template <int HD>
-__global__ __launch_bounds__(kScoreThreads) void index_score_blocks_kernel(
-    const float* __restrict__ q, const float* __restrict__ kv, const float* __restrict__ w,
-    float* __restrict__ score, int s, int n_comp, int heads, int hd_rt, int t_per_group) {
-    const int hd = HD ? HD : hd_rt;
-    const long long c = (long long)blockIdx.x * kScoreThreads + threadIdx.x;
-    const float* const kvr = kv + (size_t)(c < n_comp ? c : n_comp - 1) * hd;
-    float row[HD ? HD : 1];
-    if constexpr (HD > 0) {
+// The scalar operands of one 32-term chunk of a dot. Scalar loads return out of order, so the
+// only wait there is waits for all of them: a chunk is requested one whole chunk of
+// arithmetic (64 vector instructions) before it is used and nothing else is outstanding then.
+struct QChunk {
+    float v[32];
+};
+__device__ __forceinline__ void load_chunk(QChunk& c, const float* __restrict__ p) {
 #pragma unroll
-        for (int i = 0; i < HD; i += 4) {
-            const f32x4 v = *reinterpret_cast<const f32x4*>(kvr + i);
-            row[i] = v.x, row[i + 1] = v.y, row[i + 2] = v.z, row[i + 3] = v.w;
+    for (int i = 0; i < 32; ++i) c.v[i] = p[i];
+}
+// Waits for the chunk here: placed before the next chunk is requested, the wait covers this
+// chunk alone (requested a chunk ago); left to the first use it would also cover the request
+// just made.
+__device__ __forceinline__ void arrived(const QChunk& c) {
+    asm volatile("" ::"s"(c.v[0]), "s"(c.v[16]));
+}
+template <int OFF>
+__device__ __forceinline__ float fold_chunk(float dot, const QChunk& c, const float (&row)[128]) {
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const float prod = c.v[i] * row[OFF + i];
+        dot = dot + prod;
+    }
+    return dot;
+}
+
+// bf16 first, then the relu (blockindex.hip:224-228; the sign of a zero cannot reach the
+// output), the weight, the term's own bf16 store, the f32 head sum.
+__device__ __forceinline__ float add_head(float acc, float dot, float weight) {
+    dot = round_bf16(dot);
+    dot = dot > 0.0f ? dot : 0.0f;
+    const float term = dot * weight;
+    return acc + round_bf16(term);
+}
+
+// hd = 128: the lane's block row in registers, the (query, head) pairs of the workgroup's
+// queries walked as one run of 128-value q rows (they are contiguous), two chunk buffers.
+__global__ __launch_bounds__(kScoreThreads) void index_score_blocks_128_kernel(
+    const float* __restrict__ q, const float* __restrict__ kv, const float* __restrict__ w,
+    float* __restrict__ score, int s, int n_comp, int heads, int t_per_group) {
+    constexpr int HD = 128;
+    const long long c = (long long)blockIdx.x * kScoreThreads + threadIdx.x;
+    const float* const kvr = kv + (size_t)(c < n_comp ? c : n_comp - 1) * HD;
+    float row[HD];
+#pragma unroll
+    for (int i = 0; i < HD; i += 4) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(kvr + i);
+        row[i] = v.x, row[i + 1] = v.y, row[i + 2] = v.z, row[i + 3] = v.w;
+    }
+    const int t0 = blockIdx.y * t_per_group;
+    const int t1 = min(s, t0 + t_per_group);
+    const size_t g1 = (size_t)t1 * heads;  // one past the last (query, head) pair
+    const float* qp = q + (size_t)t0 * heads * HD;
+    QChunk a, b;
+    load_chunk(a, qp);
+    float acc = 0.0f;
+    int hh = 0, t = t0;
+    for (size_t g = (size_t)t0 * heads; g < g1; ++g) {
+        float dot = 0.0f;
+        arrived(a);
+        const float weight = w[g];
+        load_chunk(b, qp + 32);
+        __builtin_amdgcn_sched_barrier(0);
+        dot = fold_chunk<0>(dot, a, row);
+        __builtin_amdgcn_sched_barrier(0);
+        arrived(b);
+        load_chunk(a, qp + 64);
+        __builtin_amdgcn_sched_barrier(0);
+        dot = fold_chunk<32>(dot, b, row);
+        __builtin_amdgcn_sched_barrier(0);
+        arrived(a);
+        load_chunk(b, qp + 96);
+        __builtin_amdgcn_sched_barrier(0);
+        dot = fold_chunk<64>(dot, a, row);
+        __builtin_amdgcn_sched_barrier(0);
+        arrived(b);
+        load_chunk(a, g + 1 < g1 ? qp + HD : qp);  // the next pair's first chunk; the last re-reads its own
+        __builtin_amdgcn_sched_barrier(0);
+        dot = fold_chunk<96>(dot, b, row);
+        __builtin_amdgcn_sched_barrier(0);
+        acc = add_head(acc, dot, weight);
+        qp += HD;
+        if (++hh == heads) {
+            if (c < n_comp) score[(size_t)t * n_comp + c] = round_bf16(acc);
+            acc = 0.0f, hh = 0, ++t;
         }
     }
+}
+
+// Any other width: the block's row is re-read through the vector cache for every head.
+__global__ __launch_bounds__(kScoreThreads) void index_score_blocks_any_kernel(
+    const float* __restrict__ q, const float* __restrict__ kv, const float* __restrict__ w,
+    float* __restrict__ score, int s, int n_comp, int heads, int hd, int t_per_group) {
+    const long long c = (long long)blockIdx.x * kScoreThreads + threadIdx.x;
+    const float* const kvr = kv + (size_t)(c < n_comp ? c : n_comp - 1) * hd;
     const int t0 = blockIdx.y * t_per_group;
     const int t1 = min(s, t0 + t_per_group);
     for (int t = t0; t < t1; ++t) {
@@ -151,24 +230,11 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_blocks_kernel(
         for (int hh = 0; hh < heads; ++hh) {
             const float* const qh = q + ((size_t)t * heads + hh) * hd;  // wave-uniform
             float dot = 0.0f;
-            if constexpr (HD > 0) {
-#pragma unroll
-                for (int i = 0; i < HD; ++i) {
-                    const float prod = qh[i] * row[i];
-                    dot = dot + prod;
-                }
-            } else {
-                for (int i = 0; i < hd; ++i) {
-                    const float prod = qh[i] * kvr[i];
-                    dot = dot + prod;
-                }
+            for (int i = 0; i < hd; ++i) {
+                const float prod = qh[i] * kvr[i];
+                dot = dot + prod;
             }
-            // bf16 first, then the relu (blockindex.hip:224-228); the sign of a zero cannot
-            // reach the output
-            dot = round_bf16(dot);
-            dot = dot > 0.0f ? dot : 0.0f;
-            const float term = dot * w[(size_t)t * heads + hh];
-            acc = acc + round_bf16(term);
+            acc = add_head(acc, dot, w[(size_t)t * heads + hh]);
         }
         if (c < n_comp) score[(size_t)t * n_comp + c] = round_bf16(acc);
     }
@@ -217,10 +283,10 @@ extern "C" int rivoli_index_score_blocks(const float* q, const float* kv, const 
     const dim3 grid(c_groups, t_groups), block(rk::kScoreThreads);
     hipStream_t st = (hipStream_t)stream;
     if (hd == 128 && rk::aligned16(kv))
-        hipLaunchKernelGGL(rk::index_score_blocks_kernel<128>, grid, block, 0, st, q, kv, w, score, s,
-                           n_comp, heads, hd, t_per_group);
+        hipLaunchKernelGGL(rk::index_score_blocks_128_kernel, grid, block, 0, st, q, kv, w, score, s,
+                           n_comp, heads, t_per_group);
     else
-        hipLaunchKernelGGL(rk::index_score_blocks_kernel<0>, grid, block, 0, st, q, kv, w, score, s,
+        hipLaunchKernelGGL(rk::index_score_blocks_any_kernel, grid, block, 0, st, q, kv, w, score, s,
                            n_comp, heads, hd, t_per_group);
     return rk::launch_status();
 }
