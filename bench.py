@@ -83,6 +83,9 @@ def parse():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (a known-size kernel to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
+    ap.add_argument("--full-scores", action="store_true",
+                    help="v4_index: score every query against every block (the reference's rectangle) instead "
+                         "of the entries a prefill's selection can rank")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     return ap.parse_args()
@@ -555,25 +558,34 @@ def bench_v4_index(a, torch, hip):
 
     def step(events):
         bracket(torch, stream, events, "spread", lambda: hip.launch_act_quant_f4_rotated(q, s * heads, hd, sh))
-        bracket(torch, stream, events, "score",
-                lambda: hip.launch_index_score_blocks(q, kv, w, score, s, n_comp, heads, hd, sh))
+        if a.full_scores:   # the reference's rectangle: every query against every block
+            bracket(torch, stream, events, "score",
+                    lambda: hip.launch_index_score_blocks(q, kv, w, score, s, n_comp, heads, hd, sh))
+        else:               # what a prefill's selection can rank: block < (t + 1) / ratio
+            bracket(torch, stream, events, "score",
+                    lambda: hip.launch_index_score_blocks_prefill(q, kv, w, score, s, n_comp, heads, hd, ratio, sh))
 
     ms, per = timed(torch, stream, a.steps, a.warmup, step)
     spread_bytes = s * heads * hd * 8                                   # f32 in, f32 out
-    score_flops = 2 * s * n_comp * heads * hd                           # one multiply and one add per term
+    limit = np.minimum((np.arange(s) + 1) // ratio, n_comp)
+    scored = s * n_comp if a.full_scores else int((-(-limit // 64) * 64).clip(max=-(-n_comp // 64) * 64).sum())
+    score_flops = 2 * scored * heads * hd                               # one multiply and one add per term
     score_bytes = s * heads * hd * 4 + n_comp * hd * 4 + s * n_comp * 4
     # the timed steps spread the same buffer again and again; the check runs one step on a fresh copy
     q.copy_(q_raw)
     torch.cuda.synchronize()
     step(None)
     stream.synchronize()
-    res = {"metric": "v4_block_index_scores_per_s", "value": round(s * n_comp / (ms * 1e-3), 1), "unit": "scores/s",
+    legal = s * n_comp if a.full_scores else int(limit.sum())
+    res = {"metric": "v4_block_index_scores_per_s", "value": round(legal / (ms * 1e-3), 1), "unit": "scores/s",
            "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
            "config": {"workload": "second cache format, prefill: Hadamard + fp4 spread of the index queries, block "
                                   "scores of every query against every compressed block (sequential f32 folds, "
                                   "bit-identical to the reference's kernel)",
-                      "tokens": s, "heads": heads, "head_dim": hd, "ratio": ratio, "n_comp": n_comp},
+                      "tokens": s, "heads": heads, "head_dim": hd, "ratio": ratio, "n_comp": n_comp,
+                      "entries": "all" if a.full_scores else "legal (block < (t + 1) / ratio), in groups of 64 blocks",
+                      "scores_per_step": legal, "scores_computed": scored},
            "tokens_per_s": round(s / (ms * 1e-3), 1),
            "kernels": {"f4_rotated_kernel": {"avg_launch_ms": round(per["spread"], 5), "bytes_per_launch": spread_bytes,
                                              "GBps": round(spread_bytes / (per["spread"] * 1e-3) / 1e9, 1)},
@@ -602,6 +614,9 @@ def bench_v4_index(a, torch, hip):
         spent = time.perf_counter() - t0
         got_q = q.view(s, heads, hd)[rows].cpu().numpy().reshape(-1, hd)
         got_s = score[rows].cpu().numpy()
+        if not a.full_scores:   # only the legal entries are defined
+            keep = np.arange(n_comp)[None, :] < limit[rows][:, None]
+            got_s, want_s = np.where(keep, got_s, 0.0).astype(np.float32), np.where(keep, want_s, 0.0).astype(np.float32)
         if code_q != 0 or not np.array_equal(got_q.view(np.uint32), want_q.view(np.uint32)):
             raise SystemExit("bench: GPU spread differs from the CPU oracle")
         if code_s != 0 or not np.array_equal(got_s.view(np.uint32), want_s.view(np.uint32)):

@@ -286,6 +286,26 @@ launchers! {
         stream: *mut c_void,
     );
 
+    /// `launch_index_score_blocks` (crates/backend/src/hip.rs:497-520) for a prefill: only the
+    /// entries a row's selection can rank (block < (t + 1) / ratio, in groups of 64 blocks) are
+    /// computed, bit-identical to the full kernel's; the rest of `score` is left untouched.
+    ///
+    /// # Safety
+    /// As `launch_index_score_blocks`: `q` is `s * heads * hd`, `kv` `n_comp * hd`, `w`
+    /// `s * heads`, `score` `s * n_comp` f32; all live until `stream` drains.
+    launch_index_score_blocks_prefill -> rivoli_index_score_blocks_prefill, "index_score_blocks_prefill" (
+        q: *const f32,
+        kv: *const f32,
+        w: *const f32,
+        score: *mut f32,
+        s: usize as i32,
+        n_comp: usize as i32,
+        heads: usize as i32,
+        hd: usize as i32,
+        ratio: usize as i32,
+        stream: *mut c_void,
+    );
+
     /// `Sel::gather` on the device: the `[window | positional blocks]` rectangle written where the
     /// attend reads it, instead of a host fill plus `upload_selection`. The shape check stays
     /// on the host: `rivoli_sel_shape` is `Sel::shape` (1005 = multi-row decode, 1006 = past the

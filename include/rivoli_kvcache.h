@@ -316,6 +316,18 @@ int rivoli_act_quant_f4_rotated(float* x, int rows, int d, void* stream);
 int rivoli_index_score_blocks(const float* q, const float* kv, const float* w, float* score,
                               int s, int n_comp, int heads, int hd, void* stream);
 
+/* rivoli_index_score_blocks for a prefill (query row t is prompt position t), where the
+ * selection ranks block c for row t only when c < (t + 1) / ratio (select.rs:153-188: a block
+ * is legal once it has closed): every legal entry of score is written, bit-identical to
+ * rivoli_index_score_blocks; an entry whose 64-block group holds no legal block is left
+ * untouched, which is about half of the matrix and half of the time. The other entries of a
+ * group with a legal block are written too. rivoli_index_select_blocks(prefill = 1) and
+ * rivoli_sel_gather_scored read legal entries only. No counterpart in the reference, whose
+ * kernel scores the whole rectangle. Guards as rivoli_index_score_blocks; ratio <= 0: 1001. */
+int rivoli_index_score_blocks_prefill(const float* q, const float* kv, const float* w,
+                                      float* score, int s, int n_comp, int heads, int hd, int ratio,
+                                      void* stream);
+
 /* The scored block selection that crates/engine/src/v4/select.rs:153-188 (scored_rows) performs
  * on the host after a device-to-host copy of the scores, as one launch on the device. scores is
  * [rows][n_comp] f32 (what launch_index_score_blocks wrote; illegal slots need not be masked).

@@ -61,6 +61,7 @@ _SIGNATURES = {
     "rivoli_act_quant_f8_prefix": [_VP, _VP] + [_I] * 4 + [_VP],
     "rivoli_act_quant_f4_rotated": [_VP, _I, _I, _VP],
     "rivoli_index_score_blocks": [_VP] * 4 + [_I] * 4 + [_VP],
+    "rivoli_index_score_blocks_prefill": [_VP] * 4 + [_I] * 5 + [_VP],
     "rivoli_index_select_blocks": [_VP] + [_I] * 6 + [_VP, _VP],
     "rivoli_sel_shape": [_I] * 5 + [_VP, _VP],
     "rivoli_sel_gather": [_I] * 5 + [_VP, _VP],
@@ -325,6 +326,13 @@ def launch_index_score_blocks(q, kv, w, score, s, n_comp, heads, hd, stream=NULL
     """crates/backend/src/hip.rs:497-520 launch_index_score_blocks: block scores [s][n_comp]."""
     ensure_hip_status(lib().rivoli_index_score_blocks(_p(q), _p(kv), _p(w), _p(score), s, n_comp, heads, hd,
                                                       _s(stream)), "index_score_blocks")
+
+
+def launch_index_score_blocks_prefill(q, kv, w, score, s, n_comp, heads, hd, ratio, stream=NULL_STREAM) -> None:
+    """launch_index_score_blocks for a prefill: only entries a row's selection can rank
+    (block < (t + 1) / ratio, in groups of 64 blocks) are computed."""
+    ensure_hip_status(lib().rivoli_index_score_blocks_prefill(_p(q), _p(kv), _p(w), _p(score), s, n_comp, heads,
+                                                              hd, ratio, _s(stream)), "index_score_blocks_prefill")
 
 
 def launch_index_select_blocks(scores, rows, n_comp, ratio, index_topk, prefill, offset, out,

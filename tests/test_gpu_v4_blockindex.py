@@ -180,3 +180,33 @@ def test_prefill_sized_scores_on_sampled_rows_and_the_selection_they_feed(oracle
     for t in (0, 100, 255):
         want_sel = oracle.v4_scored_rows(got[t:t + 1], 4, k, False, 0)
         np.testing.assert_array_equal(got_sel[t], want_sel[0])
+
+
+@pytest.mark.parametrize("s,n_comp,heads,hd,ratio", [(700, 175, 4, 128, 4), (300, 300, 2, 128, 1), (520, 130, 3, 64, 4),
+                                                     (64, 16, 8, 128, 4), (1030, 100, 2, 128, 4)])
+def test_prefill_form_writes_every_legal_entry_and_skips_whole_groups(oracle, s, n_comp, heads, hd, ratio):
+    """score[t][c] for c < (t + 1) / ratio equals the full kernel's bit for bit; a 64-block group
+    with no legal block for row t keeps the buffer's fill; the selection built on it is the one
+    built on the full matrix."""
+    q, kv, w = score_case(s, n_comp, heads, hd, s + ratio)
+    full = device_score(q, kv, w)
+    qd, kd, wd = dev(q), dev(kv), dev(w)
+    out = dzeros(s * n_comp * 4, 0x5A)
+    hip.launch_index_score_blocks_prefill(qd, kd, wd, out, s, n_comp, heads, hd, ratio)
+    got = back(out, np.float32).reshape(s, n_comp)
+    fill = np.frombuffer(b"\x5a" * 4, np.uint32)[0]
+    limit = np.minimum((np.arange(s) + 1) // ratio, n_comp)
+    cols = np.arange(n_comp)
+    legal = cols[None, :] < limit[:, None]
+    group_live = (cols[None, :] // 64) * 64 < limit[:, None]
+    assert np.array_equal(got.view(np.uint32)[legal], full.view(np.uint32)[legal])
+    assert np.array_equal(got.view(np.uint32)[group_live], full.view(np.uint32)[group_live])
+    assert (got.view(np.uint32)[~group_live] == fill).all()
+    assert (~group_live).any() and legal.any()
+    k = min(32, n_comp)
+    sel_a, sel_b = dzeros(s * k * 4), dzeros(s * k * 4)
+    hip.launch_index_select_blocks(out, s, n_comp, ratio, k, True, 0, sel_a)
+    hip.launch_index_select_blocks(dev(full), s, n_comp, ratio, k, True, 0, sel_b)
+    assert np.array_equal(back(sel_a, np.int32), back(sel_b, np.int32))
+    assert hip.lib().rivoli_index_score_blocks_prefill(qd.data_ptr(), kd.data_ptr(), wd.data_ptr(), out.data_ptr(),
+                                                       s, n_comp, heads, hd, 0, None) == 1001
