@@ -71,3 +71,20 @@ def test_block_selection_keeps_its_masks_out_of_memory():
         assert int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b).group(1)) == 0, name
         assert int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", b).group(1)) == 8, name
     assert seen == 6, f"expected the six widths of the register form, saw {seen}"
+
+
+@pytest.mark.skipif(shutil.which(build.hipcc()) is None, reason="hipcc not found")
+def test_block_scorer_keeps_its_row_and_both_chunk_buffers_in_registers():
+    """The block scorer holds a 128-value row per lane and two 32-value chunks of the query in
+    scalar registers; a spill of either turns its two instructions per term into many."""
+    seen = 0
+    for b in _resource_blocks("block_index.hip"):
+        name = b.split()[0]
+        if "index_score_blocks_128_kernel" not in name:
+            continue
+        seen += 1
+        assert int(re.search(r"SGPRs Spill: (\d+)", b).group(1)) == 0, name
+        assert int(re.search(r"VGPRs Spill: (\d+)", b).group(1)) == 0, name
+        assert int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b).group(1)) == 0, name
+        assert int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", b).group(1)) >= 3, name
+    assert seen == 1
