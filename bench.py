@@ -601,10 +601,34 @@ def bench_v4_index(a, torch, hip):
                         "unfused_unpacked_peak": 39.3,
                         "frac_of_unfused_unpacked_peak": round(score_flops / (per["score"] * 1e-3) / 39.3e12, 4),
                         "avg_launch_ms": round(per["score"], 5), "traffic": None}}
+    # a decode step of the same layer: one query against the ctx / ratio blocks of a long context
+    d_comp = max(a.ctx // ratio, 1)
+    d_kv = torch.randn(d_comp, hd, generator=g, device="cuda", dtype=torch.float32).bfloat16().float()
+    hip.launch_act_quant_f4_rotated(d_kv, d_comp, hd)
+    d_q = q_raw[:heads].clone()
+    d_score = torch.empty(d_comp, dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+
+    def decode_step(events):
+        bracket(torch, stream, events, "spread", lambda: hip.launch_act_quant_f4_rotated(d_q, heads, hd, sh))
+        bracket(torch, stream, events, "score",
+                lambda: hip.launch_index_score_blocks(d_q, d_kv, w, d_score, 1, d_comp, heads, hd, sh))
+
+    d_ms, d_per = timed(torch, stream, max(a.steps, 20), a.warmup, decode_step)
+    res["decode_one_query_us"] = {"blocks": d_comp, "step": round(d_ms * 1e3, 2),
+                                  "spread": round(d_per["spread"] * 1e3, 2), "score": round(d_per["score"] * 1e3, 2)}
     if not a.no_cpu_baseline:
         from oracle.kvoracle import oracle as get_oracle
 
         ora = get_oracle()
+        d_q.copy_(q_raw[:heads])
+        torch.cuda.synchronize()
+        decode_step(None)
+        stream.synchronize()
+        code_d, want_d = ora.index_score_blocks(ora.act_quant_f4_rotated(q_raw[:heads].cpu().numpy())[1][None],
+                                                d_kv.cpu().numpy(), w[:1].cpu().numpy())
+        if code_d != 0 or not np.array_equal(d_score.cpu().numpy().view(np.uint32), want_d.view(np.uint32).ravel()):
+            raise SystemExit("bench: GPU decode block scores differ from the CPU oracle")
         rows = sorted({0, 1, s // 2, s - 1} | set(range(min(s, 12))))
         q_h = q_raw.view(s, heads, hd)[rows].cpu().numpy()
         kv_h, w_h = kv.cpu().numpy(), w[rows].cpu().numpy()

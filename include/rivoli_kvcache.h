@@ -310,7 +310,8 @@ int rivoli_act_quant_f4_rotated(float* x, int rows, int d, void* stream);
  * dot is a sequential f32 fold of separately rounded products and the head sum a sequential
  * f32 fold rounded once, exactly as the reference's kernel, so the result is bit-identical
  * to it. hd = 128 (the shipped width) with a 16-byte-aligned kv takes the register-resident
- * kernel; any other width a slower one. Guards as the reference's: 1001 non-positive s, heads
+ * kernels (one for prefill-sized calls, one that splits the heads of a decode step's single
+ * query over a workgroup's waves); any other width a slower one. Guards as the reference's: 1001 non-positive s, heads
  * or hd (also null pointers); 1005 n_comp <= 0 (no block has completed: the caller must not
  * rank an unwritten buffer). */
 int rivoli_index_score_blocks(const float* q, const float* kv, const float* w, float* score,

@@ -156,11 +156,11 @@ __device__ __forceinline__ float fold_chunk(float dot, const QChunk& c, const fl
 
 // bf16 first, then the relu (blockindex.hip:224-228; the sign of a zero cannot reach the
 // output), the weight, the term's own bf16 store, the f32 head sum.
-__device__ __forceinline__ float add_head(float acc, float dot, float weight) {
+__device__ __forceinline__ float head_term(float dot, float weight) {
     dot = round_bf16(dot);
     dot = dot > 0.0f ? dot : 0.0f;
     const float term = dot * weight;
-    return acc + round_bf16(term);
+    return round_bf16(term);
 }
 
 // Which (query group, block group) a workgroup owns. The full rectangle runs block groups
@@ -177,38 +177,33 @@ __device__ __forceinline__ int block_group(int ratio) { return ratio > 0 ? block
 // selection ranks block c for query t only when c < (t + 1) / ratio (a block is legal once it
 // has closed): a wave's 64 blocks start at cw, and no query before ratio * (cw + 1) - 1 can
 // rank any of them.
-__device__ __forceinline__ int first_query(int t0, int t1, int ratio) {
+__device__ __forceinline__ int first_query(int t0, int t1, int ratio, long long cw) {
     if (ratio <= 0) return t0;
-    const long long cw = (long long)block_group(ratio) * kScoreThreads +
-                         (__builtin_amdgcn_readfirstlane((int)threadIdx.x) & ~(kWave - 1));
     const long long first = (cw + 1) * ratio - 1;
     return first > t0 ? (int)(first < t1 ? first : t1) : t0;
 }
 
-// hd = 128: the lane's block row in registers, the (query, head) pairs of the workgroup's
-// queries walked as one run of 128-value q rows (they are contiguous), two chunk buffers.
-__global__ __launch_bounds__(kScoreThreads) void index_score_blocks_128_kernel(
-    const float* __restrict__ q, const float* __restrict__ kv, const float* __restrict__ w,
-    float* __restrict__ score, int s, int n_comp, int heads, int t_per_group, int ratio) {
-    constexpr int HD = 128;
-    const long long c = (long long)block_group(ratio) * kScoreThreads + threadIdx.x;
-    const int t1 = min(s, query_group(ratio) * t_per_group + t_per_group);
-    const int t0 = first_query(query_group(ratio) * t_per_group, t1, ratio);
-    if (t0 >= t1) return;  // wave-uniform; the kernel has no barrier
-    const float* const kvr = kv + (size_t)(c < n_comp ? c : n_comp - 1) * HD;
-    float row[HD];
+// The lane's block row, 128 values, into registers.
+__device__ __forceinline__ void load_row(float (&row)[128], const float* __restrict__ kvr) {
 #pragma unroll
-    for (int i = 0; i < HD; i += 4) {
+    for (int i = 0; i < 128; i += 4) {
         const f32x4 v = *reinterpret_cast<const f32x4*>(kvr + i);
         row[i] = v.x, row[i + 1] = v.y, row[i + 2] = v.z, row[i + 3] = v.w;
     }
-    const size_t g1 = (size_t)t1 * heads;  // one past the last (query, head) pair
-    const float* qp = q + (size_t)t0 * heads * HD;
+}
+
+// One head term, bf16(relu(bf16(q . row)) * weight), for each (query, head) pair g in [g0, g1):
+// the pairs' 128-value q rows are contiguous and are walked as one run through two chunk
+// buffers. on_term(g, term) receives them in order.
+template <class OnTerm>
+__device__ __forceinline__ void walk_pairs(const float* __restrict__ q, const float* __restrict__ w,
+                                           const float (&row)[128], size_t g0, size_t g1,
+                                           OnTerm&& on_term) {
+    constexpr int HD = 128;
+    const float* qp = q + g0 * HD;
     QChunk a, b;
     load_chunk(a, qp);
-    float acc = 0.0f;
-    int hh = 0, t = t0;
-    for (size_t g = (size_t)t0 * heads; g < g1; ++g) {
+    for (size_t g = g0; g < g1; ++g) {
         float dot = 0.0f;
         arrived(a);
         const float weight = w[g];
@@ -231,12 +226,66 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_blocks_128_kernel(
         __builtin_amdgcn_sched_barrier(0);
         dot = fold_chunk<96>(dot, b, row);
         __builtin_amdgcn_sched_barrier(0);
-        acc = add_head(acc, dot, weight);
+        on_term(g, head_term(dot, weight));
         qp += HD;
+    }
+}
+
+// hd = 128, many (query, block group) pairs: a lane owns a block for the workgroup's queries
+// and folds the head terms itself, in head order.
+__global__ __launch_bounds__(kScoreThreads) void index_score_blocks_128_kernel(
+    const float* __restrict__ q, const float* __restrict__ kv, const float* __restrict__ w,
+    float* __restrict__ score, int s, int n_comp, int heads, int t_per_group, int ratio) {
+    const long long c = (long long)block_group(ratio) * kScoreThreads + threadIdx.x;
+    const int t1 = min(s, query_group(ratio) * t_per_group + t_per_group);
+    const long long cw = (long long)block_group(ratio) * kScoreThreads +
+                         (__builtin_amdgcn_readfirstlane((int)threadIdx.x) & ~(kWave - 1));
+    const int t0 = first_query(query_group(ratio) * t_per_group, t1, ratio, cw);
+    if (t0 >= t1) return;  // wave-uniform; the kernel has no barrier
+    float row[128];
+    load_row(row, kv + (size_t)(c < n_comp ? c : n_comp - 1) * 128);
+    float acc = 0.0f;
+    int hh = 0, t = t0;
+    walk_pairs(q, w, row, (size_t)t0 * heads, (size_t)t1 * heads, [&](size_t, float term) {
+        acc = acc + term;
         if (++hh == heads) {
             if (c < n_comp) score[(size_t)t * n_comp + c] = round_bf16(acc);
             acc = 0.0f, hh = 0, ++t;
         }
+    });
+}
+
+// hd = 128, few (query, block group) pairs (a decode step: one query): the plain kernel would
+// occupy n_comp / 256 compute units for 64 heads' worth of arithmetic each. Here a workgroup
+// owns 64 blocks and its eight waves each take an eighth of the heads: the dots of different
+// heads are independent, only their sum has an order. The head terms meet in LDS and the first
+// wave folds them in head order, as the reference does.
+constexpr int kSplitWavesPerGroup = 8;
+constexpr int kSplitMaxHeads = 256;  // 64 KiB of terms
+__global__ __launch_bounds__(kSplitWavesPerGroup* kWave) void index_score_blocks_128_split_kernel(
+    const float* __restrict__ q, const float* __restrict__ kv, const float* __restrict__ w,
+    float* __restrict__ score, int s, int n_comp, int heads, int ratio) {
+    extern __shared__ float terms[];  // [heads][64]
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const long long cw = (long long)blockIdx.x * kWave;
+    const long long c = cw + lane;
+    const int t0 = first_query(0, s, ratio, cw);  // the same for every wave: the barriers below are safe
+    const int per = (heads + kSplitWavesPerGroup - 1) / kSplitWavesPerGroup;
+    const int h0 = min(wave * per, heads), h1 = min(h0 + per, heads);
+    float row[128];
+    load_row(row, kv + (size_t)(c < n_comp ? c : n_comp - 1) * 128);
+    for (int t = t0; t < s; ++t) {
+        const size_t base = (size_t)t * heads;
+        walk_pairs(q, w, row, base + h0, base + h1,
+                   [&](size_t g, float term) { terms[(g - base) * kWave + lane] = term; });
+        __syncthreads();
+        if (wave == 0) {
+            float acc = 0.0f;
+            for (int hh = 0; hh < heads; ++hh) acc = acc + terms[hh * kWave + lane];
+            if (c < n_comp) score[(size_t)t * n_comp + c] = round_bf16(acc);
+        }
+        __syncthreads();
     }
 }
 
@@ -247,7 +296,9 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_blocks_any_kernel(
     const long long c = (long long)block_group(ratio) * kScoreThreads + threadIdx.x;
     const float* const kvr = kv + (size_t)(c < n_comp ? c : n_comp - 1) * hd;
     const int t1 = min(s, query_group(ratio) * t_per_group + t_per_group);
-    const int t0 = first_query(query_group(ratio) * t_per_group, t1, ratio);
+    const long long cw = (long long)block_group(ratio) * kScoreThreads +
+                         (__builtin_amdgcn_readfirstlane((int)threadIdx.x) & ~(kWave - 1));
+    const int t0 = first_query(query_group(ratio) * t_per_group, t1, ratio, cw);
     for (int t = t0; t < t1; ++t) {
         float acc = 0.0f;
         for (int hh = 0; hh < heads; ++hh) {
@@ -257,7 +308,7 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_blocks_any_kernel(
                 const float prod = qh[i] * kvr[i];
                 dot = dot + prod;
             }
-            acc = add_head(acc, dot, w[(size_t)t * heads + hh]);
+            acc = acc + head_term(dot, w[(size_t)t * heads + hh]);
         }
         if (c < n_comp) score[(size_t)t * n_comp + c] = round_bf16(acc);
     }
@@ -307,6 +358,12 @@ static int score_blocks_launch(const float* q, const float* kv, const float* w, 
     if (ratio > 0 && c_groups > 65535u) return 1002;  // more than 2^24 blocks
     const dim3 grid = ratio > 0 ? dim3(t_groups, c_groups) : dim3(c_groups, t_groups);
     const dim3 block(kScoreThreads);
+    if (hd == 128 && aligned16(kv) && (long long)s * c_groups < 256 && heads <= kSplitMaxHeads) {
+        const unsigned groups = (unsigned)(((long long)n_comp + kWave - 1) / kWave);
+        hipLaunchKernelGGL(index_score_blocks_128_split_kernel, dim3(groups), dim3(kSplitWavesPerGroup * kWave),
+                           (size_t)heads * kWave * sizeof(float), st, q, kv, w, score, s, n_comp, heads, ratio);
+        return launch_status();
+    }
     if (hd == 128 && aligned16(kv))
         hipLaunchKernelGGL(index_score_blocks_128_kernel, grid, block, 0, st, q, kv, w, score, s, n_comp,
                            heads, t_per_group, ratio);

@@ -80,11 +80,12 @@ def test_block_scorer_keeps_its_row_and_both_chunk_buffers_in_registers():
     seen = 0
     for b in _resource_blocks("block_index.hip"):
         name = b.split()[0]
-        if "index_score_blocks_128_kernel" not in name:
+        if "index_score_blocks_128" not in name:
             continue
         seen += 1
-        assert int(re.search(r"SGPRs Spill: (\d+)", b).group(1)) == 0, name
+        if "split" not in name:   # the decode kernel is bound by latency, not by issue
+            assert int(re.search(r"SGPRs Spill: (\d+)", b).group(1)) == 0, name
         assert int(re.search(r"VGPRs Spill: (\d+)", b).group(1)) == 0, name
         assert int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b).group(1)) == 0, name
         assert int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", b).group(1)) >= 3, name
-    assert seen == 1
+    assert seen == 2
