@@ -261,7 +261,7 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_blocks_128_kernel(
 // heads are independent, only their sum has an order. The head terms meet in LDS and the first
 // wave folds them in head order, as the reference does.
 constexpr int kSplitWavesPerGroup = 8;
-constexpr int kSplitMaxHeads = 256;  // 64 KiB of terms
+constexpr int kSplitMaxHeads = 128;  // 32 KiB of terms
 __global__ __launch_bounds__(kSplitWavesPerGroup* kWave) void index_score_blocks_128_split_kernel(
     const float* __restrict__ q, const float* __restrict__ kv, const float* __restrict__ w,
     float* __restrict__ score, int s, int n_comp, int heads, int ratio) {

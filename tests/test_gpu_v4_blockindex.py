@@ -109,6 +109,7 @@ def score_case(s, n_comp, heads, hd, seed, spread=None):
 @pytest.mark.parametrize("s,n_comp,heads,hd,spread", [
     (1, 1, 64, 128, False), (2, 300, 64, 128, False), (33, 70, 8, 128, True), (5, 513, 64, 128, True),
     (3, 5, 4, 32, False), (2, 130, 3, 64, True), (1, 257, 2, 256, False), (40, 64, 64, 128, False),
+    (1, 200, 128, 128, False), (1, 70, 130, 128, False), (2, 65, 5, 128, True), (300, 520, 3, 128, False),
 ])
 def test_score_matches_the_oracle(oracle, s, n_comp, heads, hd, spread):
     q, kv, w = score_case(s, n_comp, heads, hd, s * 31 + n_comp, oracle if spread else None)
