@@ -32,6 +32,8 @@ def spread_rows(rows, d, seed):
         x[3] = np.float32(1e-38)
         x[4, ::32] *= np.float32(300.0)
         x[5] = np.float32(3.0)         # a constant row: one spike after the rotation
+        x[6] = rng.standard_normal(d).astype(np.float32) * np.float32(1e-40)   # denormals: below the amax floor
+        x[7] = rng.standard_normal(d).astype(np.float32) * np.float32(1e30)    # sums stay finite
     return bf16_round(x)
 
 
@@ -60,9 +62,10 @@ def test_spread_over_sixty_binades_and_the_reference_kernel(oracle):
     ref = ref_kernels()
     if ref is not None and hasattr(ref, "rivoli_act_quant_f4_rotated"):
         assert same_bits(device_spread(x, launch=ref.rivoli_act_quant_f4_rotated), want).size == 0
-        wide = spread_rows(333, 256, 5)
-        assert same_bits(device_spread(wide, launch=ref.rivoli_act_quant_f4_rotated),
-                         device_spread(wide)).size == 0
+        for rows, d in ((333, 256), (77, 128), (19, 64), (11, 32)):
+            wide = spread_rows(rows, d, 5)
+            assert same_bits(device_spread(wide, launch=ref.rivoli_act_quant_f4_rotated),
+                             device_spread(wide)).size == 0, (rows, d)
 
 
 def test_spread_guards():
