@@ -145,7 +145,32 @@ def second_format_cases(oracle) -> dict:
     g["compress_prefill_ratio4"] = {"kv_fnv": fnv(oracle, kv), "score_fnv": fnv(oracle, score),
                                     "out_u32": hexs(out.view(np.uint32))}
     g.update(consumer_cases(oracle))
+    g.update(block_index_cases(oracle))
     return g
+
+
+def block_index_inputs(oracle):
+    """Seeded inputs of the block indexer's cases: 3 queries x 4 index heads and 20 block rows
+    of 128 bf16 values, rows scaled over several binades; signed bf16 head weights."""
+    lcg = oracle.lcg(0x5EED0009)
+
+    def bf16_values(x):
+        return (oracle.f32_to_bf16(x).astype(np.uint32) << 16).view(np.float32)
+
+    q = bf16_values(lcg.fill(12 * 128).reshape(12, 128) * (np.float32(2.0) ** np.arange(-6, 6))[:, None].astype(np.float32))
+    kv = bf16_values(lcg.fill(20 * 128).reshape(20, 128) * np.float32(3.0))
+    w = bf16_values(lcg.fill(3 * 4).reshape(3, 4) * np.float32(0.1))
+    return q, kv, w
+
+
+def block_index_cases(oracle) -> dict:
+    q, kv, w = block_index_inputs(oracle)
+    (cq, sq), (ck, skv) = oracle.act_quant_f4_rotated(q), oracle.act_quant_f4_rotated(kv)
+    cs, score = oracle.index_score_blocks(sq.reshape(3, 4, 128), skv, w)
+    assert cq == ck == cs == 0
+    return {"block_index": {"q_fnv": fnv(oracle, q), "kv_fnv": fnv(oracle, kv), "w_fnv": fnv(oracle, w),
+                            "spread_q_fnv": fnv(oracle, sq), "spread_q_row0_head_u32": hexs(sq[0, :8].view(np.uint32)),
+                            "spread_kv_fnv": fnv(oracle, skv), "scores_u32": hexs(score.view(np.uint32))}}
 
 
 def consumer_inputs(oracle):
@@ -195,7 +220,8 @@ def main() -> None:
                          os.path.join(ROOT, "tests", "test_oracle_topk_hash.py"),
                          os.path.join(ROOT, "tests", "test_oracle_v4.py"),
                          os.path.join(ROOT, "tests", "test_oracle_v4_compress.py"),
-                         os.path.join(ROOT, "tests", "test_oracle_v4_select.py")], cwd=ROOT).returncode
+                         os.path.join(ROOT, "tests", "test_oracle_v4_select.py"),
+                         os.path.join(ROOT, "tests", "test_oracle_v4_blockindex.py")], cwd=ROOT).returncode
     if rc != 0:
         sys.exit("the oracle does not pass its known-answer tests: no vectors written")
     from oracle.kvoracle import oracle as get_oracle

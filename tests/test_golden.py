@@ -8,7 +8,8 @@ import numpy as np
 import pytest
 
 from tests.golden import inputs
-from tests.golden.make_golden import OUT, PT, W, build_cases, consumer_inputs, fnv, hexs, second_format_inputs
+from tests.golden.make_golden import (OUT, PT, W, block_index_inputs, build_cases, consumer_inputs, fnv, hexs,
+                                      second_format_inputs)
 from tests.test_oracle_quant import fixture_a99e
 from tests.topk_cases import reference_topk_cases
 
@@ -212,3 +213,23 @@ def test_device_reproduces_consumer_golden(oracle, golden):
     want = np.frombuffer(bytes.fromhex(g["row23_head0_u32"]), np.uint32).view(np.float32)
     # the reference's bar for this kernel: 1/128 of the largest expected element
     assert np.max(np.abs(got[23, 0] - want)) <= np.max(np.abs(want)) / 128.0
+
+
+@pytest.mark.gpu
+def test_device_reproduces_block_index_golden(oracle, golden):
+    """The Hadamard + fp4 spread and the block scores from the HIP library only."""
+    from rivoli_amd import hip
+    from tests.gpu_util import back, dev, dzeros
+
+    g = golden["block_index"]
+    q, kv, w = block_index_inputs(oracle)
+    assert (fnv(oracle, q), fnv(oracle, kv), fnv(oracle, w)) == (g["q_fnv"], g["kv_fnv"], g["w_fnv"])
+    q_d, kv_d = dev(q), dev(kv)
+    hip.launch_act_quant_f4_rotated(q_d, 12, 128)
+    hip.launch_act_quant_f4_rotated(kv_d, 20, 128)
+    sq = back(q_d, np.uint32).reshape(12, 128)
+    assert fnv(oracle, sq) == g["spread_q_fnv"] and hexs(sq[0, :8]) == g["spread_q_row0_head_u32"]
+    assert fnv(oracle, back(kv_d, np.uint32)) == g["spread_kv_fnv"]
+    out = dzeros(3 * 20 * 4, 0x5A)
+    hip.launch_index_score_blocks(q_d, kv_d, dev(w), out, 3, 20, 4, 128)
+    assert hexs(back(out, np.uint32)) == g["scores_u32"]
