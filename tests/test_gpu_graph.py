@@ -89,8 +89,9 @@ def test_decode_step_replays_from_a_graph(oracle):
 
 def test_second_format_decode_step_replays_from_a_graph(oracle):
     """The second cache format's decode step — quantize the new entry, write it into the ring,
-    deposit into the compressor (and pool the block this position closes), build the
-    [ring | scored blocks] rectangle, attend with the list shared among workgroups — captured
+    deposit into the compressor (and pool the block this position closes), spread the index
+    queries and score the blocks, build the [ring | scored blocks] rectangle from those scores,
+    attend with the list shared among workgroups — captured
     once at a position that closes a block and replayed on fresh inputs."""
     from oracle.kvoracle import CompGeom as OracleGeom
     from tests.v4_cases import bf16_round, compress_inputs
@@ -111,6 +112,13 @@ def test_second_format_decode_step_replays_from_a_graph(oracle):
     csc = torch.zeros(og.cd * 4, dtype=torch.uint8, device="cuda")
     q = torch.zeros(heads * d * 4, dtype=torch.uint8, device="cuda")
     scores = torch.zeros(n_comp * 4, dtype=torch.uint8, device="cuda")
+    # the block indexer that makes the scores: 64 index heads of 128, the blocks' spread rows
+    iheads, ihd = 64, 128
+    iq = torch.zeros(iheads * ihd * 4, dtype=torch.uint8, device="cuda")
+    iw = torch.zeros(iheads * 4, dtype=torch.uint8, device="cuda")
+    ikv_h = bf16_round(rng.standard_normal((n_comp, ihd)).astype(np.float32))
+    ikv = dev(ikv_h)
+    hip.launch_act_quant_f4_rotated(ikv, n_comp, ihd)
     cols = win + cap
     idx = torch.zeros(cols * 4, dtype=torch.uint8, device="cuda")
     o = torch.zeros(heads * d * 4, dtype=torch.uint8, device="cuda")
@@ -125,6 +133,8 @@ def test_second_format_decode_step_replays_from_a_graph(oracle):
         hip.launch_kv_compress_deposit(ckv, csc, ape_d, state_kv, state_sc, hg, 1, pos % ratio, stream)
         hip.launch_kv_compress_decode(state_kv, state_sc, fin, hg, pos, stream)
         hip.launch_act_quant_f8_prefix(block_row, block_row, 1, d, d - rd, 64, stream)
+        hip.launch_act_quant_f4_rotated(iq, iheads, ihd, stream)
+        hip.launch_index_score_blocks(iq, ikv, iw, scores, 1, n_comp, iheads, ihd, stream)
         hip.launch_sel_gather_scored(scores, n_comp, win, ratio, cap, 1, pos, idx, stream)
         hip.launch_gather_attn_shared_kv(q, cache, sink, idx, 1, heads, d, cols, d ** -0.5, o, stream, partial=part)
 
@@ -134,7 +144,8 @@ def test_second_format_decode_step_replays_from_a_graph(oracle):
                        (ckv, r.standard_normal(og.cd).astype(np.float32)),
                        (csc, r.standard_normal(og.cd).astype(np.float32)),
                        (q, bf16_round(r.standard_normal((heads, d)).astype(np.float32))),
-                       (scores, r.standard_normal(n_comp).astype(np.float32))):
+                       (iq, bf16_round(r.standard_normal((iheads, ihd)).astype(np.float32))),
+                       (iw, bf16_round((r.standard_normal(iheads) * 0.1).astype(np.float32)))):
             buf.copy_(dev(a))
 
     state = (cache, state_kv, state_sc)
@@ -159,7 +170,7 @@ def test_second_format_decode_step_replays_from_a_graph(oracle):
         for t in range(3):
             before = [b.clone() for b in state]
             load_inputs(t)
-            entry_in = entry.clone()
+            entry_in, iq_in = entry.clone(), iq.clone()
             for b in (idx, o):
                 b.fill_(0xEE)
             step(stream.cuda_stream)                               # eager, for the expectation
@@ -167,6 +178,7 @@ def test_second_format_decode_step_replays_from_a_graph(oracle):
             for b, s in zip(state, before):                        # undo the step, then replay it
                 b.copy_(s)
             entry.copy_(entry_in)
+            iq.copy_(iq_in)
             for b in (idx, o):
                 b.fill_(0xEE)
             graph.replay()
@@ -174,9 +186,15 @@ def test_second_format_decode_step_replays_from_a_graph(oracle):
             for name, g, w in zip(("cache", "compressor kv state", "compressor score state", "rectangle", "attention"),
                                   got, want):
                 assert torch.equal(g, w), (t, name)
-    # and the eager result is the oracle's: the last rectangle against the CPU rule
-    r = np.random.default_rng(902)                                  # load_inputs(2): its scores are the fifth draw
+    # and the eager result is the oracle's: the last rectangle against the CPU chain (spread the
+    # index queries, score the blocks, select)
+    r = np.random.default_rng(902)                                  # load_inputs(2): iq and iw are its last two draws
     for n in (d, og.cd, og.cd, heads * d):
         r.standard_normal(n)
-    code, want_rect = oracle.sel_gather_scored(r.standard_normal(n_comp).astype(np.float32)[None, :], win, ratio, cap, 1, pos)
+    iq_h = bf16_round(r.standard_normal((iheads, ihd)).astype(np.float32))
+    iw_h = bf16_round((r.standard_normal(iheads) * 0.1).astype(np.float32))
+    code_s, want_scores = oracle.index_score_blocks(oracle.act_quant_f4_rotated(iq_h)[1][None],
+                                                    oracle.act_quant_f4_rotated(ikv_h)[1], iw_h[None, :])
+    assert code_s == 0 and np.array_equal(scores.cpu().numpy().view(np.uint32), want_scores.view(np.uint32).ravel())
+    code, want_rect = oracle.sel_gather_scored(want_scores, win, ratio, cap, 1, pos)
     assert code == 0 and np.array_equal(got[3].cpu().numpy().view(np.int32).reshape(1, cols), want_rect)
