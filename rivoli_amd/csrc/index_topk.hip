@@ -958,6 +958,11 @@ __global__ __launch_bounds__(kSplitThreads) void topk_finish_kernel(
         const uint32_t before = wave_slots_before(s_wave[turn], wave, &all);
         turn ^= 1;
         uint32_t G = s_G[sg] + (before & 0xffffu), E = s_E[sg] + (before >> 16);
+        // the wave's 256 keys take the output positions [first, last): nothing to place when
+        // they miss this workgroup's (about half of a segment's waves; wave-uniform, and past
+        // the barrier)
+        const uint32_t first = G + min(E, need), last = G + cg + min(E + ce, need);
+        if (last <= lo || first >= hi) return;
         const uint32_t idx0 = (uint32_t)(sg * kSegKeys + wave * (4 * kWave) + lane);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
