@@ -48,16 +48,18 @@ __device__ __forceinline__ float round_bf16(float x) {
     return __uint_as_float((uint32_t)f32_to_bf16(x) << 16);
 }
 
-// formats.hpp:285-293 followed by its decode: the magnitude is the last of the eight whose
-// midpoint was passed; a tie passes an odd-indexed midpoint only. The sign is q's sign bit.
+// formats.hpp:285-293 followed by its decode, for |q| <= 6: the nearest of {0, .5, 1, 1.5, 2, 3,
+// 4, 6}, a tie to the even mantissa. The grid is spaced .5 below 2, 1 below 4 and 2 above, and
+// on each stretch "tie to the even mantissa" is "tie to the even multiple of the spacing"
+// (.25 -> 0, .75 -> 1, 1.25 -> 1, 1.75 -> 2, 2.5 -> 2, 3.5 -> 4, 5 -> 4: the reference's own
+// table), which is what adding and subtracting 2^22, 2^23 or 2^24 does in round-to-nearest-even
+// f32 arithmetic: two compares and two additions where counting midpoints takes fourteen
+// instructions. A NaN passes no midpoint there and becomes a zero with its sign; here too.
 __device__ __forceinline__ float e2m1_round_trip(float q) {
-    const float mid[7] = {0.25f, 0.75f, 1.25f, 1.75f, 2.5f, 3.5f, 5.0f};
-    const float mag[7] = {0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
     const float a = fabsf(q);
-    float v = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 7; ++i)
-        if (a > mid[i] || (a == mid[i] && (i & 1))) v = mag[i];
+    const float magic = a < 2.0f ? 4194304.0f : (a < 4.0f ? 8388608.0f : 16777216.0f);
+    float v = (a + magic) - magic;
+    v = a != a ? 0.0f : v;
     return __builtin_signbit(q) ? -v : v;
 }
 
@@ -112,10 +114,15 @@ __global__ __launch_bounds__(kSpreadThreads) void f4_rotated_kernel(float* __res
         const uint32_t b = __float_as_uint(amax * kFp4MaxInv);
         const int ex = (int)((b >> 23) & 0xffu) - 127 + ((b & 0x7fffffu) ? 1 : 0);
         const float s = __uint_as_float((uint32_t)(ex + 127) << 23);
+        // x / s for a power of two s is x * (1 / s) exactly whenever 1 / s is a normal number
+        // (one multiply instead of the divide's dozen instructions); the divide stays for the
+        // scales at the ends of the exponent range
+        const bool by_reciprocal = ex >= -126 && ex <= 126;
+        const float rinv = __uint_as_float((uint32_t)(127 - ex) << 23);
         f32x4 out;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            float q = e[i] / s;  // s is a power of two: exact unless the quotient leaves the range
+            float q = by_reciprocal ? e[i] * rinv : e[i] / s;
             q = q < -kFp4Max ? -kFp4Max : (q > kFp4Max ? kFp4Max : q);  // a NaN stays a NaN
             out[i] = round_bf16(e2m1_round_trip(q) * s);
         }
