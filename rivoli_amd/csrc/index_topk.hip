@@ -26,17 +26,25 @@
 //     has the scores in registers anyway (the indexer's score kernel) can do this step itself.
 //     `topk_cand_kernel`: every segment re-derives the pivot bin (the one holding the k-th key)
 //     from that histogram, counts its keys in higher bins and lists its keys IN the pivot bin.
-//     `topk_finish_kernel`: a query's selection is dealt to workgroups by OUTPUT position, 128
-//     slots each. Every one of them pulls the query's listed keys (a few thousand) into LDS and
-//     finishes the radix select on the low 20 bits by itself — redundant work on otherwise idle
-//     compute units instead of a hand-over — which gives the exact pivot and, per segment, how
-//     many keys precede; it then re-reads only the segments its slots fall in, emits those
-//     slots in index order and, when asked to, gathers and dequantizes the selected rows from
-//     the fp8 pages straight away: the selection never waits for a separate gather launch and
-//     the gather is balanced whatever the distribution of the selected tokens. A query whose
-//     pivot bin holds more keys than LDS can list (huge ties) finds its pivot by streaming
-//     shape (1)'s radix passes over the whole query in every workgroup — slower, same answer.
-//     The histogram is left zeroed for the next call.
+//     The finishing launch deals a query's selection to workgroups by OUTPUT position, 128
+//     slots each, and — when asked to — gathers and dequantizes those rows from the fp8 pages
+//     straight away: the selection never waits for a separate gather launch and the gather is
+//     balanced whatever the distribution of the selected tokens. Two forms.
+//     Queries of up to 64 segments (262144 scores), `topk_finish_bits_kernel`: the candidate
+//     launch has also marked every key above the pivot bin in a bitmap of the query (a wave's
+//     ballots are its words) and packed each listed key with its position, so the finishing
+//     workgroup never reads a score: it finds the exact pivot among the listed keys (two
+//     10-bit histogram passes in LDS, looked up by every wave for itself), adds the listed keys
+//     that make it to its LDS copy of the bitmap, and a popcount prefix over the bitmap gives
+//     every selected index its output position.
+//     Longer queries, `topk_finish_kernel`: every workgroup pulls the query's listed keys into
+//     LDS, finishes the radix select on the low 20 bits by itself, derives per segment how many
+//     keys precede, and re-reads only the segments its slots fall in to emit them in index
+//     order. A query whose pivot bin holds more keys than LDS can list (huge ties) finds its
+//     pivot by streaming shape (1)'s radix passes over the whole query — slower, same answer.
+//     Either way every workgroup repeats the small pivot search on otherwise idle compute
+//     units instead of waiting for a hand-over, and the histogram is left zeroed for the next
+//     call.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
 #include <mutex>
 #include <type_traits>
@@ -637,6 +645,11 @@ __global__ __launch_bounds__(kSplitThreads) void topk_hist_kernel(
 
 // Launch 2: the pivot bin from the histogram; this segment's keys above it counted, its keys
 // in it listed (in any order: only their values matter to the pivot).
+// BITS (queries of up to kBitsMaxSegs segments): the keys above the pivot bin are also marked,
+// one bit per score, in the query's bitmap — a wave's ballots ARE those words — and a listed key
+// is packed with where it sits: its low 20 bits (the top 12 are the pivot bin's) over its 12-bit
+// position in the segment. The finishing launch then never goes back to the scores.
+template <bool BITS>
 __global__ __launch_bounds__(kSplitThreads) void topk_cand_kernel(
     const float* __restrict__ scores, int stride, const int* __restrict__ nts, int nt_all, int k,
     uint32_t* __restrict__ ws, size_t ws_stride, int n_segs) {
@@ -649,11 +662,13 @@ __global__ __launch_bounds__(kSplitThreads) void topk_cand_kernel(
     const int nt = nts ? min(nts[q], nt_all) : nt_all;
     if (nt <= 0) return;
     uint32_t* w = ws + (size_t)q * ws_stride;
+    uint32_t* bits = w + topk_ws_bits_offset(n_segs) + (size_t)seg * (kSegKeys / 32);
     if (seg * kSegKeys >= nt) {  // a segment past this query's end holds nothing
         if (tid == 0) {
             w[kWsCounts + seg] = 0u;
             w[kWsCounts + n_segs + seg] = 0u;
         }
+        if (BITS && tid < kSegKeys / 32) bits[tid] = 0u;
         return;
     }
     const uint32_t kq = (uint32_t)min(k, nt);
@@ -687,20 +702,36 @@ __global__ __launch_bounds__(kSplitThreads) void topk_cand_kernel(
 
     uint32_t* list = w + topk_ws_cand_offset(n_segs) + (size_t)seg * kSegKeys;
     uint32_t higher = 0;
+    uint32_t word = 0;  // BITS: lane L < 8 keeps word L of the wave's eight bitmap words
+    unsigned long long in_pivot[4];
+    uint32_t listed = 0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const uint32_t bin = key[j] >> kLowBits;
         const bool live = j * kWave < limit;
-        higher += (uint32_t)__popcll(__ballot(live && bin > p12));
-        const bool is = live && bin == p12;
-        const unsigned long long m = __ballot(is);
-        if (m) {
-            uint32_t base = 0;
-            if (lane == 0) base = atomicAdd(&s_cnt[0], (uint32_t)__popcll(m));
-            base = __builtin_amdgcn_readfirstlane(base);
-            if (is) list[base + lanes_below(m)] = key[j];
+        const unsigned long long above_mask = __ballot(live && bin > p12);
+        higher += (uint32_t)__popcll(above_mask);
+        if (BITS) {
+            if (lane == 2 * j) word = (uint32_t)above_mask;
+            if (lane == 2 * j + 1) word = (uint32_t)(above_mask >> 32);
+        }
+        in_pivot[j] = __ballot(live && bin == p12);
+        listed += (uint32_t)__popcll(in_pivot[j]);
+    }
+    if (listed) {  // one place in the list for the wave's keys: a single LDS round trip
+        uint32_t base = 0;
+        if (lane == 0) base = atomicAdd(&s_cnt[0], listed);
+        base = __builtin_amdgcn_readfirstlane(base);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t entry =
+                BITS ? ((key[j] << kTopBits) | (uint32_t)(wave * (4 * kWave) + j * kWave + lane))
+                     : key[j];
+            if ((in_pivot[j] >> lane) & 1ull) list[base + lanes_below(in_pivot[j])] = entry;
+            base += (uint32_t)__popcll(in_pivot[j]);
         }
     }
+    if (BITS && lane < 8) bits[wave * 8 + lane] = word;
     if (lane == 0 && higher) atomicAdd(&s_cnt[1], higher);
     lds_barrier();
     if (tid == 0) {
@@ -1008,6 +1039,322 @@ __global__ __launch_bounds__(kSplitThreads) void topk_finish_kernel(
                                         out + ((size_t)q * k + lo) * width);
 }
 
+// Launch 3 for queries of up to kBitsMaxSegs segments: the selection as a bitmap.
+// The candidate launch has marked every score above the pivot bin in the query's bitmap and
+// listed the pivot bin's keys with their positions, so what is left is small and needs no score:
+// (1) one round of requests — the bitmap (a few words per thread), the segments' list lengths,
+//     the head of each list (a wave per segment, two entries per lane, asked for before the
+//     lengths are known), the query's block-table row;
+// (2) the exact pivot among the listed keys' low 20 bits: two 10-bit histogram passes, a bin per
+//     thread (or two, or four), the entries staying in registers (list entries past a
+//     segment's first 128 are read again from the workspace in each pass);
+// (3) the listed keys above the pivot — and those equal to it, all of them or the `need`
+//     lowest indices — set their bits in the LDS copy of the bitmap;
+// (4) a popcount prefix over the bitmap gives every set bit its output position; the threads
+//     whose words hold positions [lo, hi) write those indices out, resolve them through the
+//     block table, and the workgroup streams the rows.
+// Ties at the pivot value with more equal keys than the selection needs (rare) pick the lowest
+// indices by the same machinery: the equal keys alone are marked in a cleared bitmap, the
+// popcount prefix finds the index of the need-th of them, and only those up to it are kept.
+template <int THREADS>
+__device__ __forceinline__ uint32_t waves_before(const uint32_t* v, int wave, uint32_t* all) {
+    constexpr int NW = THREADS / kWave;
+    static_assert(NW <= 16, "one row of 16 lanes holds the wave slots");
+    const int lane = threadIdx.x & (kWave - 1);
+    uint32_t x = (lane & 15) < NW ? v[lane & 15] : 0u;
+    x += dpp_or_zero<0x111, 0xf>(x);
+    x += dpp_or_zero<0x112, 0xf>(x);
+    x += dpp_or_zero<0x114, 0xf>(x);
+    x += dpp_or_zero<0x118, 0xf>(x);
+    *all = (uint32_t)__builtin_amdgcn_readlane((int)x, NW - 1);
+    return wave ? (uint32_t)__builtin_amdgcn_readlane((int)x, wave - 1) : 0u;
+}
+
+// A 1024-bin histogram kept with a 64-bin summary of it (coarse bin = fine bin / 16): the
+// highest fine bin b with (count in bins > b) < need <= (count in bins >= b), found by ONE wave
+// from two LDS reads — a lane per coarse bin, then sixteen lanes over the fine bins inside the
+// one that holds it — so every wave of a workgroup can look it up for itself and nobody waits
+// for a result to be published. Returns b; *need_out = need - (count in bins > b),
+// *count_out = count in b. Bins complete and visible on entry; all 64 lanes must call it.
+__device__ __forceinline__ uint32_t find_bin_two_level(const uint32_t* coarse, const uint32_t* fine,
+                                                       uint32_t need, uint32_t* need_out,
+                                                       uint32_t* count_out) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t cc = coarse[lane];
+    const uint32_t ci = wave_inclusive_sum(cc);
+    const uint32_t above_c = wave_total(ci) - ci;  // in the coarse bins of higher lanes
+    const unsigned long long hit_c = __ballot(above_c < need && need <= above_c + cc);
+    const int cb = hit_c ? __builtin_ctzll(hit_c) : 0;
+    const uint32_t need_f = need - (uint32_t)__builtin_amdgcn_readlane((int)above_c, cb);
+    const uint32_t fc = fine[cb * 16 + (lane & 15)];
+    uint32_t fi = fc;  // inclusive over each row of 16 lanes (all four rows hold the same)
+    fi += dpp_or_zero<0x111, 0xf>(fi);
+    fi += dpp_or_zero<0x112, 0xf>(fi);
+    fi += dpp_or_zero<0x114, 0xf>(fi);
+    fi += dpp_or_zero<0x118, 0xf>(fi);
+    const uint32_t above_f = (uint32_t)__builtin_amdgcn_readlane((int)fi, 15) - fi;
+    const unsigned long long hit_f =
+        __ballot(above_f < need_f && need_f <= above_f + fc) & 0xffffull;
+    const int fb = hit_f ? __builtin_ctzll(hit_f) : 0;
+    *need_out = need_f - (uint32_t)__builtin_amdgcn_readlane((int)above_f, fb);
+    *count_out = (uint32_t)__builtin_amdgcn_readlane((int)fc, fb);
+    return (uint32_t)(cb * 16 + fb);
+}
+
+template <int W, int PT, int THREADS, int SLOTS, int WPT>
+__global__ __launch_bounds__(THREADS) void topk_finish_bits_kernel(
+    const int* __restrict__ nts, int nt_all, int k, uint32_t* __restrict__ rows,
+    uint32_t* __restrict__ ws, size_t ws_stride, int n_segs, const uint8_t* __restrict__ pool,
+    const int* __restrict__ block_table, uint16_t* __restrict__ out, int max_blocks_per_seq,
+    int width_rt, int page_tokens_rt, int n_pages, size_t page_bytes,
+    unsigned int* __restrict__ bad_rows) {
+    constexpr int NW = THREADS / kWave;
+    constexpr int ROUNDS = (kBitsMaxSegs + NW - 1) / NW;  // segments a wave may own
+    constexpr int TPT = 1024 / THREADS;                   // block-table entries a thread caches
+    constexpr int kMini = kWave;  // keys of the pivot's 10-bit bin one wave ranks by itself
+    __shared__ uint32_t s_bm[THREADS * WPT];
+    __shared__ uint32_t s_fine[2][1024];  // [0]: bits 19..10 of the listed keys, [1]: bits 9..0
+    __shared__ uint32_t s_coarse[2][64];  // their 64-bin summaries
+    __shared__ uint32_t s_mini[kMini + 1];  // [kMini]: how many
+    __shared__ uint32_t s_inc[THREADS];
+    __shared__ uint32_t s_wv[16];
+    __shared__ uint32_t s_tie[2];
+    __shared__ int s_skipped;
+    __shared__ int s_table[1024];
+    __shared__ unsigned long long s_base[SLOTS];
+    __shared__ unsigned long long s_scale_at[SLOTS];
+
+    const int q = blockIdx.y, tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nt = nts ? min(nts[q], nt_all) : nt_all;
+    if (nt <= 0) return;
+    const uint32_t kq = (uint32_t)min(k, nt);
+    const uint32_t lo = (uint32_t)blockIdx.x * SLOTS;
+    if (lo >= kq) return;  // (workgroup 0, which also puts the histogram back to zero, never is)
+    const uint32_t hi = min(lo + (uint32_t)SLOTS, kq);
+    uint32_t* w = ws + (size_t)q * ws_stride;
+    const uint32_t* lists = w + topk_ws_cand_offset(n_segs);
+    const int n_words = n_segs * (kSegKeys / 32);
+
+    // ---- (1) requests ----
+    uint32_t need = w[kWsNeed];
+    uint32_t n_listed[ROUNDS];
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+        const int sg = wave + r * NW;
+        n_listed[r] = sg < n_segs ? w[kWsCounts + sg] : 0u;  // one address per wave
+    }
+    uint32_t head[2] = {0u, 0u};
+    if (wave < n_segs) {  // entries past the list's length are junk and never used
+        head[0] = lists[(size_t)wave * kSegKeys + lane];
+        head[1] = lists[(size_t)wave * kSegKeys + lane + kWave];
+    }
+    uint32_t bw[WPT];
+    {
+        const uint32_t* bits = w + topk_ws_bits_offset(n_segs);
+#pragma unroll
+        for (int j = 0; j < WPT; ++j) bw[j] = tid * WPT + j < n_words ? bits[tid * WPT + j] : 0u;
+    }
+    const bool table_cached = pool && max_blocks_per_seq <= 1024;
+    int my_page[TPT];
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) {
+        my_page[i] = -1;
+        if (table_cached && tid + i * THREADS < max_blocks_per_seq)
+            my_page[i] = block_table[(size_t)q * max_blocks_per_seq + tid + i * THREADS];
+    }
+    if (blockIdx.x == 0)  // the histogram has served: left zeroed for the next call
+        for (int i = tid; i < kTopBins / 4; i += THREADS)
+            reinterpret_cast<u32x4*>(w)[i] = u32x4{0u, 0u, 0u, 0u};
+    for (int i = tid; i < 2 * 1024; i += THREADS) (&s_fine[0][0])[i] = 0u;
+    if (tid < 2 * 64) (&s_coarse[0][0])[tid] = 0u;
+    if (tid == 0) {
+        s_skipped = 0;
+        s_mini[kMini] = 0u;
+    }
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) n_listed[r] = __builtin_amdgcn_readfirstlane(n_listed[r]);
+#pragma unroll
+    for (int j = 0; j < WPT; ++j) s_bm[tid * WPT + j] = bw[j];
+#pragma unroll
+    for (int i = 0; i < TPT; ++i)
+        if (table_cached && tid + i * THREADS < max_blocks_per_seq)
+            s_table[tid + i * THREADS] = my_page[i];
+    lds_barrier();
+
+    // every listed entry of the segments this wave owns: f(entry, segment)
+    auto for_each_listed = [&](auto&& f) {
+#pragma unroll
+        for (int r = 0; r < ROUNDS; ++r) {
+            const int sg = wave + r * NW;
+            const uint32_t n = n_listed[r];
+            const uint32_t* src = lists + (size_t)sg * kSegKeys;
+            if (r == 0) {
+                if ((uint32_t)lane < n) f(head[0], sg);
+                if ((uint32_t)(lane + kWave) < n) f(head[1], sg);
+            }
+            for (uint32_t i = (r == 0 ? 2 * kWave : 0) + lane; i < n; i += kWave) f(src[i], sg);
+        }
+    };
+
+    // ---- (2) the exact pivot: bits 19..10 of the listed keys, then bits 9..0 ----
+    for_each_listed([&](uint32_t e, int) {
+        atomicAdd(&s_fine[0][e >> 22], 1u);
+        atomicAdd(&s_coarse[0][e >> 26], 1u);
+    });
+    lds_barrier();
+    uint32_t n_hi;
+    const uint32_t p_hi = find_bin_two_level(s_coarse[0], s_fine[0], need, &need, &n_hi);
+    // the keys of that bin: few enough (about one, on scores without heavy ties) for a wave to
+    // rank among themselves — every wave does, so nothing is published — else a second histogram
+    const bool mini = n_hi <= (uint32_t)kMini;
+    for_each_listed([&](uint32_t e, int) {
+        if ((e >> 22) != p_hi) return;
+        if (mini) {
+            s_mini[atomicAdd(&s_mini[kMini], 1u)] = e >> 12;
+        } else {
+            atomicAdd(&s_fine[1][(e >> 12) & 1023u], 1u);
+            atomicAdd(&s_coarse[1][(e >> 16) & 63u], 1u);
+        }
+    });
+    lds_barrier();
+    uint32_t pivot, n_equal;  // low 20 bits of the k-th largest key; how many keys equal it
+    if (mini) {
+        const uint32_t mine = (uint32_t)lane < n_hi ? s_mini[lane] : 0u;
+        uint32_t gt = 0, eq = 0;
+        for (uint32_t j = 0; j < n_hi; ++j) {
+            const uint32_t other = (uint32_t)__builtin_amdgcn_readlane((int)mine, (int)j);
+            gt += other > mine ? 1u : 0u;
+            eq += other == mine ? 1u : 0u;
+        }
+        const unsigned long long hit =
+            __ballot((uint32_t)lane < n_hi && gt < need && need <= gt + eq);
+        const int at = hit ? __builtin_ctzll(hit) : 0;
+        pivot = (uint32_t)__builtin_amdgcn_readlane((int)mine, at);
+        need -= (uint32_t)__builtin_amdgcn_readlane((int)gt, at);
+        n_equal = (uint32_t)__builtin_amdgcn_readlane((int)eq, at);
+    } else {
+        pivot = (p_hi << 10) | find_bin_two_level(s_coarse[1], s_fine[1], need, &need, &n_equal);
+    }
+    // need: keys equal to the pivot that are selected
+
+    // ---- (3) the listed keys' bits ----
+    uint32_t last_equal = 0xffffffffu;  // equal keys at indices up to this one are selected
+    if (n_equal > need) {               // uniform: ties by index, lowest first
+#pragma unroll
+        for (int j = 0; j < WPT; ++j) s_bm[tid * WPT + j] = 0u;
+        lds_barrier();
+        for_each_listed([&](uint32_t e, int sg) {
+            if ((e >> 12) == pivot) {
+                const uint32_t idx = (uint32_t)sg * kSegKeys + (e & 4095u);
+                atomicOr(&s_bm[idx >> 5], 1u << (idx & 31u));
+            }
+        });
+        lds_barrier();
+        uint32_t ew[WPT], cnt = 0;
+#pragma unroll
+        for (int j = 0; j < WPT; ++j) cnt += (uint32_t)__popc(ew[j] = s_bm[tid * WPT + j]);
+        const uint32_t incl = wave_inclusive_sum(cnt);
+        if (lane == kWave - 1) s_wv[wave] = incl;
+        lds_barrier();
+        uint32_t all;
+        uint32_t before = waves_before<THREADS>(s_wv, wave, &all) + incl - cnt;
+        if (before < need && need <= before + cnt) {  // the need-th equal key is in these words
+#pragma unroll
+            for (int j = 0; j < WPT; ++j) {
+                uint32_t x = ew[j];
+                while (x) {
+                    const int b = __builtin_ctz(x);
+                    x &= x - 1u;
+                    if (++before == need) s_tie[0] = (uint32_t)(tid * WPT + j) * 32u + (uint32_t)b;
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < WPT; ++j) s_bm[tid * WPT + j] = bw[j];
+        lds_barrier();
+        last_equal = s_tie[0];
+    }
+    for_each_listed([&](uint32_t e, int sg) {
+        const uint32_t low = e >> 12, idx = (uint32_t)sg * kSegKeys + (e & 4095u);
+        if (low > pivot || (low == pivot && idx <= last_equal))
+            atomicOr(&s_bm[idx >> 5], 1u << (idx & 31u));
+    });
+    lds_barrier();
+
+    // ---- (4) output positions from a popcount prefix; this workgroup's are [lo, hi) ----
+    // Position p belongs to the thread whose prefix is the last one <= p; one thread per
+    // position looks its own bit up (the wave from the sixteen wave totals, the thread by a
+    // search over that wave's running counts, then a select inside the word), so a word with
+    // every bit set costs what an almost empty one costs.
+    uint32_t cnt = 0;
+#pragma unroll
+    for (int j = 0; j < WPT; ++j) cnt += (uint32_t)__popc(s_bm[tid * WPT + j]);
+    const uint32_t incl = wave_inclusive_sum(cnt);
+    s_inc[tid] = incl;
+    if (lane == kWave - 1) s_wv[wave] = incl;  // (the tie path's readers are a barrier back)
+    lds_barrier();
+    const int width = W ? W : width_rt;
+    const int pt = PT ? PT : page_tokens_rt;
+    if (tid < (int)(hi - lo)) {
+        // (no cross-lane operation in here: the lanes of a partly filled last wave are off)
+        const uint32_t p = lo + (uint32_t)tid;
+        int wv = 0;
+        uint32_t before = 0, upto = 0;  // selected before wave wv, which holds position p
+#pragma unroll
+        for (int i = 0; i < NW - 1; ++i) {
+            upto += s_wv[i];
+            const bool past = upto <= p;
+            wv += past ? 1 : 0;
+            before = past ? upto : before;
+        }
+        const uint32_t* inc = s_inc + wv * kWave;
+        int at = 0;  // threads of that wave wholly before p
+#pragma unroll
+        for (int step = kWave / 2; step > 0; step >>= 1)
+            if (before + inc[at + step - 1] <= p) at += step;
+        if (at) before += inc[at - 1];
+        const int t = wv * kWave + at;
+        uint32_t r = p - before, x = 0;
+        int j = 0;
+#pragma unroll
+        for (int i = 0; i < WPT; ++i) {  // the word that holds it
+            const uint32_t y = s_bm[t * WPT + i];
+            const uint32_t c = (uint32_t)__popc(y);
+            const bool here = i == j && r < c;
+            x = here ? y : x;
+            const bool past = i == j && !here;
+            r -= past ? c : 0u;
+            j += past ? 1 : 0;
+        }
+        uint32_t bit = 0;  // its r-th set bit
+#pragma unroll
+        for (int half = 16; half > 0; half >>= 1) {
+            const uint32_t c = (uint32_t)__popc(x & ((1u << half) - 1u));
+            if (r >= c) {
+                r -= c;
+                bit += (uint32_t)half;
+                x >>= half;
+            }
+        }
+        const uint32_t tok = (uint32_t)(t * WPT + j) * 32u + bit;
+        rows[(size_t)q * k + p] = tok;
+        if (pool &&
+            !resolve_row(tok, table_cached ? s_table : block_table + (size_t)q * max_blocks_per_seq,
+                         max_blocks_per_seq, width, pt, n_pages, page_bytes, bad_rows, &s_base[tid],
+                         &s_scale_at[tid]))
+            s_skipped = 1;
+    }
+    if (!pool) return;
+    lds_barrier();
+    const int n_mine = (int)(hi - lo);
+    constexpr int kUnroll = W ? (SLOTS * (W / 8) + THREADS - 1) / THREADS : 4;
+    const bool plain = !s_skipped && n_mine * (width >> 3) == THREADS * kUnroll;
+    stream_rows<THREADS, kUnroll>(pool, s_base, s_scale_at, n_mine, width, plain,
+                                  out + ((size_t)q * k + lo) * width);
+}
+
 struct GatherArgs {  // the page pool a selection gathers from; pool == nullptr: indices only
     const uint8_t* pool;
     const int* block_table;
@@ -1015,6 +1362,37 @@ struct GatherArgs {  // the page pool a selection gathers from; pool == nullptr:
     int max_blocks_per_seq, width, page_tokens, n_pages;
     unsigned int* bad_rows;
 };
+
+// The bitmap finishing kernel in the shape the query length asks for: WPT bitmap words per
+// thread hold 16 segments (WPT x THREADS = 2048 words) or kBitsMaxSegs of them.
+template <int THREADS, int SLOTS, class... Args>
+static void finish_bits_launch_shape(bool fixed, int n_segs, int kmax, int n_queries,
+                                     hipStream_t stream, Args... args) {
+    const dim3 grid((unsigned)((kmax + SLOTS - 1) / SLOTS), (unsigned)n_queries), block(THREADS);
+    constexpr int kShort = 16 * (kSegKeys / 32) / THREADS, kLong = kBitsMaxSegs * (kSegKeys / 32) / THREADS;
+    if (n_segs <= 16) {
+        if (fixed)
+            hipLaunchKernelGGL((topk_finish_bits_kernel<576, 64, THREADS, SLOTS, kShort>), grid, block,
+                               0, stream, args...);
+        else
+            hipLaunchKernelGGL((topk_finish_bits_kernel<0, 0, THREADS, SLOTS, kShort>), grid, block, 0,
+                               stream, args...);
+    } else {
+        if (fixed)
+            hipLaunchKernelGGL((topk_finish_bits_kernel<576, 64, THREADS, SLOTS, kLong>), grid, block,
+                               0, stream, args...);
+        else
+            hipLaunchKernelGGL((topk_finish_bits_kernel<0, 0, THREADS, SLOTS, kLong>), grid, block, 0,
+                               stream, args...);
+    }
+}
+template <class... Args>
+static void finish_bits_launch(bool fixed, int n_segs, int kmax, int n_queries, hipStream_t stream,
+                               Args... args) {
+    // 128 output positions per 1024-thread workgroup: 256 workgroups for 16 queries x 2048, one
+    // per compute unit (64 per 512 threads and 32 per 256 measure 3 % and 20 % slower there)
+    finish_bits_launch_shape<1024, 128>(fixed, n_segs, kmax, n_queries, stream, args...);
+}
 
 static int index_topk_launch(const float* scores, int n_queries, int stride, const int* nts,
                              int nt, int k, unsigned int* rows, void* workspace, bool hist_ready,
@@ -1033,13 +1411,23 @@ static int index_topk_launch(const float* scores, int n_queries, int stride, con
         if (!hist_ready)
             hipLaunchKernelGGL(topk_hist_kernel, seg_grid, block, 0, stream, scores, stride, nts, nt,
                                ws, ws_stride);
-        hipLaunchKernelGGL(topk_cand_kernel, seg_grid, block, 0, stream, scores, stride, nts, nt, k,
-                           ws, ws_stride, n_segs);
         const int kmax = k < nt ? k : nt;
+        const size_t page_bytes = (size_t)ga.page_tokens * ga.width + (size_t)ga.page_tokens * 4;
+        const bool fixed = ga.pool && ga.width == 576 && ga.page_tokens == 64;
+        if (n_segs <= kBitsMaxSegs) {
+            hipLaunchKernelGGL(topk_cand_kernel<true>, seg_grid, block, 0, stream, scores, stride,
+                               nts, nt, k, ws, ws_stride, n_segs);
+            finish_bits_launch(fixed, n_segs, kmax, n_queries, stream, nts, nt, k, rows, ws,
+                               ws_stride, n_segs, ga.pool, ga.block_table, ga.out,
+                               ga.max_blocks_per_seq, ga.width, ga.page_tokens, ga.n_pages,
+                               page_bytes, ga.bad_rows);
+            return launch_status();
+        }
+        hipLaunchKernelGGL(topk_cand_kernel<false>, seg_grid, block, 0, stream, scores, stride, nts,
+                           nt, k, ws, ws_stride, n_segs);
         const dim3 out_grid((unsigned)((kmax + kSlotsPerGroup - 1) / kSlotsPerGroup),
                             (unsigned)n_queries);
-        const size_t page_bytes = (size_t)ga.page_tokens * ga.width + (size_t)ga.page_tokens * 4;
-        if (ga.pool && ga.width == 576 && ga.page_tokens == 64)
+        if (fixed)
             hipLaunchKernelGGL((topk_finish_kernel<576, 64>), out_grid, block, 0, stream, scores,
                                stride, nts, nt, k, rows, ws, ws_stride, n_segs, ga.pool,
                                ga.block_table, ga.out, ga.max_blocks_per_seq, ga.width,

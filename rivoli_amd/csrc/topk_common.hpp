@@ -48,13 +48,19 @@ constexpr int kSplitMinScores = 16384;   // shorter queries stay on one workgrou
 //   [4100, 4100 + S)     per segment: keys in the pivot bin (the candidates)
 //   [4100 + S, 4100+2S)  per segment: keys in higher bins (selected whatever the low bits say)
 //   (padded to 4 words)  S x 4096 candidate keys, segment s at s * 4096
+//   S x 128              one bit per score: set where the key's bin is above the pivot bin
+//                        (queries of up to kBitsMaxSegs segments, see index_topk.hip)
+constexpr int kBitsMaxSegs = 64;         // longer queries take the list-only finishing kernel
 constexpr int kWsPivot = kTopBins, kWsNeed = kTopBins + 1, kWsCounts = kTopBins + 4;
 __host__ __device__ inline int topk_segments(int nt) { return (nt + kSegKeys - 1) / kSegKeys; }
 __host__ __device__ inline size_t topk_ws_cand_offset(int n_segs) {
     return ((size_t)kWsCounts + 2 * (size_t)n_segs + 3) & ~(size_t)3;
 }
-__host__ __device__ inline size_t topk_ws_words(int n_segs) {
+__host__ __device__ inline size_t topk_ws_bits_offset(int n_segs) {
     return topk_ws_cand_offset(n_segs) + (size_t)n_segs * kSegKeys;
+}
+__host__ __device__ inline size_t topk_ws_words(int n_segs) {
+    return topk_ws_bits_offset(n_segs) + (size_t)n_segs * (kSegKeys / 32);
 }
 // Whether a call of this shape runs split (so whether a producer should fill the histogram).
 inline bool topk_runs_split(int n_queries, int nt) {

@@ -75,7 +75,7 @@ def dsa_scores(n_q, nt, seed):
 
 @pytest.mark.parametrize("split", [False, True])
 @pytest.mark.parametrize("nt", [1, 63, 64, 65, 1023, 1024, 1025, 4096, 4097, 5185, 8192, 16384,
-                                16385, 65535, 65536, 65537, 200_000])
+                                16385, 65535, 65536, 65537, 200_000, 300_000])
 def test_batched_topk_sizes(oracle, nt, split):
     """Every register-resident variant's boundary, the streaming path past 65536, and the
     segment boundaries of the split form."""
