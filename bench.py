@@ -17,6 +17,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -127,7 +128,8 @@ def main():
     short = min(a.cpu_seconds, 2.0)
     others = (("cfg3_ragged", "decode", dict(ragged=True, cpu_seconds=short)),
               ("cfg4_dsa", "dsa", dict(cpu_seconds=short)),
-              ("cfg4_dsa_scored", "dsa_scored", {}),
+              ("cfg4_dsa_scored", "dsa_scored", dict(cpu_seconds=short)),
+              ("cfg4_dsa_attend", "dsa_attend", dict(precise=4)),
               ("cfg2_prefill_8192", "prefill", dict(tokens=8192, cpu_seconds=short)),
               ("cfg2_prefill_1048576", "prefill", dict(tokens=1048576, cpu_seconds=short)),
               # the cache's consumer at configuration 3's shape: inside the reference's own bar on
@@ -165,14 +167,44 @@ def run_workload(workload, a, torch, hip):
 
 
 def brief(res):
-    """What a secondary configuration contributes to the default run's line."""
-    keep = ("metric", "value", "unit", "ms_per_step", "layer_us", "hbm_peak_frac", "tokens_per_s", "rows_per_s",
-            "kernels_ms", "kernels", "roofline", "index_score", "decode_one_query_us", "queries_per_s", "config")
-    out = {k: res[k] for k in keep if k in res}
+    """What a secondary configuration contributes to the default run's line: the figures, not
+    the prose (`--workload X` prints the full record of one configuration). frac = the dominant
+    kernel's algorithmic bytes (or flops) per launch / its bracketed launch time / the peak;
+    frac_step, where present, is the same bytes over the step time per launch (the plain pass,
+    whose launches queue ahead of the device). checked: how the GPU result compared with the
+    CPU oracle ("equal", or the error it stayed within); cpu: the oracle's rate in `unit`."""
+    r = res.get("roofline", {})
+    out = {"value": res["value"], "unit": res["unit"], "ms": res["ms_per_step"]}
+    if "layer_us" in res:
+        out["layer_us"] = res["layer_us"]
+    out["kernel"] = r.get("kernel")
+    if r.get("bound", "hbm") != "hbm":
+        out["bound"] = r["bound"]
+    out["frac"] = r.get("frac")
+    if "frac_step" in r:
+        out["frac_step"] = r["frac_step"]
+    out["launch_ms"] = r.get("avg_launch_ms")
+    out["per_launch"] = r.get("bytes_per_launch", r.get("flops_per_launch"))
+    out["traffic"] = r.get("traffic")
+    if "kernels_ms" in res:
+        out["kernels_ms"] = res["kernels_ms"]
+    elif "kernels" in res:
+        out["kernels_ms"] = {k: v["avg_launch_ms"] for k, v in res["kernels"].items()}
+    if "index_score" in res:
+        out["score_frac"] = res["index_score"]["frac"]
+    if "decode_one_query_us" in res:
+        out["decode_one_query_us"] = res["decode_one_query_us"]
+    cfg = res.get("config", {})
+    out["shape"] = " ".join(f"{k}={v}" for k, v in cfg.items()
+                            if isinstance(v, (int, float)) and not isinstance(v, bool)
+                            and k not in ("width", "page_tokens", "head_dim", "quantized_dims", "block"))
     if "cpu_baseline" in res:
-        out["checked"] = res["cpu_baseline"]["sample"]
-        out["cpu_baseline"] = {k: res["cpu_baseline"][k] for k in ("value", "unit", "cores", "nproc", "kind")
-                               if k in res["cpu_baseline"]}
+        c = res["cpu_baseline"]
+        m = re.search(r"within ([0-9.e+-]+)", c["sample"])
+        out["checked"] = m.group(1) if m else "equal"
+        out["cpu"] = {"value": c["value"], "cores": c["cores"]}
+        if c["unit"] != res["unit"]:
+            out["cpu"]["unit"] = c["unit"]
     return out
 
 
@@ -291,8 +323,9 @@ def bench_decode(a, torch, hip):
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "batched decode (benchmark configuration 3, metric point): append 1 token/"
-                               "seq/layer then gather+dequantize every sequence's full context",
+        "config": {"workload": ("cfg3 batched decode, contexts ~U[1024, ctx]" if a.ragged else
+                                "cfg3 batched decode at its metric point") +
+                               ": per layer append 1 token/seq, then gather+dequantize every context",
                    "layers": L, "batch": B, "ctx": ctx, "page_tokens": PT, "width": W,
                    "stored": "fp8 e4m3 + 1 f32 scale/token", "out": "bf16",
                    "contexts": "uniform in [1024, ctx]" if a.ragged else "all at ctx",
@@ -387,10 +420,13 @@ def bench_prefill(a, torch, hip):
            "config": {"workload": "prefill bulk append (benchmark configuration 2)", "tokens": n,
                       "pages": n_pages, "width": W, "page_tokens": PT},
            "tokens_per_s": round(n / (ms * 1e-3), 1),
-           "roofline": {"bound": "hbm", "kernel": "kv_append_paged_kernel",
+           # (kv_append.hip: batches under 16384 tokens take the wave-per-token kernel)
+           "roofline": {"bound": "hbm",
+                        "kernel": "kv_append_paged_token_kernel<2>" if n < 16384 else "kv_append_paged_kernel<72>",
                         "achieved": round(nbytes / (per["append"] * 1e-3) / 1e9, 2),
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                         "frac": round(nbytes / (per["append"] * 1e-3) / HBM_PEAK, 5),
+                        "frac_step": round(nbytes / (ms * 1e-3) / HBM_PEAK, 5),
                         "avg_launch_ms": round(per["append"], 5), "bytes_per_launch": nbytes,
                         "traffic": measured_traffic(f"prefill:tokens{n}")}}
     if not a.no_cpu_baseline:
@@ -814,10 +850,11 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
 
     fused = not attend and not a.unfused
 
+    score = hip.launch_index_score_paged_hist if fused else hip.launch_index_score_paged
+
     def step(events):
         for layer in range(L):
             if scored:
-                score = hip.launch_index_score_paged_hist if fused else hip.launch_index_score_paged
                 tail = (ws_topk, sh) if fused else (sh,)
                 bracket(torch, stream, events, "score",
                         lambda: score(qs[layer], ws[layer], kpools[layer], tables, None, None, B, blocks, nt,
@@ -870,6 +907,8 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
                         "avg_launch_ms": round(per[rows_kernel], 5),
                         "bytes_per_launch": dom_bytes,
                         "traffic": measured_traffic(f"dsa:b{B}:ctx{nt}:k{k}") if fused and not scored else None}}
+    if fused and not scored:  # the step IS one such call per layer
+        res["roofline"]["frac_step"] = round(dom_bytes / (ms * 1e-3 / L) / HBM_PEAK, 5)
     if not fused:
         res["topk"] = {"achieved": round(topk_bytes / (per["topk"] * 1e-3) / 1e9, 2), "unit": "GB/s",
                        "avg_launch_ms": round(per["topk"], 5), "bytes_per_launch": topk_bytes}
@@ -885,34 +924,77 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
         res["config"]["workload"] = ("DSA sparse path with the consumer fused: top-k, then MLA latent attention "
                                      "over the selected rows straight from the fp8 pages")
         res["config"]["heads"], res["config"]["precise"] = H, a.precise
-    if not a.no_cpu_baseline and not scored and not attend:
+    if not a.no_cpu_baseline:
         from oracle.kvoracle import oracle as get_oracle
 
         ora = get_oracle()
         cores, usable, nproc = host_threads()
-        sc_h, pool_h = scores[0].cpu().numpy(), pools[0].cpu().numpy()
+        pool_h = pools[0].cpu().numpy()
+        note = ""
+        if scored:
+            # layer 0's scores as the device computed them: a sample of them against the oracle's
+            # scorer (the reference's bar for that kernel, 1e-5 of the largest score:
+            # crates/engine/tests/indexer_kernel.rs:351-366), then the selection and the gather
+            # on exactly those scores
+            score(qs[0], ws[0], kpools[0], tables, None, None, B, blocks, nt, nt, NH, NH, HD, PT, n_pages,
+                  HD ** -0.5, 1.0, score_buf, *((ws_topk,) if fused else ()))
+            torch.cuda.synchronize()
+            sc_h = score_buf.cpu().numpy()
+            n_s = 4096
+            want_sc = ora.index_score_paged(qs[0][:1].cpu().numpy(), ws[0][:1].cpu().numpy(),
+                                            kpools[0].view(torch.int16).cpu().numpy().view(np.uint16),
+                                            tables_np[:1], np.array([n_s], np.int32), None, n_s, HD, PT,
+                                            HD ** -0.5, 1.0, n_threads=cores)
+            err = float(np.abs(sc_h[0, :n_s] - want_sc[0]).max() / np.abs(want_sc[0]).max())
+            if not err <= 1e-5:
+                raise SystemExit(f"bench: device scores differ from the CPU oracle ({err:.2e} of the largest)")
+            note = f"; device scores of query 0's first {n_s} tokens: error {err:.1e} of the largest (bar 1e-5)"
+        else:
+            sc_h = scores[0].cpu().numpy()
         reps, spent = 0, 0.0
         while spent < a.cpu_seconds and reps < 50:
             t0 = time.perf_counter()
             want_sel = ora.topk_batched(sc_h, k, n_threads=cores)
-            want_rows = ora.kv_gather_rows_paged(pool_h, tables_np, want_sel, W, PT)
+            want_rows = None if attend else ora.kv_gather_rows_paged(pool_h, tables_np, want_sel, W, PT)
             spent += time.perf_counter() - t0
             reps += 1
+        sc_d = score_buf if scored else scores[0]
         if fused:
-            hip.launch_dsa_select_gather_paged(scores[0], B, nt, None, nt, k, sel, ws_topk, False, pools[0], tables,
+            hip.launch_dsa_select_gather_paged(sc_d, B, nt, None, nt, k, sel, ws_topk, scored, pools[0], tables,
                                                out, blocks, W, PT, n_pages)
         else:
-            hip.launch_index_topk_batched(scores[0], B, nt, None, nt, k, sel, ws_topk)
-            hip.launch_kv_gather_rows_paged(pools[0], tables, sel, None, out, B, k, blocks, W, PT, n_pages)
+            hip.launch_index_topk_batched(sc_d, B, nt, None, nt, k, sel, ws_topk)
+            if not attend:
+                hip.launch_kv_gather_rows_paged(pools[0], tables, sel, None, out, B, k, blocks, W, PT, n_pages)
         torch.cuda.synchronize()
         if not np.array_equal(sel.cpu().numpy().view(np.uint32).reshape(B, k), want_sel):
             raise SystemExit("bench: GPU top-k differs from the CPU oracle")
-        if not np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16).reshape(B, k, W), want_rows):
-            raise SystemExit("bench: GPU sparse gather differs from the CPU oracle")
-        res["cpu_baseline"] = {"value": round(layer_bytes / (spent / reps) / 1e9, 3), "unit": "GB/s",
+        if attend:
+            # the attention over the selected rows: two queries through the oracle (the reference's
+            # bar for that kernel, crates/engine/tests/kernel_attend.rs:267)
+            n_chk = 2
+            hip.launch_mla_attend_paged(qabs[0], qrope[0], pools[0], tables, None, sel, None, B, H, k, blocks, 512,
+                                        64, PT, n_pages, float(W) ** -0.5, a.precise, clat, partial)
+            torch.cuda.synchronize()
+            want_att = ora.mla_attend_paged(qabs[0][:n_chk].cpu().numpy(), qrope[0][:n_chk].cpu().numpy(), pool_h,
+                                            tables_np[:n_chk], np.full(n_chk, nt, np.int32), want_sel[:n_chk], None,
+                                            512, 64, PT, float(W) ** -0.5, n_threads=cores)
+            got_att = clat.cpu().numpy()[:n_chk]
+            err = float(np.abs(got_att - want_att).max() / np.abs(want_att).max())
+            if not err <= 1e-3:
+                raise SystemExit(f"bench: attention over the selected rows differs from the oracle ({err:.2e})")
+            sample = (f"one layer's top-k on {cores} host threads x{reps} reps, GPU indices checked equal; attention "
+                      f"of {n_chk} queries over their {k} rows within {err:.1e} of the oracle's")
+            cpu_bytes = topk_bytes
+        else:
+            if not np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16).reshape(B, k, W), want_rows):
+                raise SystemExit("bench: GPU sparse gather differs from the CPU oracle")
+            sample = (f"one layer (top-k on {cores} host threads, sparse gather single-threaded) x{reps} reps; "
+                      "GPU indices and rows checked equal" + note)
+            cpu_bytes = topk_bytes + rows_bytes
+        res["cpu_baseline"] = {"value": round(cpu_bytes / (spent / reps) / 1e9, 3), "unit": "GB/s",
                                "cores": cores, "nproc": nproc, "usable": usable, "kind": "port",
-                               "sample": f"one layer (top-k on {cores} host threads, sparse gather "
-                                         f"single-threaded) x{reps} reps; GPU indices and rows checked equal"}
+                               "sample": sample}
     return res
 
 

@@ -89,6 +89,28 @@ launchers! {
         stream: *mut c_void,
     );
 
+    /// A decode step's cache work in one launch: append one new row per sequence (`seq_lens`
+    /// already counts it, `slot_mapping[s]` is that token's slot), then gather every context.
+    /// See `include/rivoli_kvcache.h` for the full contract.
+    launch_kv_append_gather_paged -> rivoli_kv_append_gather_paged, "kv_append_gather_paged" (
+        new_rows: *const u16,
+        slot_mapping: *const i32,
+        pool: *mut u8,
+        block_table: *const i32,
+        seq_lens: *const i32,
+        cu_seqlens: *const i32,
+        out: *mut u16,
+        n_seqs: usize as i32,
+        max_blocks_per_seq: usize as i32,
+        total_tokens: usize as i64,
+        width: usize as i32,
+        page_tokens: usize as i32,
+        n_pages: usize as i32,
+        bad_slots: *mut u32,
+        bad_pages: *mut u32,
+        stream: *mut c_void,
+    );
+
     /// Sparse row gather + dequantize: `rows[q*k + j]` of sequence `q`, `j < n_rows[q]`.
     launch_kv_gather_rows_paged -> rivoli_kv_gather_rows_paged, "kv_gather_rows_paged" (
         pool: *const u8,

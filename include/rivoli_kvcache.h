@@ -124,6 +124,29 @@ int rivoli_kv_gather_paged_packed(const unsigned char* pool, const int* block_ta
                                   int width, int page_tokens, int n_pages, unsigned int* bad_pages,
                                   void* stream);
 
+/* A decode step's cache work in ONE launch: rivoli_kv_append_paged of one new row per sequence
+ * (new_rows [n_seqs][width] bf16, slot_mapping [n_seqs]) followed by rivoli_kv_gather_paged_packed
+ * (rivoli_kv_gather_paged when total_tokens < 0) — what the reference runs per layer as
+ * append_kv (crates/backend/kernels/fwd.hip:51-71) and then the tile loads of the attend
+ * (attn.hip:168-177), one launch each per token. seq_lens ALREADY COUNTS the new token, and
+ * slot_mapping[s] must be the slot the block table gives token seq_lens[s] - 1 of sequence s:
+ * that token's output row is written from the row just quantized (dequantized from its new
+ * codes and scale, so bit-identical to gathering the stored record), every other token is
+ * gathered from the pool, and no workgroup reads what another one writes. Under that condition
+ * pool and out end up exactly as after the two separate calls. A negative slot is a sequence
+ * without a new token (all of it is gathered); a slot >= n_pages * page_tokens is counted in
+ * *bad_slots, written nowhere, and the sequence is gathered whole. A slot_mapping that names
+ * another token's slot is outside the contract (the separate calls would gather the new row
+ * there; this call gathers what the pool held).
+ * Guards: those of the two calls (1001 null / non-positive, 1002 width > 1024, 1004 alignment
+ * of pool, out and new_rows or a width that is not a multiple of 16). */
+int rivoli_kv_append_gather_paged(const unsigned short* new_rows, const int* slot_mapping,
+                                  unsigned char* pool, const int* block_table, const int* seq_lens,
+                                  const int* cu_seqlens, unsigned short* out, int n_seqs,
+                                  int max_blocks_per_seq, long long total_tokens, int width,
+                                  int page_tokens, int n_pages, unsigned int* bad_slots,
+                                  unsigned int* bad_pages, void* stream);
+
 /* Sparse row gather + dequantize (the `rows` argument of rivoli_mla_attend,
  * crates/backend/kernels/attn.hip:125,175): for query q < n_queries and j < n_rows[q]
  * (k when n_rows is null): out[(q*k + j)*width ..] = dequantized token rows[q*k + j] of
@@ -220,7 +243,9 @@ int rivoli_index_score_paged(const float* q, const float* w, const unsigned shor
  * indexer.hip:1-13): while a score is still in a register its selection key's top 12 bits are
  * counted into topk_workspace (the rivoli_index_topk_workspace_bytes(n_queries, nt) buffer the
  * selection will be handed, zero-filled as described there), so rivoli_dsa_select_gather_paged
- * (hist_ready = 1) does not sweep the scores for it. For shapes the selection does not split
+ * (hist_ready = 1) does not sweep the scores for it. A token whose key page is outside the pool
+ * is written as -inf here (and counted as such), not left unwritten: the histogram and the
+ * scores the selection reads next must describe the same keys. For shapes the selection does not split
  * (nt <= 16384) the workspace is left alone. Guards as rivoli_index_score_paged, plus 1001 for a
  * null workspace and 1004 for one that is not 16-byte aligned. */
 int rivoli_index_score_paged_hist(const float* q, const float* w, const unsigned short* kpool,
@@ -323,8 +348,11 @@ int rivoli_index_score_blocks(const float* q, const float* kv, const float* w, f
  * rivoli_index_score_blocks; an entry whose 64-block group holds no legal block is left
  * untouched, which is about half of the matrix and half of the time. The other entries of a
  * group with a legal block are written too. rivoli_index_select_blocks(prefill = 1) and
- * rivoli_sel_gather_scored read legal entries only. No counterpart in the reference, whose
- * kernel scores the whole rectangle. Guards as rivoli_index_score_blocks; ratio <= 0: 1001. */
+ * rivoli_sel_gather_scored read legal entries only. ITS OUTPUT FEEDS A PREFILL SELECTION
+ * ONLY: a consumer that ranks whole rows (rivoli_index_select_blocks with prefill = 0, a
+ * host-side scored_rows over all n_comp blocks) would rank entries this call never wrote, and
+ * nothing in the buffer marks them. No counterpart in the reference, whose kernel scores the
+ * whole rectangle. Guards as rivoli_index_score_blocks; ratio <= 0: 1001. */
 int rivoli_index_score_blocks_prefill(const float* q, const float* kv, const float* w,
                                       float* score, int s, int n_comp, int heads, int hd, int ratio,
                                       void* stream);

@@ -7,6 +7,7 @@ architecture here is gfx950 and the product is one shared library behind a C ABI
 from __future__ import annotations
 
 import os
+import re
 import subprocess
 import sys
 
@@ -21,6 +22,33 @@ KERNELS = ["kv_append.hip", "kv_gather.hip", "index_topk.hip", "index_score.hip"
 # kernels of the same file time the same either way.
 EXTRA_FLAGS = {"mla_attend.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 HOST_SOURCES = ["pagepool.cpp"]
+# Kernels whose design rests on "no scratch memory": source file -> (substring of the mangled
+# name, suffix of it). The 8-bit attention kernels run one wave per SIMD on the whole register
+# file and order their own LDS transfers (hand-placed waits, an m0 swap around each transfer): a
+# build of them that spills is a different program, so the build refuses to produce one (a
+# compile without EXTRA_FLAGS, an ablation with a piece compiled out).
+NO_SCRATCH = {"mla_attend.hip": ("mla_attend_paged_kernel", "Lb1EEEvNS_10AttendArgsE")}
+
+
+def check_resources(k: str, report: str) -> None:
+    """Raises when a kernel of NO_SCRATCH[k] in hipcc's resource report uses scratch memory or
+    more LDS than a compute unit has."""
+    if k not in NO_SCRATCH:
+        return
+    part, suffix = NO_SCRATCH[k]
+    seen = 0
+    for block in re.split(r"remark: Function Name: ", report)[1:]:
+        name = block.split()[0]
+        if part not in name or not name.endswith(suffix):
+            continue
+        seen += 1
+        scratch = int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", block).group(1))
+        lds = int(re.search(r"LDS Size \[bytes/block\]: (\d+)", block).group(1))
+        if scratch or lds > 160 * 1024:
+            raise RuntimeError(f"{k}: {name} uses {scratch} bytes of scratch per lane and {lds} bytes of LDS; "
+                               "this kernel must compile to 0 and at most 163840")
+    if not seen:
+        raise RuntimeError(f"{k}: no kernel matching {part}...{suffix} in the resource report")
 
 
 def hipcc() -> str:
@@ -44,12 +72,18 @@ def build_kernels(verbose: bool = False) -> str:
 
     def compile_one(k: str) -> str:
         obj = os.path.join(objdir, k.replace(".hip", ".o"))
-        res = subprocess.run(common + EXTRA_FLAGS.get(k, []) + ["-c", os.path.join(CSRC, k), "-o", obj],
+        report = ["-Rpass-analysis=kernel-resource-usage"] if k in NO_SCRATCH else []
+        res = subprocess.run(common + EXTRA_FLAGS.get(k, []) + report + ["-c", os.path.join(CSRC, k), "-o", obj],
                              capture_output=True, text=True)
-        if verbose or res.returncode != 0:
+        if res.returncode != 0 or (verbose and not report):
             sys.stderr.write(res.stdout + res.stderr)
         if res.returncode != 0:
             raise RuntimeError("hipcc failed compiling " + k)
+        try:
+            check_resources(k, res.stderr)
+        except RuntimeError:
+            os.remove(obj)  # never link it
+            raise
         return obj
 
     with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:

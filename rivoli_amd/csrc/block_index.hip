@@ -207,6 +207,7 @@ __device__ __forceinline__ void walk_pairs(const float* __restrict__ q, const fl
                                            const float (&row)[128], size_t g0, size_t g1,
                                            OnTerm&& on_term) {
     constexpr int HD = 128;
+    if (g0 >= g1) return;  // (wave-uniform) no pair: the first chunk below would be pair g1's
     const float* qp = q + g0 * HD;
     QChunk a, b;
     load_chunk(a, qp);

@@ -134,13 +134,14 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
     constexpr int kChunks = 32 * kScoreMaxHd / 8 / kWave;  // 16-byte chunks per lane per block
     uint16_t(*tile)[kScoreMaxHd + kScoreRowPad] = s_k[wave];
     const int cprk = hd >> 3;                               // 16-byte chunks per key row
+    // rows_ok < 0: the block's page is outside the pool, -rows_ok of its tokens are in range
     auto block_base = [&](int tb, int& rows_ok) -> const uint16_t* {
         rows_ok = min(32, nt - tb);
         size_t slot = (size_t)tb;
         if (block_table) {
             const int page = block_table[(size_t)qi * max_blocks_per_seq + tb / page_tokens];
             if ((unsigned)page >= (unsigned)n_pages) {
-                rows_ok = 0;  // nothing of this block is readable or written
+                rows_ok = -rows_ok;  // nothing of this block is readable
                 return kpool;
             }
             slot = (size_t)page * page_tokens + (size_t)(tb % page_tokens);
@@ -207,7 +208,12 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_kernel(
 #pragma unroll
             for (int v = 0; v < 16; ++v) sum += wv[rb][v] * fmaxf(acc[rb][v] * dscale, 0.0f);
         sum += __shfl_xor(sum, 32, kWave);
-        if (lane < 32 && valid) {
+        // With the selection's histogram: a token of an unreadable page gets the score -inf and
+        // is counted like any other, so that the histogram and the scores the selection reads
+        // next agree. Without it such a token is left unwritten, as the plain form documents.
+        const bool lost = topk_ws && col < -rows_ok;
+        if (lost) sum = -INFINITY;
+        if (lane < 32 && (valid || lost)) {
             scores[(size_t)qi * stride + token] = sum;
             if (topk_ws) {
                 const uint32_t bin = topk_key(sum) >> kLowBits;
@@ -266,7 +272,15 @@ __global__ __launch_bounds__(kScoreThreads) void index_score_plain_kernel(
         size_t slot = (size_t)t;
         if (block_table) {
             const int page = block_table[(size_t)qi * max_blocks_per_seq + t / page_tokens];
-            if ((unsigned)page >= (unsigned)n_pages) continue;  // not readable: not written
+            if ((unsigned)page >= (unsigned)n_pages) {
+                // not readable: not written — except with the selection's histogram, where the
+                // token scores -inf and is counted, so that histogram and scores agree
+                if (topk_ws && lane == 0) {
+                    scores[(size_t)qi * stride + t] = -INFINITY;
+                    atomicAdd(&topk_ws[(size_t)qi * ws_stride + (topk_key(-INFINITY) >> kLowBits)], 1u);
+                }
+                continue;
+            }
             slot = (size_t)page * page_tokens + (size_t)(t % page_tokens);
         }
         const uint16_t* krow = kpool + slot * hd;

@@ -12,7 +12,7 @@
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
 #include <type_traits>
 
-#include "codec.hpp"
+#include "append_common.hpp"
 
 namespace rk {
 
@@ -171,54 +171,11 @@ __global__ __launch_bounds__(kAppendWaves* kWave) void kv_append_paged_token_ker
     const uint16_t* __restrict__ rows, const int* __restrict__ slot_mapping,
     uint8_t* __restrict__ pool, int n_tokens, int width, int page_tokens, long long n_slots,
     size_t page_bytes, unsigned int* __restrict__ bad_slots) {
-    const int lane = threadIdx.x & (kWave - 1);
     const int token =
         __builtin_amdgcn_readfirstlane((int)(blockIdx.x * kAppendWaves + (threadIdx.x >> 6)));
     if (token >= n_tokens) return;
-    const int n_chunks = width >> 3;
-    const u32x4* src = reinterpret_cast<const u32x4*>(rows + (size_t)token * width);
-
-    // the row is requested before the slot is looked at: the two fetches overlap instead of
-    // queueing one memory round trip behind the other (a padding token costs a wasted read)
-    u32x4 raw[STEPS];
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-        int c = lane + s * kWave;
-        raw[s] = c < n_chunks ? __builtin_nontemporal_load(src + c) : u32x4{0, 0, 0, 0};
-    }
-    const int slot = slot_mapping[token];
-    if (slot < 0) return;  // padding
-    if ((long long)slot >= n_slots) {
-        if (lane == 0 && bad_slots) atomicAdd(bad_slots, 1u);
-        return;
-    }
-    float amax = 0.0f;
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-        const uint32_t w[4] = {raw[s].x, raw[s].y, raw[s].z, raw[s].w};
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            amax = fmaxf(amax, fmaxf(fabsf(bf16_lo_to_f32(w[i])), fabsf(bf16_hi_to_f32(w[i]))));
-    }
-    amax = wave_max(amax);
-    const float scl = amax > 0.0f ? amax / 448.0f : 1.0f;
-    const float rinv = 1.0f / scl;
-    const uint32_t band = row_band(scl);
-
-    const int page = slot / page_tokens;
-    const int off = slot - page * page_tokens;
-    uint8_t* pg = pool + (size_t)page * page_bytes;
-    u32x2* dst = reinterpret_cast<u32x2*>(pg + (size_t)off * width);
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-        int c = lane + s * kWave;
-        if (c < n_chunks) {
-            const uint32_t w[4] = {raw[s].x, raw[s].y, raw[s].z, raw[s].w};
-            dst[c] = quantize8(w, scl, rinv, band);
-        }
-    }
-    if (lane == 0)
-        *reinterpret_cast<float*>(pg + (size_t)page_tokens * width + (size_t)off * 4) = scl;
+    append_token_wave<STEPS>(rows + (size_t)token * width, slot_mapping + token, pool, width,
+                             page_tokens, n_slots, page_bytes, bad_slots, nullptr);
 }
 
 // Linear slabs, reference layout. One wave per token; a lane owns elements lane*2, lane*2+1

@@ -15,13 +15,51 @@
 // Sparse: one workgroup per 32 selected rows of one query; the 32 row bases and scales are
 // resolved once into LDS (block-table lookup), then the same 8-in/16-out streaming body runs
 // over the 32 x width bytes.
+// A decode step's "append one token per sequence, then gather every context" is one launch of
+// the same kernels (APPEND): n_seqs extra workgroups quantize the new rows, store their records
+// and write those tokens' bf16 rows themselves (dequantized from the codes they just made), and
+// the gather units stop one token short of such a sequence's end — no workgroup reads what
+// another one writes, so nothing has to be ordered inside the launch.
 // Launch-only; see include/rivoli_kvcache.h for the contract of every entry point.
-#include "gather_common.hpp"
+#include "append_common.hpp"
 
 namespace rk {
 
 constexpr int kGatherThreads = 256;
 constexpr int kRowsPerGroup = 32;  // sparse gather: rows resolved per workgroup
+
+// What the APPEND forms carry besides the gather's arguments.
+struct AppendArgs {
+    const uint16_t* new_rows;  // [n_seqs][width] bf16
+    const int* slot_mapping;   // [n_seqs]: where sequence s's new token goes (negative: none)
+    uint8_t* pool;             // the same pool, writable
+    long long n_slots;
+    unsigned int* bad_slots;
+};
+// Whether sequence s's last token is written by its append workgroup (and so skipped by the
+// gather units): its slot is a slot of the pool and the sequence has a token to be the last.
+__device__ __forceinline__ bool appends_last(const AppendArgs& ap, int s, int len) {
+    const int slot = ap.slot_mapping[s];
+    return len > 0 && slot >= 0 && (long long)slot < ap.n_slots;
+}
+// The append workgroup of sequence s: its first wave quantizes the row into the pool and writes
+// the token's output row; the other waves have nothing to do.
+template <int W>
+__device__ __forceinline__ void append_unit(const AppendArgs& ap, const int* __restrict__ seq_lens,
+                                            const int* __restrict__ cu_seqlens,
+                                            uint16_t* __restrict__ out, int s, int width_rt,
+                                            int page_tokens, size_t page_bytes) {
+    if (threadIdx.x >= kWave) return;
+    const int width = W ? W : width_rt;
+    const int len = seq_lens[s];
+    uint16_t* out_row = len > 0 ? out + ((size_t)cu_seqlens[s] + len - 1) * width : nullptr;
+    if (width <= 512)
+        append_token_wave<1>(ap.new_rows + (size_t)s * width, ap.slot_mapping + s, ap.pool, width,
+                             page_tokens, ap.n_slots, page_bytes, ap.bad_slots, out_row);
+    else
+        append_token_wave<2>(ap.new_rows + (size_t)s * width, ap.slot_mapping + s, ap.pool, width,
+                             page_tokens, ap.n_slots, page_bytes, ap.bad_slots, out_row);
+}
 
 // W / PT are the compile-time row width and page size (0 = take the runtime value), so the
 // flagship 576 x 64 shape gets constant divisors and a fully unrolled body. A workgroup owns
@@ -78,17 +116,23 @@ __device__ __forceinline__ void gather_unit(const uint8_t* __restrict__ pool,
 // The grid spans what the block tables could hold: blockIdx.y = sequence, blockIdx.x = its
 // (page, part). Right when every sequence is about as long as the longest; with uneven lengths
 // most workgroups only find out that they have nothing to do.
-template <int W, int PT, int THREADS, int ROWS>
+template <int W, int PT, int THREADS, int ROWS, bool APPEND>
 __global__ __launch_bounds__(THREADS) void kv_gather_paged_kernel(
     const uint8_t* __restrict__ pool, const int* __restrict__ block_table,
     const int* __restrict__ seq_lens, const int* __restrict__ cu_seqlens,
     uint16_t* __restrict__ out, int max_blocks_per_seq, int width_rt, int page_tokens_rt,
-    int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_pages) {
+    int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_pages, AppendArgs ap) {
     const int parts = (PT ? PT : page_tokens_rt) / ROWS;
     const int s = blockIdx.y;
+    if (APPEND && (int)blockIdx.x == max_blocks_per_seq * parts) {  // one more column: the appends
+        append_unit<W>(ap, seq_lens, cu_seqlens, out, s, width_rt, PT ? PT : page_tokens_rt, page_bytes);
+        return;
+    }
     const int blk = (int)blockIdx.x / parts;
     const int part = (int)blockIdx.x - blk * parts;
-    gather_unit<W, PT, THREADS, ROWS>(pool, block_table, cu_seqlens, out, s, blk, part, seq_lens[s],
+    int len = seq_lens[s];
+    if (APPEND && appends_last(ap, s, len)) --len;
+    gather_unit<W, PT, THREADS, ROWS>(pool, block_table, cu_seqlens, out, s, blk, part, len,
                                       max_blocks_per_seq, width_rt, page_tokens_rt, n_pages,
                                       page_bytes, bad_pages);
 }
@@ -101,16 +145,21 @@ __global__ __launch_bounds__(THREADS) void kv_gather_paged_kernel(
 // the compute unit's one scalar pipe (measured: 0.63 against 0.66 of peak at 32 sequences,
 // 0.37 against 0.63 at 128). No LDS, no barrier; at most n_seqs workgroups of the launch (the
 // rounding of each sequence's last unit) find nothing to do.
-template <int W, int PT, int THREADS, int ROWS>
+template <int W, int PT, int THREADS, int ROWS, bool APPEND>
 __global__ __launch_bounds__(THREADS) void kv_gather_flat_kernel(
     const uint8_t* __restrict__ pool, const int* __restrict__ block_table,
     const int* __restrict__ seq_lens, const int* __restrict__ cu_seqlens,
     uint16_t* __restrict__ out, int n_seqs, int max_blocks_per_seq, int width_rt,
-    int page_tokens_rt, int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_pages) {
+    int page_tokens_rt, int n_pages, size_t page_bytes, unsigned int* __restrict__ bad_pages,
+    AppendArgs ap) {
     static_assert(THREADS % kWave == 0, "the scan below runs in every wave and needs all 64 lanes of each");
     const int pt = PT ? PT : page_tokens_rt;
     const int parts = pt / ROWS;
-    const uint32_t u = blockIdx.x;
+    if (APPEND && (int)blockIdx.x < n_seqs) {  // the first n_seqs workgroups: the appends
+        append_unit<W>(ap, seq_lens, cu_seqlens, out, (int)blockIdx.x, width_rt, pt, page_bytes);
+        return;
+    }
+    const uint32_t u = blockIdx.x - (APPEND ? (uint32_t)n_seqs : 0u);
     const int cap = max_blocks_per_seq * pt;  // rows a block-table row can address
     uint32_t first = 0;                       // units of the sequences before s
     int s = -1, my_len = 0;
@@ -118,6 +167,7 @@ __global__ __launch_bounds__(THREADS) void kv_gather_flat_kernel(
         const int lane = threadIdx.x & (kWave - 1);
         for (int s0 = 0; s0 < n_seqs; s0 += kWave) {
             int len = seq_lens[min(s0 + lane, n_seqs - 1)];
+            if (APPEND && s0 + lane < n_seqs && appends_last(ap, s0 + lane, len)) --len;
             len = s0 + lane < n_seqs ? min(max(len, 0), cap) : 0;
             const uint32_t units = (uint32_t)(len + ROWS - 1) / ROWS;
             const uint32_t incl = first + wave_inclusive_sum(units);
@@ -187,17 +237,19 @@ __global__ void e4m3_dequant_bf16_kernel(const uint8_t* __restrict__ codes, floa
 }  // namespace rk
 
 // total_tokens < 0: not known, the grid spans what the block tables could hold.
+// ap.new_rows != nullptr: the APPEND forms.
 static int gather_paged_launch(const unsigned char* pool, const int* block_table,
                                const int* seq_lens, const int* cu_seqlens, unsigned short* out,
                                int n_seqs, int max_blocks_per_seq, long long total_tokens,
                                int width, int page_tokens, int n_pages, unsigned int* bad_pages,
-                               void* stream) {
+                               rk::AppendArgs ap, void* stream) {
     using namespace rk;
     if (!pool || !block_table || !seq_lens || !cu_seqlens || !out) return 1001;
     if (n_seqs <= 0 || max_blocks_per_seq <= 0 || width <= 0 || page_tokens <= 0 || n_pages <= 0)
         return 1001;
     if (n_seqs > 65535) return 1002;
     if (!gather_shape_ok(width, page_tokens) || !aligned16(pool) || !aligned16(out)) return 1004;
+    const bool append = ap.new_rows != nullptr;
     const size_t page_bytes = (size_t)page_tokens * width + (size_t)page_tokens * 4;
     const long long capacity = (long long)n_seqs * max_blocks_per_seq * page_tokens;
     // The flat grid pays for finding each workgroup's sequence and saves the idle workgroups of
@@ -207,23 +259,31 @@ static int gather_paged_launch(const unsigned char* pool, const int* block_table
     // flat when the batch fills less than 0.7 of what its block tables could hold.
     const bool flat = total_tokens >= 0 && total_tokens * 10 < capacity * 7;
     (void)hipGetLastError();
-#define RK_GATHER(WV, PTV, THREADS, FLAT_THREADS, ROWS)                                            \
+#define RK_GATHER_AS(WV, PTV, THREADS, FLAT_THREADS, ROWS, APPEND)                                 \
     do {                                                                                           \
         const unsigned parts = (unsigned)(page_tokens / (ROWS));                                   \
         if (flat) {                                                                                \
-            const long long units = (total_tokens + (ROWS) - 1) / (ROWS) + n_seqs;                 \
+            const long long units = (total_tokens + (ROWS) - 1) / (ROWS) + n_seqs + ((APPEND) ? n_seqs : 0); \
             if (units > 0x7fffffffLL) return 1002;                                                 \
-            hipLaunchKernelGGL((kv_gather_flat_kernel<WV, PTV, FLAT_THREADS, ROWS>),               \
+            hipLaunchKernelGGL((kv_gather_flat_kernel<WV, PTV, FLAT_THREADS, ROWS, APPEND>),       \
                                dim3((unsigned)units), dim3(FLAT_THREADS), 0, (hipStream_t)stream, pool, \
                                block_table, seq_lens, cu_seqlens, out, n_seqs, max_blocks_per_seq, \
-                               width, page_tokens, n_pages, page_bytes, bad_pages);                \
+                               width, page_tokens, n_pages, page_bytes, bad_pages, ap);            \
         } else {                                                                                   \
-            hipLaunchKernelGGL((kv_gather_paged_kernel<WV, PTV, THREADS, ROWS>),                   \
-                               dim3((unsigned)max_blocks_per_seq * parts, (unsigned)n_seqs),       \
+            hipLaunchKernelGGL((kv_gather_paged_kernel<WV, PTV, THREADS, ROWS, APPEND>),           \
+                               dim3((unsigned)max_blocks_per_seq * parts + ((APPEND) ? 1u : 0u),   \
+                                    (unsigned)n_seqs),                                             \
                                dim3(THREADS), 0, (hipStream_t)stream, pool, block_table, seq_lens, \
                                cu_seqlens, out, max_blocks_per_seq, width, page_tokens, n_pages,   \
-                               page_bytes, bad_pages);                                             \
+                               page_bytes, bad_pages, ap);                                         \
         }                                                                                          \
+    } while (0)
+#define RK_GATHER(WV, PTV, THREADS, FLAT_THREADS, ROWS)                                            \
+    do {                                                                                           \
+        if (append)                                                                                \
+            RK_GATHER_AS(WV, PTV, THREADS, FLAT_THREADS, ROWS, true);                              \
+        else                                                                                       \
+            RK_GATHER_AS(WV, PTV, THREADS, FLAT_THREADS, ROWS, false);                             \
     } while (0)
     if (width == 576 && page_tokens == 64)
         RK_GATHER(576, 64, 768, 576, 16);  // flat: 576 threads = two 8-byte chunks each
@@ -232,6 +292,7 @@ static int gather_paged_launch(const unsigned char* pool, const int* block_table
     else
         RK_GATHER(0, 0, kGatherThreads, kGatherThreads, 4);
 #undef RK_GATHER
+#undef RK_GATHER_AS
     return launch_status();
 }
 
@@ -241,7 +302,8 @@ extern "C" int rivoli_kv_gather_paged(const unsigned char* pool, const int* bloc
                                       int width, int page_tokens, int n_pages,
                                       unsigned int* bad_pages, void* stream) {
     return gather_paged_launch(pool, block_table, seq_lens, cu_seqlens, out, n_seqs,
-                               max_blocks_per_seq, -1, width, page_tokens, n_pages, bad_pages, stream);
+                               max_blocks_per_seq, -1, width, page_tokens, n_pages, bad_pages,
+                               rk::AppendArgs{nullptr, nullptr, nullptr, 0, nullptr}, stream);
 }
 
 extern "C" int rivoli_kv_gather_paged_packed(const unsigned char* pool, const int* block_table,
@@ -253,7 +315,25 @@ extern "C" int rivoli_kv_gather_paged_packed(const unsigned char* pool, const in
     if (total_tokens < 0) return 1001;
     return gather_paged_launch(pool, block_table, seq_lens, cu_seqlens, out, n_seqs,
                                max_blocks_per_seq, total_tokens, width, page_tokens, n_pages,
-                               bad_pages, stream);
+                               bad_pages, rk::AppendArgs{nullptr, nullptr, nullptr, 0, nullptr},
+                               stream);
+}
+
+extern "C" int rivoli_kv_append_gather_paged(const unsigned short* new_rows, const int* slot_mapping,
+                                             unsigned char* pool, const int* block_table,
+                                             const int* seq_lens, const int* cu_seqlens,
+                                             unsigned short* out, int n_seqs,
+                                             int max_blocks_per_seq, long long total_tokens,
+                                             int width, int page_tokens, int n_pages,
+                                             unsigned int* bad_slots, unsigned int* bad_pages,
+                                             void* stream) {
+    if (!new_rows || !slot_mapping) return 1001;
+    if (width > 1024) return 1002;  // the append's widest row
+    if (!rk::aligned16(new_rows)) return 1004;
+    const rk::AppendArgs ap = {new_rows, slot_mapping, pool, (long long)n_pages * page_tokens, bad_slots};
+    return gather_paged_launch(pool, block_table, seq_lens, cu_seqlens, out, n_seqs,
+                               max_blocks_per_seq, total_tokens, width, page_tokens, n_pages,
+                               bad_pages, ap, stream);
 }
 
 // Query q gathers its first min(n_rows[q], nr_cap) listed rows (nr_cap when n_rows is null);

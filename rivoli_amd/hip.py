@@ -55,6 +55,7 @@ _SIGNATURES = {
     "rivoli_kv_append_paged": [_VP, _VP, _VP, _I, _I, _I, _I, _VP, _VP],
     "rivoli_kv_gather_paged": [_VP] * 5 + [_I] * 5 + [_VP, _VP],
     "rivoli_kv_gather_paged_packed": [_VP] * 5 + [_I, _I, _LL] + [_I] * 3 + [_VP, _VP],
+    "rivoli_kv_append_gather_paged": [_VP] * 7 + [_I, _I, _LL] + [_I] * 3 + [_VP, _VP, _VP],
     "rivoli_kv_gather_rows_paged": [_VP] * 5 + [_I] * 6 + [_VP, _VP],
     "rivoli_mla_attend": [_VP] * 6 + [_I] * 5 + [_F, _VP, _VP],
     "rivoli_mla_attend_paged": [_VP] * 7 + [_I] * 8 + [_F, _I, _VP, _VP, _VP, _VP],
@@ -232,6 +233,17 @@ def launch_kv_gather_paged_packed(pool, block_table, seq_lens, cu_seqlens, out, 
     ensure_hip_status(lib().rivoli_kv_gather_paged_packed(
         _p(pool), _p(block_table), _p(seq_lens), _p(cu_seqlens), _p(out), n_seqs, max_blocks_per_seq,
         total_tokens, width, page_tokens, n_pages, _p(bad_pages), _s(stream)), "kv_gather_paged_packed")
+
+
+def launch_kv_append_gather_paged(new_rows, slot_mapping, pool, block_table, seq_lens, cu_seqlens, out, n_seqs,
+                                  max_blocks_per_seq, total_tokens, width, page_tokens, n_pages,
+                                  bad_slots=None, bad_pages=None, stream=NULL_STREAM) -> None:
+    """One launch for a decode step's cache work: append one new row per sequence (seq_lens already
+    counts it; slot_mapping[s] is that token's slot), then gather every context."""
+    ensure_hip_status(lib().rivoli_kv_append_gather_paged(
+        _p(new_rows), _p(slot_mapping), _p(pool), _p(block_table), _p(seq_lens), _p(cu_seqlens), _p(out), n_seqs,
+        max_blocks_per_seq, total_tokens, width, page_tokens, n_pages, _p(bad_slots), _p(bad_pages),
+        _s(stream)), "kv_append_gather_paged")
 
 
 def launch_kv_gather_rows_paged(pool, block_table, rows, n_rows, out, n_queries, k,

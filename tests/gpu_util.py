@@ -37,6 +37,19 @@ def back(t, dtype=np.uint8) -> np.ndarray:
 _REF = None
 
 
+def need_ref(*symbols):
+    """The reference's own launchers (ref_kernels), or a SKIP when that build is not there or
+    lacks one of `symbols`: a test whose only claim is "the reference's kernel agrees" must not
+    read as passed on a box that never ran it."""
+    ref = ref_kernels()
+    if ref is None:
+        pytest.skip("oracle/_ref not built: the reference's own kernels were not run")
+    for name in symbols:
+        if not hasattr(ref, name):
+            pytest.skip(f"oracle/_ref lacks {name}: the reference's own kernel was not run")
+    return ref
+
+
 def ref_kernels():
     """The reference's own launchers compiled for gfx950 (oracle/Makefile `ref`), or None.
     They run on the null stream like every launch in these tests."""

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from rivoli_amd import hip
-from tests.gpu_util import back, dev, dzeros, ref_kernels
+from tests.gpu_util import back, dev, dzeros, need_ref
 from tests.test_oracle_quant import fixture_a99e
 from tests.util import f32_to_bf16_rne, make_rows_bf16, shuffled_block_tables, slots_for
 
@@ -26,15 +26,23 @@ def test_append_kv_reference_fixture(oracle):
     assert np.array_equal(back(c8), want[0])
     assert np.array_equal(back(ls, np.uint32), want[1].view(np.uint32))
     assert np.array_equal(back(rc, np.uint16), want[2])
-    ref = ref_kernels()
-    if ref is not None:  # the reference's own kernel, compiled for this GPU, agrees too
-        r8, rs, rr = dzeros(rows * kvl), dzeros(rows * nb * 4), dzeros(rows * ropn * 2)
-        lat_d, rope_d = dev(latent), dev(rope)
-        assert ref.rivoli_append_kv(lat_d.data_ptr(), rope_d.data_ptr(), r8.data_ptr(),
-                                    rs.data_ptr(), rr.data_ptr(), pos, kvl, ropn, nb) == 0
-        assert np.array_equal(back(r8), want[0])
-        assert np.array_equal(back(rs, np.uint32), want[1].view(np.uint32))
-        assert np.array_equal(back(rr, np.uint16), want[2])
+
+
+def test_reference_append_kv_agrees_with_the_oracle(oracle):
+    """The reference's own kernel (fwd.hip compiled for this GPU) on the same fixture."""
+    ref = need_ref("rivoli_append_kv")
+    rows, kvl, ropn, pos, nb = 5, 256, 64, 3, 2
+    latent, rope = fixture_a99e(oracle)
+    want = [np.zeros(rows * kvl, np.uint8), np.zeros(rows * nb, np.float32),
+            np.zeros(rows * ropn, np.uint16)]
+    assert oracle.append_kv(latent, rope, *want, pos, kvl, ropn, nb) == 0
+    r8, rs, rr = dzeros(rows * kvl), dzeros(rows * nb * 4), dzeros(rows * ropn * 2)
+    lat_d, rope_d = dev(latent), dev(rope)
+    assert ref.rivoli_append_kv(lat_d.data_ptr(), rope_d.data_ptr(), r8.data_ptr(),
+                                rs.data_ptr(), rr.data_ptr(), pos, kvl, ropn, nb) == 0
+    assert np.array_equal(back(r8), want[0])
+    assert np.array_equal(back(rs, np.uint32), want[1].view(np.uint32))
+    assert np.array_equal(back(rr, np.uint16), want[2])
 
 
 def test_append_kv_guards():
@@ -75,13 +83,20 @@ def test_index_append_reference_fixture(oracle):
     cache = dzeros(rows * hd * 2)
     hip.launch_index_append(dev(k), cache, pos, hd)
     assert np.array_equal(back(cache, np.uint16), want)
-    ref = ref_kernels()
-    if ref is not None:
-        rcache, kd = dzeros(rows * hd * 2), dev(k)
-        assert ref.rivoli_index_append(kd.data_ptr(), rcache.data_ptr(), pos, hd) == 0
-        assert np.array_equal(back(rcache, np.uint16), want)
     with pytest.raises(hip.LaunchError):
         hip.launch_index_append(dev(k), cache, -1, hd)
+
+
+def test_reference_index_append_agrees_with_the_oracle(oracle):
+    """The reference's own kernel (indexer.hip compiled for this GPU) on the same fixture."""
+    ref = need_ref("rivoli_index_append")
+    rows, hd, pos = 7, 128, 5
+    k = oracle.lcg(0xC0DE).fill(hd) * np.float32(8.0)
+    want = np.zeros(rows * hd, np.uint16)
+    oracle.index_append(k, want, pos, hd)
+    rcache, kd = dzeros(rows * hd * 2), dev(k)
+    assert ref.rivoli_index_append(kd.data_ptr(), rcache.data_ptr(), pos, hd) == 0
+    assert np.array_equal(back(rcache, np.uint16), want)
 
 
 def paged_append_both(oracle, rows, slots, n_pages, fill=0xA5):

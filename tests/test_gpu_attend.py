@@ -317,17 +317,29 @@ def check_linear(got, want, what):
 ])
 def test_linear_attend_reference_cases(oracle, seed, h, nt, kvl, rope):
     from tests.attend_cases import reference_attend_case
-    from tests.gpu_util import ref_kernels
 
     case = reference_attend_case(oracle, seed, h, nt, kvl, rope)
     code, want = oracle.mla_attend(*case[:5], None, h, nt, kvl, rope, case[5], case[6])
     assert code == 0
     check_linear(run_linear(case, h, nt, kvl, rope), want, "multi-split")
     check_linear(run_linear(case, h, nt, kvl, rope, scratch=False), want, "single split (null scratch)")
-    ref = ref_kernels()
-    if ref is not None and hasattr(ref, "rivoli_mla_attend"):
-        # the reference's own kernel, compiled for this GPU, agrees with the oracle too
-        check_linear(run_linear(case, h, nt, kvl, rope, launch=ref.rivoli_mla_attend), want, "reference kernel")
+
+
+@pytest.mark.parametrize("seed,h,nt,kvl,rope", [
+    (0x0A5E1102, 64, 300, 512, 64), (0x5F117BAD, 64, 704, 512, 64), (0xC1A39ED0, 64, 4608, 512, 64),
+    (0x00C0FFEE, 4, 1, 128, 8), (0xB10CC0DE, 20, 130, 512, 64), (0x0DD5A4E5, 3, 50, 256, 200),
+    (0x0DD5A4E6, 130, 9000, 384, 6),
+])
+def test_reference_mla_attend_agrees_with_the_oracle(oracle, seed, h, nt, kvl, rope):
+    """The reference's own kernel (attn.hip compiled for this GPU) on the same cases."""
+    from tests.attend_cases import reference_attend_case
+    from tests.gpu_util import need_ref
+
+    ref = need_ref("rivoli_mla_attend")
+    case = reference_attend_case(oracle, seed, h, nt, kvl, rope)
+    code, want = oracle.mla_attend(*case[:5], None, h, nt, kvl, rope, case[5], case[6])
+    assert code == 0
+    check_linear(run_linear(case, h, nt, kvl, rope, launch=ref.rivoli_mla_attend), want, "reference kernel")
 
 
 def test_linear_attend_rows_and_guards(oracle):

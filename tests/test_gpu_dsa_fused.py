@@ -166,6 +166,47 @@ def test_score_kernel_fills_the_selection_histogram(oracle, nh):
         assert not back(ws, np.uint32).reshape(n_q, -1)[:, :4096].any()
 
 
+@pytest.mark.parametrize("nh", [32, 72])
+def test_a_key_page_outside_the_pool_scores_minus_infinity_in_the_histogram_form(oracle, nh):
+    """A block-table entry of the key cache that is not a page of the pool: the score kernel
+    that also fills the selection histogram writes -inf for that page's tokens and counts them,
+    so the histogram, the scores and the selection that follows (hist_ready) agree; the plain
+    score kernel leaves those tokens unwritten."""
+    hd, pt, nt, k, n_q = 128, 64, 20000, 700, 2
+    rng = np.random.default_rng(77)
+    blocks = -(-nt // pt)
+    n_pages = n_q * blocks
+    tables = shuffled_block_tables(n_q, blocks, n_pages, seed=3)
+    kpool_h = (rng.standard_normal((n_pages * pt, hd), dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    tables[0, 5] = n_pages + 7                       # tokens 320..383 of query 0
+    tables[1, blocks - 1] = -1                       # the last (partial) page of query 1
+    q = rng.standard_normal((n_q, nh, hd), dtype=np.float32)
+    w = np.abs(rng.standard_normal((n_q, nh), dtype=np.float32))
+    kv_tables, kv_pages, pool_h = paged_cache(oracle, rng, n_q, nt)
+    ws = dzeros(hip.index_topk_workspace_bytes(n_q, nt))
+    sc = dev(np.full((n_q, nt), 123.0, np.float32))
+    rows, out = dzeros(n_q * k * 4, 0xFF), dzeros(n_q * k * W * 2, 0xEE)
+    hip.launch_index_score_paged_hist(dev(q), dev(w), dev(kpool_h), dev(tables), None, None, n_q, blocks, nt, nt, nh,
+                                      nh, hd, pt, n_pages, 0.1, 0.1, sc, ws)
+    hist = back(ws, np.uint32).reshape(n_q, -1)[:, :4096].copy()
+    scores = back(sc, np.float32).reshape(n_q, nt).copy()
+    lost0, lost1 = slice(5 * pt, 6 * pt), slice((blocks - 1) * pt, nt)
+    assert np.all(np.isneginf(scores[0, lost0])) and np.all(np.isneginf(scores[1, lost1]))
+    assert np.isfinite(np.delete(scores[0], np.r_[lost0])).all() and int(hist[0].sum()) == nt == int(hist[1].sum())
+    hip.launch_dsa_select_gather_paged(sc, n_q, nt, None, nt, k, rows, ws, True, dev(pool_h), dev(kv_tables), out,
+                                       kv_tables.shape[1], W, PT, kv_pages)
+    got_rows, got_out = back(rows, np.uint32).reshape(n_q, k), back(out, np.uint16).reshape(n_q, k, W)
+    check_against_oracle(oracle, scores, None, k, kv_tables, pool_h, got_rows, got_out)
+    plain = dev(np.full((n_q, nt), 123.0, np.float32))
+    hip.launch_index_score_paged(dev(q), dev(w), dev(kpool_h), dev(tables), None, None, n_q, blocks, nt, nt, nh, nh,
+                                 hd, pt, n_pages, 0.1, 0.1, plain)
+    plain_h = back(plain, np.float32).reshape(n_q, nt)
+    assert np.all(plain_h[0, lost0] == 123.0) and np.all(plain_h[1, lost1] == 123.0)
+    keep = np.ones((n_q, nt), bool)
+    keep[0, lost0] = keep[1, lost1] = False
+    assert np.array_equal(plain_h[keep], scores[keep])
+
+
 def test_config4_layer_fused(oracle):
     """benchmark configuration 4's layer: 16 queries x 65536 scores, k = 2048, fragmented pages."""
     rng = np.random.default_rng(0x5EED0004)

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 from rivoli_amd import hip
-from tests.gpu_util import back, dev, dzeros, ref_kernels
+from tests.gpu_util import back, dev, dzeros, need_ref
 from tests.v4_cases import attend_inputs, sparse_attn_f64
 
 pytestmark = pytest.mark.gpu
@@ -166,9 +166,7 @@ def test_window_selection_feeds_the_attention(oracle):
 def test_reference_kernel_agrees_with_the_oracle(oracle):
     """The reference's own kernel compiled for this GPU, where that build exists: it and the
     oracle follow the same folds, so they agree far inside the bar."""
-    ref = ref_kernels()
-    if ref is None or not hasattr(ref, "rivoli_gather_attn_shared_kv"):
-        pytest.skip("reference kernels not built")
+    ref = need_ref("rivoli_gather_attn_shared_kv")
     for (m, h, d, topk, rows) in ((3, 8, 512, 40, 64), (2, 4, 64, 8, 12)):
         q, kv, sink = attend_inputs(oracle, m, h, d, rows, seed=31 + d)
         idx = random_lists(np.random.default_rng(5), m, topk, rows)

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from rivoli_amd import hip
-from tests.gpu_util import back, dev, dzeros, ref_kernels
+from tests.gpu_util import back, dev, dzeros, need_ref
 from tests.topk_cases import brute_force_topk, reference_topk_cases
 
 pytestmark = pytest.mark.gpu
@@ -29,11 +29,14 @@ def test_index_topk_reference_cases(oracle):
     for name, scores, k in reference_topk_cases(oracle):
         want = oracle.topk(scores, k)
         check_topk_case(name, scores, k, want, hip.launch_index_topk)
-    ref = ref_kernels()
-    if ref is not None:  # the reference kernel itself agrees with the oracle on its own cases
-        for name, scores, k in reference_topk_cases(oracle):
-            check_topk_case("ref:" + name, scores, k, oracle.topk(scores, k),
-                            lambda s, n, kk, r: ref.rivoli_index_topk(s.data_ptr(), n, kk, r.data_ptr()))
+
+
+def test_reference_index_topk_agrees_with_the_oracle(oracle):
+    """The reference's own kernel (indexer.hip compiled for this GPU) on its own cases."""
+    ref = need_ref("rivoli_index_topk")
+    for name, scores, k in reference_topk_cases(oracle):
+        check_topk_case("ref:" + name, scores, k, oracle.topk(scores, k),
+                        lambda s, n, kk, r: ref.rivoli_index_topk(s.data_ptr(), n, kk, r.data_ptr()))
 
 
 def test_index_topk_guards():
@@ -170,10 +173,15 @@ def test_hash_rows_matches_the_host_fold(oracle):
     assert int(back(twice, np.uint64)[0]) == 0
     big = np.random.default_rng(1).integers(0, 2 ** 32, 3_000_001, dtype=np.uint64).astype(np.uint32)
     assert fold(big.view(np.float32)) == oracle.xor_fold(big)
-    ref = ref_kernels()
-    if ref is not None:
-        out = dzeros(8)
-        assert ref.rivoli_hash_rows(xd.data_ptr(), n, 1, 0, out.data_ptr(), None) == 0
-        assert int(back(out, np.uint64)[0]) == want
     with pytest.raises(hip.LaunchError):
         hip.launch_hash_rows(xd, 0, 1, 0, twice)
+
+
+def test_reference_hash_rows_agrees_with_the_host_fold(oracle):
+    """The reference's own kernel (compiled for this GPU) on the same 1000 values."""
+    ref = need_ref("rivoli_hash_rows")
+    n = 1000
+    x = oracle.lcg(0x8AD5).fill(n)
+    xd, out = dev(x), dzeros(8)
+    assert ref.rivoli_hash_rows(xd.data_ptr(), n, 1, 0, out.data_ptr(), None) == 0
+    assert int(back(out, np.uint64)[0]) == oracle.xor_fold(x)

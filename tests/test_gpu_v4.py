@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from rivoli_amd import hip
-from tests.gpu_util import back, dev, dzeros, ref_kernels
+from tests.gpu_util import back, dev, dzeros, need_ref
 from tests.test_oracle_v4 import brute_force_rows, reference_tie_block
 
 pytestmark = pytest.mark.gpu
@@ -42,11 +42,19 @@ def test_act_quant_reference_tie_fixture(oracle):
     row = reference_tie_block()[None, :]
     got = check_act_quant(oracle, row, 64, 64, what="tie block")
     assert np.count_nonzero((got != 0) & (np.abs(got) < 0.015625)) >= 8
-    ref = ref_kernels()
-    if ref is not None and hasattr(ref, "rivoli_act_quant_f8_prefix"):
-        # the reference's own kernel, compiled for this GPU, agrees with the oracle too
-        theirs = device_act_quant(row, 64, 64, launch=ref.rivoli_act_quant_f8_prefix)
-        assert same_bits(theirs, oracle.act_quant_f8_prefix(row, 64, 64)[1]).size == 0
+
+
+def test_reference_act_quant_agrees_with_the_oracle(oracle):
+    """The reference's own kernel (mla.hip compiled for this GPU): the tie fixture against the
+    oracle, 300 cache rows against the oracle and this library."""
+    ref = need_ref("rivoli_act_quant_f8_prefix")
+    row = reference_tie_block()[None, :]
+    theirs = device_act_quant(row, 64, 64, launch=ref.rivoli_act_quant_f8_prefix)
+    assert same_bits(theirs, oracle.act_quant_f8_prefix(row, 64, 64)[1]).size == 0
+    x = cache_rows(300, seed=64)
+    theirs = device_act_quant(x, 448, 64, launch=ref.rivoli_act_quant_f8_prefix)
+    assert same_bits(theirs, oracle.act_quant_f8_prefix(x, 448, 64)[1]).size == 0
+    assert same_bits(theirs, device_act_quant(x, 448, 64)).size == 0
 
 
 def cache_rows(rows, seed):
@@ -69,10 +77,6 @@ def test_act_quant_cache_rows_block_64_prefix(oracle):
     x = cache_rows(3001, seed=64)
     got = check_act_quant(oracle, x, 448, 64, what="kv rows")
     assert np.array_equal(got[:, 448:].view(np.uint32), x[:, 448:].view(np.uint32))
-    ref = ref_kernels()
-    if ref is not None and hasattr(ref, "rivoli_act_quant_f8_prefix"):
-        theirs = device_act_quant(x[:300], 448, 64, launch=ref.rivoli_act_quant_f8_prefix)
-        assert same_bits(theirs, got[:300]).size == 0
 
 
 def test_act_quant_block_128_into_a_second_buffer(oracle):

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from rivoli_amd import hip
-from tests.gpu_util import back, dev, dzeros, ref_kernels
+from tests.gpu_util import back, dev, dzeros, need_ref
 from tests.test_gpu_v4 import same_bits
 from tests.test_oracle_v4_blockindex import bf16_round
 
@@ -48,24 +48,33 @@ def test_spread_matches_the_oracle(oracle, rows, d):
     assert bad.size == 0, [(int(i) // d, int(i) % d, got.ravel()[i], want.ravel()[i]) for i in bad[:6]]
 
 
-def test_spread_over_sixty_binades_and_the_reference_kernel(oracle):
-    """crates/engine/tests/kernel_v4_indexer.rs:246-277: row r scaled into binade r - 30, so the
-    block scale lands on 60 powers of two; the reference's own kernel, compiled for this GPU,
-    is held to the oracle on the same rows."""
+def sixty_binades():
     rng = np.random.default_rng(60)
     base = bf16_round(rng.standard_normal((60, 128)).astype(np.float32))
-    x = bf16_round(base * (2.0 ** (np.arange(60) - 30))[:, None].astype(np.float32))
+    return bf16_round(base * (2.0 ** (np.arange(60) - 30))[:, None].astype(np.float32))
+
+
+def test_spread_over_sixty_binades(oracle):
+    """crates/engine/tests/kernel_v4_indexer.rs:246-277: row r scaled into binade r - 30, so the
+    block scale lands on 60 powers of two."""
+    x = sixty_binades()
     code, want = oracle.act_quant_f4_rotated(x)
     assert same_bits(device_spread(x), want).size == 0
     scales = {float(np.abs(r[r != 0]).min()) for r in want if (r != 0).any()}
     assert len(scales) >= 55
-    ref = ref_kernels()
-    if ref is not None and hasattr(ref, "rivoli_act_quant_f4_rotated"):
-        assert same_bits(device_spread(x, launch=ref.rivoli_act_quant_f4_rotated), want).size == 0
-        for rows, d in ((333, 256), (77, 128), (19, 64), (11, 32)):
-            wide = spread_rows(rows, d, 5)
-            assert same_bits(device_spread(wide, launch=ref.rivoli_act_quant_f4_rotated),
-                             device_spread(wide)).size == 0, (rows, d)
+
+
+def test_reference_spread_agrees_with_the_oracle_and_this_library(oracle):
+    """The reference's own kernel (blockindex.hip compiled for this GPU): the sixty binades
+    against the oracle, other widths against this library."""
+    ref = need_ref("rivoli_act_quant_f4_rotated")
+    x = sixty_binades()
+    want = oracle.act_quant_f4_rotated(x)[1]
+    assert same_bits(device_spread(x, launch=ref.rivoli_act_quant_f4_rotated), want).size == 0
+    for rows, d in ((333, 256), (77, 128), (19, 64), (11, 32)):
+        wide = spread_rows(rows, d, 5)
+        assert same_bits(device_spread(wide, launch=ref.rivoli_act_quant_f4_rotated),
+                         device_spread(wide)).size == 0, (rows, d)
 
 
 def test_spread_guards():
@@ -124,10 +133,8 @@ def test_score_matches_the_oracle(oracle, s, n_comp, heads, hd, spread):
     assert np.count_nonzero(want) > 0 or n_comp * s < 4
 
 
-def test_score_known_answer_and_the_reference_kernel(oracle):
-    """kernel_v4_indexer.rs:689-726 (f32 accumulation, one bf16 round: 1.125, not 1.0), and the
-    reference's own kernel held to the oracle and to this library on rounding-sensitive
-    operands."""
+def test_score_known_answer(oracle):
+    """kernel_v4_indexer.rs:689-726 (f32 accumulation, one bf16 round: 1.125, not 1.0)."""
     heads, hd = 64, 128
     kv = np.zeros((1, hd), np.float32)
     kv[0, 0] = 1.0
@@ -136,13 +143,17 @@ def test_score_known_answer_and_the_reference_kernel(oracle):
     q[0, 0, 0] = 1.0
     got = device_score(q, kv, np.ones((1, heads), np.float32))
     assert got[0, 0] == np.float32(1.125)
-    ref = ref_kernels()
-    if ref is not None and hasattr(ref, "rivoli_index_score_blocks"):
-        for shape in [(4, 200, 64, 128), (3, 77, 5, 64)]:
-            q, kv, w = score_case(*shape, seed=9)
-            theirs = device_score(q, kv, w, launch=ref.rivoli_index_score_blocks)
-            assert same_bits(theirs, oracle.index_score_blocks(q, kv, w)[1]).size == 0
-            assert same_bits(theirs, device_score(q, kv, w)).size == 0
+
+
+def test_reference_scorer_agrees_with_the_oracle_and_this_library(oracle):
+    """The reference's own kernel (blockindex.hip compiled for this GPU) on rounding-sensitive
+    operands."""
+    ref = need_ref("rivoli_index_score_blocks")
+    for shape in [(4, 200, 64, 128), (3, 77, 5, 64)]:
+        q, kv, w = score_case(*shape, seed=9)
+        theirs = device_score(q, kv, w, launch=ref.rivoli_index_score_blocks)
+        assert same_bits(theirs, oracle.index_score_blocks(q, kv, w)[1]).size == 0
+        assert same_bits(theirs, device_score(q, kv, w)).size == 0
 
 
 def test_score_guards():

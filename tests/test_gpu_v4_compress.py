@@ -10,7 +10,7 @@ import pytest
 
 from oracle.kvoracle import CompGeom as OracleGeom
 from rivoli_amd import hip
-from tests.gpu_util import back, dev, dzeros, ref_kernels
+from tests.gpu_util import back, dev, dzeros, need_ref
 from tests.v4_cases import compress_gap, compress_inputs
 
 pytestmark = pytest.mark.gpu
@@ -57,11 +57,20 @@ def test_prefill_matches_oracle(oracle, ratio, d, rd, s):
     assert code == 0
     got = device_prefill(hg, kv, score, ape, norm, freqs, nblk)
     assert_clean(oracle, got, want, f"ratio {ratio} d {d}", rd)
-    ref = ref_kernels()
-    if ref is not None and hasattr(ref, "rivoli_kv_compress_prefill") and d <= 1024:
-        # the reference's own kernel, compiled for this GPU, agrees with the oracle too
-        theirs = device_prefill(hg, kv, score, ape, norm, freqs, nblk, launch=ref.rivoli_kv_compress_prefill)
-        assert_clean(oracle, theirs, want, f"reference kernel, ratio {ratio} d {d}", rd)
+
+
+@pytest.mark.parametrize("ratio,d,rd,s", [(4, 512, 64, 1024), (128, 512, 64, 1024), (4, 64, 16, 45),
+                                          (8, 34, 8, 80), (16, 128, 32, 160), (32, 130, 64, 96)])
+def test_reference_prefill_agrees_with_the_oracle(oracle, ratio, d, rd, s):
+    """The reference's own kernel (kvcompress.hip compiled for this GPU; widths it accepts)."""
+    ref = need_ref("rivoli_kv_compress_prefill")
+    og, hg = geoms(ratio, d, rd)
+    kv, score, ape, norm, freqs = compress_inputs(og, s, seed=ratio * 31 + d)
+    nblk = s // ratio
+    code, want = oracle.kv_compress_prefill(kv, score, ape, norm, freqs, og, nblk)
+    assert code == 0
+    theirs = device_prefill(hg, kv, score, ape, norm, freqs, nblk, launch=ref.rivoli_kv_compress_prefill)
+    assert_clean(oracle, theirs, want, f"reference kernel, ratio {ratio} d {d}", rd)
 
 
 def test_masked_and_peaked_windows(oracle):

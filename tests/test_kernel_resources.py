@@ -89,3 +89,15 @@ def test_block_scorer_keeps_its_row_and_both_chunk_buffers_in_registers():
         assert int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b).group(1)) == 0, name
         assert int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", b).group(1)) >= 3, name
     assert seen == 2
+
+
+def test_the_build_refuses_an_attention_object_that_spills():
+    """build.check_resources is what build_kernels applies to mla_attend.hip's resource report:
+    scratch memory or too much LDS in an 8-bit attention kernel raises instead of linking."""
+    head = "x.hip:1:1: remark: Function Name: _ZN2rk23mla_attend_paged_kernelILi2ELi2ELi0ELb0ELb1EEEvNS_10AttendArgsE\n"
+    fine = head + "    ScratchSize [bytes/lane]: 0\n    LDS Size [bytes/block]: 85632\n"
+    build.check_resources("mla_attend.hip", fine)
+    build.check_resources("kv_gather.hip", "")                        # other files are not held to it
+    for bad in (fine.replace("lane]: 0", "lane]: 44"), fine.replace("85632", "170000"), ""):
+        with pytest.raises(RuntimeError):
+            build.check_resources("mla_attend.hip", bad)

@@ -55,3 +55,43 @@ def test_noalloc_size_limit_and_guards():
         with pytest.raises(hip.LaunchError) as e:
             call(**kw)
         assert e.value.code == code, kw
+
+
+def test_noalloc_call_replays_from_a_graph(oracle):
+    """The callers it is for: the call captured into a HIP graph (the first call on the device,
+    which looks the array's address up, made before the capture) and replayed on fresh scores,
+    with eager work between the replays; every replay equals the workspace form."""
+    from tests.gpu_util import torch_cuda
+
+    torch = torch_cuda()
+    rng = np.random.default_rng(77)
+    n_q, nt, k = 3, 30000, 400
+    tables, n_pages, pool_h = paged_cache(oracle, rng, n_q, nt)
+    pool_d, tables_d = dev(pool_h), dev(tables)
+    scores = torch.zeros(n_q * nt * 4, dtype=torch.uint8, device="cuda")
+    rows, out = dzeros(n_q * k * 4, 0xFF), dzeros(n_q * k * W * 2, 0xEE)
+
+    def call(stream):
+        hip.launch_dsa_select_gather_paged_noalloc(scores, n_q, nt, None, nt, k, rows, pool_d, tables_d, out,
+                                                   tables.shape[1], W, PT, n_pages, None, stream)
+
+    call(hip.NULL_STREAM)                                      # the address lookup happens here
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    for t in range(3):                                         # replays on the null stream, like the eager work
+        s = rng.standard_normal((n_q, nt), dtype=np.float32)
+        s[1, ::7] = np.float32(0.25)
+        scores.copy_(dev(s))
+        rows.fill_(0xFF)
+        out.fill_(0xEE)
+        graph.replay()
+        torch.cuda.synchronize()
+        got_rows, got_out = back(rows, np.uint32).reshape(n_q, k), back(out, np.uint16).reshape(n_q, k, W)
+        want_rows, want_out, _ = run_fused(s, None, k, tables, n_pages, pool_d, split=True)   # eager work between
+        assert np.array_equal(got_rows, want_rows), t
+        assert np.array_equal(got_out, want_out), t
