@@ -81,6 +81,10 @@ def parse():
     ap.add_argument("--unfused", action="store_true",
                     help="dsa / dsa_scored: run the selection and the sparse gather as two separate "
                          "entry points instead of the one fused call")
+    ap.add_argument("--one-launch", action="store_true",
+                    help="decode: the step's append and gather as one launch (rivoli_kv_append_gather_paged) "
+                         "instead of two calls; it pays where the step is launch-bound (configuration 1), and "
+                         "measures equal at configuration 3's size")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (a known-size kernel to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
@@ -126,7 +130,11 @@ def main():
     # line, the other configurations, each with its own oracle check
     res = bench_decode(a, torch, hip)
     short = min(a.cpu_seconds, 2.0)
+    small = dict(layers=1, batch=1, ctx=4096, steps=200, warmup=20, cpu_seconds=short)
     others = (("cfg3_ragged", "decode", dict(ragged=True, cpu_seconds=short)),
+              # configuration 1 (append one token, gather 4096): as two calls and as one launch
+              ("cfg1_step", "decode", small),
+              ("cfg1_step_one_launch", "decode", dict(small, one_launch=True)),
               ("cfg4_dsa", "dsa", dict(cpu_seconds=short)),
               ("cfg4_dsa_scored", "dsa_scored", dict(cpu_seconds=short)),
               ("cfg4_dsa_attend", "dsa_attend", dict(precise=4)),
@@ -279,14 +287,20 @@ def bench_decode(a, torch, hip):
     stream = torch.cuda.Stream()
     sh = stream.cuda_stream
 
+    fused = a.one_launch and a.gather_form == "packed"
+
     def step(events=None):
         for layer in range(L):
-            hip.launch_kv_append_paged(new_rows[layer], new_slots, pools[layer], B, W, PT, n_pages,
-                                       None, sh)
+            if not fused:
+                hip.launch_kv_append_paged(new_rows[layer], new_slots, pools[layer], B, W, PT, n_pages,
+                                           None, sh)
             if events is not None:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)
-            if a.gather_form == "packed":
+            if fused:    # the step's two calls as one launch
+                hip.launch_kv_append_gather_paged(new_rows[layer], new_slots, pools[layer], tables, seq_lens, cu,
+                                                  out, B, cols, n_att, W, PT, n_pages, None, None, sh)
+            elif a.gather_form == "packed":
                 hip.launch_kv_gather_paged_packed(pools[layer], tables, seq_lens, cu, out, B, cols, n_att, W,
                                                   PT, n_pages, None, sh)
             else:
@@ -315,6 +329,9 @@ def bench_decode(a, torch, hip):
     table_entries = int((-(-seq_lens_np // PT)).sum())
     gather_bytes_layer = n_att * (REC + ROW_IN) + table_entries * 4  # records + table in, bf16 out
     step_bytes = append_bytes + L * gather_bytes_layer
+    if fused:  # the launch that is bracketed also appends: its new rows in, their records out
+        # (the new tokens' bf16 rows come from the rows just quantized, not from their records)
+        gather_bytes_layer += B * (ROW_IN + 4 + REC) - B * REC
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     achieved = gather_bytes_layer / (gather_ms * 1e-3) / 1e9
 
@@ -329,7 +346,8 @@ def bench_decode(a, torch, hip):
                    "layers": L, "batch": B, "ctx": ctx, "page_tokens": PT, "width": W,
                    "stored": "fp8 e4m3 + 1 f32 scale/token", "out": "bf16",
                    "contexts": "uniform in [1024, ctx]" if a.ragged else "all at ctx",
-                   "tokens_per_layer": n_att, "table_blocks": cols, "gather_form": a.gather_form},
+                   "tokens_per_layer": n_att, "table_blocks": cols, "gather_form": a.gather_form,
+                   "launches_per_layer": 1 if fused else 2},
         "decode_step_kv_ms": round(ms_per_step, 4),
         "tokens_per_s": round(L * n_att / (ms_per_step * 1e-3), 1),
         "hbm_peak_frac": round(value * 1e9 / HBM_PEAK, 4),
@@ -337,7 +355,7 @@ def bench_decode(a, torch, hip):
         # less than 0.7 of what its block tables could hold (kv_gather.hip: gather_paged_launch)
         "roofline": {"bound": "hbm",
                      "kernel": ("kv_gather_flat_kernel" if a.gather_form == "packed" and n_att * 10 < B * cols * PT * 7
-                                else "kv_gather_paged_kernel"),
+                                else "kv_gather_paged_kernel") + (" (with the step's appends)" if fused else ""),
                      "achieved": round(achieved, 1),
                      "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": round(achieved * 1e9 / HBM_PEAK, 4),
                      "avg_launch_ms": round(gather_ms, 5), "bytes_per_launch": gather_bytes_layer,
@@ -345,8 +363,12 @@ def bench_decode(a, torch, hip):
     }
 
     if not a.no_cpu_baseline:
+        regather = None
+        if fused:   # layer 0's step again: the append rewrites the same record, the gather is checked
+            regather = lambda: hip.launch_kv_append_gather_paged(new_rows[0], new_slots, pools[0], tables, seq_lens,
+                                                                 cu, out, B, cols, n_att, W, PT, n_pages)
         result["cpu_baseline"] = cpu_baseline(pools[0], tables_np, seq_lens_np, out, a.cpu_seconds,
-                                              hip, tables, seq_lens, cu, B, cols, n_pages)
+                                              hip, tables, seq_lens, cu, B, cols, n_pages, regather)
     return result
 
 
@@ -1104,7 +1126,7 @@ def bench_attend(a, torch, hip):
 
 
 def cpu_baseline(pool0, tables_np, seq_lens_np, out, budget_s, hip, tables, seq_lens, cu, B, blocks,
-                 n_pages):
+                 n_pages, regather=None):
     """The CPU oracle's gather over layer 0 of the same pool, on the host cores, repeated until
     about `budget_s` seconds have been spent; its output is also compared with the GPU's."""
     import torch
@@ -1131,8 +1153,13 @@ def cpu_baseline(pool0, tables_np, seq_lens_np, out, budget_s, hip, tables, seq_
     ora.kv_gather_paged(pool_host, tables_np[:1], one_len, W, PT, n_threads=1, out=one_out)
     one_s = time.perf_counter() - t0
     one_bytes = int(one_len[0]) * (REC + ROW_IN)
-    # full-size parity of one layer: GPU gather of the same pool vs the oracle's bytes
-    hip.launch_kv_gather_paged(pool0, tables, seq_lens, cu, out, B, blocks, W, PT, n_pages)
+    # full-size parity of one layer: GPU gather of the same pool vs the oracle's bytes (through
+    # the entry point that was timed, when the caller hands it over)
+    out.fill_(0)
+    if regather is not None:
+        regather()
+    else:
+        hip.launch_kv_gather_paged(pool0, tables, seq_lens, cu, out, B, blocks, W, PT, n_pages)
     torch.cuda.synchronize()
     same = bool(np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1, W)[:n_tok],
                                out_host))

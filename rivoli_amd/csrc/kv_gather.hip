@@ -166,8 +166,11 @@ __global__ __launch_bounds__(THREADS) void kv_gather_flat_kernel(
     {
         const int lane = threadIdx.x & (kWave - 1);
         for (int s0 = 0; s0 < n_seqs; s0 += kWave) {
-            int len = seq_lens[min(s0 + lane, n_seqs - 1)];
-            if (APPEND && s0 + lane < n_seqs && appends_last(ap, s0 + lane, len)) --len;
+            // (both loads unconditional, from an index that always exists: a load under a
+            // condition is a branch with a wait of its own)
+            const int at = min(s0 + lane, n_seqs - 1);
+            int len = seq_lens[at];
+            if (APPEND) len -= appends_last(ap, at, len) ? 1 : 0;
             len = s0 + lane < n_seqs ? min(max(len, 0), cap) : 0;
             const uint32_t units = (uint32_t)(len + ROWS - 1) / ROWS;
             const uint32_t incl = first + wave_inclusive_sum(units);
