@@ -442,9 +442,10 @@ def bench_prefill(a, torch, hip):
            "config": {"workload": "prefill bulk append (benchmark configuration 2)", "tokens": n,
                       "pages": n_pages, "width": W, "page_tokens": PT},
            "tokens_per_s": round(n / (ms * 1e-3), 1),
-           # (kv_append.hip: batches under 16384 tokens take the wave-per-token kernel)
+           # (kv_append.hip picks the kernel by the batch's size)
            "roofline": {"bound": "hbm",
-                        "kernel": "kv_append_paged_token_kernel<2>" if n < 16384 else "kv_append_paged_kernel<72>",
+                        "kernel": ("kv_append_paged_token_kernel<2>" if n < 512 else
+                                   "kv_append_paged_wide_kernel" if n < 20480 else "kv_append_paged_kernel<72>"),
                         "achieved": round(nbytes / (per["append"] * 1e-3) / 1e9, 2),
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                         "frac": round(nbytes / (per["append"] * 1e-3) / HBM_PEAK, 5),

@@ -20,11 +20,19 @@ constexpr int kAppendWaves = 4;   // linear-slab kernel: tokens per workgroup
 constexpr int kRowsPerWave = 8;   // paged kernel: tokens per (one-wave) workgroup
 constexpr int kMaxChunksPerRow = 128;  // width <= 1024
 // Batches at least this large take the 8-rows-per-wave kernel (throughput); smaller ones the
-// one-wave-per-token kernel (latency). RIVOLI_BULK_APPEND_TOKENS overrides it at build time.
+// one-wave-per-token kernel (latency) — except 576-wide rows, which have a kernel of their own
+// for the sizes in between (kWideAppendTokens .. kWideAppendBelow).
+// RIVOLI_BULK_APPEND_TOKENS overrides it at build time.
 #ifndef RIVOLI_BULK_APPEND_TOKENS
 #define RIVOLI_BULK_APPEND_TOKENS 16384
 #endif
 constexpr int kBulkAppendTokens = RIVOLI_BULK_APPEND_TOKENS;
+// From this many tokens (of 576-wide rows) up to the bulk threshold: the 576-thread kernel.
+#ifndef RIVOLI_WIDE_APPEND_TOKENS
+#define RIVOLI_WIDE_APPEND_TOKENS 512
+#endif
+constexpr int kWideAppendTokens = RIVOLI_WIDE_APPEND_TOKENS;
+constexpr int kWideAppendBelow = 20480;  // from here on the one-wave-per-8-tokens kernel is faster
 
 // Paged append. One wave64 workgroup owns 8 consecutive tokens = one contiguous run of the
 // input, cut into 16-byte chunks (8 bf16) dealt round-robin to the lanes: for a 576-wide row
@@ -160,6 +168,104 @@ __global__ __launch_bounds__(kWave) void kv_append_paged_kernel(
         *reinterpret_cast<float*>(pool + s_sdst[lane]) = __uint_as_float(s_row[lane].x);
 }
 
+// Paged append, mid-sized batches of 576-wide rows (a prefill chunk of a few thousand tokens):
+// the bulk kernel's work unit — 8 consecutive tokens = 576 16-byte chunks — dealt to 576
+// threads, one chunk each, so a launch of a few thousand tokens still fills the chip with
+// loads in flight (the one-wave form keeps 9 chunks per lane and, below ~16 K tokens, too few
+// waves per compute unit; the wave-per-token form below issues a second, almost empty step for
+// the row's last 8 chunks). A chunk's maximum is taken NaN-free on the spot (a chunk holding a
+// NaN folds its other values with float maxima), wave 0 folds the 72 chunk maxima of each row
+// (8 lanes per row) and derives the row's scale, its reciprocal and the exact-path band.
+constexpr int kWideThreads = kRowsPerWave * 72;
+// J chunks per thread: a workgroup owns 8 J consecutive tokens.
+template <int J>
+__global__ __launch_bounds__(kWideThreads) void kv_append_paged_wide_kernel(
+    const uint16_t* __restrict__ rows, const int* __restrict__ slot_mapping,
+    uint8_t* __restrict__ pool, int n_tokens, int page_tokens, long long n_slots,
+    size_t page_bytes, unsigned int* __restrict__ bad_slots) {
+    constexpr int CPR = 72, W = CPR * 8, ROWS = kRowsPerWave * J;
+    constexpr int PARTS = kWave / ROWS, PER = CPR / PARTS;  // wave 0: lanes per row, chunks per lane
+    static_assert(PARTS * ROWS == kWave && PER * PARTS == CPR, "a wave folds the rows' chunk maxima");
+    constexpr unsigned long long kSkip = ~0ull;
+    __shared__ uint32_t s_amax[kWideThreads * J];
+    __shared__ u32x4 s_row[ROWS];
+    __shared__ unsigned long long s_dst[ROWS], s_sdst[ROWS];
+    const int tid = threadIdx.x;
+    const int t0 = (int)blockIdx.x * ROWS;
+    const int nrows = min(ROWS, n_tokens - t0);
+    const u32x4* src = reinterpret_cast<const u32x4*>(rows + (size_t)t0 * W);
+    u32x4 raw[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j)
+        raw[j] = tid + j * kWideThreads < nrows * CPR ? __builtin_nontemporal_load(src + tid + j * kWideThreads)
+                                                      : u32x4{0, 0, 0, 0};
+    if (tid < ROWS) {  // where each row goes (or nowhere)
+        unsigned long long dst = kSkip, sdst = 0;
+        if (tid < nrows) {
+            const int slot = slot_mapping[t0 + tid];
+            if (slot >= 0) {
+                if ((long long)slot < n_slots) {
+                    const int page = slot / page_tokens, off = slot - page * page_tokens;
+                    dst = (size_t)page * page_bytes + (size_t)off * W;
+                    sdst = (size_t)page * page_bytes + (size_t)page_tokens * W + (size_t)off * 4;
+                } else if (bad_slots) {
+                    atomicAdd(bad_slots, 1u);
+                }
+            }
+        }
+        s_dst[tid] = dst;
+        s_sdst[tid] = sdst;
+    }
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+        // |bf16| patterns order like their values: a packed 16-bit integer maximum
+        u16x2 m = {0, 0};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2, w[i] & 0x7fff7fffu));
+        uint32_t top = (uint32_t)max(m.x, m.y) << 16;
+        if (top > 0x7f800000u) {  // the chunk holds a NaN, which the rule's max ignores
+            float f = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                f = fmaxf(f, fmaxf(fabsf(bf16_lo_to_f32(w[i])), fabsf(bf16_hi_to_f32(w[i]))));
+            top = __float_as_uint(f);
+        }
+        s_amax[tid + j * kWideThreads] = top;
+    }
+    __syncthreads();
+    if (tid < kWave) {
+        const int r = tid / PARTS, part = tid - r * PARTS;
+        uint32_t m = 0u;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) m = max(m, s_amax[r * CPR + part * PER + i]);
+#pragma unroll
+        for (int off = 1; off < PARTS; off <<= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
+        if (part == 0) {
+            const float amax = __uint_as_float(m);
+            const float scl = amax > 0.0f ? amax / 448.0f : 1.0f;
+            s_row[r] = u32x4{__float_as_uint(scl), __float_as_uint(1.0f / scl), row_band(scl), 0u};
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const int c = tid + j * kWideThreads;
+        const int r = c / CPR, col = c - r * CPR;
+        if (c < nrows * CPR) {
+            const unsigned long long dst = s_dst[r];
+            if (dst != kSkip) {
+                const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+                const u32x4 row = s_row[r];
+                __builtin_nontemporal_store(quantize8(w, __uint_as_float(row.x), __uint_as_float(row.y), row.z),
+                                            reinterpret_cast<u32x2*>(pool + dst) + col);
+                if (col == 0) *reinterpret_cast<float*>(pool + s_sdst[r]) = __uint_as_float(row.x);
+            }
+        }
+    }
+}
+
 // Paged append, low-latency form for small batches (decode steps, short prefill chunks): one
 // wave64 per token, 4 tokens per workgroup, no LDS and no barrier. A lane holds 8 consecutive
 // elements per step (one 16-byte load), so a 576-wide row is one full step plus an 8-lane
@@ -243,6 +349,25 @@ extern "C" int rivoli_kv_append_paged(const unsigned short* rows, const int* slo
     const size_t page_bytes = rivoli_kv_page_bytes(page_tokens, width);
     const long long n_slots = (long long)n_pages * page_tokens;
     (void)hipGetLastError();
+    // measured on MI355X, 576-wide rows: 512 tokens 4.0 us either way; 8192 tokens 5.6 us (wave per
+    // token: 6.7); 16384 tokens 8.6 us (one wave per 8 tokens: 9.6); 24576: 12.3 against 11.7
+    if (width == 576 && n_tokens >= kWideAppendTokens && n_tokens < kWideAppendBelow) {
+        // chunks per thread by size (8192 tokens: 5.5 / 5.25 / 5.8 us with 1 / 2 / 4; 16384 tokens:
+        // 8.4 / 8.0 / 7.7; 4096 tokens: 4.15 / 4.4 with 1 / 2)
+#define RK_WIDE(J)                                                                                     \
+    hipLaunchKernelGGL(kv_append_paged_wide_kernel<J>,                                                 \
+                       dim3((unsigned)((n_tokens + kRowsPerWave * (J) - 1) / (kRowsPerWave * (J)))),   \
+                       dim3(kWideThreads), 0, (hipStream_t)stream, rows, slot_mapping, pool, n_tokens, \
+                       page_tokens, n_slots, page_bytes, bad_slots)
+        if (n_tokens < 6144)
+            RK_WIDE(1);
+        else if (n_tokens < 12288)
+            RK_WIDE(2);
+        else
+            RK_WIDE(4);
+#undef RK_WIDE
+        return launch_status();
+    }
     if (n_tokens < kBulkAppendTokens) {
         dim3 grid((unsigned)((n_tokens + kAppendWaves - 1) / kAppendWaves));
         dim3 block(kAppendWaves * kWave);

@@ -246,7 +246,7 @@ def test_append_other_widths(oracle):
 
 
 def test_large_batch_kernel_on_the_census_and_the_special_rows(oracle):
-    """Batches of 16 384 tokens and more take the eight-rows-per-wave kernel, which has its own
+    """Large batches (20 480 tokens and more at this width) take the eight-rows-per-wave kernel, which has its own
     row maxima (packed 16-bit integer maxima, float maxima when a row holds a NaN) and its own
     per-row record: the same census and special rows, interleaved so that NaN rows share a wave
     with ordinary ones, repeated up to 40 000 tokens into shuffled slots."""
@@ -263,6 +263,32 @@ def test_large_batch_kernel_on_the_census_and_the_special_rows(oracle):
     got = back(pool)
     mism = np.flatnonzero(got != want)
     assert int(back(bad, np.uint32)[0]) == 0 and mism.size == 0, [(int(j), hex(got[j]), hex(want[j])) for j in mism[:8]]
+
+
+def test_each_batch_size_class_on_the_census_and_the_special_rows(oracle):
+    """kv_append_paged picks its kernel by the batch's size: a wave per token below 512 tokens,
+    576 threads per 8 tokens from 512 up to the large-batch kernel's 20 480. The census and the
+    special rows, shuffled, go through the first in batches of 500 and through the second in
+    batches of 4 001 (not a multiple of eight) with padding tokens in between; the pool must
+    equal the oracle's after every batch."""
+    base = np.concatenate([special_rows(), census_rows()])
+    base = np.concatenate([base, base])[np.random.default_rng(21).permutation(2 * base.shape[0])]
+    n_pages = -(-base.shape[0] // PT) + 2
+    page_bytes = oracle.kv_page_bytes(PT, W)
+    for batch in (500, 4001, 9000, 13001):      # (the second kernel in its three shapes)
+        slots = np.random.default_rng(batch).permutation(n_pages * PT)[: base.shape[0]].astype(np.int32)
+        slots[::131] = -1
+        want = np.full(n_pages * page_bytes, 0xA5, np.uint8)
+        pool, bad = dzeros(n_pages * page_bytes, 0xA5), dzeros(4)
+        rows_d, slots_d = dev(base), dev(slots)
+        for at in range(0, base.shape[0], batch):
+            n = min(batch, base.shape[0] - at)
+            assert oracle.kv_append_paged(base[at: at + n], slots[at: at + n], want, W, PT, n_pages) == 0
+            hip.launch_kv_append_paged(rows_d[at * W * 2:], slots_d[at * 4:], pool, n, W, PT, n_pages, bad)
+        got = back(pool)
+        mism = np.flatnonzero(got != want)
+        assert int(back(bad, np.uint32)[0]) == 0 and mism.size == 0, \
+            (batch, [(int(j), hex(got[j]), hex(want[j])) for j in mism[:8]])
 
 
 def test_large_batch_kernel_other_widths(oracle):
