@@ -45,6 +45,23 @@ constexpr int kGaXchBytes = 2 * kGaWaves * kWave * 8 * 4;
 constexpr int kGaSmemBytes = kGaBufs * kGaTileBytes + kGaBufs * kGaTile * 4 + kGaXchBytes;
 static_assert(kGaSmemBytes <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
 
+// Which row of a 16-row half of the LDS tile holds slot s of the half (the slot is the row index
+// of the score MFMA's A operand and the contraction index of the value MFMA). The two ways the
+// tile is read want different things of the row stride (1040 B = 65 granules of 16 B): the score
+// side's 16-byte reads go eight lanes — eight consecutive slots — at a time and need their rows
+// distinct mod 8; the transposing reads of the value side go sixteen lanes at a time, slots
+// 4g .. 4g+3 with 32 bytes each, and need those four rows two apart mod 8 or neighbouring rows
+// meet in half their banks (measured: one stalled LDS cycle for every cycle of those reads).
+// Slots 0..3 -> rows 0 2 4 6, 4..7 -> 1 3 5 7, 8..11 -> 8 10 12 14, 12..15 -> 9 11 13 15.
+__device__ __forceinline__ int row_of_slot(int s) { return 2 * (s & 7) + (s >> 3); }
+__device__ __forceinline__ int slot_of_row(int p) { return 8 * (p & 1) + (p >> 1); }
+// Staging wave w writes rows tile_pos_of(w, i) of the tile; the mask bias of such a row is kept
+// at its slot's contraction index, 8 (s >> 2) + 4 half + (s & 3).
+__device__ __forceinline__ int bias_index_of(int wave, int i) {
+    const int s = slot_of_row(4 * (wave >> 1) + i);
+    return 8 * (s >> 2) + 4 * (wave & 1) + (s & 3);
+}
+
 struct GatherAttnArgs {
     const float* q;      // [m][h][512]
     const float* kv;     // [rows][512]
@@ -141,7 +158,7 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
             if (!((r.live >> i) & 1)) v = u32x4{0u, 0u, 0u, 0u};
             *(lds_ptr<u32x4>)(krb + (my_pos0 + i) * kGaRowBytes + 16 * lane) = v;
         }
-        if (lane < 4) sbias[buf * kGaTile + 4 * wave + lane] = r.bias;
+        if (lane < 4) sbias[buf * kGaTile + bias_index_of(wave, lane)] = r.bias;
     };
 
     // ---- prologue ------------------------------------------------------------------------
@@ -157,11 +174,11 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
     {
         const int head = hb * 64 + 16 * hw + n16;
         const bool live = head < a.h;
-        const float* qa = a.q + (t * a.h + (live ? head : 0)) * kGaD + half * (kGaD / 2) + 8 * g;
+        const float* qa = a.q + (t * a.h + (live ? head : 0)) * kGaD + half * (kGaD / 2) + 128 * (g & 1) + 8 * (g >> 1);
         float4 qv[kGaKStepsHalf][2];
 #pragma unroll
         for (int j = 0; j < kGaKStepsHalf; ++j) {
-            const float4* src = reinterpret_cast<const float4*>(qa + 32 * j);
+            const float4* src = reinterpret_cast<const float4*>(qa + 16 * j);
             qv[j][0] = src[0], qv[j][1] = src[1];  // a head past h reads head 0 and is zeroed below
         }
         const int e0 = list_entry(0, f0), e1 = list_entry(1, f1);
@@ -193,28 +210,42 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
     float m_ref = -INFINITY, l_sum = 0.0f;
 
     // Scores of one staged tile: this wave's half of the dims, S^T[slot][head], two 16-slot
-    // halves. The operand fragments of a block of K-steps are all requested before the first
-    // MFMA of the block; left alone the compiler keeps two reads in flight and every pair of
-    // MFMAs then waits out a full LDS round trip.
+    // halves. The operand fragments of a block of K-steps are requested one block ahead of the
+    // MFMAs that use them: every wave of the workgroup runs the same phase at the same time, so
+    // without the lookahead LDS sits idle while the matrix cores work and the matrix cores while
+    // LDS delivers — the tile then costs the sum of the two, not the larger.
     auto scores_of = [&](int b, f32x4& s0, f32x4& s1) {
         const lds_ptr<uint8_t> krb = kr + b * kGaTileBytes + half * (kGaKStepsHalf * 64);
-        const lds_ptr<bf16x8> a0p = (lds_ptr<bf16x8>)(krb + n16 * kGaRowBytes + 16 * g);
-        const lds_ptr<bf16x8> a1p = (lds_ptr<bf16x8>)(krb + (16 + n16) * kGaRowBytes + 16 * g);
+        // K-step j, lane group g: the 8 dims at bytes 256 (g & 1) + 32 j + 16 (g >> 1) of the
+        // wave's half row (the query fragments follow the same rule). A 16-byte LDS read is
+        // served sixteen lanes at a time, and those are lanes 0-3, 12-15, 20-23, 24-27 of a
+        // 32-lane half, then the rest: eight rows from one lane group, the other eight from
+        // the next. With rows an odd number of 16-byte granules apart the sixteen meet in no
+        // bank exactly when the two lane groups read the same position mod 256 bytes.
+        const int col = 256 * (g & 1) + 16 * (g >> 1);
+        const lds_ptr<bf16x8> a0p = (lds_ptr<bf16x8>)(krb + row_of_slot(n16) * kGaRowBytes + col);
+        const lds_ptr<bf16x8> a1p = (lds_ptr<bf16x8>)(krb + (16 + row_of_slot(n16)) * kGaRowBytes + col);
         s0 = f32x4{0, 0, 0, 0}, s1 = f32x4{0, 0, 0, 0};
+        bf16x8 fa0[2][kFragBlock], fa1[2][kFragBlock];
+#pragma unroll
+        for (int i = 0; i < kFragBlock; ++i) fa0[0][i] = a0p[i * 2], fa1[0][i] = a1p[i * 2];
 #pragma unroll
         for (int j0 = 0; j0 < kGaKStepsHalf; j0 += kFragBlock) {
-            bf16x8 fa0[kFragBlock], fa1[kFragBlock];
+            const int cur = (j0 / kFragBlock) & 1;
+            if (j0 + kFragBlock < kGaKStepsHalf) {
 #pragma unroll
-            for (int i = 0; i < kFragBlock; ++i) fa0[i] = a0p[(j0 + i) * 4], fa1[i] = a1p[(j0 + i) * 4];
+                for (int i = 0; i < kFragBlock; ++i)
+                    fa0[cur ^ 1][i] = a0p[(j0 + kFragBlock + i) * 2], fa1[cur ^ 1][i] = a1p[(j0 + kFragBlock + i) * 2];
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < kFragBlock; ++i) {
                 const int j = j0 + i;
-                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[i], qh[j], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[i], qh[j], s1, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[cur][i], qh[j], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[cur][i], qh[j], s1, 0, 0, 0);
                 if (QSPLIT == 2) {
-                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[i], ql[j], s0, 0, 0, 0);
-                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[i], ql[j], s1, 0, 0, 0);
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[cur][i], ql[j], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[cur][i], ql[j], s1, 0, 0, 0);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -244,7 +275,7 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
         // transposing load hands a lane element e of the 8-byte chunk that lane
         // 4e + (n16 >> 2) of its 16-lane row addressed, position n16 & 3 — so lane i
         // addresses slot 4g + (i >> 2), columns 16*nt' + 4*(i & 3) .. +3.
-        const lds_ptr<uint8_t> vrow = kr + buf * kGaTileBytes + (4 * g + (n16 >> 2)) * kGaRowBytes +
+        const lds_ptr<uint8_t> vrow = kr + buf * kGaTileBytes + row_of_slot(4 * g + (n16 >> 2)) * kGaRowBytes +
                                       (half * (kGaD / 2) + 4 * (n16 & 3)) * 2;
         auto vt_frag = [&](int nt) -> bf16x8 {
             typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -255,10 +286,6 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
             const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             return __builtin_bit_cast(bf16x8, both);
         };
-        bf16x8 fb[kValueAhead];
-#pragma unroll
-        for (int i = 0; i < kValueAhead; ++i) fb[i] = vt_frag(i);
-        __builtin_amdgcn_sched_barrier(0);
         const f32x4 ba = *(lds_ptr<f32x4>)(sbias + buf * kGaTile + 8 * g);
         const f32x4 bb = *(lds_ptr<f32x4>)(sbias + buf * kGaTile + 8 * g + 4);
         __syncthreads();  // both halves of every score of this tile are in LDS
@@ -311,29 +338,39 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
             }
         };
         // the next tile's scores go to the matrix cores before this tile's softmax occupies
-        // the vector ALU (the two waves of a pair share a SIMD; running them in opposite order
-        // from two copies of the loop measured the same)
+        // the vector ALU (the two waves of a pair share a SIMD; running them in opposite order —
+        // one starting an iteration with the scores, the other ending it with them — measured
+        // 4 % slower)
         f32x4 ns0, ns1;
         const bool more = tile + 1 < n_tiles;
-        if (more) scores_of(buf_next, ns0, ns1);
-        softmax_tile();
-
-        // ---- values: O[head][col] += P . V over this wave's 256 columns -------------------
+        auto softmax_and_values = [&]() {
+            // the value side's first fragments come out of LDS while the softmax runs, every
+            // later block while the block before it is in the matrix cores
+            bf16x8 fb[2][kValueAhead];
 #pragma unroll
-        for (int n0 = 0; n0 < kGaColTilesHalf; n0 += kValueAhead) {
-            if (n0 > 0) {
+            for (int i = 0; i < kValueAhead; ++i) fb[0][i] = vt_frag(i);
+            __builtin_amdgcn_sched_barrier(0);
+            softmax_tile();
+            // O[head][col] += P . V over this wave's 256 columns
 #pragma unroll
-                for (int i = 0; i < kValueAhead; ++i) fb[i] = vt_frag(n0 + i);
+            for (int n0 = 0; n0 < kGaColTilesHalf; n0 += kValueAhead) {
+                const int cur = (n0 / kValueAhead) & 1;
+                if (n0 + kValueAhead < kGaColTilesHalf) {
+#pragma unroll
+                    for (int i = 0; i < kValueAhead; ++i) fb[cur ^ 1][i] = vt_frag(n0 + kValueAhead + i);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < kValueAhead; ++i) {
+                    o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p, fb[cur][i], o[n0 + i], 0, 0, 0);
+                    if (PSPLIT == 2)
+                        o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_lo, fb[cur][i], o[n0 + i], 0, 0, 0);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
-#pragma unroll
-            for (int i = 0; i < kValueAhead; ++i) {
-                o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p, fb[i], o[n0 + i], 0, 0, 0);
-                if (PSPLIT == 2)
-                    o[n0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_lo, fb[i], o[n0 + i], 0, 0, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        };
+        if (more) scores_of(buf_next, ns0, ns1);
+        softmax_and_values();
 
         if (more) {
             xch_next[0] = ns0, xch_next[1] = ns1;
