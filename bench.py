@@ -922,7 +922,7 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
            "kernels_ms": {n: round(v, 5) for n, v in per.items()},
            "roofline": {"bound": "hbm",
                         "kernel": "mla_attend_paged_kernel" if attend else
-                                  ("topk_hist + topk_cand + topk_finish (select and gather)" if fused
+                                  ("topk_hist + topk_cand + topk_finish_bits (select and gather)" if fused
                                    else "kv_gather_rows_kernel"),
                         "achieved": round(dom_bytes / (per[rows_kernel] * 1e-3) / 1e9, 2),
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
@@ -941,7 +941,8 @@ def bench_dsa(a, torch, hip, scored=False, attend=False):
         res["index_score"] = {"achieved": round(score_bytes / (per["score"] * 1e-3) / 1e9, 2),
                               "unit": "GB/s", "frac": round(score_bytes / (per["score"] * 1e-3) / HBM_PEAK, 4),
                               "avg_launch_ms": round(per["score"], 5), "bytes_per_launch": score_bytes,
-                              "tflops": round(B * nt * NH * HD * 2 * 2 / (per["score"] * 1e-3) / 1e12, 1)}
+                              "tflops": round(B * nt * NH * HD * 2 * 2 / (per["score"] * 1e-3) / 1e12, 1),
+                              "traffic": measured_traffic(f"dsa_scored:b{B}:ctx{nt}:h{NH}")}
     if attend:
         res["metric"] = "kv_dsa_topk_attend_GBps"
         res["config"]["workload"] = ("DSA sparse path with the consumer fused: top-k, then MLA latent attention "
