@@ -180,20 +180,28 @@ def brief(res):
     kernel's algorithmic bytes (or flops) per launch / its bracketed launch time / the peak;
     frac_step, where present, is the same bytes over the step time per launch (the plain pass,
     whose launches queue ahead of the device). checked: how the GPU result compared with the
-    CPU oracle ("equal", or the error it stayed within); cpu: the oracle's rate in `unit`."""
+    CPU oracle ("equal", or the error it stayed within); cpu: the oracle's rate in `unit`
+    (GB/s where no unit is given)."""
     r = res.get("roofline", {})
-    out = {"value": res["value"], "unit": res["unit"], "ms": res["ms_per_step"]}
+    out = {"value": res["value"], "ms": res["ms_per_step"]}
+    if res["unit"] != "GB/s":  # (the headline's unit is the default)
+        out["unit"] = res["unit"]
     if "layer_us" in res:
         out["layer_us"] = res["layer_us"]
-    out["kernel"] = r.get("kernel")
+    out["kernel"] = (r.get("kernel") or "").split(" (")[0]
     if r.get("bound", "hbm") != "hbm":
         out["bound"] = r["bound"]
     out["frac"] = r.get("frac")
     if "frac_step" in r:
         out["frac_step"] = r["frac_step"]
     out["launch_ms"] = r.get("avg_launch_ms")
-    out["per_launch"] = r.get("bytes_per_launch", r.get("flops_per_launch"))
-    out["traffic"] = r.get("traffic")
+    per_launch = r.get("bytes_per_launch", r.get("flops_per_launch"))
+    if per_launch is not None:
+        out["per_launch"] = int(per_launch)
+    if r.get("traffic") is not None:  # (absent: not measured for this shape)
+        out["traffic"] = r["traffic"]
+    elif "index_score" in res and res["index_score"].get("traffic") is not None:
+        out["score_traffic"] = res["index_score"]["traffic"]
     if "kernels_ms" in res:
         out["kernels_ms"] = res["kernels_ms"]
     elif "kernels" in res:
@@ -205,7 +213,9 @@ def brief(res):
     cfg = res.get("config", {})
     out["shape"] = " ".join(f"{k}={v}" for k, v in cfg.items()
                             if isinstance(v, (int, float)) and not isinstance(v, bool)
-                            and k not in ("width", "page_tokens", "head_dim", "quantized_dims", "block"))
+                            and k not in ("width", "page_tokens", "head_dim", "quantized_dims", "block",
+                                          "table_blocks", "launches_per_layer", "live_slots", "scores_computed",
+                                          "pages", "slots_per_query"))
     if "cpu_baseline" in res:
         c = res["cpu_baseline"]
         m = re.search(r"within ([0-9.e+-]+)", c["sample"])
@@ -342,7 +352,7 @@ def bench_decode(a, torch, hip):
         "data": "synthetic",
         "config": {"workload": ("cfg3 batched decode, contexts ~U[1024, ctx]" if a.ragged else
                                 "cfg3 batched decode at its metric point") +
-                               ": per layer append 1 token/seq, then gather+dequantize every context",
+                               ": per layer append 1 token/seq, gather+dequantize every context",
                    "layers": L, "batch": B, "ctx": ctx, "page_tokens": PT, "width": W,
                    "stored": "fp8 e4m3 + 1 f32 scale/token", "out": "bf16",
                    "contexts": "uniform in [1024, ctx]" if a.ragged else "all at ctx",
@@ -1169,11 +1179,11 @@ def cpu_baseline(pool0, tables_np, seq_lens_np, out, budget_s, hip, tables, seq_
         raise SystemExit("bench: GPU gather differs from the CPU oracle at full size")
     return {"value": round(bytes_layer / per_layer_s / 1e9, 3), "unit": "GB/s", "cores": cores, "nproc": nproc,
             "usable": usable, "kind": "port",
-            "sample": f"gather+dequantize of one layer ({n_tok} tokens, same pool and block "
-                      f"tables) x{reps} reps, {cores} host threads; GPU output checked equal",
+            "sample": f"one layer's gather+dequantize ({n_tok} tokens, same pool and tables) x{reps}, "
+                      f"{cores} threads; GPU output equal",
             "tokens_per_s": round(n_tok / per_layer_s, 1),
             "one_thread": {"value": round(one_bytes / one_s / 1e9, 3), "unit": "GB/s",
-                           "sample": f"the first sequence of the same layer ({int(one_len[0])} tokens), once"}}
+                           "sample": f"the layer's first sequence ({int(one_len[0])} tokens), once"}}
 
 
 if __name__ == "__main__":
