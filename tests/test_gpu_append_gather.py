@@ -122,3 +122,64 @@ def test_guards():
         with pytest.raises(hip.LaunchError) as e:
             call(**kw)
         assert e.value.code == code, kw
+
+
+def test_the_one_launch_step_replays_from_a_graph(oracle):
+    """A serving loop's use: the call captured once, replayed per token on inputs the host
+    refills in place; every replay equals append-then-gather launched eagerly."""
+    from tests.gpu_util import torch_cuda
+
+    torch = torch_cuda()
+    lens0 = [700, 64, 1500, 129]
+    n_seqs = len(lens0)
+    n_pages = n_seqs * -(-(max(lens0) + 4) // PT) + 3
+    pool_h, tables = build_pool(oracle, lens0, n_pages, seed=404)
+    blocks = tables.shape[1]
+    max_tok = sum(lens0) + 4 * n_seqs
+    pool, table_d = dev(pool_h), dev(tables)
+    new_rows = torch.zeros(n_seqs * W * 2, dtype=torch.uint8, device="cuda")
+    new_slots = torch.zeros(n_seqs * 4, dtype=torch.uint8, device="cuda")
+    seq_lens = torch.zeros(n_seqs * 4, dtype=torch.uint8, device="cuda")
+    cu = torch.zeros((n_seqs + 1) * 4, dtype=torch.uint8, device="cuda")
+    out = torch.zeros(max_tok * W * 2, dtype=torch.uint8, device="cuda")
+
+    def load_inputs(t):
+        now = np.array([n + t + 1 for n in lens0], np.int32)
+        rows = make_rows_bf16(n_seqs, W, seed=900 + t)
+        slots = np.array([slots_for(tables[s], np.array([lens0[s] + t]), PT)[0] for s in range(n_seqs)], np.int32)
+        for buf, a in ((new_rows, rows), (new_slots, slots), (seq_lens, now),
+                       (cu, np.concatenate([[0], np.cumsum(now)]).astype(np.int32))):
+            buf.copy_(dev(a))
+        return int(now.sum())
+
+    # the captured call is told the largest token count the graph will see: the flat grid is sized
+    # by it, and units past the batch's real end find no sequence and leave
+    def fused(stream):
+        hip.launch_kv_append_gather_paged(new_rows, new_slots, pool, table_d, seq_lens, cu, out, n_seqs, blocks,
+                                          max_tok, W, PT, n_pages, None, None, stream)
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        load_inputs(0)
+        pool_start = pool.clone()
+        fused(stream.cuda_stream)                                  # warm-up outside the capture
+        stream.synchronize()
+        pool.copy_(pool_start)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            fused(torch.cuda.current_stream().cuda_stream)
+        for t in range(3):
+            n_now = load_inputs(t)
+            pool_before = pool.clone()
+            out.fill_(0xEE)
+            hip.launch_kv_append_paged(new_rows, new_slots, pool, n_seqs, W, PT, n_pages, None, stream.cuda_stream)
+            hip.launch_kv_gather_paged_packed(pool, table_d, seq_lens, cu, out, n_seqs, blocks, max_tok, W, PT,
+                                              n_pages, None, stream.cuda_stream)
+            torch.cuda.synchronize()
+            want_pool, want_out = pool.clone(), out.clone()
+            pool.copy_(pool_before)
+            out.fill_(0xEE)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(pool, want_pool), t
+            assert torch.equal(out[: n_now * W * 2], want_out[: n_now * W * 2]), t
