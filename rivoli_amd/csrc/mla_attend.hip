@@ -766,7 +766,7 @@ __global__ __launch_bounds__(F8 ? kF8Threads : kAttThreads) void mla_attend_page
             return;
         }
     }
-    if constexpr (F8) attend_part_f8<QSPLIT, PSPLIT, MODE == kSparse>(a, seq, hb, r_begin, r_end, whole, pa, pml);
+    if constexpr (F8) attend_part_f8<QSPLIT, PSPLIT, MODE == kSparse, MODE == kSparse ? 64 : 128>(a, seq, hb, r_begin, r_end, whole, pa, pml);
     else attend_part<QSPLIT, PSPLIT, MODE, ANY>(a, seq, hb, r_begin, r_end, whole, pa, pml);
     if (a.n_items == 0) break;
   }  // parts of this workgroup

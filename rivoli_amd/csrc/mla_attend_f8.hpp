@@ -40,22 +40,33 @@ typedef int i32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kF8Threads = 256;              // four waves, one per SIMD, each with the full register file
 constexpr int kF8Waves = kF8Threads / kWave;
-constexpr int kF8Tile = 64;                  // tokens per tile
 constexpr int kF8Bufs = 2;
 constexpr int kF8RowBytes = 592;             // 576 codes + 16 of padding
-constexpr int kF8TileBytes = kF8Tile * kF8RowBytes;
 constexpr int kF8ZeroBytes = 64;
 constexpr int kF8Steps = 5;                  // K-steps of the scores: four of 128 latent dims, one for the rope
-constexpr int kF8RowBlocks = kF8Tile / 16;   // 4 score row blocks per tile
 constexpr int kF8ColTiles = kKvl / 16;       // 32 output column tiles per wave
 constexpr int kF8RowGranules = kF8RowBytes / 16;  // 37: 36 of codes, one of padding
-constexpr int kF8WaveRows = kF8Tile / kF8Waves;    // rows of a tile one wave brings in
-constexpr int kF8Requests = (kF8WaveRows * kF8RowGranules + kWave - 1) / kWave;
-template <int TQ>
-constexpr int f8_q_bytes() { return TQ > 2 ? (TQ - 2) * 64 * kF8RowBytes : 16; }  // q terms past the second: the block's 64 heads, rows padded like the tiles'
-constexpr int kF8SmemBytes =
-    kF8Bufs * kF8TileBytes + kF8ZeroBytes + 3 * kF8Bufs * kF8Tile * 4 + kF8Tile * 8 + kTableLds * 4;
-static_assert(kF8SmemBytes + f8_q_bytes<3>() + (1024 + 8 + 8) * 4 <= 160 * 1024, "one workgroup per CU must fit the 160 KiB of LDS");
+// What follows from the tile size. TILE = 128 (dense rows): the value contraction's K is the
+// tile's 128 tokens, one matrix instruction per weight term, and every q term lives in
+// registers. TILE = 64 (listed rows, whose calls are a tile or two long): K is the 64 tokens
+// once per weight term, the value operand repeats its 16 bytes, a third q term lives in LDS.
+template <int TILE>
+struct F8Shape {
+    static_assert(TILE == 64 || TILE == 128, "the value contraction is written for these two");
+    static constexpr int kTileBytes = TILE * kF8RowBytes;
+    static constexpr int kRowBlocks = TILE / 16;        // score row blocks per tile
+    static constexpr int kWaveRows = TILE / kF8Waves;   // rows of a tile one wave brings in
+    static constexpr int kRequests = (kWaveRows * kF8RowGranules + kWave - 1) / kWave;
+    static constexpr int kTable = TILE == 128 ? 512 : kTableLds;  // block-table entries staged in LDS
+    static constexpr int kQTermsInRegs(int tq) { return TILE == 128 ? tq : (tq > 2 ? 2 : tq); }
+    // q terms that do not live in registers: the block's 64 heads, rows padded like the tiles'
+    static constexpr int kQBytes(int tq) { return tq > kQTermsInRegs(tq) ? (tq - kQTermsInRegs(tq)) * 64 * kF8RowBytes : 16; }
+    static constexpr int kSmemBytes =
+        kF8Bufs * kTileBytes + kF8ZeroBytes + 3 * kF8Bufs * TILE * 4 + TILE * 8 + kTable * 4;
+};
+static_assert(F8Shape<64>::kSmemBytes + F8Shape<64>::kQBytes(3) + (1024 + 8 + 8) * 4 <= 160 * 1024 &&
+              F8Shape<128>::kSmemBytes + F8Shape<128>::kQBytes(3) + (1024 + 8 + 8) * 4 <= 160 * 1024,
+              "one workgroup per CU must fit the 160 KiB of LDS");
 constexpr int kWaitLds0 = 0xC07F;           // s_waitcnt lgkmcnt(0), the other counters left alone
 constexpr int kScaleOne = 0x7f7f7f7f;        // E8M0 1.0 in every byte
 
@@ -88,30 +99,33 @@ __device__ __forceinline__ void dma16(const uint8_t* src, lds_ptr<uint8_t> dst) 
                  : "memory");
 }
 
-template <int TQ, int TP, bool SPARSE>
+template <int TQ, int TP, bool SPARSE, int TILE>
 __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int hb, int r_begin, int r_end,
                                                bool whole, float* pa, float* pml) {
-    __shared__ __attribute__((aligned(16))) uint8_t smem8[kF8SmemBytes + f8_q_bytes<TQ>()];
-    const lds_ptr<uint8_t> tiles = (lds_ptr<uint8_t>)smem8;               // [2][64] rows of codes
-    const lds_ptr<uint8_t> zeros = tiles + kF8Bufs * kF8TileBytes;
-    const lds_ptr<float> sc = (lds_ptr<float>)(zeros + kF8ZeroBytes);     // [2][64] token scales (0 = not there)
-    const lds_ptr<float> sbias = sc + kF8Bufs * kF8Tile;                     // [2][64] log2 scale, or -inf
-    const lds_ptr<float> rsc = sbias + kF8Bufs * kF8Tile;                    // [2][64] 1 / scale (0 = not there)
-    const lds_ptr<unsigned long long> rowbase = (lds_ptr<unsigned long long>)(rsc + kF8Bufs * kF8Tile);  // [64] where a row's codes are
-    const lds_ptr<int> tbl = (lds_ptr<int>)(rowbase + kF8Tile);
-    const lds_ptr<uint8_t> qlds = (lds_ptr<uint8_t>)(tbl + kTableLds);  // [TQ - 2][64 heads] rows of q codes
+    using Sh = F8Shape<TILE>;
+    constexpr int kTileBytes = Sh::kTileBytes, kRowBlocks = Sh::kRowBlocks, kWaveRows = Sh::kWaveRows;
+    constexpr int kRequests = Sh::kRequests, kTable = Sh::kTable;
+    __shared__ __attribute__((aligned(16))) uint8_t smem8[Sh::kSmemBytes + Sh::kQBytes(TQ)];
+    const lds_ptr<uint8_t> tiles = (lds_ptr<uint8_t>)smem8;               // [2][TILE] rows of codes
+    const lds_ptr<uint8_t> zeros = tiles + kF8Bufs * kTileBytes;
+    const lds_ptr<float> sc = (lds_ptr<float>)(zeros + kF8ZeroBytes);     // [2][TILE] token scales (0 = not there)
+    const lds_ptr<float> sbias = sc + kF8Bufs * TILE;                        // [2][TILE] log2 scale, or -inf
+    const lds_ptr<float> rsc = sbias + kF8Bufs * TILE;                       // [2][TILE] 1 / scale (0 = not there)
+    const lds_ptr<unsigned long long> rowbase = (lds_ptr<unsigned long long>)(rsc + kF8Bufs * TILE);  // [TILE] where a row's codes are
+    const lds_ptr<int> tbl = (lds_ptr<int>)(rowbase + TILE);
+    const lds_ptr<uint8_t> qlds = (lds_ptr<uint8_t>)(tbl + kTable);  // [TQ - TQR][64 heads] rows of q codes
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // = which 16 heads of the block
     const int g = lane >> 4, n16 = lane & 15;
-    const int n_tiles = (r_end - r_begin + kF8Tile - 1) / kF8Tile;
+    const int n_tiles = (r_end - r_begin + TILE - 1) / TILE;
 
     // ---- block-table slice, zero area -------------------------------------------------------
     const int* const table_g = a.block_table + (size_t)seq * a.max_blocks;
     const int tbl_first = SPARSE ? 0 : r_begin / a.page_tokens;
     const int tbl_last = SPARSE ? a.max_blocks - 1 : min(a.max_blocks - 1, (r_end - 1) / a.page_tokens);
-    const int tbl_count = min(kTableLds, tbl_last - tbl_first + 1);
+    const int tbl_count = min(kTable, tbl_last - tbl_first + 1);
     for (int i = tid; i < tbl_count; i += kF8Threads) tbl[i] = table_g[tbl_first + i];
     if (tid < kF8ZeroBytes / 4) ((lds_ptr<int>)zeros)[tid] = 0;
 
@@ -124,8 +138,8 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     // from lane group k: term 0 sits in blocks 0 and 2, term 1 in blocks 1 and 3, hence a scale
     // register that alternates between the two terms' scales by lane group (qscale_rope). A
     // third term keeps the half-empty form (zeros in lane groups 2 and 3).
-    constexpr int TQR = TQ > 2 ? 2 : TQ;  // terms in (accumulation) registers; a third one lives in LDS
-    static_assert(TQR == 2, "the rope step pairs the first two terms");
+    constexpr int TQR = Sh::kQTermsInRegs(TQ);  // terms in (accumulation) registers; one past them lives in LDS
+    static_assert(TQR >= 2, "the rope step pairs the first two terms");
     i32x8 qt[TQR][kF8Steps];  // qt[1][4] is not used
     int qscale_lo[TQ], qscale_hi[TQ];  // E8M0 scales: bytes 0..3 = steps 0..3, byte 0 of _hi = step 4
     int qscale_rope = kScaleOne;
@@ -174,10 +188,11 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
                     uint32_t w4 = e4m3x4_and_residual(y);
                     if (s == 4 && t == 0) first_term[c] = w4;
                     if (s == 4 && t == 1) w4 = g < 2 ? first_term[c] : w4;
+                    if (s == 4 && t >= 2 && t < TQR) w4 = g < 2 ? w4 : 0u;  // half-empty: zeros in lane groups 2 and 3
                     if (t < TQR && !(s == 4 && t == 0)) {
                         int qa;
                         asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(qa) : "v"(w4));
-                        qt[s == 4 ? 0 : t][s][c] = qa;
+                        qt[s == 4 && t == 1 ? 0 : t][s][c] = qa;
                     } else if (t >= TQR && (s < 4 || g < 2))
                         *(lds_ptr<uint32_t>)(qlds + ((t - TQR) * 64 + 16 * wave + n16) * kF8RowBytes + 128 * s + 32 * g + 4 * c) = w4;
                     // what is left over, at the next term's scale (16 times finer)
@@ -198,13 +213,13 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         return (rel >= 0 && rel < tbl_count) ? tbl[rel] : table_g[blk];
     };
 
-    // ---- where the wave's 16 rows of a tile are: lanes 0..15 resolve one each ------------------
+    // ---- where the wave's rows of a tile are: lanes 0..kWaveRows-1 resolve one each -------------
     constexpr unsigned long long kNone = ~0ull;
     const unsigned int* const rows_g = SPARSE ? a.rows + (size_t)seq * a.k : nullptr;
     auto resolve = [&](int t, unsigned long long& code_off, unsigned long long& scale_off) {
         code_off = kNone, scale_off = 0;
-        const int pos = r_begin + t * kF8Tile + kF8WaveRows * wave + lane;
-        if (lane >= kF8WaveRows || t >= n_tiles || pos >= r_end) return;
+        const int pos = r_begin + t * TILE + kWaveRows * wave + lane;
+        if (lane >= kWaveRows || t >= n_tiles || pos >= r_end) return;
         const unsigned int tok = SPARSE ? rows_g[pos] : (unsigned)pos;
         unsigned int blk, off;
         if (a.page_shift >= 0) blk = tok >> a.page_shift, off = tok & (unsigned)(a.page_tokens - 1);
@@ -219,39 +234,39 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         }
     };
     // A tile goes from memory straight into LDS (16 bytes per lane, a wave's 64 lanes filling
-    // 1 KiB of consecutive LDS). The wave's 16 rows of 37 granules (36 of codes + the padding one)
+    // 1 KiB of consecutive LDS). The wave's rows of 37 granules (36 of codes + the padding one)
     // are that consecutive range, so lane L of request I fills granule 64 I + L = row
     // (64 I + L) / 37, granule (64 I + L) % 37 of the row, from wherever that row's page is. A row
     // that is not there is zero-filled by hand: its codes must be finite, they meet a zero weight
     // and a -inf bias, never a NaN.
-    float next_scale = 0.0f;  // lanes 0..15: the scale of the row this lane resolved
-    // Dense fast path: the wave's 16 rows of a tile are 16 consecutive rows of one page (tiles
-    // start on multiples of 32 tokens and the page holds a multiple of 16), so granule 64 i +
-    // lane comes from byte goff[i] past the first of them: no lookups, one request per 1 KiB.
-    int goff[kF8Requests];
+    float next_scale = 0.0f;  // lanes 0..kWaveRows-1: the scale of the row this lane resolved
+    // Dense fast path: the wave's rows of a tile are consecutive rows of one page (tiles start
+    // on multiples of 32 tokens and the page holds a multiple of the wave's share), so granule
+    // 64 i + lane comes from byte goff[i] past the first of them: no lookups, one request per 1 KiB.
+    int goff[kRequests];
 #pragma unroll
-    for (int i = 0; i < kF8Requests; ++i) {
-        const int gi = min(kWave * i + lane, kF8WaveRows * kF8RowGranules - 1);
+    for (int i = 0; i < kRequests; ++i) {
+        const int gi = min(kWave * i + lane, kWaveRows * kF8RowGranules - 1);
         const int row = gi / kF8RowGranules, c = min(gi - row * kF8RowGranules, kRowW / 16 - 1);
         goff[i] = row * kRowW + 16 * c;  // (the padding granule repeats the one before it)
     }
-    const bool pages_hold_runs = !SPARSE && a.page_shift >= 4;
+    const bool pages_hold_runs = !SPARSE && a.page_shift >= (TILE == 128 ? 5 : 4);
     auto request_tile = [&](int t, lds_ptr<uint8_t> dst_tile) {
-        const lds_ptr<uint8_t> dst_w = dst_tile + (kF8WaveRows * wave) * kF8RowBytes;
+        const lds_ptr<uint8_t> dst_w = dst_tile + (kWaveRows * wave) * kF8RowBytes;
         if (pages_hold_runs) {
-            const int pos0 = r_begin + t * kF8Tile + kF8WaveRows * wave;
-            if (pos0 + kF8WaveRows <= r_end) {
+            const int pos0 = r_begin + t * TILE + kWaveRows * wave;
+            if (pos0 + kWaveRows <= r_end) {
                 const int blk = pos0 >> a.page_shift, off = pos0 & (a.page_tokens - 1);
                 const int page = blk < a.max_blocks ? __builtin_amdgcn_readfirstlane(table_at(blk)) : -1;
                 if ((unsigned)page < (unsigned)a.n_pages) {
                     const uint8_t* const pg = a.pool + (size_t)page * a.page_bytes;
                     const uint8_t* const src = pg + (size_t)off * kRowW;
                     next_scale = 0.0f;
-                    if (lane < kF8WaveRows)
+                    if (lane < kWaveRows)
                         next_scale = reinterpret_cast<const float*>(pg + (size_t)a.page_tokens * kRowW)[off + lane];
 #pragma unroll
-                    for (int i = 0; i < kF8Requests; ++i)
-                        if (kWave * (i + 1) <= kF8WaveRows * kF8RowGranules || lane < kF8WaveRows * kF8RowGranules - kWave * i)
+                    for (int i = 0; i < kRequests; ++i)
+                        if (kWave * (i + 1) <= kWaveRows * kF8RowGranules || lane < kWaveRows * kF8RowGranules - kWave * i)
                             dma16(src + goff[i], dst_w + 1024 * i);
                     return;
                 }
@@ -259,20 +274,20 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         }
         unsigned long long code_off, scale_off;
         resolve(t, code_off, scale_off);
-        if (lane < kF8WaveRows) rowbase[kF8WaveRows * wave + lane] = code_off;
+        if (lane < kWaveRows) rowbase[kWaveRows * wave + lane] = code_off;
         next_scale = 0.0f;
         if (code_off != kNone) next_scale = *reinterpret_cast<const float*>(a.pool + scale_off);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
         const lds_ptr<uint8_t> dst0 = dst_w;
 #pragma unroll
-        for (int i = 0; i < kF8Requests; ++i) {
+        for (int i = 0; i < kRequests; ++i) {
             int ln = lane;
             asm volatile("" : "+v"(ln));  // (kept out of the registers that live across the tile loop)
             const int gi = kWave * i + ln;
             const int row = gi / kF8RowGranules, c = gi - row * kF8RowGranules;
-            if (row < kF8WaveRows && c < kRowW / 16) {
-                const unsigned long long base = rowbase[kF8WaveRows * wave + row];
+            if (row < kWaveRows && c < kRowW / 16) {
+                const unsigned long long base = rowbase[kWaveRows * wave + row];
                 if (base != kNone) {
                     dma16(a.pool + base + 16 * c, dst0 + 1024 * i);
                 } else {
@@ -282,15 +297,15 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         }
     };
     auto publish_scales = [&](int buf) {  // the scales of the tile request_tile last asked for
-        if (lane < kF8WaveRows) {
+        if (lane < kWaveRows) {
             const bool ok = next_scale > 0.0f;  // a token that is not there has scale 0
-            sc[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? next_scale : 0.0f;
+            sc[buf * TILE + kWaveRows * wave + lane] = ok ? next_scale : 0.0f;
             // the bias added to a token's scores: log2 of its scale (its weights then carry the
             // scale the value contraction needs), -inf for a token that is not there
-            sbias[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? __builtin_amdgcn_logf(next_scale) : -INFINITY;
+            sbias[buf * TILE + kWaveRows * wave + lane] = ok ? __builtin_amdgcn_logf(next_scale) : -INFINITY;
             // the denominator divides every held weight by its token's scale: the reciprocal is
             // taken once per token here, not once per (token, head) in the softmax
-            rsc[buf * kF8Tile + kF8WaveRows * wave + lane] = ok ? __builtin_amdgcn_rcpf(next_scale) : 0.0f;
+            rsc[buf * TILE + kWaveRows * wave + lane] = ok ? __builtin_amdgcn_rcpf(next_scale) : 0.0f;
         }
     };
 
@@ -301,14 +316,15 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     const int a_rope = n16 * kF8RowBytes + kKvl + 32 * (g & 1);  // both pairs of lane groups read the rope
     const bool rope_zero = g >= 2;  // a third q term's rope fragment
     const int q_row = (16 * wave + n16) * kF8RowBytes + 32 * g;
-    // values: transposing load r (of 4) hands this lane bytes 8 r .. 8 r + 7 of its operand = the
+    // values: transposing load r hands this lane bytes 8 r .. 8 r + 7 of its operand = the
     // tokens 16 (2 r + e / 4) + 4 g + e % 4, e = 0..7, of column 16 nt + n16; source lane pair e
     // addresses token e's row, its two lanes the two 8-byte halves of the 16 columns.
-    int v_off[2];
+    constexpr int kReads = TILE / 32;  // transposing loads per column tile: 16 tokens each... 8 bytes a lane
+    int v_off[kReads];
     {
         const int e = n16 >> 1;
 #pragma unroll
-        for (int r = 0; r < 2; ++r)
+        for (int r = 0; r < kReads; ++r)
             v_off[r] = (16 * (2 * r + (e >> 2)) + 4 * g + (e & 3)) * kF8RowBytes + 8 * (n16 & 1);
     }
 
@@ -325,29 +341,31 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
 
     for (int t = 0; t < n_tiles; ++t) {
         const int buf = t & 1;
-        const lds_ptr<uint8_t> tile = tiles + buf * kF8TileBytes, next = tiles + (buf ^ 1) * kF8TileBytes;
-        const lds_ptr<float> sc_t = sc + buf * kF8Tile, sbias_t = sbias + buf * kF8Tile, rsc_t = rsc + buf * kF8Tile;
+        const lds_ptr<uint8_t> tile = tiles + buf * kTileBytes, next = tiles + (buf ^ 1) * kTileBytes;
+        const lds_ptr<float> sc_t = sc + buf * TILE, sbias_t = sbias + buf * TILE, rsc_t = rsc + buf * TILE;
 
         // ---- scores: S^T[token][head] over the five K-steps ---------------------------------
-        // A K-step's four operand fragments are requested while the matrix instructions of the
-        // step before run; the scheduling fences keep that order.
-        f32x4 acc[kF8RowBlocks];
+        // A unit's operand fragments are requested while the matrix instructions of the unit
+        // before run; the scheduling fences keep that order.
+        f32x4 acc[kRowBlocks];
 #pragma unroll
-        for (int mb = 0; mb < kF8RowBlocks; ++mb) acc[mb] = f32x4{0, 0, 0, 0};
+        for (int mb = 0; mb < kRowBlocks; ++mb) acc[mb] = f32x4{0, 0, 0, 0};
         i32x8 af[2][2], qf[2][TQ > TQR ? TQ - TQR : 1];
-        f32x4 s4[kF8RowBlocks], r4[kF8RowBlocks], b4[kF8RowBlocks];  // token scales, their reciprocals, biases
+        f32x4 s4[kRowBlocks], r4[kRowBlocks], b4[kRowBlocks];  // token scales, their reciprocals, biases
         auto read32 = [&](lds_ptr<uint8_t> src) -> i32x8 {
             const u32x4 lo4 = *(lds_ptr<u32x4>)(src), hi4 = *(lds_ptr<u32x4>)(src + 16);
             return i32x8{(int)lo4.x, (int)lo4.y, (int)lo4.z, (int)lo4.w, (int)hi4.x, (int)hi4.y, (int)hi4.z, (int)hi4.w};
         };
-        // unit u: K-step u / 2, row blocks 2 (u & 1) + {0, 1}; a step's q fragments come with its first unit
+        // unit u: K-step u / UPS, row blocks 2 (u % UPS) + {0, 1}; a step's q fragments (those
+        // that live in LDS) come with its first unit
+        constexpr int UPS = kRowBlocks / 2, kUnits = UPS * kF8Steps;
         auto load_unit = [&](int u) {
-            const int s = u >> 1;
+            const int s = u / UPS;
             const bool z = s == 4 && rope_zero;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                af[u & 1][j] = read32(tile + (2 * (u & 1) + j) * 16 * kF8RowBytes + (s == 4 ? a_rope : a_row + 128 * s));
-            if ((u & 1) == 0) {
+                af[u & 1][j] = read32(tile + (2 * (u % UPS) + j) * 16 * kF8RowBytes + (s == 4 ? a_rope : a_row + 128 * s));
+            if ((u % UPS) == 0) {
 #pragma unroll
                 for (int tq = 0; tq < TQ - TQR; ++tq)
                     qf[s & 1][tq] = read32(z ? zeros : qlds + tq * 64 * kF8RowBytes + q_row + 128 * s);
@@ -360,29 +378,29 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         // its requests runs while the first fragments above come out of LDS
         if (t + 1 < n_tiles) request_tile(t + 1, next);
 #pragma unroll
-        for (int u = 0; u < 2 * kF8Steps; ++u) {
+        for (int u = 0; u < kUnits; ++u) {
             __builtin_amdgcn_s_waitcnt(kWaitLds0);  // this unit's fragments are in
             __builtin_amdgcn_sched_barrier(0);
-            if (u + 1 < 2 * kF8Steps) {
+            if (u + 1 < kUnits) {
                 load_unit(u + 1);
             } else {
                 // under the last unit's matrix instructions: what the softmax reads first
 #pragma unroll
-                for (int mb = 0; mb < kF8RowBlocks; ++mb) {
+                for (int mb = 0; mb < kRowBlocks; ++mb) {
                     s4[mb] = *(lds_ptr<f32x4>)(sc_t + 16 * mb + 4 * g);
-                    r4[mb] = *(lds_ptr<f32x4>)(rsc_t + 16 * mb + 4 * g);
                     b4[mb] = *(lds_ptr<f32x4>)(sbias_t + 16 * mb + 4 * g);
+                    if (TILE == 64) r4[mb] = *(lds_ptr<f32x4>)(rsc_t + 16 * mb + 4 * g);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
-            const int s = u >> 1;
+            const int s = u / UPS;
 #pragma unroll
             for (int tq = 0; tq < TQ; ++tq)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     if (s == 4 && tq == 1) continue;  // the rope's second term rode with the first
                     const i32x8 fa = af[u & 1][j], fq = tq < TQR ? qt[tq < TQR ? tq : 0][s] : qf[s & 1][tq < TQR ? 0 : tq - TQR];
-                    const int mb = 2 * (u & 1) + j;
+                    const int mb = 2 * (u % UPS) + j;
                     if (s == 0)
                         acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa, fq, acc[mb], 0, 0, 0, kScaleOne, 0, qscale_lo[tq]);
                     else if (s == 1)
@@ -400,28 +418,35 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         // the value contraction's first operands are requested now: they do not depend on the
         // softmax, whose arithmetic then hides their way out of LDS
         static_assert(TP == 2, "two terms fill the value contraction's K exactly");
-        constexpr int CU = 8;  // column tiles per unit
+        constexpr int CU = TILE == 128 ? 4 : 8;  // column tiles per unit (eight matrix instructions)
         i32x8 vf[2][CU];
         auto load_cols = [&](int n0, i32x8 (&f)[CU]) {
 #pragma unroll
             for (int j = 0; j < CU; ++j) {
-                const i32x2 r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr<i32x2>)(tile + v_off[0] + 16 * (n0 + j)));
-                const i32x2 r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr<i32x2>)(tile + v_off[1] + 16 * (n0 + j)));
-                f[j] = i32x8{r0[0], r0[1], r1[0], r1[1], r0[0], r0[1], r1[0], r1[1]};
+                i32x2 r[kReads];
+#pragma unroll
+                for (int k = 0; k < kReads; ++k)
+                    r[k] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr<i32x2>)(tile + v_off[k] + 16 * (n0 + j)));
+                if constexpr (TILE == 128) f[j] = i32x8{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]};
+                else f[j] = i32x8{r[0][0], r[0][1], r[1][0], r[1][1], r[0][0], r[0][1], r[1][0], r[1][1]};
             }
         };
         load_cols(0, vf[0]);
         __builtin_amdgcn_sched_barrier(0);
 
-        // ---- online softmax over the lane's 16 tokens of head n16: tokens 16 mb + 4 g + i ----
+        // ---- online softmax over the lane's tokens of head n16: tokens 16 mb + 4 g + i ---------
         float tmax = -INFINITY;
 #pragma unroll
-        for (int mb = 0; mb < kF8RowBlocks; ++mb) {
+        for (int mb = 0; mb < kRowBlocks; ++mb) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 acc[mb][i] = __builtin_fmaf(acc[mb][i], s4[mb][i], b4[mb][i]);  // -inf where the token is not there
                 tmax = fmaxf(tmax, acc[mb][i]);
             }
+        }
+        if constexpr (TILE == 128) {  // (asked for here: the registers of the scales above are free again)
+#pragma unroll
+            for (int mb = 0; mb < kRowBlocks; ++mb) r4[mb] = *(lds_ptr<f32x4>)(rsc_t + 16 * mb + 4 * g);
         }
         tmax = rows_max(tmax);
         const bool grow = tmax > m_ref + kLazyRescale;  // false while everything is masked
@@ -440,25 +465,33 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         const float mu = m_ref == -INFINITY ? 0.0f : m_ref;
         // weights w_t = 2^(v_t - mu) * s_t = 2^(v'_t - mu) with v' = v + log2 s_t (the published
         // bias carries log2 s_t, so the token scale costs nothing here), as TP e4m3 terms under
-        // one scale 2^pe per (head, tile). The largest weight of the head's 64 tokens is
+        // one scale 2^pe per (head, tile). The largest weight of the head's tokens is
         // 2^(tmax - mu), exp2 being monotonic: no second maximum is taken. The terms are cut from
         // y = w / 2^pe, computed as one exponential.
         const int pe = block_exp(__builtin_amdgcn_exp2f(tmax - mu));
         const float shift = mu + (float)pe, unit = pow2i(pe);
-        i32x8 pt;  // bytes 0..15: the first term of the lane's 16 tokens, 16..31: the second
-        // (the instruction takes K block b's scale from lane 16 b + row: blocks 0, 1 are the
-        // first term of lane groups 0,1 / 2,3, blocks 2, 3 the second term, 16 times finer)
-        const int pscale = (int)((uint32_t)max(pe - 4 * (g >> 1) + 127, 1) * 0x01010101u);
+        // TILE = 64: one operand, bytes 0..15 the first term of the lane's 16 tokens, 16..31 the
+        // second (the instruction takes K block b's scale from lane 16 b + row: blocks 0, 1 are
+        // the first term of lane groups 0,1 / 2,3, blocks 2, 3 the second term, 16 times finer).
+        // TILE = 128: an operand per term, byte b the token 16 (b / 4) + 4 g + b % 4.
+        constexpr int kOperands = TILE == 128 ? TP : 1;
+        i32x8 pt[kOperands];
+        int pscale[kOperands];
+#pragma unroll
+        for (int k = 0; k < kOperands; ++k)
+            pscale[k] = (int)((uint32_t)max(pe - 4 * (TILE == 128 ? k : (g >> 1)) + 127, 1) * 0x01010101u);
         float l_tile = 0.0f;  // in units of 2^pe
 #pragma unroll
-        for (int mb = 0; mb < kF8RowBlocks; ++mb) {
+        for (int mb = 0; mb < kRowBlocks; ++mb) {
             float y[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) y[i] = acc[mb][i] = __builtin_amdgcn_exp2f(acc[mb][i] - shift);  // not there -> 0
-            pt[mb] = (int)e4m3x4_and_residual(y);
+            const int first = (int)e4m3x4_and_residual(y);
 #pragma unroll
             for (int i = 0; i < 4; ++i) y[i] *= 16.0f;
-            pt[4 + mb] = (int)e4m3x4_and_residual(y);
+            const int second = (int)e4m3x4_and_residual(y);
+            if constexpr (TILE == 128) pt[0][mb] = first, pt[1][mb] = second;
+            else pt[0][mb] = first, pt[0][4 + mb] = second;
             // The denominator sums the weights the numerator really holds (w_t less the last
             // residual), over the token scale: the result is an exactly normalised average under
             // weights perturbed by 2^-8 each.
@@ -480,7 +513,16 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < CU; ++j)
-                o[n0 + j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pt, vf[(n0 / CU) & 1][j], o[n0 + j], 0, 0, 0, pscale, 0, kScaleOne);
+#pragma unroll
+                for (int k = 0; k < kOperands; ++k)
+                    o[n0 + j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pt[k], vf[(n0 / CU) & 1][j], o[n0 + j], 0, 0, 0, pscale[k], 0, kScaleOne);
+            // TILE = 128: the products stay here, under the next unit's operands on their way out
+            // of LDS. Left free, the compiler sinks them all below the end of the tile (nothing
+            // reads the sums before the next tile) and has to hold every unit's operands at once.
+            if constexpr (TILE == 128) {
+#pragma unroll
+                for (int j = 0; j < CU; ++j) asm volatile("" : "+v"(o[n0 + j]));
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
 
