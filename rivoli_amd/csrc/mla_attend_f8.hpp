@@ -99,6 +99,22 @@ __device__ __forceinline__ void dma16(const uint8_t* src, lds_ptr<uint8_t> dst) 
                  : "memory");
 }
 
+// The same from a wave-uniform address plus a 32-bit offset per lane (the instruction's scalar
+// base form: no 64-bit add, and offsets kept across a loop cost one register each). The base is
+// made scalar here: an operand that reaches the statement through a loop-carried value may
+// otherwise sit in vector registers, which the assembler accepts and the instruction misreads.
+__device__ __forceinline__ void dma16_from(const uint8_t* base_uniform, uint32_t off, lds_ptr<uint8_t> dst) {
+    const uint32_t lds_base = (uint32_t)(uintptr_t)dst;
+    const uint64_t b = (uint64_t)(uintptr_t)base_uniform;
+    const uint64_t sb = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(b >> 32)) << 32) |
+                        (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    uint32_t keep;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b32 m0, %0"
+                 : "=&s"(keep)
+                 : "v"(off), "s"(sb), "s"(lds_base)
+                 : "memory");
+}
+
 template <int TQ, int TP, bool SPARSE, int TILE>
 __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int hb, int r_begin, int r_end,
                                                bool whole, float* pa, float* pml) {
@@ -251,7 +267,17 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         goff[i] = row * kRowW + 16 * c;  // (the padding granule repeats the one before it)
     }
     const bool pages_hold_runs = !SPARSE && a.page_shift >= (TILE == 128 ? 5 : 4);
-    auto request_tile = [&](int t, lds_ptr<uint8_t> dst_tile) {
+    // Request i of such a run, from `run` (the first of the wave's rows in its page).
+    auto request_of_run = [&](const uint8_t* run, lds_ptr<uint8_t> dst_tile, int i) {
+        if (kWave * (i + 1) <= kWaveRows * kF8RowGranules || lane < kWaveRows * kF8RowGranules - kWave * i)
+            dma16_from(run, (uint32_t)goff[i], dst_tile + (kWaveRows * wave) * kF8RowBytes + 1024 * i);
+    };
+    // Tile t on its way into dst_tile. Returns the run's address when the tile is one (then
+    // `spread` leaves the requests to the caller, who issues them one at a time between other
+    // work: more than about forty transfers in flight per compute unit and each further
+    // request holds its wave until one of them has landed), nullptr when everything was
+    // requested here.
+    auto request_tile = [&](int t, lds_ptr<uint8_t> dst_tile, bool spread) -> const uint8_t* {
         const lds_ptr<uint8_t> dst_w = dst_tile + (kWaveRows * wave) * kF8RowBytes;
         if (pages_hold_runs) {
             const int pos0 = r_begin + t * TILE + kWaveRows * wave;
@@ -264,11 +290,10 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
                     next_scale = 0.0f;
                     if (lane < kWaveRows)
                         next_scale = reinterpret_cast<const float*>(pg + (size_t)a.page_tokens * kRowW)[off + lane];
+                    if (spread) return src;
 #pragma unroll
-                    for (int i = 0; i < kRequests; ++i)
-                        if (kWave * (i + 1) <= kWaveRows * kF8RowGranules || lane < kWaveRows * kF8RowGranules - kWave * i)
-                            dma16(src + goff[i], dst_w + 1024 * i);
-                    return;
+                    for (int i = 0; i < kRequests; ++i) request_of_run(src, dst_tile, i);
+                    return nullptr;
                 }
             }
         }
@@ -295,6 +320,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
                 }
             }
         }
+        return nullptr;
     };
     auto publish_scales = [&](int buf) {  // the scales of the tile request_tile last asked for
         if (lane < kWaveRows) {
@@ -334,7 +360,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     float m_ref = -INFINITY, l_sum = 0.0f;
 
     // prologue: tile 0 into LDS
-    request_tile(0, tiles);
+    request_tile(0, tiles, false);
     publish_scales(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -376,7 +402,9 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         // tile t + 1 starts on its way into the other buffer (which held tile t - 1: every wave
         // left it before the barrier that ended the previous iteration); the address arithmetic of
         // its requests runs while the first fragments above come out of LDS
-        if (t + 1 < n_tiles) request_tile(t + 1, next);
+        constexpr int kPerUnit = 2;  // requests behind each of the first units
+        static_assert(kUnits * kPerUnit >= kRequests, "the units take every request");
+        const uint8_t* const run = t + 1 < n_tiles ? request_tile(t + 1, next, true) : nullptr;
 #pragma unroll
         for (int u = 0; u < kUnits; ++u) {
             __builtin_amdgcn_s_waitcnt(kWaitLds0);  // this unit's fragments are in
@@ -412,6 +440,16 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
                     else
                         acc[mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa, fq, acc[mb], 0, 0, 0, kScaleOne, 0, tq == 0 ? qscale_rope : qscale_hi[tq]);
                 }
+            if (kPerUnit * u < kRequests) {
+                // (the sums are used here so that the unit's matrix instructions stay in front
+                // of the branch: the compiler would sink them past it)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(acc[2 * (u % UPS) + j]));
+                if (run) {
+#pragma unroll
+                    for (int i = kPerUnit * u; i < kPerUnit * (u + 1) && i < kRequests; ++i) request_of_run(run, next, i);
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
 
