@@ -12,19 +12,22 @@
 //
 // Mapping: a 256-thread workgroup — one wave per SIMD, each with the whole register file — owns
 // 64 heads and a run of rows; wave w owns heads 16 w .. +15 and all 512 output columns (128
-// accumulators). Two q terms live in the accumulation half of the register file, which the
-// matrix instructions read directly (a third, when there is one, in LDS). Tiles are 64 tokens,
-// two buffers of raw code rows in LDS. Per tile a wave
-//   requests the next tile into the other buffer;
-//   scores: S^T[token][head] = rows x q, 4 row blocks x 5 K-steps (128 dims; the rope's 64 fill
-//     half a step) x TQ terms, A = 32 contiguous bytes of a row per lane;
+// accumulators). The q terms live in the accumulation half of the register file, which the
+// matrix instructions read directly. Two buffers of raw code rows in LDS; tiles are 128 tokens
+// for dense rows, 64 for listed rows (whose calls are a tile or two long; there a third q term
+// lives in LDS). Per tile a wave
+//   requests the next tile into the other buffer (dense rows: two requests behind each of the
+//     first score units; else all of them first);
+//   scores: S^T[token][head] = rows x q, row blocks of 16 tokens x 5 K-steps (128 dims; the
+//     rope's 64 fill half a step) x TQ terms, A = 32 contiguous bytes of a row per lane;
 //   online softmax in base 2 with a lazily moved reference, the weights to two e4m3 terms in
-//     registers: a lane's 16 weights per term are exactly its share of the next operand;
-//   values: O[head][col] += P V. The contraction's K is 128 = the tile's 64 tokens once per
-//     term: bytes 0..15 of a lane's weight operand hold the first term of its 16 tokens, bytes
-//     16..31 the second (the instruction takes K block b's scale from lane 16 b + row, so lane
-//     groups 2 and 3 carry the finer scale), and the value operand — the same tile, read through
-//     the transposing byte load (ds_read_b64_tr_b8) — repeats its 16 bytes;
+//     registers: a lane's weights per term are exactly its share of the next operand;
+//   values: O[head][col] += P V on the same tile, read through the transposing byte load
+//     (ds_read_b64_tr_b8). 128-token tiles: the contraction's K = 128 is the tile's tokens, one
+//     matrix instruction per weight term. 64-token tiles: K is the 64 tokens once per term —
+//     bytes 0..15 of a lane's weight operand hold the first term of its 16 tokens, bytes 16..31
+//     the second (the instruction takes K block b's scale from lane 16 b + row, so lane groups
+//     2 and 3 carry the finer scale) and the value operand repeats its 16 bytes;
 //   waits for its part of the next tile and meets the other waves at the one barrier of the step.
 // Operand fragments are requested one unit ahead of the matrix instructions that use them.
 // The file must be compiled with -mllvm -amdgpu-mfma-vgpr-form (the build does): the kernel's
