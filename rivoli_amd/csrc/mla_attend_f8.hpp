@@ -65,7 +65,7 @@ struct F8Shape {
     // q terms that do not live in registers: the block's 64 heads, rows padded like the tiles'
     static constexpr int kQBytes(int tq) { return tq > kQTermsInRegs(tq) ? (tq - kQTermsInRegs(tq)) * 64 * kF8RowBytes : 16; }
     static constexpr int kSmemBytes =
-        kF8Bufs * kTileBytes + kF8ZeroBytes + 3 * kF8Bufs * TILE * 4 + TILE * 8 + kTable * 4;
+        kF8Bufs * kTileBytes + kF8ZeroBytes + 3 * kF8Bufs * TILE * 4 + kTable * 4;
 };
 static_assert(F8Shape<64>::kSmemBytes + F8Shape<64>::kQBytes(3) + (1024 + 8 + 8) * 4 <= 160 * 1024 &&
               F8Shape<128>::kSmemBytes + F8Shape<128>::kQBytes(3) + (1024 + 8 + 8) * 4 <= 160 * 1024,
@@ -130,8 +130,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     const lds_ptr<float> sc = (lds_ptr<float>)(zeros + kF8ZeroBytes);     // [2][TILE] token scales (0 = not there)
     const lds_ptr<float> sbias = sc + kF8Bufs * TILE;                        // [2][TILE] log2 scale, or -inf
     const lds_ptr<float> rsc = sbias + kF8Bufs * TILE;                       // [2][TILE] 1 / scale (0 = not there)
-    const lds_ptr<unsigned long long> rowbase = (lds_ptr<unsigned long long>)(rsc + kF8Bufs * TILE);  // [TILE] where a row's codes are
-    const lds_ptr<int> tbl = (lds_ptr<int>)(rowbase + TILE);
+    const lds_ptr<int> tbl = (lds_ptr<int>)(rsc + kF8Bufs * TILE);
     const lds_ptr<uint8_t> qlds = (lds_ptr<uint8_t>)(tbl + kTable);  // [TQ - TQR][64 heads] rows of q codes
 
     const int tid = threadIdx.x;
@@ -139,6 +138,17 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // = which 16 heads of the block
     const int g = lane >> 4, n16 = lane & 15;
     const int n_tiles = (r_end - r_begin + TILE - 1) / TILE;
+
+    // ---- listed rows: a tile's list entries are asked for a tile ahead (the first two tiles'
+    // here, in front of everything), so that their way from memory is not waited for in front of
+    // the tile's requests. Lanes 0..kWaveRows-1 hold one entry each; the address always exists.
+    const unsigned int* const rows_g = SPARSE ? a.rows + (size_t)seq * a.k : nullptr;
+    auto list_entry = [&](int t) -> unsigned int {
+        if constexpr (!SPARSE) return 0u;
+        const int pos = r_begin + t * TILE + kWaveRows * wave + (lane & (kWaveRows - 1));
+        return rows_g[min(pos, r_end - 1)];
+    };
+    unsigned int entry_now = list_entry(0), entry_next = list_entry(1);
 
     // ---- block-table slice, zero area -------------------------------------------------------
     const int* const table_g = a.block_table + (size_t)seq * a.max_blocks;
@@ -181,21 +191,22 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         }
 #pragma unroll
         for (int s = 0; s < kF8Steps; ++s) {
+            // x = q * qscale / 2^e in one multiply per value (2^e is exact, so the product rounds
+            // as the two multiplies would); a head past H keeps its loaded values times zero
+            // (the rope step: lane groups 2, 3 hold what 0, 1 hold)
             float x[32];
-            const bool there = live;  // (the rope step: lane groups 2, 3 hold what 0, 1 hold)
-            const float keep = there ? a.qscale : 0.0f;
+            const float keep = live ? a.qscale : 0.0f;
+            float amax = 0.0f;
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
                 const float4 v = raw[s][c];
-                x[4 * c] = there ? v.x * keep : 0.0f, x[4 * c + 1] = there ? v.y * keep : 0.0f;
-                x[4 * c + 2] = there ? v.z * keep : 0.0f, x[4 * c + 3] = there ? v.w * keep : 0.0f;
+                x[4 * c] = v.x, x[4 * c + 1] = v.y, x[4 * c + 2] = v.z, x[4 * c + 3] = v.w;
             }
-            float amax = 0.0f;
 #pragma unroll
             for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(x[i]));
-            amax = rows_max(amax);  // over the head's four lanes: one scale per (head, step)
+            amax = rows_max(amax * keep);  // over the head's four lanes: one scale per (head, step)
             const int e = block_exp(amax);
-            const float inv = pow2i(-e);
+            const float inv = keep * pow2i(-e);
 #pragma unroll
             for (int i = 0; i < 32; ++i) x[i] *= inv;
             uint32_t first_term[8];  // the rope step: term 0's codes, until term 1's join them
@@ -234,12 +245,11 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
 
     // ---- where the wave's rows of a tile are: lanes 0..kWaveRows-1 resolve one each -------------
     constexpr unsigned long long kNone = ~0ull;
-    const unsigned int* const rows_g = SPARSE ? a.rows + (size_t)seq * a.k : nullptr;
-    auto resolve = [&](int t, unsigned long long& code_off, unsigned long long& scale_off) {
+    auto resolve = [&](int t, unsigned int entry, unsigned long long& code_off, unsigned long long& scale_off) {
         code_off = kNone, scale_off = 0;
         const int pos = r_begin + t * TILE + kWaveRows * wave + lane;
         if (lane >= kWaveRows || t >= n_tiles || pos >= r_end) return;
-        const unsigned int tok = SPARSE ? rows_g[pos] : (unsigned)pos;
+        const unsigned int tok = SPARSE ? entry : (unsigned)pos;
         unsigned int blk, off;
         if (a.page_shift >= 0) blk = tok >> a.page_shift, off = tok & (unsigned)(a.page_tokens - 1);
         else blk = tok / (unsigned)a.page_tokens, off = tok - blk * (unsigned)a.page_tokens;
@@ -252,16 +262,15 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             atomicAdd(a.bad_rows, 1u);
         }
     };
-    // A tile goes from memory straight into LDS (16 bytes per lane, a wave's 64 lanes filling
-    // 1 KiB of consecutive LDS). The wave's rows of 37 granules (36 of codes + the padding one)
-    // are that consecutive range, so lane L of request I fills granule 64 I + L = row
-    // (64 I + L) / 37, granule (64 I + L) % 37 of the row, from wherever that row's page is. A row
-    // that is not there is zero-filled by hand: its codes must be finite, they meet a zero weight
-    // and a -inf bias, never a NaN.
+    // A tile goes from memory straight into LDS, 16 bytes per lane, a request's lanes filling
+    // consecutive LDS. The wave's rows of 37 granules (36 of codes + the padding one) are one
+    // consecutive range of the tile. A row that is not there is zero-filled by hand: its codes
+    // must be finite, they meet a zero weight and a -inf bias, never a NaN.
     float next_scale = 0.0f;  // lanes 0..kWaveRows-1: the scale of the row this lane resolved
     // Dense fast path: the wave's rows of a tile are consecutive rows of one page (tiles start
-    // on multiples of 32 tokens and the page holds a multiple of the wave's share), so granule
-    // 64 i + lane comes from byte goff[i] past the first of them: no lookups, one request per 1 KiB.
+    // on multiples of 32 tokens and the page holds a multiple of the wave's share), so lane L of
+    // request i fills granule 64 i + L = row (64 i + L) / 37, granule (64 i + L) % 37 of the row,
+    // from byte goff[i] past the first row: no lookups, one request per 1 KiB.
     int goff[kRequests];
 #pragma unroll
     for (int i = 0; i < kRequests; ++i) {
@@ -275,12 +284,10 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         if (kWave * (i + 1) <= kWaveRows * kF8RowGranules || lane < kWaveRows * kF8RowGranules - kWave * i)
             dma16_from(run, (uint32_t)goff[i], dst_tile + (kWaveRows * wave) * kF8RowBytes + 1024 * i);
     };
-    // Tile t on its way into dst_tile. Returns the run's address when the tile is one (then
-    // `spread` leaves the requests to the caller, who issues them one at a time between other
-    // work: more than about forty transfers in flight per compute unit and each further
-    // request holds its wave until one of them has landed), nullptr when everything was
-    // requested here.
-    auto request_tile = [&](int t, lds_ptr<uint8_t> dst_tile, bool spread) -> const uint8_t* {
+    // Tile t on its way into dst_tile. Returns the run's address when the tile is one and
+    // `spread` leaves the requests to the caller (who issues them between the score units: a
+    // little faster than one burst), nullptr when everything was requested here.
+    auto request_tile = [&](int t, unsigned int entry, lds_ptr<uint8_t> dst_tile, bool spread) -> const uint8_t* {
         const lds_ptr<uint8_t> dst_w = dst_tile + (kWaveRows * wave) * kF8RowBytes;
         if (pages_hold_runs) {
             const int pos0 = r_begin + t * TILE + kWaveRows * wave;
@@ -300,27 +307,24 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
                 }
             }
         }
+        // General path: a request per row, 37 lanes of 16 bytes from the row's own address (held by
+        // the lane that resolved it, handed over as a scalar: one page per request, no address
+        // arithmetic per lane). A row that is not there is zero-filled by hand.
         unsigned long long code_off, scale_off;
-        resolve(t, code_off, scale_off);
-        if (lane < kWaveRows) rowbase[kWaveRows * wave + lane] = code_off;
+        resolve(t, entry, code_off, scale_off);
         next_scale = 0.0f;
         if (code_off != kNone) next_scale = *reinterpret_cast<const float*>(a.pool + scale_off);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-        const lds_ptr<uint8_t> dst0 = dst_w;
+        const uint32_t granule = (uint32_t)min(lane, kRowW / 16 - 1) * 16u;  // (the padding granule repeats the one before it)
 #pragma unroll
-        for (int i = 0; i < kRequests; ++i) {
-            int ln = lane;
-            asm volatile("" : "+v"(ln));  // (kept out of the registers that live across the tile loop)
-            const int gi = kWave * i + ln;
-            const int row = gi / kF8RowGranules, c = gi - row * kF8RowGranules;
-            if (row < kWaveRows && c < kRowW / 16) {
-                const unsigned long long base = rowbase[kWaveRows * wave + row];
-                if (base != kNone) {
-                    dma16(a.pool + base + 16 * c, dst0 + 1024 * i);
-                } else {
-                    *(lds_ptr<u32x4>)(dst0 + 16 * (kWave * i + lane)) = u32x4{0, 0, 0, 0};
-                }
+        for (int r = 0; r < kWaveRows; ++r) {
+            const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)code_off, r);
+            const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(code_off >> 32), r);
+            const lds_ptr<uint8_t> dst_r = dst_w + r * kF8RowBytes;
+            if ((lo & hi) != 0xffffffffu) {
+                if (lane < kF8RowGranules)
+                    dma16_from(a.pool + (((unsigned long long)hi << 32) | lo), granule, dst_r);
+            } else if (lane < kF8RowGranules) {
+                *(lds_ptr<u32x4>)(dst_r + 16 * lane) = u32x4{0, 0, 0, 0};
             }
         }
         return nullptr;
@@ -363,7 +367,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
     float m_ref = -INFINITY, l_sum = 0.0f;
 
     // prologue: tile 0 into LDS
-    request_tile(0, tiles, false);
+    request_tile(0, entry_now, tiles, false);
     publish_scales(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -407,7 +411,8 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         // its requests runs while the first fragments above come out of LDS
         constexpr int kPerUnit = 2;  // requests behind each of the first units
         static_assert(kUnits * kPerUnit >= kRequests, "the units take every request");
-        const uint8_t* const run = t + 1 < n_tiles ? request_tile(t + 1, next, true) : nullptr;
+        const uint8_t* const run = t + 1 < n_tiles ? request_tile(t + 1, entry_next, next, true) : nullptr;
+        if constexpr (SPARSE) entry_next = list_entry(t + 2);
 #pragma unroll
         for (int u = 0; u < kUnits; ++u) {
             __builtin_amdgcn_s_waitcnt(kWaitLds0);  // this unit's fragments are in
