@@ -80,14 +80,33 @@ __device__ __forceinline__ int block_exp(float amax) {
     const int e = (int)((__float_as_uint(amax) >> 23) & 0xffu) - 127 - 7;
     return amax > 0.0f ? max(min(e, 100), -100) : 0;  // (a tile of vanishing weights keeps a scale whose finer terms still exist)
 }
-// x[0..3] (already divided by the block scale) -> four e4m3 codes, and x -= their values.
-__device__ __forceinline__ uint32_t e4m3x4_and_residual(float (&x)[4]) {
-    int w = 0;
-    w = __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], w, false);
-    w = __builtin_amdgcn_cvt_pk_fp8_f32(x[2], x[3], w, true);
-    const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
-    x[0] -= lo[0], x[1] -= lo[1], x[2] -= hi[0], x[3] -= hi[1];
-    return (uint32_t)w;
+// x[0..3] (already divided by the block scale) -> four e4m3 codes of x * 16^T, the T-th term of
+// a sum whose terms are 16 times finer each; val[i] = what the codes stand for (their values /
+// 16^T) and x -= val. Terms past the first use the scaled conversions (the instruction divides
+// by a power of two on the way in and multiplies on the way out: no multiplies of our own).
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+template <int T>
+__device__ __forceinline__ uint32_t e4m3x4_term(float (&x)[4], float (&val)[4]) {
+    uint32_t u;
+    if constexpr (T == 0) {
+        int w = 0;
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], w, false);
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(x[2], x[3], w, true);
+        const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+        val[0] = lo[0], val[1] = lo[1], val[2] = hi[0], val[3] = hi[1];
+        u = (uint32_t)w;
+    } else {
+        constexpr float kFiner = T == 1 ? 0.0625f : T == 2 ? 0.00390625f : 0.000244140625f;
+        static_assert(T <= 3, "up to four terms");
+        i16x2 w = {0, 0};
+        w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w, x[0], x[1], kFiner, false);
+        w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w, x[2], x[3], kFiner, true);
+        u = ((uint32_t)(uint16_t)w[1] << 16) | (uint16_t)w[0];
+        const auto lo = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(u, kFiner, false), hi = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(u, kFiner, true);
+        val[0] = lo[0], val[1] = lo[1], val[2] = hi[0], val[3] = hi[1];
+    }
+    x[0] -= val[0], x[1] -= val[1], x[2] -= val[2], x[3] -= val[3];
+    return u;
 }
 
 // Sixteen bytes per lane from memory straight into LDS: lane L's land at dst + 16 L (dst is
@@ -214,8 +233,8 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             for (int t = 0; t < TQ; ++t) {
 #pragma unroll
                 for (int c = 0; c < 8; ++c) {
-                    float y[4] = {x[4 * c], x[4 * c + 1], x[4 * c + 2], x[4 * c + 3]};
-                    uint32_t w4 = e4m3x4_and_residual(y);
+                    float y[4] = {x[4 * c], x[4 * c + 1], x[4 * c + 2], x[4 * c + 3]}, val[4];
+                    uint32_t w4 = t == 0 ? e4m3x4_term<0>(y, val) : t == 1 ? e4m3x4_term<1>(y, val) : e4m3x4_term<2>(y, val);
                     if (s == 4 && t == 0) first_term[c] = w4;
                     if (s == 4 && t == 1) w4 = g < 2 ? first_term[c] : w4;
                     if (s == 4 && t >= 2 && t < TQR) w4 = g < 2 ? w4 : 0u;  // half-empty: zeros in lane groups 2 and 3
@@ -225,9 +244,8 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
                         qt[s == 4 && t == 1 ? 0 : t][s][c] = qa;
                     } else if (t >= TQR && (s < 4 || g < 2))
                         *(lds_ptr<uint32_t>)(qlds + ((t - TQR) * 64 + 16 * wave + n16) * kF8RowBytes + 128 * s + 32 * g + 4 * c) = w4;
-                    // what is left over, at the next term's scale (16 times finer)
-                    x[4 * c] = y[0] * 16.0f, x[4 * c + 1] = y[1] * 16.0f, x[4 * c + 2] = y[2] * 16.0f,
-                    x[4 * c + 3] = y[3] * 16.0f;
+                    // what is left over, for the next term
+                    x[4 * c] = y[0], x[4 * c + 1] = y[1], x[4 * c + 2] = y[2], x[4 * c + 3] = y[3];
                 }
                 const int byte = max(e - 4 * t + 127, 1);
                 if (s < 4) qscale_lo[t] = (qscale_lo[t] & ~(0xff << (8 * s))) | (byte << (8 * s));
@@ -529,13 +547,11 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
         float l_tile = 0.0f;  // in units of 2^pe
 #pragma unroll
         for (int mb = 0; mb < kRowBlocks; ++mb) {
-            float y[4];
+            float y[4], val[4], back[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) y[i] = acc[mb][i] = __builtin_amdgcn_exp2f(acc[mb][i] - shift);  // not there -> 0
-            const int first = (int)e4m3x4_and_residual(y);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) y[i] *= 16.0f;
-            const int second = (int)e4m3x4_and_residual(y);
+            for (int i = 0; i < 4; ++i) y[i] = __builtin_amdgcn_exp2f(acc[mb][i] - shift);  // not there -> 0
+            const int first = (int)e4m3x4_term<0>(y, val);
+            const int second = (int)e4m3x4_term<1>(y, back);
             if constexpr (TILE == 128) pt[0][mb] = first, pt[1][mb] = second;
             else pt[0][mb] = first, pt[0][4 + mb] = second;
             // The denominator sums the weights the numerator really holds (w_t less the last
@@ -543,7 +559,7 @@ __device__ __forceinline__ void attend_part_f8(const AttendArgs& a, int seq, int
             // weights perturbed by 2^-8 each.
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float held = __builtin_fmaf(y[i], -0.0625f, acc[mb][i]);  // 0 for a token that is not there
+                const float held = val[i] + back[i];  // 0 for a token that is not there
                 l_tile = __builtin_fmaf(held, r4[mb][i], l_tile);
             }
         }
