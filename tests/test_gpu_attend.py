@@ -136,12 +136,12 @@ def test_more_sequences_than_the_dealing_plan_holds(oracle):
 
 
 @pytest.mark.parametrize("precise", [2, 4, 3])
-@pytest.mark.parametrize("pt", [16, 48, 128, 4])
+@pytest.mark.parametrize("pt", [16, 32, 48, 128, 4])
 def test_other_page_sizes(oracle, pt, precise):
-    """Pages of 128 tokens keep the one-lookup-per-tile path; 16 (smaller than a tile), 48 (not
-    a power of two) and 4 take the per-token lookup. Dense and row lists. (In the 8-bit modes a
-    wave brings in 16 consecutive rows at a time: pages of 16 and 128 keep that path, 48 and 4
-    resolve every row on its own.)"""
+    """Pages of 128 tokens keep the one-lookup-per-tile path; 16 and 32 (smaller than a tile), 48
+    (not a power of two) and 4 take the per-token lookup. Dense and row lists. (In the 8-bit
+    modes a wave brings in 32 consecutive rows of a dense tile at a time: pages of 32 and 128
+    keep that path, 16, 48 and 4 resolve every row on its own, as listed rows always do.)"""
     lens = [700, 33, 1300]
     c = paged_case(oracle, lens, H=64, seed=700 + pt, page_tokens=pt)
     want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], c["lens"], None, None,
@@ -191,7 +191,8 @@ def test_peaked_softmax(oracle):
     check(run_paged(c, 3000), want, 2, "peaked", tight_bound=False)
 
 
-def test_sparse_rows(oracle):
+@pytest.mark.parametrize("precise", [2, 4])
+def test_sparse_rows(oracle, precise):
     """The DSA selection: ascending row lists, ragged through n_rows, over fragmented pages."""
     lens = [5000, 3000, 2100]
     c = paged_case(oracle, lens, H=64, seed=400)
@@ -203,17 +204,42 @@ def test_sparse_rows(oracle):
         rows[s] = np.sort(rng.choice(lens[s], k, replace=False))
     want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], None, rows, n_rows,
                                    KVL, ROPE, PT, c["scale"], n_threads=3)
-    got = run_paged(c, k, rows=rows, n_rows=n_rows, use_lens=False)
-    check(got, want, 2, "sparse")
+    got = run_paged(c, k, rows=rows, n_rows=n_rows, use_lens=False, precise=precise)
+    check(got, want, precise, "sparse")
     assert not got[2].any()
     # without n_rows every sequence attends all k rows; an unsorted list is the same softmax
     want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], None, rows, None,
                                    KVL, ROPE, PT, c["scale"], n_threads=3)
-    check(run_paged(c, k, rows=rows, use_lens=False), want, 2, "sparse, all k")
+    check(run_paged(c, k, rows=rows, use_lens=False, precise=precise), want, precise, "sparse, all k")
     shuffled = rows.copy()
     for s in range(3):
         rng.shuffle(shuffled[s])
-    check(run_paged(c, k, rows=shuffled, use_lens=False), want, 2, "sparse, shuffled rows")
+    check(run_paged(c, k, rows=shuffled, use_lens=False, precise=precise), want, precise, "sparse, shuffled rows")
+
+
+@pytest.mark.parametrize("precise", [2, 4])
+def test_listed_rows_in_a_missing_page_are_left_out_and_counted(oracle, precise):
+    """A row list that names tokens of a page the table does not have: those rows take no part
+    (the softmax runs over the others) and are counted once each."""
+    c = paged_case(oracle, [600, 600], H=64, seed=620)
+    table = c["table"].copy()
+    table[0, 3] = -1                                     # tokens 192..255 of sequence 0
+    table[1, 0] = c["n_pages"] + 1                       # tokens 0..63 of sequence 1
+    rng = np.random.default_rng(62)
+    k = 200
+    rows = np.stack([np.sort(rng.choice(600, k, replace=False)) for _ in range(2)]).astype(np.uint32)
+    gone = [(rows[0] >= 192) & (rows[0] < 256), rows[1] < 64]
+    assert gone[0].any() and gone[1].any()
+    want = []
+    for s in range(2):
+        keep = rows[s][~gone[s]]
+        want.append(oracle.mla_attend_paged(c["qabs"][s:s + 1], c["qrope"][s:s + 1], c["pool"], c["table"][s:s + 1],
+                                            None, keep[None, :], None, KVL, ROPE, PT, c["scale"]))
+    bad = dzeros(4)
+    got = run_paged(dict(c, table=table), k, rows=rows, use_lens=False, bad=bad, precise=precise)
+    for s in range(2):
+        check(got[s:s + 1], want[s], precise, f"sequence {s}")
+    assert back(bad, np.uint32)[0] == int(gone[0].sum() + gone[1].sum())
 
 
 def test_sparse_equals_dense_on_the_full_row_list(oracle):
@@ -226,7 +252,8 @@ def test_sparse_equals_dense_on_the_full_row_list(oracle):
     assert np.array_equal(dense.view(np.uint32), run_paged(c, 1000).view(np.uint32))   # and repeatable
 
 
-def test_bad_pages_are_left_out_and_counted(oracle):
+@pytest.mark.parametrize("precise", [2, 4])
+def test_bad_pages_are_left_out_and_counted(oracle, precise):
     c = paged_case(oracle, [200, 200], H=64, seed=600)
     table = c["table"].copy()
     table[1, 1] = c["n_pages"] + 5                      # tokens 64..127 of sequence 1 are not there
@@ -237,13 +264,14 @@ def test_bad_pages_are_left_out_and_counted(oracle):
                                     None, None, KVL, ROPE, PT, c["scale"])
     bad = dzeros(4)
     c2 = dict(c, table=table)
-    got = run_paged(c2, 200, bad=bad)
-    check(got[:1], want0, 2, "untouched sequence")
-    check(got[1:], want1, 2, "sequence with a missing page")
+    got = run_paged(c2, 200, bad=bad, precise=precise)
+    check(got[:1], want0, precise, "untouched sequence")
+    check(got[1:], want1, precise, "sequence with a missing page")
     assert back(bad, np.uint32)[0] == 64
 
 
-def test_lengths_past_the_block_table_are_left_out_and_counted(oracle):
+@pytest.mark.parametrize("precise", [2, 4])
+def test_lengths_past_the_block_table_are_left_out_and_counted(oracle, precise):
     """A length that claims more rows than the block table can address (4 blocks = 256 rows
     here): the rows past the table are skipped and counted, the neighbouring sequence's table
     row is never used in their place, and nothing past the table is read."""
@@ -252,8 +280,8 @@ def test_lengths_past_the_block_table_are_left_out_and_counted(oracle):
     want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], c["lens"], None, None,
                                    KVL, ROPE, PT, c["scale"])
     bad = dzeros(4)
-    got = run_paged(dict(c, lens=np.array([300, 300], np.int32)), 300, bad=bad)
-    check(got, want, 2, "rows past the table")
+    got = run_paged(dict(c, lens=np.array([300, 300], np.int32)), 300, bad=bad, precise=precise)
+    check(got, want, precise, "rows past the table")
     assert back(bad, np.uint32)[0] == 2 * (300 - 256)
 
 
