@@ -200,6 +200,20 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
         stage(raw, 0);
         if (n_tiles > 1) stage(second, 1);
     }
+    // A query that is bf16-valued (the model's is: its rotary stores bf16, crates/backend/kernels/
+    // mla.hip:432) has no remainder: its lo fragments are zeros, their products exact zeros, and
+    // the wave leaves those matrix instructions out — a quarter of the kernel's — with the same
+    // sums to the bit.
+    bool q_has_lo = false;
+    if (QSPLIT == 2) {
+        uint32_t any = 0;
+#pragma unroll
+        for (int j = 0; j < kGaKStepsHalf; ++j) {
+            const u32x4 w = __builtin_bit_cast(u32x4, ql[j]);
+            any |= w.x | w.y | w.z | w.w;
+        }
+        q_has_lo = __builtin_amdgcn_ballot_w64((any & 0x7fff7fffu) != 0) != 0;
+    }
     if (n_tiles > 2) issue_loads(raw, list_entry(2, f2));
     int entry_next = list_entry(3, f3);
     __syncthreads();
@@ -243,9 +257,17 @@ __global__ __launch_bounds__(kGaThreads) void gather_attn_d512_kernel(const Gath
                 const int j = j0 + i;
                 s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[cur][i], qh[j], s0, 0, 0, 0);
                 s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[cur][i], qh[j], s1, 0, 0, 0);
-                if (QSPLIT == 2) {
-                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[cur][i], ql[j], s0, 0, 0, 0);
-                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[cur][i], ql[j], s1, 0, 0, 0);
+            }
+            if (QSPLIT == 2) {
+                // (the sums are used here so that the products above stay in front of the branch)
+                asm volatile("" : "+v"(s0), "+v"(s1));
+                if (q_has_lo) {
+#pragma unroll
+                    for (int i = 0; i < kFragBlock; ++i) {
+                        const int j = j0 + i;
+                        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa0[cur][i], ql[j], s0, 0, 0, 0);
+                        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa1[cur][i], ql[j], s1, 0, 0, 0);
+                    }
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
