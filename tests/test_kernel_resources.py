@@ -1,7 +1,7 @@
 """Register budgets that are part of a kernel's design, held to the build's own resource report.
 
 The 8-bit attention kernels' register budget is part of their design: one wave per SIMD with
-the whole register file, 128 accumulators in ordinary registers, two q terms in the accumulation
+the whole register file, 128 accumulators in ordinary registers, the q terms in the accumulation
 registers (rivoli_amd/csrc/mla_attend_f8.hpp). A compiler or source change that makes them spill
 still gives right answers, only several times slower, so the build's own resource report is held
 to "no scratch memory" here. The scored block selection keeps a row's keys in registers and its
