@@ -145,9 +145,11 @@ def main():
               ("attend_decode", "attend", dict(precise=4)),
               ("attend_decode_bf16x2", "attend", dict(precise=2)),
               # the second cache format's own operators, at prefill
-              ("v4_prefill_32768", "v4", dict(tokens=32768)),
-              ("v4_attend_prefill_8192", "v4_attend", dict(tokens=8192, precise=2)),
-              ("v4_index_prefill_4096", "v4_index", dict(tokens=4096)))
+              # (one layer a step, a millisecond or so: more steps than the default three, so that
+              # the first launches' cold caches do not set the figure)
+              ("v4_prefill_32768", "v4", dict(tokens=32768, steps=20, warmup=3)),
+              ("v4_attend_prefill_8192", "v4_attend", dict(tokens=8192, precise=2, steps=20, warmup=3)),
+              ("v4_index_prefill_4096", "v4_index", dict(tokens=4096, steps=20, warmup=3)))
     res["configs"] = {}
     for name, workload, over in others:
         torch.cuda.empty_cache()
