@@ -58,6 +58,19 @@ def test_dense_ragged_batch(oracle, precise):
     check(run_paged(c, 300, precise=precise), want, precise, "ragged batch, no outliers", mild=True)
 
 
+@pytest.mark.parametrize("precise", [4, 3])
+def test_lengths_around_the_tile_and_run_sizes_of_the_eight_bit_modes(oracle, precise):
+    """Dense rows move in 128-token tiles, a wave's share of a tile is a run of 32 rows of one
+    page: lengths one short of, at and one past 32, 64, 96, 128, 256 and 384, in one batch (a
+    partial last tile, a run cut short by the sequence's end, a tile of which one wave has
+    nothing)."""
+    lens = [31, 32, 33, 63, 64, 65, 95, 96, 97, 127, 128, 129, 255, 256, 257, 383, 384, 385]
+    c = paged_case(oracle, lens, H=64, seed=130, outlier_frac=0.0)
+    want = oracle.mla_attend_paged(c["qabs"], c["qrope"], c["pool"], c["table"], c["lens"], None, None,
+                                   KVL, ROPE, PT, c["scale"], n_threads=8)
+    check(run_paged(c, max(lens), precise=precise), want, precise, "lengths around tile sizes", mild=precise == 4)
+
+
 @pytest.mark.parametrize("lens,H", [([4608], 64), ([5000, 704, 2049], 64), ([1500, 130], 20), ([900], 128),
                                     ([700, 650], 80), ([333, 1, 2100], 1), ([40, 777], 4)])
 def test_dense_split_regimes_and_head_counts(oracle, lens, H):
