@@ -57,6 +57,27 @@ def test_matrix_core_kernel_matches_oracle(oracle, m, h, topk, rows, cache_like,
             float(np.max(np.abs(got - exact)))
 
 
+def test_queries_with_and_without_a_bf16_remainder_in_one_call(oracle):
+    """A wave whose 16 heads x 256 dims of q are bf16 values leaves the remainder's products out;
+    its partner on the other half of the dims, or its neighbour on other heads, may not. Heads 5
+    and 40 get a remainder on dims 0..255 only, head 20 on all dims, query 1 on every head."""
+    d, m, h, topk, rows = 512, 3, 64, 200, 300
+    q, kv, sink = attend_inputs(oracle, m, h, d, rows, seed=77, cache_like=True)
+    rng = np.random.default_rng(7)
+    noise = (rng.standard_normal(q.shape) * 2.0 ** -12).astype(np.float32)
+    q = q.copy()
+    q[0, 5, :256] += noise[0, 5, :256]
+    q[0, 40, :256] += noise[0, 40, :256]
+    q[0, 20] += noise[0, 20]
+    q[1] += noise[1]
+    idx = random_lists(rng, m, topk, rows)
+    exact = sparse_attn_f64(q, kv, sink, idx, d ** -0.5)
+    got = device_attend(q, kv, sink, idx, d ** -0.5, precise=2)
+    assert worst_rel(got, oracle.sparse_attn(q, kv, sink, idx, d ** -0.5)) <= ATTEND_TOL
+    assert np.all(np.abs(got - exact) <= 2.0 ** -8 * np.abs(exact) + 2.0 ** -10 * np.abs(exact).max()), \
+        float(np.max(np.abs(got - exact)))
+
+
 def test_peaked_and_flat_softmax(oracle):
     """Logits far apart (one slot holds the whole softmax; the lazily moved maximum must move)
     and logits all equal."""
